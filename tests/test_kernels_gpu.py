@@ -1,0 +1,409 @@
+"""Each HIP kernel alone against a plain float64 reference, at sizes other than the
+engine's: odd widths, head sizes in steps of 16, page sizes 8/16/32, far keys,
+a window's edge.  Vectors marked (ref) are the ones the reference's own tests hold."""
+import math
+
+import pytest
+import torch
+
+import plain_llama as plain
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def ops():
+    from tiny_llm_amd.kernels import ops as o
+    return o
+
+
+def tol(dtype, f32=1e-5, bf16=1.2e-2):
+    return f32 if dtype == torch.float32 else bf16
+
+
+def rel(got, ref):
+    got, ref = got.double().cpu(), ref.double().cpu()
+    return float((got - ref).abs().max() / ref.abs().max().clamp_min(1e-30))
+
+
+# ------------------------------------------------------------------- embedding
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embedding_rows(dtype):
+    # (ref) tests/ops/cuda/test_embedding.cpp:19-43: rows 2,3,1,7,9,0 of a table of width 2011
+    table = (torch.arange(10 * 2011, dtype=torch.float32).reshape(10, 2011) % 97 / 97).to(dtype).to(DEV)
+    ids = torch.tensor([2, 3, 1, 7, 9, 0], dtype=torch.int32, device=DEV)
+    out = torch.empty(6, 2011, dtype=torch.float32, device=DEV)
+    ops().embedding(ids, table, out)
+    assert torch.equal(out.cpu(), table.float().cpu()[ids.cpu().long()])
+
+
+# --------------------------------------------------------------------- rmsnorm
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden", [241, 64, 2048, 5120])
+def test_rmsnorm(dtype, hidden):
+    # width 241 and eps 1.192e-7 as in tests/ops/cuda/test_norm.cpp:8-47
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(23, hidden, generator=g) * 3
+    w = (1 + 0.1 * torch.randn(hidden, generator=g))
+    for wdt in (torch.float32, dtype):
+        out = torch.empty(23, hidden, dtype=dtype, device=DEV)
+        ops().rmsnorm(x.to(DEV), w.to(wdt).to(DEV), 1.192e-7, out)
+        ref = plain.rms_norm(x.double(), w.to(wdt).double(), 1.192e-7)
+        assert rel(out, ref) < tol(dtype, 2e-6, 5e-3)
+
+
+def test_rmsnorm_gathers_rows():
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(10, 96, generator=g)
+    w = torch.randn(96, generator=g)
+    rows = torch.tensor([9, 0, 4], dtype=torch.int32, device=DEV)
+    out = torch.empty(3, 96, dtype=torch.float32, device=DEV)
+    ops().rmsnorm(x.to(DEV), w.to(DEV), 1e-5, out, rows)
+    ref = plain.rms_norm(x.double()[[9, 0, 4]], w.double(), 1e-5)
+    assert rel(out, ref) < 2e-6
+
+
+def test_rmsnorm_reduces_to_library_routine():
+    x = torch.randn(5, 128, generator=torch.Generator().manual_seed(3))
+    out = torch.empty(5, 128, dtype=torch.float32, device=DEV)
+    ops().rmsnorm(x.to(DEV), torch.ones(128, device=DEV), 1e-6, out)
+    ref = torch.nn.functional.rms_norm(x.double(), (128,), eps=1e-6)
+    assert rel(out, ref) < 2e-6
+
+
+# ---------------------------------------------------------------------- linear
+def test_linear_reference_vectors():
+    # (ref) tests/ops/cuda/test_gemm.cpp:8-40
+    a = torch.tensor([[0., 1, 2], [3, 4, 5]], device=DEV)
+    w = torch.arange(12, dtype=torch.float32, device=DEV).reshape(4, 3)
+    out = torch.empty(2, 4, device=DEV)
+    ops().linear(a, w, out)
+    assert out.cpu().tolist() == [[5, 14, 23, 32], [14, 50, 86, 122]]
+    # one row (the reference's q == 1 path) gives the same numbers
+    out1 = torch.empty(1, 4, device=DEV)
+    ops().linear(a[1:2], w, out1)
+    assert out1.cpu().tolist() == [[14, 50, 86, 122]]
+
+
+def test_lm_head_last_rows_reference_vector():
+    # (ref) tests/runtime/cuda/test_linear_runtime.cpp:332-387: rows 1, 4, 9 of a [10, 3] ramp
+    x = torch.arange(30, dtype=torch.float32, device=DEV).reshape(10, 3)
+    w = torch.tensor([[0., 1, 2], [3, 4, 5]], device=DEV)
+    rows = x[[1, 4, 9]].contiguous()
+    out = torch.empty(3, 2, device=DEV)
+    ops().linear(rows, w, out)
+    assert out.cpu().tolist() == [[14, 50], [41, 158], [86, 338]]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,K,N", [(127, 255, 353), (1, 64, 251), (7, 176, 64), (130, 96, 517), (64, 2048, 256),
+                                   (300, 5632, 136)])
+def test_linear_sizes(dtype, M, K, N):
+    if dtype == torch.bfloat16 and K % 8:
+        K = K + 8 - K % 8
+    g = torch.Generator().manual_seed(M * 1000 + N)
+    a = torch.randn(M, K, generator=g).to(dtype)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(dtype)
+    res = torch.randn(M, N, generator=g)
+    ref = a.double() @ w.double().T
+    for out_dtype in {dtype, torch.float32}:
+        out = torch.empty(M, N, dtype=out_dtype, device=DEV)
+        ops().linear(a.to(DEV), w.to(DEV), out)
+        assert rel(out, ref) < (1e-5 if out_dtype == torch.float32 and dtype == torch.float32 else
+                                1e-5 if out_dtype == torch.float32 else 6e-3)
+    out = torch.empty(M, N, dtype=torch.float32, device=DEV)
+    ops().linear(a.to(DEV), w.to(DEV), out, res.to(DEV))
+    assert rel(out, ref + res.double()) < 1e-5
+    # in place on the residual, as the blocks use it
+    x = res.clone().to(DEV)
+    ops().linear(a.to(DEV), w.to(DEV), x, x)
+    assert rel(x, ref + res.double()) < 1e-5
+
+
+def test_linear_row_alone_equals_row_in_batch_fp32():
+    g = torch.Generator().manual_seed(5)
+    a = torch.randn(70, 200, generator=g).to(DEV)
+    w = torch.randn(90, 200, generator=g).to(DEV)
+    full = torch.empty(70, 90, device=DEV)
+    ops().linear(a, w, full)
+    one = torch.empty(1, 90, device=DEV)
+    ops().linear(a[37:38], w, one)
+    assert torch.equal(full[37:38], one)
+
+
+def test_linear_refuses_bad_inner_size_in_bf16():
+    from tiny_llm_amd.kernels import KernelError
+    a = torch.zeros(4, 12, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(8, 12, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(KernelError):
+        ops().linear(a, w, torch.empty(4, 8, dtype=torch.bfloat16, device=DEV))
+
+
+# -------------------------------------------------------------------- silu_mul
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_mul(dtype):
+    # (ref) tests/ops/cuda/test_silu.cpp:8-28: silu(0) = 0, silu(1) = 1 / (1 + e^-1)
+    gu = torch.tensor([[0., 1., -2., 2., 3., 0.5]], dtype=dtype, device=DEV)
+    out = torch.empty(1, 3, dtype=dtype, device=DEV)
+    ops().silu_mul(gu, out)
+    ref = torch.tensor([[0.0, 1 / (1 + math.exp(-1)) * 3, -2 / (1 + math.exp(2)) * 0.5]])
+    assert rel(out, ref) < tol(dtype, 1e-6, 4e-3)
+    g = torch.Generator().manual_seed(7)
+    gu = torch.randn(9, 2 * 176, generator=g).to(dtype)
+    out = torch.empty(9, 176, dtype=dtype, device=DEV)
+    ops().silu_mul(gu.to(DEV), out)
+    ref = plain.silu(gu.double()[:, :176]) * gu.double()[:, 176:]
+    assert rel(out, ref) < tol(dtype, 1e-6, 4e-3)
+
+
+# ------------------------------------------------------------------ rope_store
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hd,nq,nkv,bs", [(96, 4, 4, 8), (16, 4, 2, 16), (48, 3, 1, 32), (128, 8, 2, 16)])
+def test_rope_store(dtype, hd, nq, nkv, bs):
+    # head size 96 and base 1e4 as in tests/ops/cuda/test_rope.cpp:8-37; the paged write follows
+    # test_rope.cpp:100-213 (positions deep in a block table, neighbours must stay untouched)
+    from tiny_llm_amd.parts.rotary import RotaryEmbedding
+    T, max_pos, nblocks = 11, 64, 12
+    rot = RotaryEmbedding("r", dtype, DEV, head_dim=hd, theta=10000.0, max_position=max_pos)
+    cos, sin, rd = rot.rotary_tables()
+    pc, ps = plain.rope_table(max_pos, hd, 10000.0)
+    assert torch.equal(cos.cpu().double(), pc) and torch.equal(sin.cpu().double(), ps)
+    g = torch.Generator().manual_seed(11)
+    qkv = torch.randn(T, (nq + 2 * nkv) * hd, generator=g).to(dtype)
+    positions = torch.tensor([0, 1, 2, 3, 4, 5, 6, 40, 41, 17, 63], dtype=torch.int32)
+    slots = torch.tensor([3 * bs + 0, 3 * bs + 1, 3 * bs + 2, 3 * bs + 3, 3 * bs + 4, 3 * bs + 5, 3 * bs + 6,
+                          7 * bs + bs - 1, 9 * bs, 1 * bs + 1, -1], dtype=torch.int32)
+    kc = torch.ones(nblocks, nkv, bs, hd, dtype=dtype, device=DEV)
+    vc = torch.ones(nblocks, nkv, bs, hd, dtype=dtype, device=DEV)
+    dq = qkv.clone().to(DEV)
+    ops().rope_store(dq, positions.to(DEV), cos, sin, slots.to(DEV), kc, vc, nq, nkv, hd, rd)
+    q_ref = plain.apply_rope(qkv.double()[:, :nq * hd].reshape(T, nq, hd), positions.tolist(), pc, ps)
+    k_ref = plain.apply_rope(qkv.double()[:, nq * hd:(nq + nkv) * hd].reshape(T, nkv, hd), positions.tolist(), pc, ps)
+    v_ref = qkv.double()[:, (nq + nkv) * hd:].reshape(T, nkv, hd)
+    t = tol(dtype, 1e-6, 4e-3)
+    assert rel(dq[:, :nq * hd].reshape(T, nq, hd), q_ref) < t
+    exp_k = torch.ones(nblocks, nkv, bs, hd, dtype=torch.float64)
+    exp_v = torch.ones(nblocks, nkv, bs, hd, dtype=torch.float64)
+    for i in range(T):
+        s = int(slots[i])
+        if s < 0:
+            continue
+        exp_k[s // bs, :, s % bs] = k_ref[i].to(dtype).double()
+        exp_v[s // bs, :, s % bs] = v_ref[i]
+    assert rel(kc, exp_k) < t
+    assert torch.equal(vc.cpu().double(), exp_v)
+    untouched = exp_k == 1.0
+    assert torch.equal(kc.cpu().double()[untouched], exp_k[untouched])
+
+
+def test_rope_invariants():
+    """Position 0 is the identity; pair norms are kept; q.k depends only on the distance."""
+    from tiny_llm_amd.parts.rotary import RotaryEmbedding
+    hd = 32
+    rot = RotaryEmbedding("r", torch.float32, DEV, head_dim=hd, theta=500000.0, max_position=512)
+    cos, sin, rd = rot.rotary_tables()
+    g = torch.Generator().manual_seed(13)
+    base = torch.randn(1, 3 * hd, generator=g)     # one q head, one k head, one v head
+
+    def rotated(p):
+        x = base.clone().to(DEV)
+        ops().rope_store(x, torch.tensor([p], dtype=torch.int32, device=DEV), cos, sin, None, None, None, 1, 1, hd, rd)
+        return x.cpu()[0, :hd], x.cpu()[0, hd:2 * hd]
+
+    q0, k0 = rotated(0)
+    assert torch.equal(q0, base[0, :hd]) and torch.equal(k0, base[0, hd:2 * hd])
+    q7, _ = rotated(7)
+    pair = lambda v: v[:hd // 2] ** 2 + v[hd // 2:] ** 2
+    assert torch.allclose(pair(q7), pair(base[0, :hd]), rtol=1e-5, atol=1e-6)
+    dots = []
+    for m, n in [(5, 2), (105, 102), (303, 300)]:
+        qm, _ = rotated(m)
+        _, kn = rotated(n)
+        dots.append(float(qm.double() @ kn.double()))
+    assert abs(dots[0] - dots[1]) < 1e-4 and abs(dots[0] - dots[2]) < 1e-4
+    qa, _ = rotated(9)
+    _, kb = rotated(2)
+    assert abs(float(qa.double() @ kb.double()) - dots[0]) > 1e-3   # another distance, another score
+
+
+# ------------------------------------------------------------- paged attention
+def _paged_case(dtype, lens, q_lens, nq, nkv, hd, bs, window=0, seed=0, boost=None, shuffle=True):
+    """Builds a batch: request r has lens[r] cached tokens, the last q_lens[r] are this step's
+    queries.  Returns engine output and the plain result, both [T, nq, hd]."""
+    g = torch.Generator().manual_seed(seed)
+    R = len(lens)
+    nblocks = sum(-(-l // bs) for l in lens) + 3
+    perm = torch.randperm(nblocks, generator=g).tolist() if shuffle else list(range(nblocks))
+    kc = torch.full((nblocks, nkv, bs, hd), float("nan"), dtype=dtype)
+    vc = torch.full((nblocks, nkv, bs, hd), float("nan"), dtype=dtype)
+    max_blocks = max(-(-l // bs) for l in lens)
+    bt = torch.zeros(R, max_blocks, dtype=torch.int32)
+    qs, refs, req_of, pos = [], [], [], []
+    for r, (L, ql) in enumerate(zip(lens, q_lens)):
+        k = torch.randn(L, nkv, hd, generator=g).to(dtype)
+        v = torch.randn(L, nkv, hd, generator=g).to(dtype)
+        q = torch.randn(L, nq, hd, generator=g).to(dtype)
+        if boost is not None:               # make one far key stand out for the last query
+            far = boost
+            k[far] = 0
+            k[far, :, 0] = 6.0
+            q[L - 1] = 0
+            q[L - 1, :, 0] = 6.0 * math.sqrt(hd) / 6.0 * 3
+        for b in range(-(-L // bs)):
+            blk = perm.pop()
+            bt[r, b] = blk
+            n = min(bs, L - b * bs)
+            kc[blk, :, :n] = k[b * bs:b * bs + n].transpose(0, 1)
+            vc[blk, :, :n] = v[b * bs:b * bs + n].transpose(0, 1)
+        full = plain.attention_fast(q.double(), k.double(), v.double(), list(range(L)), window)
+        qs.append(q[L - ql:])
+        refs.append(full[L - ql:])
+        req_of += [r] * ql
+        pos += list(range(L - ql, L))
+    q = torch.cat(qs).reshape(-1, nq * hd).contiguous()
+    out = torch.empty_like(q).to(DEV)
+    ops().paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), bt.to(DEV),
+                          torch.tensor(req_of, dtype=torch.int32, device=DEV),
+                          torch.tensor(pos, dtype=torch.int32, device=DEV), out, nq, nkv, hd,
+                          1.0 / math.sqrt(hd), window)
+    return out.reshape(-1, nq, hd), torch.cat(refs)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,hd,bs", [(4, 2, 48, 32), (4, 2, 64, 16), (3, 1, 32, 8), (8, 8, 16, 16),
+                                          (6, 2, 80, 16), (2, 1, 128, 64), (5, 5, 112, 8), (2, 2, 256, 16)])
+def test_paged_attention_mixed_batch(dtype, nq, nkv, hd, bs):
+    # shapes after tests/ops/cuda/test_flash_attention.cpp:172-271 (q 107, kv 123, heads 4:2), generalised:
+    # a whole prompt, a portion with earlier context, single decoded tokens, a one-token request
+    out, ref = _paged_case(dtype, lens=[123, 107, 65, 1, 300], q_lens=[123, 40, 1, 1, 1], nq=nq, nkv=nkv,
+                           hd=hd, bs=bs, seed=hd + bs)
+    assert not torch.isnan(out).any()
+    assert rel(out, ref) < tol(dtype, 2e-6, 8e-3)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_paged_attention_far_key_among_hundreds(dtype):
+    # one early key dominates the last query: a kernel that drops or misplaces it shows at once
+    for far in (0, 15, 16, 255, 256, 511):
+        out, ref = _paged_case(dtype, lens=[700], q_lens=[1], nq=4, nkv=2, hd=64, bs=16, seed=far, boost=far)
+        assert rel(out, ref) < tol(dtype, 2e-6, 8e-3), far
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [1, 7, 16, 33])
+def test_paged_attention_window_edge(dtype, window):
+    out, ref = _paged_case(dtype, lens=[90, 40, 64], q_lens=[90, 1, 5], nq=4, nkv=2, hd=32, bs=8,
+                           window=window, seed=window)
+    assert rel(out, ref) < tol(dtype, 2e-6, 8e-3)
+
+
+def test_paged_attention_reduces_to_library_routine():
+    """One request, whole prompt, identity block table: plain causal attention."""
+    nq = nkv = 2
+    hd, L, bs = 64, 50, 16
+    g = torch.Generator().manual_seed(17)
+    q, k, v = (torch.randn(L, nq, hd, generator=g) for _ in range(3))
+    nb = -(-L // bs)
+    kc = torch.zeros(nb, nkv, bs, hd)
+    vc = torch.zeros(nb, nkv, bs, hd)
+    for b in range(nb):
+        n = min(bs, L - b * bs)
+        kc[b, :, :n] = k[b * bs:b * bs + n].transpose(0, 1)
+        vc[b, :, :n] = v[b * bs:b * bs + n].transpose(0, 1)
+    out = torch.empty(L, nq * hd, device=DEV)
+    ops().paged_attention(q.reshape(L, -1).to(DEV), kc.to(DEV), vc.to(DEV),
+                          torch.arange(nb, dtype=torch.int32, device=DEV).reshape(1, nb),
+                          torch.zeros(L, dtype=torch.int32, device=DEV),
+                          torch.arange(L, dtype=torch.int32, device=DEV), out, nq, nkv, hd, hd ** -0.5, 0)
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        q.double().transpose(0, 1), k.double().transpose(0, 1), v.double().transpose(0, 1), is_causal=True)
+    assert rel(out.reshape(L, nq, hd), ref.transpose(0, 1)) < 2e-6
+
+
+# -------------------------------------------------------------------- sampling
+def _sample(logits, **kw):
+    n = logits.shape[0]
+    out = torch.empty(n, dtype=torch.int32, device=DEV)
+    dev = {k: (v.to(DEV) if v is not None else None) for k, v in kw.items()}
+    ops().sample(logits.to(DEV), out, **dev)
+    return out.cpu().tolist()
+
+
+def test_argmax_reference_vector_and_first_maximum():
+    # (ref) tests/logit_processors/test_argmax_processor.cpp:19-31: ramps -> id 19
+    ramps = torch.arange(40, dtype=torch.float32).reshape(2, 20)
+    assert _sample(ramps) == [19, 19]
+    ties = torch.zeros(3, 1000)
+    ties[0, [5, 700]] = 2.0
+    ties[1, 999] = 1.0
+    ties[2] = -1.0
+    assert _sample(ties) == [5, 999, 0]
+    big = torch.randn(4, 32003, generator=torch.Generator().manual_seed(19))
+    assert _sample(big) == big.argmax(dim=1).tolist()
+
+
+def test_sampling_single_finite_logit():
+    # (ref) tests/logit_processors/test_sample_processors.cpp:20-34: one finite logit is always drawn
+    l = torch.full((2, 64), -1e30)
+    l[0, 17] = 0.3
+    l[1, 63] = -2.0
+    got = _sample(l, temperature=torch.tensor([1.0, 0.5]), top_k=torch.tensor([0, 0], dtype=torch.int32),
+                  top_p=torch.tensor([1.0, 1.0]), seeds=torch.tensor([1, 2]), counters=torch.tensor([0, 9], dtype=torch.int32))
+    assert got == [17, 63]
+
+
+def test_sampling_matches_plain_chain():
+    """Temperature -> top-k -> top-p -> multinomial gives the plain chain's token for the same u."""
+    g = torch.Generator().manual_seed(23)
+    cases = []
+    for vocab in (20, 251, 517, 32000):
+        for (t, k, p) in [(0.7, 50, 0.95), (1.0, 0, 1.0), (0.8, 5, 1.0), (1.3, 0, 0.2), (0.5, 1, 0.9),
+                          (1.0, 10, 0.0), (2.0, 0, 0.6)]:
+            cases.append((vocab, t, min(k, vocab), p))
+    mismatches = 0
+    for vocab, t, k, p in cases:
+        n = 12
+        logits = torch.randn(n, vocab, generator=g) * 3
+        seeds = torch.arange(n, dtype=torch.int64) * 7919 + vocab
+        ctrs = torch.arange(n, dtype=torch.int32) + 3
+        got = _sample(logits, temperature=torch.full((n,), t), top_k=torch.full((n,), k, dtype=torch.int32),
+                      top_p=torch.full((n,), p), seeds=seeds, counters=ctrs)
+        for i in range(n):
+            u = plain.uniform_for(int(seeds[i]), int(ctrs[i]))
+            want = plain.sample_token(logits[i], t, k, p, u)
+            if got[i] != want:
+                # allowed only when u sits on a boundary of the cumulative distribution (rounding)
+                near = {plain.sample_token(logits[i], t, k, p, min(max(u + d, 0.0), 0.999999)) for d in (-2e-6, 2e-6)}
+                assert got[i] in near, (vocab, t, k, p, i, got[i], want)
+                mismatches += 1
+    assert mismatches <= 2
+
+
+def test_sampling_top_p_reference_vectors():
+    # (ref) tests/logit_processors/test_sort_processors.cpp:120-200: with logits i/40 and logit[0] = 0.5,
+    # p = 0.2 keeps ids {0, 19, 18, 17}; with logit[0] = 2 it keeps {0, 19}
+    for first, keep in ((0.5, {0, 19, 18, 17}), (2.0, {0, 19})):
+        l = (torch.arange(20, dtype=torch.float32) / 40) + (0.5 if first == 2.0 else 0.0)
+        l[0] = first
+        assert set(plain.top_k_top_p_ids(l, 0, 0.2)) == keep
+        n = 400
+        got = _sample(l.repeat(n, 1), temperature=torch.ones(n), top_k=torch.zeros(n, dtype=torch.int32),
+                      top_p=torch.full((n,), 0.2), seeds=torch.arange(n, dtype=torch.int64),
+                      counters=torch.zeros(n, dtype=torch.int32))
+        assert set(got) == keep
+
+
+def test_sampling_distribution():
+    """Frequencies follow softmax(logits / T) over the kept ids."""
+    l = torch.tensor([2.0, 1.0, 0.0, -1.0, 3.0, 0.5])
+    n = 20000
+    got = _sample(l.repeat(n, 1), temperature=torch.full((n,), 0.8), top_k=torch.full((n,), 4, dtype=torch.int32),
+                  top_p=torch.ones(n), seeds=torch.full((n,), 12345, dtype=torch.int64),
+                  counters=torch.arange(n, dtype=torch.int32))
+    kept = [4, 0, 1, 5]
+    probs = torch.softmax(l[kept].double() / 0.8, 0)
+    counts = torch.tensor([got.count(i) for i in kept], dtype=torch.float64) / n
+    assert set(got) == set(kept)
+    assert (counts - probs).abs().max() < 0.015

@@ -1,0 +1,217 @@
+"""The cache manager: paged keys and values with a block table per request, in
+groups of layers with the same needs, and slots for per-request state of fixed size.
+
+Differences from the reference, which keeps one pool per layer sized so that it can
+never run out and frees everything when the whole batch is done
+(tiny_llm/runtime/cuda/cuda_runtime.cpp:505-526, 683-709, 804-819):
+
+* Layers whose mixers declare the same CacheSpec form a group.  A group has ONE
+  block-id space and one block table per request that serves all its layers; each
+  layer has its own key and value tensor [blocks, kv_heads, block_size, head_dim]
+  indexed by those ids.
+* A "window" group gives a request's blocks back as soon as every position in them
+  is more than `window` behind the next query; a "full" group when the request ends.
+* Blocks that are given back are used again by later growth, most recently freed first.
+* `grow` is all-or-nothing over all groups, so a step that cannot be held changes nothing.
+
+Everything here is host bookkeeping; device tensors are only allocated (by
+`allocate_tensors`) and handed to the mixers as views.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, Hashable, List, Optional, Sequence, Tuple
+
+import torch
+
+from ..parts.base import CacheSpec, LayerCache, StateSpec
+from .block_pool import BlockPool, CacheError, OutOfBlocks
+
+RELEASED = -1
+
+
+class NoFreeSlot(CacheError):
+    pass
+
+
+@dataclass
+class CacheGroup:
+    spec: CacheSpec
+    entries: List[int]                 # plan entries that own a cache in this group
+    pool: BlockPool
+    k: Optional[torch.Tensor] = None   # [len(entries), blocks, kv_heads, block_size, head_dim]
+    v: Optional[torch.Tensor] = None
+
+    @property
+    def bytes_per_block_per_layer(self) -> int:
+        return 0 if self.k is None else 2 * self.k[0, 0].numel() * self.k.element_size()
+
+
+@dataclass
+class RequestCache:
+    slot: int
+    num_tokens: int = 0
+    blocks: List[List[int]] = field(default_factory=list)   # per group: logical block -> id or RELEASED
+
+
+class CacheManager:
+    def __init__(self, cache_specs: Sequence[Optional[CacheSpec]], state_specs: Sequence[Optional[StateSpec]],
+                 block_size: int, num_blocks: int, max_seqs: int):
+        """cache_specs / state_specs: per plan entry, None where the entry has none."""
+        if block_size <= 0:
+            raise ValueError("block_size must be positive")
+        self.block_size = int(block_size)
+        self.num_blocks = int(num_blocks)
+        self.max_seqs = int(max_seqs)
+        self.groups: List[CacheGroup] = []
+        self.group_of_entry: Dict[int, int] = {}
+        self.index_in_group: Dict[int, int] = {}
+        by_key: Dict[Tuple, int] = {}
+        for i, cs in enumerate(cache_specs):
+            if cs is None:
+                continue
+            key = cs.group_key()
+            if key not in by_key:
+                by_key[key] = len(self.groups)
+                self.groups.append(CacheGroup(cs, [], BlockPool(self.num_blocks)))
+            g = by_key[key]
+            self.group_of_entry[i] = g
+            self.index_in_group[i] = len(self.groups[g].entries)
+            self.groups[g].entries.append(i)
+        self.state_specs = list(state_specs)
+        self.states: List[Optional[torch.Tensor]] = [None] * len(self.state_specs)
+        self._free_slots: List[int] = list(range(self.max_seqs - 1, -1, -1))
+        self.requests: Dict[Hashable, RequestCache] = {}
+
+    # ------------------------------------------------------------------- tensors
+    def allocate_tensors(self, dtype: torch.dtype, device) -> None:
+        for g in self.groups:
+            shape = (len(g.entries), self.num_blocks, g.spec.num_kv_heads, self.block_size, g.spec.head_dim)
+            g.k = torch.zeros(shape, dtype=dtype, device=device)
+            g.v = torch.zeros(shape, dtype=dtype, device=device)
+        for i, ss in enumerate(self.state_specs):
+            if ss is not None:
+                self.states[i] = torch.zeros((self.max_seqs, *ss.shape), dtype=ss.dtype, device=device)
+
+    def layer_cache(self, entry: int, cache_of: Optional[int] = None) -> Optional[LayerCache]:
+        """The view a plan entry's mixer gets: its own cache, or (read-only) the cache of `cache_of`."""
+        owner = entry if cache_of is None else cache_of
+        if owner not in self.group_of_entry:
+            return None
+        g = self.group_of_entry[owner]
+        grp = self.groups[g]
+        j = self.index_in_group[owner]
+        return LayerCache(k=grp.k[j], v=grp.v[j], group=g, write=cache_of is None)
+
+    # ------------------------------------------------------------------ requests
+    def has(self, req_id) -> bool:
+        return req_id in self.requests
+
+    @property
+    def free_slots(self) -> int:
+        return len(self._free_slots)
+
+    def add_request(self, req_id) -> int:
+        if req_id in self.requests:
+            raise CacheError(f"request {req_id!r} is already live")
+        if not self._free_slots:
+            raise NoFreeSlot(f"all {self.max_seqs} request slots are taken")
+        slot = self._free_slots.pop()
+        self.requests[req_id] = RequestCache(slot, 0, [[] for _ in self.groups])
+        for st in self.states:
+            if st is not None:
+                st[slot].zero_()
+        return slot
+
+    def num_tokens(self, req_id) -> int:
+        return self.requests[req_id].num_tokens
+
+    def slot(self, req_id) -> int:
+        return self.requests[req_id].slot
+
+    def block_table(self, req_id, group: int) -> List[int]:
+        return self.requests[req_id].blocks[group]
+
+    def _first_needed_block(self, g: CacheGroup, context_len: int) -> int:
+        """Lowest logical block a query at position >= context_len can still read."""
+        if g.spec.kind != "window" or g.spec.window <= 0:
+            return 0
+        first_pos = max(0, context_len - g.spec.window + 1)
+        return first_pos // self.block_size
+
+    def blocks_needed(self, req_id, new_len: int) -> List[int]:
+        """New blocks per group to hold positions up to new_len - 1."""
+        rc = self.requests.get(req_id)
+        have = [len(b) for b in rc.blocks] if rc else [0] * len(self.groups)
+        want = -(-new_len // self.block_size)
+        return [max(0, want - h) for h in have]
+
+    def can_grow(self, needs: Sequence[Sequence[int]]) -> bool:
+        """needs: for several requests, their `blocks_needed`; true if all fit together."""
+        for gi, g in enumerate(self.groups):
+            if sum(n[gi] for n in needs) > g.pool.free_count:
+                return False
+        return True
+
+    def grow(self, req_id, new_len: int) -> None:
+        """Blocks for positions < new_len in every group, or none at all."""
+        rc = self.requests[req_id]
+        if new_len < rc.num_tokens:
+            raise CacheError("a request's cache cannot shrink")
+        need = self.blocks_needed(req_id, new_len)
+        for g, n in zip(self.groups, need):
+            if n > g.pool.free_count:
+                raise OutOfBlocks(f"request {req_id!r} needs {n} more blocks, {g.pool.free_count} are free")
+        for gi, (g, n) in enumerate(zip(self.groups, need)):
+            rc.blocks[gi].extend(g.pool.allocate(n))
+
+    def commit(self, req_id, new_len: int) -> None:
+        """The step has written positions < new_len.  Gives back what a window has passed."""
+        rc = self.requests[req_id]
+        if new_len < rc.num_tokens:
+            raise CacheError("a request's cache cannot shrink")
+        want = -(-new_len // self.block_size)
+        for gi, g in enumerate(self.groups):
+            if len(rc.blocks[gi]) < want:
+                raise CacheError(f"request {req_id!r} commits {new_len} tokens without blocks for them")
+        rc.num_tokens = new_len
+        for gi, g in enumerate(self.groups):
+            first = self._first_needed_block(g, new_len)
+            gone = [b for b in rc.blocks[gi][:first] if b != RELEASED]
+            if gone:
+                g.pool.free(gone)
+                for i in range(first):
+                    rc.blocks[gi][i] = RELEASED
+
+    def free_request(self, req_id) -> None:
+        rc = self.requests.pop(req_id, None)
+        if rc is None:
+            raise CacheError(f"request {req_id!r} is not live")
+        for gi, g in enumerate(self.groups):
+            g.pool.free([b for b in rc.blocks[gi] if b != RELEASED])
+        self._free_slots.append(rc.slot)
+
+    # -------------------------------------------------------------------- checks
+    def free_blocks(self) -> List[int]:
+        return [g.pool.free_count for g in self.groups]
+
+    def audit(self) -> None:
+        """Every block is either free or held by exactly one request; every slot likewise."""
+        for gi, g in enumerate(self.groups):
+            held: Dict[int, Hashable] = {}
+            for rid, rc in self.requests.items():
+                for b in rc.blocks[gi]:
+                    if b == RELEASED:
+                        continue
+                    if b in held:
+                        raise CacheError(f"group {gi}: block {b} is held by {held[b]!r} and {rid!r}")
+                    if g.pool.is_free(b):
+                        raise CacheError(f"group {gi}: block {b} of {rid!r} is on the free list")
+                    held[b] = rid
+            if len(held) + g.pool.free_count != g.pool.num_blocks:
+                raise CacheError(f"group {gi}: {g.pool.num_blocks - len(held) - g.pool.free_count} blocks are lost")
+        slots = [rc.slot for rc in self.requests.values()]
+        if len(set(slots)) != len(slots) or set(slots) & set(self._free_slots):
+            raise CacheError("a state slot is held twice")
+        if len(slots) + len(self._free_slots) != self.max_seqs:
+            raise CacheError("a state slot is lost")

@@ -1,0 +1,192 @@
+// Memory-bound kernels of the step: embedding gather, RMSNorm (with optional
+// row gather), SiLU-gate, residual add, and rotary position encoding fused with
+// the write of keys and values into the paged cache.
+//
+// Formulas follow the reference's kernels: tiny_llm/ops/cuda/embedding.cu:10-29,
+// norm.cu:29-48, silu.cu:10, arithmetic.cu:13, rope.cu:46-54 and 73-93.
+// The residual stream is float32 in both precisions; T is the element type of
+// weights, activations and cache (float or bf16).
+#include "common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / TL_WAVE;
+
+// ------------------------------------------------------------------ embedding
+template <typename T>
+__global__ void embedding_kernel(const int32_t* __restrict__ tokens, const T* __restrict__ table,
+                                 float* __restrict__ out, int hidden, int vocab) {
+  const int t = blockIdx.x;
+  const int tok = tokens[t];
+  float* dst = out + (int64_t)t * hidden;
+  if (tok < 0 || tok >= vocab) {  // ids are checked on the host; poison instead of reading outside
+    for (int j = threadIdx.x; j < hidden; j += kThreads) dst[j] = __builtin_nanf("");
+    return;
+  }
+  const T* src = table + (int64_t)tok * hidden;
+  for (int j = threadIdx.x; j < hidden; j += kThreads) dst[j] = to_f32(src[j]);
+}
+
+// -------------------------------------------------------------------- RMSNorm
+// y = w * x / sqrt(mean(x^2) + eps), statistics in float32.  One workgroup per
+// output row; `rows` (optional) selects the input row of each output row.
+template <typename TW, typename TO>
+__global__ void rmsnorm_kernel(const float* __restrict__ x, const TW* __restrict__ w,
+                               const int32_t* __restrict__ rows, TO* __restrict__ out, int hidden,
+                               float eps) {
+  __shared__ float red[kWaves];
+  const int64_t in_row = rows ? rows[blockIdx.x] : blockIdx.x;
+  const float* src = x + in_row * hidden;
+  float ss = 0.f;
+  for (int j = threadIdx.x; j < hidden; j += kThreads) {
+    const float v = src[j];
+    ss += v * v;
+  }
+  ss = block_sum<kWaves>(ss, red);
+  const float r = sqrtf(ss / (float)hidden + eps);
+  TO* dst = out + (int64_t)blockIdx.x * hidden;
+  for (int j = threadIdx.x; j < hidden; j += kThreads) dst[j] = from_f32<TO>(to_f32(w[j]) * src[j] / r);
+}
+
+// ------------------------------------------------------------------ SiLU-gate
+// z[t, j] = silu(gate_up[t, j]) * gate_up[t, I + j]
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gate_up, T* __restrict__ z, int64_t total, int inter) {
+  const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (i >= total) return;
+  const int64_t t = i / inter;
+  const int j = (int)(i - t * inter);
+  const float g = to_f32(gate_up[t * 2 * inter + j]);
+  const float u = to_f32(gate_up[t * 2 * inter + inter + j]);
+  z[i] = from_f32<T>(g / (1.f + expf(-g)) * u);
+}
+
+// --------------------------------------------------------------- residual add
+template <typename T>
+__global__ void add_residual_kernel(float* __restrict__ x, const T* __restrict__ y, int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (i < total) x[i] += to_f32(y[i]);
+}
+
+// ------------------------------------------------------ rotary + cache write
+// qkv row t = [q heads | k heads | v heads], each head `hd` wide.  The first
+// `rot` dims of every q and k head are rotated in the rotate-half pairing
+// (i, i + rot/2) by the angle table row positions[t]; q is rewritten in place,
+// k (rotated) and v go to the cache slot slot_mapping[t] (a negative slot
+// stores nothing).  Cache layout: [block, kv_head, slot_in_block, hd].
+template <typename T>
+__global__ void rope_store_kernel(T* __restrict__ qkv, const int32_t* __restrict__ positions,
+                                  const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                  const int32_t* __restrict__ slot_mapping, T* __restrict__ k_cache,
+                                  T* __restrict__ v_cache, int nq, int nkv, int hd, int rot,
+                                  int block_size, int64_t row_stride) {
+  const int t = blockIdx.x;
+  const int pos = positions[t];
+  const int half = rot / 2;
+  const int slot = slot_mapping ? slot_mapping[t] : -1;
+  T* row = qkv + (int64_t)t * row_stride;
+  const float* cs = cos_t + (int64_t)pos * half;
+  const float* sn = sin_t + (int64_t)pos * half;
+  const int64_t blk = slot >= 0 ? slot / block_size : 0;
+  const int in_blk = slot >= 0 ? slot % block_size : 0;
+
+  // rotated pairs of q and k heads
+  const int pairs = (nq + nkv) * half;
+  for (int i = threadIdx.x; i < pairs; i += kThreads) {
+    const int head = i / half, j = i - head * half;
+    T* h = row + (int64_t)head * hd;
+    const float a = to_f32(h[j]), b = to_f32(h[j + half]);
+    const float c = cs[j], s = sn[j];
+    const T ra = from_f32<T>(c * a - s * b);
+    const T rb = from_f32<T>(s * a + c * b);
+    if (head < nq) {
+      h[j] = ra;
+      h[j + half] = rb;
+    } else if (slot >= 0) {
+      T* dst = k_cache + ((blk * nkv + (head - nq)) * block_size + in_blk) * hd;
+      dst[j] = ra;
+      dst[j + half] = rb;
+    }
+  }
+  if (slot < 0) return;
+  // dims of k beyond the rotated part, and all of v, are copied as they are
+  const int tail = hd - rot;
+  for (int i = threadIdx.x; i < nkv * tail; i += kThreads) {
+    const int head = i / tail, j = rot + (i - head * tail);
+    k_cache[((blk * nkv + head) * block_size + in_blk) * hd + j] = row[(int64_t)(nq + head) * hd + j];
+  }
+  for (int i = threadIdx.x; i < nkv * hd; i += kThreads) {
+    const int head = i / hd, j = i - head * hd;
+    v_cache[((blk * nkv + head) * block_size + in_blk) * hd + j] = row[(int64_t)(nq + nkv + head) * hd + j];
+  }
+}
+
+}  // namespace
+
+#define TL_DISPATCH_T(dtype, ...)                 \
+  if ((dtype) == 0) { using T = float; __VA_ARGS__ } \
+  else if ((dtype) == 1) { using T = bf16_t; __VA_ARGS__ } \
+  else return TL_ERR_ARG;
+
+extern "C" {
+
+int tl_embedding(const int32_t* tokens, const void* table, float* out, int n_tokens, int hidden,
+                 int vocab, int dtype, hipStream_t stream) {
+  if (n_tokens <= 0) return TL_OK;
+  if (hidden <= 0 || vocab <= 0) return TL_ERR_ARG;
+  TL_DISPATCH_T(dtype, hipLaunchKernelGGL(embedding_kernel<T>, dim3(n_tokens), dim3(kThreads), 0, stream,
+                                          tokens, (const T*)table, out, hidden, vocab);)
+  return tl_launch_status();
+}
+
+// w_dtype / out_dtype: 0 float32, 1 bfloat16.  rows may be null.
+int tl_rmsnorm(const float* x, const void* w, const int32_t* rows, void* out, int n_rows, int hidden,
+               float eps, int w_dtype, int out_dtype, hipStream_t stream) {
+  if (n_rows <= 0) return TL_OK;
+  if (hidden <= 0) return TL_ERR_ARG;
+  dim3 g(n_rows), b(kThreads);
+  if (w_dtype == 0 && out_dtype == 0)
+    hipLaunchKernelGGL((rmsnorm_kernel<float, float>), g, b, 0, stream, x, (const float*)w, rows, (float*)out, hidden, eps);
+  else if (w_dtype == 1 && out_dtype == 0)
+    hipLaunchKernelGGL((rmsnorm_kernel<bf16_t, float>), g, b, 0, stream, x, (const bf16_t*)w, rows, (float*)out, hidden, eps);
+  else if (w_dtype == 0 && out_dtype == 1)
+    hipLaunchKernelGGL((rmsnorm_kernel<float, bf16_t>), g, b, 0, stream, x, (const float*)w, rows, (bf16_t*)out, hidden, eps);
+  else if (w_dtype == 1 && out_dtype == 1)
+    hipLaunchKernelGGL((rmsnorm_kernel<bf16_t, bf16_t>), g, b, 0, stream, x, (const bf16_t*)w, rows, (bf16_t*)out, hidden, eps);
+  else
+    return TL_ERR_ARG;
+  return tl_launch_status();
+}
+
+int tl_silu_mul(const void* gate_up, void* z, int n_tokens, int inter, int dtype, hipStream_t stream) {
+  if (n_tokens <= 0) return TL_OK;
+  if (inter <= 0) return TL_ERR_ARG;
+  const int64_t total = (int64_t)n_tokens * inter;
+  TL_DISPATCH_T(dtype, hipLaunchKernelGGL(silu_mul_kernel<T>, dim3((unsigned)ceil_div64(total, kThreads)),
+                                          dim3(kThreads), 0, stream, (const T*)gate_up, (T*)z, total, inter);)
+  return tl_launch_status();
+}
+
+int tl_add_residual(float* x, const void* y, int64_t total, int dtype, hipStream_t stream) {
+  if (total <= 0) return TL_OK;
+  TL_DISPATCH_T(dtype, hipLaunchKernelGGL(add_residual_kernel<T>, dim3((unsigned)ceil_div64(total, kThreads)),
+                                          dim3(kThreads), 0, stream, x, (const T*)y, total);)
+  return tl_launch_status();
+}
+
+int tl_rope_store(void* qkv, const int32_t* positions, const float* cos_t, const float* sin_t,
+                  const int32_t* slot_mapping, void* k_cache, void* v_cache, int n_tokens, int nq,
+                  int nkv, int hd, int rot, int block_size, int64_t row_stride, int dtype,
+                  hipStream_t stream) {
+  if (n_tokens <= 0) return TL_OK;
+  if (nq < 0 || nkv < 0 || hd <= 0 || rot < 0 || rot > hd || (rot & 1) || block_size <= 0) return TL_ERR_ARG;
+  if (rot > 0 && (!cos_t || !sin_t)) return TL_ERR_ARG;
+  if (slot_mapping && (!k_cache || !v_cache)) return TL_ERR_ARG;
+  TL_DISPATCH_T(dtype, hipLaunchKernelGGL(rope_store_kernel<T>, dim3(n_tokens), dim3(kThreads), 0, stream,
+                                          (T*)qkv, positions, cos_t, sin_t, slot_mapping, (T*)k_cache,
+                                          (T*)v_cache, nq, nkv, hd, rot, block_size, row_stride);)
+  return tl_launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,219 @@
+// Linear layers: out[m, n] = sum_k a[m, k] * w[n, k] (+ residual[m, n]).
+// Weights are [out, in] row-major as in the checkpoint, the contraction the
+// reference's GEMM family computes (tiny_llm/ops/cuda/gemm.cu:86-100); the
+// residual add that the reference runs as a separate kernel
+// (tiny_llm/ops/cuda/arithmetic.cu:13) is folded into the epilogue.
+//
+//  * gemm_f32_kernel: true float32, FMA on the vector units, no reduced-precision
+//    matrix mode.  The k order of the accumulation does not depend on M, so a row
+//    gives the same bits whether it is computed alone or in a batch.
+//  * gemm_bf16_kernel: bf16 inputs on the MFMA matrix cores
+//    (v_mfma_f32_32x32x16_bf16), float32 accumulation, 128x128x32 tiles staged
+//    through LDS, four wave64 per workgroup.
+#include "common.h"
+
+namespace {
+
+// ===================================================================== float32
+constexpr int F_BM = 64, F_BN = 64, F_BK = 16, F_THREADS = 256;
+
+template <typename TO>
+__global__ __launch_bounds__(F_THREADS) void gemm_f32_kernel(const float* __restrict__ a,
+                                                             const float* __restrict__ w,
+                                                             TO* __restrict__ out,
+                                                             const float* __restrict__ residual, int M,
+                                                             int N, int K, int64_t lda, int64_t ldo) {
+  __shared__ float As[F_BK][F_BM + 4];
+  __shared__ float Ws[F_BK][F_BN + 4];
+  const int tid = threadIdx.x;
+  const int m0 = blockIdx.y * F_BM, n0 = blockIdx.x * F_BN;
+  const int ty = tid / 16, tx = tid % 16;
+  float acc[4][4] = {};
+  // each thread stages 4 consecutive k of one row of each operand
+  const int lr = tid / 4, lk = (tid % 4) * 4;
+  for (int k0 = 0; k0 < K; k0 += F_BK) {
+    float av[4], wv[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int k = k0 + lk + i;
+      av[i] = (m0 + lr < M && k < K) ? a[(int64_t)(m0 + lr) * lda + k] : 0.f;
+      wv[i] = (n0 + lr < N && k < K) ? w[(int64_t)(n0 + lr) * K + k] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      As[lk + i][lr] = av[i];
+      Ws[lk + i][lr] = wv[i];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < F_BK; ++k) {
+      float ar[4], wr[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        ar[i] = As[k][ty * 4 + i];
+        wr[i] = Ws[k][tx * 4 + i];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(ar[i], wr[j], acc[i][j]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = m0 + ty * 4 + i;
+    if (m >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx * 4 + j;
+      if (n >= N) continue;
+      float v = acc[i][j];
+      if (residual) v += residual[(int64_t)m * ldo + n];
+      out[(int64_t)m * ldo + n] = from_f32<TO>(v);
+    }
+  }
+}
+
+// ==================================================================== bfloat16
+constexpr int B_BM = 128, B_BN = 128, B_BK = 32, B_THREADS = 256;
+constexpr int B_LD = B_BK + 8;  // LDS row stride in elements: 80 bytes, keeps 16-byte alignment
+
+// K must be a multiple of 8 (16-byte chunks of bf16 never straddle the end).
+template <typename TO>
+__global__ __launch_bounds__(B_THREADS) void gemm_bf16_kernel(const bf16_t* __restrict__ a,
+                                                              const bf16_t* __restrict__ w,
+                                                              TO* __restrict__ out,
+                                                              const float* __restrict__ residual, int M,
+                                                              int N, int K, int64_t lda, int64_t ldo) {
+  __shared__ __attribute__((aligned(16))) bf16_t As[B_BM * B_LD];
+  __shared__ __attribute__((aligned(16))) bf16_t Ws[B_BN * B_LD];
+  const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
+  const int wm = wave / 2, wn = wave % 2;
+  const int m0 = blockIdx.y * B_BM, n0 = blockIdx.x * B_BN;
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // staging: 512 16-byte chunks per operand tile, two per thread
+  bf16x8 ra[2], rw[2];
+  auto load_tiles = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int c = tid + i * B_THREADS;
+      const int row = c / 4, kc = (c % 4) * 8;
+      const int k = k0 + kc;
+      bf16x8 z = {};
+      ra[i] = (m0 + row < M && k < K) ? *(const bf16x8*)(a + (int64_t)(m0 + row) * lda + k) : z;
+      rw[i] = (n0 + row < N && k < K) ? *(const bf16x8*)(w + (int64_t)(n0 + row) * K + k) : z;
+    }
+  };
+  auto store_tiles = [&]() {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int c = tid + i * B_THREADS;
+      const int row = c / 4, kc = (c % 4) * 8;
+      *(bf16x8*)(As + row * B_LD + kc) = ra[i];
+      *(bf16x8*)(Ws + row * B_LD + kc) = rw[i];
+    }
+  };
+
+  load_tiles(0);
+  for (int k0 = 0; k0 < K; k0 += B_BK) {
+    __syncthreads();
+    store_tiles();
+    __syncthreads();
+    if (k0 + B_BK < K) load_tiles(k0 + B_BK);
+#pragma unroll
+    for (int ks = 0; ks < B_BK; ks += 16) {
+      bf16x8 fa[2], fw[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        fa[i] = *(const bf16x8*)(As + (wm * 64 + i * 32 + lane % 32) * B_LD + ks + (lane / 32) * 8);
+        fw[i] = *(const bf16x8*)(Ws + (wn * 64 + i * 32 + lane % 32) * B_LD + ks + (lane / 32) * 8);
+      }
+      // result tile is transposed (rows = n, columns = m) so that a lane holds four
+      // consecutive n of one output row and can store them as one vector
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[j], fa[i], acc[i][j], 0, 0, 0);
+    }
+  }
+
+  const bool vec_ok = (N % 4 == 0) && (ldo % 4 == 0);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int m = m0 + wm * 64 + i * 32 + lane % 32;
+    if (m >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = n0 + wn * 64 + j * 32 + q * 8 + (lane / 32) * 4;
+        if (n >= N) continue;
+        float v[4] = {acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
+        const int64_t o = (int64_t)m * ldo + n;
+        if (vec_ok) {  // n + 3 < N because n and N are both multiples of 4
+          if (residual) {
+            const f32x4 r = *(const f32x4*)(residual + o);
+            v[0] += r[0]; v[1] += r[1]; v[2] += r[2]; v[3] += r[3];
+          }
+          if constexpr (sizeof(TO) == 4) {
+            f32x4 s = {v[0], v[1], v[2], v[3]};
+            *(f32x4*)((float*)out + o) = s;
+          } else {
+            bf16x4 s = {(bf16_t)v[0], (bf16_t)v[1], (bf16_t)v[2], (bf16_t)v[3]};
+            *(bf16x4*)((bf16_t*)out + o) = s;
+          }
+        } else {
+          for (int e = 0; e < 4 && n + e < N; ++e) {
+            float x = v[e];
+            if (residual) x += residual[o + e];
+            out[o + e] = from_f32<TO>(x);
+          }
+        }
+      }
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+// dtype: element type of a and w (0 float32, 1 bfloat16); out_dtype: of out.
+// lda: row stride of a in elements; ldo: row stride of out and residual.
+int tl_linear(const void* a, const void* w, void* out, const float* residual, int M, int N, int K,
+              int64_t lda, int64_t ldo, int dtype, int out_dtype, hipStream_t stream) {
+  if (M <= 0) return TL_OK;
+  if (N <= 0 || K <= 0 || lda < K || ldo < N) return TL_ERR_ARG;
+  if (dtype == 0) {
+    if (out_dtype != 0) return TL_ERR_ARG;
+    dim3 g((N + F_BN - 1) / F_BN, (M + F_BM - 1) / F_BM);
+    hipLaunchKernelGGL(gemm_f32_kernel<float>, g, dim3(F_THREADS), 0, stream, (const float*)a, (const float*)w,
+                       (float*)out, residual, M, N, K, lda, ldo);
+  } else if (dtype == 1) {
+    if (K % 8 || lda % 8) return TL_ERR_ARG;
+    dim3 g((N + B_BN - 1) / B_BN, (M + B_BM - 1) / B_BM);
+    if (out_dtype == 0)
+      hipLaunchKernelGGL(gemm_bf16_kernel<float>, g, dim3(B_THREADS), 0, stream, (const bf16_t*)a,
+                         (const bf16_t*)w, (float*)out, residual, M, N, K, lda, ldo);
+    else if (out_dtype == 1)
+      hipLaunchKernelGGL(gemm_bf16_kernel<bf16_t>, g, dim3(B_THREADS), 0, stream, (const bf16_t*)a,
+                         (const bf16_t*)w, (bf16_t*)out, residual, M, N, K, lda, ldo);
+    else
+      return TL_ERR_ARG;
+  } else {
+    return TL_ERR_ARG;
+  }
+  return tl_launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,200 @@
+"""The step function: one batch of (request, its next tokens) through the model.
+
+A step runs only the tokens it is given, against the cache that earlier steps
+left, and returns the logits at the wanted places.  Entries may be portions of
+prompts beside single decoded tokens, cut anywhere.  The reference's runtime needs
+five calls and allows either whole prompts from position 0 or exactly one token per
+request (tiny_llm/pipeline/pipeline.cpp:132-140, 184-190,
+tiny_llm/runtime/cuda/cuda_runtime.cpp:673, 690); here it is one call for any mix.
+
+Step metadata is built on the host in one pinned int32 buffer and uploaded with
+one copy (the reference uploads a block table per layer with a stream sync each,
+cuda_runtime.cpp:758-773).  Token rows map to requests through `req_of_token`, so
+kernels need no search over sequence separators (tiny_llm/ops/details.hpp:19-36).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, Hashable, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache import CacheManager, OutOfBlocks
+
+
+@dataclass
+class StepEntry:
+    req_id: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = ()        # places among `tokens` whose logits are asked for
+
+
+@dataclass
+class StepContext:
+    """Who is in the batch and where each token sits; device tensors are int32."""
+    num_tokens: int
+    num_requests: int
+    tokens: torch.Tensor            # [T]
+    positions: torch.Tensor         # [T] absolute position of each token in its request
+    req_of_token: torch.Tensor      # [T] row of the block tables
+    cu_seqlens_q: torch.Tensor      # [R+1]
+    seq_lens: torch.Tensor          # [R] cached length after this step
+    state_slots: torch.Tensor       # [R] per-request state slot
+    logit_rows: Optional[torch.Tensor]      # [n_out] token rows whose logits are wanted
+    block_tables: List[torch.Tensor]        # per cache group [R, max_blocks]
+    slot_mappings: List[torch.Tensor]       # per cache group [T] flat slot = block * block_size + offset
+    # host copies
+    q_lens: List[int] = field(default_factory=list)
+    context_lens: List[int] = field(default_factory=list)
+    slots_host: List[int] = field(default_factory=list)
+    max_q_len: int = 0
+    max_seq_len: int = 0
+    block_size: int = 0
+
+    @property
+    def decode_only(self) -> bool:
+        return self.max_q_len == 1
+
+
+class StepError(ValueError):
+    pass
+
+
+class ModelRunner:
+    """Owns the decoder's cache views and turns step entries into one forward pass."""
+
+    def __init__(self, decoder, cache: CacheManager, max_num_batched_tokens: int, max_model_len: int):
+        self.decoder = decoder
+        self.cache = cache
+        self.device = decoder.device
+        self.max_tokens = int(max_num_batched_tokens)
+        self.max_model_len = int(max_model_len)
+        self.vocab_size = decoder.spec.vocab_size
+        for i, e in enumerate(decoder.spec.plan):
+            decoder.caches[i] = cache.layer_cache(i, e.cache_of)
+            decoder.states[i] = cache.states[i]
+        self._pinned: Optional[torch.Tensor] = None
+        self._uploaded: Optional[torch.cuda.Event] = None
+
+    # ----------------------------------------------------------------- metadata
+    def _host_buffer(self, n: int) -> torch.Tensor:
+        if self._pinned is None or self._pinned.numel() < n:
+            self._pinned = torch.empty(max(n, 1 << 16), dtype=torch.int32, pin_memory=True)
+        return self._pinned[:n]
+
+    def prepare(self, entries: Sequence[StepEntry]) -> StepContext:
+        """Checks the entries, takes the cache blocks they need (all or nothing) and
+        builds the step metadata on the device."""
+        cm = self.cache
+        bs = cm.block_size
+        if not entries:
+            raise StepError("a step needs at least one entry")
+        seen = set()
+        T = 0
+        for e in entries:
+            if e.req_id in seen:
+                raise StepError(f"request {e.req_id!r} appears twice in one step")
+            seen.add(e.req_id)
+            n = len(e.tokens)
+            if n == 0:
+                raise StepError(f"request {e.req_id!r} brings no tokens")
+            for t in e.tokens:
+                if not (0 <= int(t) < self.vocab_size):
+                    raise StepError(f"token id {t} of request {e.req_id!r} is outside the vocabulary")
+            for w in e.want:
+                if not (0 <= int(w) < n):
+                    raise StepError(f"wanted place {w} of request {e.req_id!r} is outside its {n} tokens")
+            T += n
+        if T > self.max_tokens:
+            raise StepError(f"step brings {T} tokens, the budget is {self.max_tokens}")
+
+        new_reqs = [e.req_id for e in entries if not cm.has(e.req_id)]
+        if len(new_reqs) > cm.free_slots:
+            raise OutOfBlocks(f"{len(new_reqs)} new requests, {cm.free_slots} request slots are free")
+        ctx_lens, new_lens, needs = [], [], []
+        for e in entries:
+            c = cm.num_tokens(e.req_id) if cm.has(e.req_id) else 0
+            n = c + len(e.tokens)
+            if n > self.max_model_len:
+                raise StepError(f"request {e.req_id!r} would reach {n} tokens, the limit is {self.max_model_len}")
+            ctx_lens.append(c)
+            new_lens.append(n)
+            needs.append(cm.blocks_needed(e.req_id, n))
+        if not cm.can_grow(needs):
+            raise OutOfBlocks("the step needs more cache blocks than are free: "
+                              f"needs {[sum(n[g] for n in needs) for g in range(len(cm.groups))]}, "
+                              f"free {cm.free_blocks()}")
+        for rid in new_reqs:
+            cm.add_request(rid)
+        for e, n in zip(entries, new_lens):
+            cm.grow(e.req_id, n)
+
+        R, G = len(entries), len(cm.groups)
+        max_blocks = max(1, max(-(-n // bs) for n in new_lens))
+        n_out = sum(len(e.want) for e in entries)
+        sizes = [T, T, T, R + 1, R, R, n_out] + [T] * G + [R * max_blocks] * G
+        offs = [0]
+        for s in sizes:
+            offs.append(offs[-1] + ((s + 3) // 4) * 4)   # 16-byte aligned sections
+        if self._uploaded is not None:
+            self._uploaded.synchronize()      # the last step's upload has left the pinned buffer
+        buf = self._host_buffer(offs[-1])
+        host = buf.numpy()
+        host[:offs[-1]] = 0
+        tok, pos, rot = host[offs[0]:], host[offs[1]:], host[offs[2]:]
+        cu, sl, ss, lr = host[offs[3]:], host[offs[4]:], host[offs[5]:], host[offs[6]:]
+        t = 0
+        k = 0
+        q_lens, slots = [], []
+        for r, e in enumerate(entries):
+            n = len(e.tokens)
+            c = ctx_lens[r]
+            tok[t:t + n] = e.tokens
+            pos[t:t + n] = range(c, c + n)
+            rot[t:t + n] = r
+            cu[r] = t
+            sl[r] = new_lens[r]
+            ss[r] = cm.slot(e.req_id)
+            slots.append(cm.slot(e.req_id))
+            for w in e.want:
+                lr[k] = t + int(w)
+                k += 1
+            for g in range(G):
+                table = cm.block_table(e.req_id, g)
+                sm = host[offs[7 + g]:]
+                bt = host[offs[7 + G + g]:]
+                tb = np.maximum(np.asarray(table, dtype=np.int32), 0)   # released blocks are never read
+                bt[r * max_blocks: r * max_blocks + len(table)] = tb
+                p = np.arange(c, c + n, dtype=np.int32)
+                sm[t:t + n] = tb[p // bs] * bs + p % bs
+            q_lens.append(n)
+            t += n
+        cu[R] = T
+        dev = buf.to(self.device, non_blocking=True)
+        self._uploaded = torch.cuda.Event()
+        self._uploaded.record()
+        sec = lambda i, n: dev[offs[i]:offs[i] + n]
+        return StepContext(
+            num_tokens=T, num_requests=R,
+            tokens=sec(0, T), positions=sec(1, T), req_of_token=sec(2, T), cu_seqlens_q=sec(3, R + 1),
+            seq_lens=sec(4, R), state_slots=sec(5, R), logit_rows=sec(6, n_out) if n_out else None,
+            block_tables=[sec(7 + G + g, R * max_blocks).view(R, max_blocks) for g in range(G)],
+            slot_mappings=[sec(7 + g, T) for g in range(G)],
+            q_lens=q_lens, context_lens=ctx_lens, slots_host=slots, max_q_len=max(q_lens),
+            max_seq_len=max(new_lens), block_size=bs)
+
+    # --------------------------------------------------------------------- step
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Runs the entries as one batch.  Returns float32 logits [wanted, vocab] on the
+        device, in the order of the entries and of each entry's `want`."""
+        ctx = self.prepare(entries)
+        logits = self.decoder.forward(ctx)
+        for e, c, n in zip(entries, ctx.context_lens, ctx.q_lens):
+            self.cache.commit(e.req_id, c + n)
+        return logits
+
+    def finish(self, req_id) -> None:
+        """The request is done: its blocks and its state slot are given back."""
+        if self.cache.has(req_id):
+            self.cache.free_request(req_id)

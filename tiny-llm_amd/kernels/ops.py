@@ -1,0 +1,237 @@
+"""Python face of the HIP kernels: one function per kernel entry point.
+
+Every function checks on the host that device, dtype, contiguity, alignment and
+shapes are what the kernel and its grid assume, then hands raw pointers and the
+current stream to the library.  A refused size raises `KernelError`; nothing is
+computed on the CPU or by a library op.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import library
+
+c_void_p = ctypes.c_void_p
+c_int = ctypes.c_int
+c_int64 = ctypes.c_int64
+c_float = ctypes.c_float
+
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _lib():
+    return library.load()
+
+
+def _stream():
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise KernelError(f"element type {t.dtype} is not float32 or bfloat16") from None
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _dev(*tensors) -> None:
+    for t in tensors:
+        if t is not None:
+            _need(t.is_cuda, "kernel operands must live on the GPU (there is no CPU path)")
+
+
+def _ptr(t: Optional[torch.Tensor], align: int = 1) -> c_void_p:
+    if t is None:
+        return c_void_p(0)
+    p = t.data_ptr()
+    _need(p % align == 0, f"operand is not {align}-byte aligned")
+    return c_void_p(p)
+
+
+def _check(code: int, what: str) -> None:
+    if code == 1:
+        raise KernelError(f"{what}: the kernel refuses these sizes")
+    if code != 0:
+        raise KernelError(f"{what}: launch failed (status {code})")
+
+
+def _rows_2d(t: torch.Tensor, name: str) -> None:
+    _need(t.dim() == 2 and t.stride(1) == 1, f"{name} must be 2-D with unit inner stride")
+
+
+# --------------------------------------------------------------------------- ops
+def embedding(tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t, :] = table[tokens[t], :] as float32."""
+    _dev(tokens, table, out)
+    T = tokens.numel()
+    V, H = table.shape
+    _need(tokens.dtype == torch.int32 and tokens.is_contiguous(), "tokens must be contiguous int32")
+    _need(table.is_contiguous(), "embedding table must be contiguous")
+    _need(out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (T, H),
+          f"embedding output must be float32 [{T}, {H}]")
+    _check(_lib().tl_embedding(_ptr(tokens), _ptr(table), _ptr(out), c_int(T), c_int(H), c_int(V),
+                               c_int(_dt(table)), _stream()), "embedding")
+    return out
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
+            rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[i] = weight * x[rows[i] or i] / sqrt(mean(x^2) + eps); x is float32."""
+    _dev(x, weight, out, rows)
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous(), "norm input must be contiguous float32 [T, H]")
+    H = x.shape[1]
+    n = out.shape[0]
+    _need(weight.is_contiguous() and weight.numel() == H, f"norm weight must have {H} elements")
+    _need(out.dim() == 2 and out.is_contiguous() and out.shape[1] == H, "norm output must be contiguous [n, H]")
+    if rows is None:
+        _need(n == x.shape[0], "norm output rows must match input rows")
+    else:
+        _need(rows.dtype == torch.int32 and rows.is_contiguous() and rows.numel() == n,
+              "row index must be contiguous int32, one per output row")
+    _check(_lib().tl_rmsnorm(_ptr(x), _ptr(weight), _ptr(rows), _ptr(out), c_int(n), c_int(H),
+                             c_float(eps), c_int(_dt(weight)), c_int(_dt(out)), _stream()), "rmsnorm")
+    return out
+
+
+def linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor,
+           residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out = a @ w.T (+ residual).  a [M, K], w [N, K] share an element type;
+    out [M, N] is that type or float32; residual float32 with out's strides."""
+    _dev(a, w, out, residual)
+    _rows_2d(a, "linear input")
+    _rows_2d(out, "linear output")
+    M, K = a.shape
+    N = w.shape[0]
+    _need(w.dim() == 2 and w.is_contiguous() and w.shape[1] == K, f"weight must be contiguous [N, {K}]")
+    _need(a.dtype == w.dtype, "input and weight must share an element type")
+    _need(tuple(out.shape) == (M, N), f"linear output must be [{M}, {N}]")
+    dt, odt = _dt(a), _dt(out)
+    _need(odt == dt or odt == 0, "linear output must have the input's type or float32")
+    if residual is not None:
+        _need(residual.dtype == torch.float32 and residual.shape == out.shape
+              and residual.stride() == out.stride(), "residual must be float32 with the output's layout")
+    if dt == 1:
+        _need(K % 8 == 0 and a.stride(0) % 8 == 0,
+              f"bfloat16 linear needs an inner size that is a multiple of 8, got K={K}")
+    _check(_lib().tl_linear(_ptr(a, 16), _ptr(w, 16), _ptr(out, 16), _ptr(residual, 16), c_int(M), c_int(N),
+                            c_int(K), c_int64(a.stride(0)), c_int64(out.stride(0)), c_int(dt), c_int(odt),
+                            _stream()), "linear")
+    return out
+
+
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t, j] = silu(gate_up[t, j]) * gate_up[t, I + j]."""
+    _dev(gate_up, out)
+    T, I2 = gate_up.shape
+    _need(I2 % 2 == 0 and gate_up.is_contiguous(), "gate_up must be contiguous [T, 2I]")
+    _need(out.dtype == gate_up.dtype and out.is_contiguous() and tuple(out.shape) == (T, I2 // 2),
+          "silu_mul output must be contiguous [T, I] of the input's type")
+    _check(_lib().tl_silu_mul(_ptr(gate_up), _ptr(out), c_int(T), c_int(I2 // 2), c_int(_dt(gate_up)),
+                              _stream()), "silu_mul")
+    return out
+
+
+def add_residual(x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+    """x += y with x float32."""
+    _dev(x, y)
+    _need(x.dtype == torch.float32 and x.is_contiguous() and y.is_contiguous() and x.shape == y.shape,
+          "residual add needs contiguous operands of one shape, the sum in float32")
+    _check(_lib().tl_add_residual(_ptr(x), _ptr(y), c_int64(x.numel()), c_int(_dt(y)), _stream()), "add_residual")
+    return x
+
+
+def rope_store(qkv: torch.Tensor, positions: torch.Tensor, cos: Optional[torch.Tensor],
+               sin: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor],
+               k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+               num_heads: int, num_kv_heads: int, head_dim: int, rotary_dim: int) -> None:
+    """Rotate q and k of every row of qkv in place by the row's position and
+    store k, v at the row's cache slot.  Caches: [blocks, kv_heads, block, head_dim]."""
+    _dev(qkv, positions, cos, sin, slot_mapping, k_cache, v_cache)
+    _rows_2d(qkv, "qkv")
+    T = qkv.shape[0]
+    width = (num_heads + 2 * num_kv_heads) * head_dim
+    _need(qkv.shape[1] == width, f"qkv rows must be {width} wide")
+    _need(positions.dtype == torch.int32 and positions.is_contiguous() and positions.numel() == T,
+          "positions must be contiguous int32, one per row")
+    block_size = 1
+    if rotary_dim:
+        _need(cos is not None and sin is not None and cos.dtype == torch.float32 and sin.dtype == torch.float32
+              and cos.is_contiguous() and sin.is_contiguous() and cos.shape == sin.shape
+              and cos.shape[1] == rotary_dim // 2, "angle tables must be float32 [positions, rotary_dim/2]")
+    if slot_mapping is not None:
+        _need(slot_mapping.dtype == torch.int32 and slot_mapping.is_contiguous() and slot_mapping.numel() == T,
+              "slot mapping must be contiguous int32, one per row")
+        for c in (k_cache, v_cache):
+            _need(c is not None and c.dtype == qkv.dtype and c.is_contiguous() and c.dim() == 4
+                  and c.shape[1] == num_kv_heads and c.shape[3] == head_dim,
+                  "cache must be contiguous [blocks, kv_heads, block, head_dim] of the activations' type")
+        _need(k_cache.shape == v_cache.shape, "key and value caches must have one shape")
+        block_size = k_cache.shape[2]
+    _check(_lib().tl_rope_store(_ptr(qkv), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(slot_mapping),
+                                _ptr(k_cache), _ptr(v_cache), c_int(T), c_int(num_heads), c_int(num_kv_heads),
+                                c_int(head_dim), c_int(rotary_dim), c_int(block_size), c_int64(qkv.stride(0)),
+                                c_int(_dt(qkv)), _stream()), "rope_store")
+
+
+def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                    block_tables: torch.Tensor, req_of_token: torch.Tensor, positions: torch.Tensor,
+                    out: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, scale: float,
+                    window: int = 0) -> torch.Tensor:
+    """Causal attention of every row of q (at its absolute position) over its
+    request's cached keys 0..position (the last `window` of them if window > 0)."""
+    _dev(q, k_cache, v_cache, block_tables, req_of_token, positions, out)
+    _rows_2d(q, "q")
+    _rows_2d(out, "attention output")
+    T = q.shape[0]
+    _need(q.shape[1] == num_heads * head_dim and tuple(out.shape) == (T, num_heads * head_dim),
+          "q and the attention output must be [T, heads * head_dim]")
+    _need(q.dtype == k_cache.dtype == v_cache.dtype == out.dtype, "q, caches and output must share an element type")
+    _need(k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dim() == 4
+          and k_cache.shape == v_cache.shape and k_cache.shape[1] == num_kv_heads
+          and k_cache.shape[3] == head_dim, "cache must be contiguous [blocks, kv_heads, block, head_dim]")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(),
+          "block tables must be contiguous int32 [requests, max_blocks]")
+    for t in (req_of_token, positions):
+        _need(t.dtype == torch.int32 and t.is_contiguous() and t.numel() == T,
+              "per-token request ids and positions must be contiguous int32")
+    _need(num_kv_heads > 0 and num_heads % num_kv_heads == 0, "heads must be a multiple of kv heads")
+    _need(head_dim <= 256, f"head_dim {head_dim} exceeds the attention kernel's limit of 256")
+    _check(_lib().tl_paged_attention(
+        _ptr(q), c_int64(q.stride(0)), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
+        c_int(block_tables.shape[1]), _ptr(req_of_token), _ptr(positions), _ptr(out), c_int64(out.stride(0)),
+        c_int(T), c_int(num_heads), c_int(num_kv_heads), c_int(head_dim), c_int(k_cache.shape[2]),
+        c_float(scale), c_int(window), c_int(_dt(q)), _stream()), "paged_attention")
+    return out
+
+
+def sample(logits: torch.Tensor, out: torch.Tensor, temperature: Optional[torch.Tensor] = None,
+           top_k: Optional[torch.Tensor] = None, top_p: Optional[torch.Tensor] = None,
+           seeds: Optional[torch.Tensor] = None, counters: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One token per row of float32 logits.  temperature <= 0 (or None): first
+    maximum.  Otherwise temperature -> top-k -> top-p -> multinomial with the
+    uniform number drawn from (seeds[row], counters[row])."""
+    _dev(logits, out, temperature, top_k, top_p, seeds, counters)
+    _rows_2d(logits, "logits")
+    n, V = logits.shape
+    _need(logits.dtype == torch.float32, "logits must be float32")
+    _need(out.dtype == torch.int32 and out.is_contiguous() and out.numel() == n, "token output must be int32 [rows]")
+    for t, dt, name in ((temperature, torch.float32, "temperature"), (top_k, torch.int32, "top_k"),
+                        (top_p, torch.float32, "top_p"), (seeds, torch.int64, "seeds"),
+                        (counters, torch.int32, "counters")):
+        if t is not None:
+            _need(t.dtype == dt and t.is_contiguous() and t.numel() == n, f"{name} must be contiguous {dt} [rows]")
+    _check(_lib().tl_sample(_ptr(logits), c_int64(logits.stride(0)), c_int(n), c_int(V), _ptr(temperature),
+                            _ptr(top_k), _ptr(top_p), _ptr(seeds), _ptr(counters), _ptr(out), _stream()), "sample")
+    return out

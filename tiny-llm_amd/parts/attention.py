@@ -1,0 +1,79 @@
+"""Grouped-query causal attention over the paged cache (the Llama mixer).
+
+Per token: q, k, v = h Wq^T, h Wk^T, h Wv^T (tiny_llm/ops/cuda/gemm.cu:86-100,
+head-major columns gemm.cu:119-123); q and k rotated by the token's position
+(rope.cu:46-54); k (rotated) and v written to the cache (gemm.cu:400-407);
+scores q.k * hd^-0.5 against the request's cached keys with a causal mask, online
+softmax, weighted sum of values (flash_attention.cu:374-405); output projection
+with the residual add folded in (gemm.cu:171-190, arithmetic.cu:13).
+
+Q, K and V weights are concatenated on load into one [(nq + 2 nkv) * hd, H]
+matrix: row concatenation leaves every dot product as it was.
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, List, Optional
+
+import torch
+
+from ..kernels import ops
+from .base import (CacheSpec, LayerCache, Mixer, POSITION_ENCODINGS, WeightSpec, register_mixer)
+
+
+class Attention(Mixer):
+    def __init__(self, prefix, dtype, device, *, hidden_size: int, num_heads: int, num_kv_heads: int,
+                 head_dim: int, position: dict = None, window: int = 0, scale: float = None,
+                 max_position: int = 0):
+        super().__init__(prefix, dtype, device)
+        self.hidden_size = int(hidden_size)
+        self.num_heads = int(num_heads)
+        self.num_kv_heads = int(num_kv_heads)
+        self.head_dim = int(head_dim)
+        if self.num_heads % self.num_kv_heads:
+            raise ValueError("num_heads must be a multiple of num_kv_heads")
+        self.window = int(window or 0)
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
+        pos = dict(position or {"kind": "none"})
+        kind = pos.pop("kind")
+        self.position = POSITION_ENCODINGS.get(kind)(f"{prefix}.position", dtype, device, **pos)
+        self.q_size = self.num_heads * self.head_dim
+        self.kv_size = self.num_kv_heads * self.head_dim
+        self.w_qkv: Optional[torch.Tensor] = None
+        self.w_o: Optional[torch.Tensor] = None
+
+    # ---------------------------------------------------------------- declarations
+    def weights(self) -> List[WeightSpec]:
+        p, H = self.prefix, self.hidden_size
+        return [WeightSpec(f"{p}.q_proj.weight", (self.q_size, H)),
+                WeightSpec(f"{p}.k_proj.weight", (self.kv_size, H)),
+                WeightSpec(f"{p}.v_proj.weight", (self.kv_size, H)),
+                WeightSpec(f"{p}.o_proj.weight", (H, self.q_size))]
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        p = self.prefix
+        self.w_qkv = torch.cat([tensors[f"{p}.q_proj.weight"], tensors[f"{p}.k_proj.weight"],
+                                tensors[f"{p}.v_proj.weight"]], dim=0).contiguous()
+        self.w_o = tensors[f"{p}.o_proj.weight"].contiguous()
+
+    def cache_spec(self) -> CacheSpec:
+        return CacheSpec(self.num_kv_heads, self.head_dim, "window" if self.window else "full", self.window)
+
+    # --------------------------------------------------------------------- compute
+    def forward(self, h, ctx, cache: LayerCache, state, residual):
+        T = h.shape[0]
+        qkv = torch.empty((T, self.q_size + 2 * self.kv_size), dtype=self.dtype, device=h.device)
+        ops.linear(h, self.w_qkv, qkv)
+        tables = self.position.rotary_tables()
+        cos, sin, rot = tables if tables is not None else (None, None, 0)
+        slots = ctx.slot_mappings[cache.group] if cache.write else None
+        ops.rope_store(qkv, ctx.positions, cos, sin, slots, cache.k if cache.write else None,
+                       cache.v if cache.write else None, self.num_heads, self.num_kv_heads, self.head_dim, rot)
+        attn = torch.empty((T, self.q_size), dtype=self.dtype, device=h.device)
+        ops.paged_attention(qkv[:, :self.q_size], cache.k, cache.v, ctx.block_tables[cache.group],
+                            ctx.req_of_token, ctx.positions, attn, self.num_heads, self.num_kv_heads,
+                            self.head_dim, self.scale, self.window)
+        return ops.linear(attn, self.w_o, residual, residual)
+
+
+register_mixer("attention", Attention)

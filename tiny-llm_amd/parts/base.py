@@ -1,0 +1,174 @@
+"""Interfaces of the parts a layer is made of, and the registries that name them.
+
+A part is built from a PartSpec's parameters alone: it knows its own sizes and
+constants and nothing about the model it sits in.  The generic decoder
+(models/decoder.py) looks parts up here by name, layer by layer, so one model
+may mix kinds.  Tests and other architectures add kinds with the `register_*`
+functions; no framework file changes.
+
+Calling conventions
+-------------------
+* The residual stream `x` is float32 [tokens, hidden].
+* A norm maps x (float32) to the activation type of the engine.
+* A mixer and a feed-forward receive the normed activations `h` and the
+  residual, and return `residual + f(h)` as float32 (writing into `residual`
+  is allowed); `add_to_residual` does that for parts that do not fuse it.
+* A mixer additionally receives the step context (who is in the batch, where
+  each token sits), its view of the paged cache (or None) and its per-request
+  state tensor [slots, ...] (or None).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+
+# ------------------------------------------------------------------ declarations
+@dataclass(frozen=True)
+class WeightSpec:
+    """One checkpoint tensor a part needs.
+
+    role: "matrix" - operand of a matrix product, takes the engine's element type;
+          "vector" - norm weights and the like: engine type, except that a tensor
+                     stored in 32 bits stays in 32 bits;
+          "table"  - integer tables, kept as int32.
+    init: how random-weights mode fills it ("normal" | "ones" | "around_one").
+    alias_of: a tensor to use when the file does not hold `name` (tied weights).
+    """
+    name: str
+    shape: Tuple[int, ...]
+    role: str = "matrix"
+    init: str = "normal"
+    alias_of: Optional[str] = None
+
+
+@dataclass(frozen=True)
+class CacheSpec:
+    """What a mixer keeps per token: keys and values of `num_kv_heads` heads.
+    kind "full" keeps every position, "window" the last `window` positions."""
+    num_kv_heads: int
+    head_dim: int
+    kind: str = "full"
+    window: int = 0
+
+    def group_key(self):
+        return (self.kind, self.window, self.num_kv_heads, self.head_dim)
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """Per-request state of fixed size: one tensor of `shape` per live request."""
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class LayerCache:
+    """A mixer's view of the paged cache for one plan entry."""
+    k: torch.Tensor            # [blocks, kv_heads, block_size, head_dim]
+    v: torch.Tensor
+    group: int                 # which block table / slot mapping of the context applies
+    write: bool = True         # False: the entry reads a cache that another entry fills
+
+
+class Part:
+    """Base of every part: declares weights, receives them, computes."""
+
+    def __init__(self, prefix: str, dtype: torch.dtype, device: torch.device):
+        self.prefix = prefix
+        self.dtype = dtype
+        self.device = device
+
+    def weights(self) -> List[WeightSpec]:
+        return []
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        """Receives the device tensors named by `weights()` (full names)."""
+
+
+class Norm(Part):
+    def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """How positions enter a mixer.  `rotary_tables()` returns
+    (cos, sin, rotary_dim) for encodings that rotate queries and keys, or None."""
+
+    def rotary_tables(self):
+        return None
+
+
+class Mixer(Part):
+    def cache_spec(self) -> Optional[CacheSpec]:
+        return None
+
+    def state_spec(self) -> Optional[StateSpec]:
+        return None
+
+    def forward(self, h: torch.Tensor, ctx, cache: Optional[LayerCache], state: Optional[torch.Tensor],
+                residual: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, h: torch.Tensor, ctx, residual: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block:
+    """Arrangement of (mixer_norm, mixer, ffn_norm, ffn) around the residual stream."""
+
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Norm, ffn: FeedForward):
+        self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
+
+    def parts(self):
+        return [self.mixer_norm, self.mixer, self.ffn_norm, self.ffn]
+
+    def forward(self, x, ctx, cache, state):
+        raise NotImplementedError
+
+
+def add_to_residual(residual: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+    """residual += y in float32, for parts whose last kernel does not fuse the add."""
+    from ..kernels import ops
+    return ops.add_residual(residual, y.contiguous())
+
+
+# -------------------------------------------------------------------- registries
+class Registry:
+    def __init__(self, what: str):
+        self.what = what
+        self._items: Dict[str, Callable[..., Any]] = {}
+
+    def register(self, name: str, factory: Callable[..., Any], *, replace: bool = False) -> None:
+        if name in self._items and not replace:
+            raise ValueError(f"{self.what} {name!r} is already registered")
+        self._items[name] = factory
+
+    def unregister(self, name: str) -> None:
+        self._items.pop(name, None)
+
+    def get(self, name: str) -> Callable[..., Any]:
+        if name not in self._items:
+            raise KeyError(f"no {self.what} named {name!r}; known: {', '.join(sorted(self._items))}")
+        return self._items[name]
+
+    def names(self):
+        return sorted(self._items)
+
+
+NORMS = Registry("norm")
+MIXERS = Registry("mixer")
+FEED_FORWARDS = Registry("feed-forward")
+POSITION_ENCODINGS = Registry("position encoding")
+BLOCKS = Registry("block arrangement")
+
+
+def register_norm(name, factory, **kw): NORMS.register(name, factory, **kw)
+def register_mixer(name, factory, **kw): MIXERS.register(name, factory, **kw)
+def register_feed_forward(name, factory, **kw): FEED_FORWARDS.register(name, factory, **kw)
+def register_position_encoding(name, factory, **kw): POSITION_ENCODINGS.register(name, factory, **kw)
+def register_block(name, factory, **kw): BLOCKS.register(name, factory, **kw)

@@ -1,0 +1,48 @@
+"""Token embedding (a row gather, no scale: tiny_llm/ops/cuda/embedding.cu:10-29)
+and the output head (logits = xn W^T at the wanted rows only:
+tiny_llm/ops/cuda/gemm_q1_helper.cu:99-124).  A tied head uses the embedding
+table; the reference never reads `tie_word_embeddings`."""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from ..kernels import ops
+from .base import Part, WeightSpec
+
+
+class TokenEmbedding(Part):
+    def __init__(self, prefix, dtype, device, *, vocab_size: int, hidden_size: int):
+        super().__init__(prefix, dtype, device)
+        self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+        self.weight: Optional[torch.Tensor] = None
+
+    def weights(self) -> List[WeightSpec]:
+        return [WeightSpec(f"{self.prefix}.weight", (self.vocab_size, self.hidden_size))]
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.weight = tensors[f"{self.prefix}.weight"].contiguous()
+
+    def forward(self, tokens: torch.Tensor) -> torch.Tensor:
+        out = torch.empty((tokens.numel(), self.hidden_size), dtype=torch.float32, device=tokens.device)
+        return ops.embedding(tokens, self.weight, out)
+
+
+class LMHead(Part):
+    def __init__(self, prefix, dtype, device, *, vocab_size: int, hidden_size: int, tied_to: str = None):
+        super().__init__(prefix, dtype, device)
+        self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+        self.tied_to = tied_to
+        self.weight: Optional[torch.Tensor] = None
+
+    def weights(self) -> List[WeightSpec]:
+        alias = f"{self.tied_to}.weight" if self.tied_to else None
+        return [WeightSpec(f"{self.prefix}.weight", (self.vocab_size, self.hidden_size), alias_of=alias)]
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.weight = tensors[f"{self.prefix}.weight"].contiguous()
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        out = torch.empty((h.shape[0], self.vocab_size), dtype=torch.float32, device=h.device)
+        return ops.linear(h, self.weight, out)
