@@ -208,9 +208,14 @@ def test_rope_invariants():
     base = torch.randn(1, 3 * hd, generator=g)     # one q head, one k head, one v head
 
     def rotated(p):
+        """(q rotated in place, k as it lands in the cache) for a token at position p."""
         x = base.clone().to(DEV)
-        ops().rope_store(x, torch.tensor([p], dtype=torch.int32, device=DEV), cos, sin, None, None, None, 1, 1, hd, rd)
-        return x.cpu()[0, :hd], x.cpu()[0, hd:2 * hd]
+        kc = torch.zeros(1, 1, 4, hd, device=DEV)
+        vc = torch.zeros(1, 1, 4, hd, device=DEV)
+        ops().rope_store(x, torch.tensor([p], dtype=torch.int32, device=DEV), cos, sin,
+                         torch.tensor([2], dtype=torch.int32, device=DEV), kc, vc, 1, 1, hd, rd)
+        assert torch.equal(vc.cpu()[0, 0, 2], base[0, 2 * hd:])
+        return x.cpu()[0, :hd], kc.cpu()[0, 0, 2]
 
     q0, k0 = rotated(0)
     assert torch.equal(q0, base[0, :hd]) and torch.equal(k0, base[0, hd:2 * hd])

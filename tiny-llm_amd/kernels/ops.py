@@ -125,7 +125,8 @@ def linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor,
     if dt == 1:
         _need(K % 8 == 0 and a.stride(0) % 8 == 0,
               f"bfloat16 linear needs an inner size that is a multiple of 8, got K={K}")
-    _check(_lib().tl_linear(_ptr(a, 16), _ptr(w, 16), _ptr(out, 16), _ptr(residual, 16), c_int(M), c_int(N),
+    al = 16 if dt == 1 else 4      # the bfloat16 kernel moves 16-byte vectors
+    _check(_lib().tl_linear(_ptr(a, al), _ptr(w, al), _ptr(out, al), _ptr(residual, al), c_int(M), c_int(N),
                             c_int(K), c_int64(a.stride(0)), c_int64(out.stride(0)), c_int(dt), c_int(odt),
                             _stream()), "linear")
     return out
