@@ -6,5 +6,7 @@ scheduler, sampling, and hand-written HIP kernels for gfx950.
 """
 from . import config, parts, models, weights, cache, kernels  # noqa: F401
 from .config import EngineConfig, LlamaConfig
+from .sampling import SamplingParams
+from .engine import Engine, StepEntry
 
 __version__ = "0.1.0"

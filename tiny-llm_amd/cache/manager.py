@@ -165,6 +165,28 @@ class CacheManager:
         for gi, (g, n) in enumerate(zip(self.groups, need)):
             rc.blocks[gi].extend(g.pool.allocate(n))
 
+    def reserve_step(self, entries: Sequence[Tuple[Hashable, int]]) -> List[int]:
+        """entries: (request, number of new tokens) of one step.  Admits the requests that are
+        new (a state slot each) and takes the blocks every entry needs, or changes nothing and
+        raises.  Returns each request's cached length before the step."""
+        new = [rid for rid, _ in entries if rid not in self.requests]
+        if len(new) > len(self._free_slots):
+            raise NoFreeSlot(f"{len(new)} new requests, {len(self._free_slots)} request slots are free")
+        before, needs = [], []
+        for rid, n in entries:
+            c = self.requests[rid].num_tokens if rid in self.requests else 0
+            before.append(c)
+            needs.append(self.blocks_needed(rid, c + n))
+        if not self.can_grow(needs):
+            raise OutOfBlocks("the step needs more cache blocks than are free: needs "
+                              f"{[sum(n[g] for n in needs) for g in range(len(self.groups))]}, "
+                              f"free {self.free_blocks()}")
+        for rid in new:
+            self.add_request(rid)
+        for (rid, n), c in zip(entries, before):
+            self.grow(rid, c + n)
+        return before
+
     def commit(self, req_id, new_len: int) -> None:
         """The step has written positions < new_len.  Gives back what a window has passed."""
         rc = self.requests[req_id]

@@ -1,1 +1,3 @@
 from .step import StepEntry, StepContext, ModelRunner, StepError
+from .scheduler import Scheduler, Request, StepPlan, Scheduled
+from .engine import Engine

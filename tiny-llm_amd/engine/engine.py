@@ -1,0 +1,109 @@
+"""The Python entry point: a model, its cache, the scheduler and the sampler behind
+`generate(prompt_token_ids, SamplingParams) -> token ids`.
+
+It stands where the reference's `Pipeline` stands (tiny_llm/pipeline/pipeline.hpp:14-29:
+constructor from a model folder and a config, `apply(prompts, max_new_tokens, do_sample,
+temperature, top_k, top_p)`), with token ids instead of text on both sides; text is the
+command line's business.
+"""
+from __future__ import annotations
+
+import itertools
+from typing import Dict, Hashable, List, Mapping, Optional, Sequence, Union
+
+import torch
+
+from ..config import EngineConfig
+from ..sampling import Sampler, SamplingParams
+from .loading import build_runner, load_model, random_model
+from .scheduler import Request, Scheduler, StepPlan
+from .step import StepEntry
+
+
+class Engine:
+    def __init__(self, model_path: Optional[str] = None, *, config: Optional[Mapping] = None,
+                 engine_config: Optional[EngineConfig] = None, weights_seed: int = 0,
+                 init_std: Optional[float] = None, norm_std: float = 0.0, **engine_kwargs):
+        """Either `model_path` (a folder with config.json and safetensors) or `config`
+        (config.json keys as a dict: seeded random weights are made on the device)."""
+        self.engine_config = engine_config or EngineConfig(**engine_kwargs)
+        if (model_path is None) == (config is None):
+            raise ValueError("give exactly one of model_path and config")
+        if model_path is not None:
+            self.model_config, self.decoder = load_model(model_path, self.engine_config)
+        else:
+            self.model_config, self.decoder = random_model(config, self.engine_config, weights_seed, init_std, norm_std)
+        self.runner = build_runner(self.decoder, self.engine_config)
+        self.eos_token_id = self.decoder.spec.eos_token_id
+        self.scheduler = Scheduler(self.runner.cache, self.engine_config.max_num_seqs,
+                                   self.engine_config.max_num_batched_tokens, self.runner.max_model_len,
+                                   self.eos_token_id)
+        self.sampler = Sampler(self.decoder.device)
+        self._ids = itertools.count()
+        self.requests: Dict[Hashable, Request] = {}
+        self.steps_run = 0
+
+    # ---------------------------------------------------------------- requests
+    def add_request(self, prompt_token_ids: Sequence[int], params: Optional[SamplingParams] = None,
+                    req_id: Optional[Hashable] = None) -> Hashable:
+        n = next(self._ids)
+        req_id = n if req_id is None else req_id
+        if req_id in self.requests and self.requests[req_id].status != "finished":
+            raise ValueError(f"request {req_id!r} is already live")
+        params = params or SamplingParams()
+        vocab = self.decoder.spec.vocab_size
+        prompt = [int(t) for t in prompt_token_ids]
+        for t in prompt:
+            if not (0 <= t < vocab):
+                raise ValueError(f"token id {t} is outside the vocabulary of {vocab}")
+        seed = params.seed if params.seed is not None else (self.engine_config.seed * 1000003 + n)
+        req = Request(req_id, prompt, params, seed=seed)
+        if params.max_new_tokens == 0:
+            req.status, req.finish_reason = "finished", "length"
+            self.requests[req_id] = req
+            return req_id
+        self.scheduler.add(req)
+        self.requests[req_id] = req
+        return req_id
+
+    def abort(self, req_id: Hashable) -> None:
+        self.scheduler.abort(req_id)
+
+    def has_unfinished(self) -> bool:
+        return self.scheduler.has_work()
+
+    # -------------------------------------------------------------------- step
+    def step(self) -> List[Request]:
+        """One scheduler decision, one forward pass, one sampling call.  Returns the requests
+        that finished in this step."""
+        plan = self.scheduler.schedule()
+        done = list(plan.finished)
+        if not plan.entries:
+            return done
+        entries, rows = [], []
+        for e in plan.entries:
+            toks = e.request.tokens[e.start:e.start + e.count]
+            entries.append(StepEntry(e.request.req_id, toks, [e.count - 1] if e.samples else []))
+            if e.samples:
+                rows.append(e.request)
+        logits = self.runner.step(entries)
+        sampled = {}
+        if rows:
+            toks = self.sampler(logits, [r.params for r in rows], [r.seed for r in rows],
+                                [r.num_tokens for r in rows])
+            sampled = {r.req_id: t for r, t in zip(rows, toks)}
+        done += self.scheduler.update(plan, sampled)
+        self.steps_run += 1
+        return done
+
+    # ---------------------------------------------------------------- generate
+    def generate(self, prompt_token_ids: Sequence[Sequence[int]],
+                 params: Union[SamplingParams, Sequence[SamplingParams], None] = None) -> List[List[int]]:
+        """Generated token ids of every prompt (eos, when it ends a request, is part of them,
+        as in tiny_llm/pipeline/pipeline.cpp:216-223)."""
+        if params is None or isinstance(params, SamplingParams):
+            params = [params or SamplingParams()] * len(prompt_token_ids)
+        ids = [self.add_request(p, sp) for p, sp in zip(prompt_token_ids, params)]
+        while self.scheduler.has_work():
+            self.step()
+        return [list(self.requests[i].output) for i in ids]

@@ -1,0 +1,238 @@
+"""The scheduler: admits requests, cuts prompts into portions under a token budget,
+decodes, finishes and frees.
+
+The reference's `Pipeline::apply` has none of this: a fixed list of prompts is
+prefilled whole in one step, every request then decodes in lockstep, finished
+requests are fed eos until request 0 reaches `max_new_tokens`, and all pages go back
+at the very end (tiny_llm/pipeline/pipeline.cpp:118-130, 181-231).  Kept from it: the
+position rule `pos = prompt_len + generated - 1` for a decoded token (:224-225), eos
+ends a request and is part of its output (:216-223), `max_new_tokens` bounds it.
+
+Decisions (all host-side, testable without a GPU):
+* A request's tokens are prompt + output; `num_computed` of them are in the cache.
+  Each step it is fed the next portion; when the portion reaches the end, the last
+  logits are wanted and a token is sampled.  Decoding is the portion of one.
+* Order within a step: running requests first, those that decode before those still
+  in their prompt, each group in order of admission; then waiting requests are
+  admitted in arrival order while a request slot, blocks for their first portion and
+  token budget are left.
+* Budget: at most `max_num_batched_tokens` tokens per step; a prompt portion is
+  `min(remaining, budget left, blocks that fit)`.
+* When pages run out for a running request, the request admitted last (other than
+  ones already scheduled this step) is preempted: its blocks and slot are given
+  back at once and it returns to the FRONT of the waiting queue with nothing
+  computed; prompt and output so far are recomputed when it is admitted again.  A
+  request that cannot fit even alone, with every other block free, is finished with
+  reason "capacity": the engine never deadlocks.
+"""
+from __future__ import annotations
+
+from collections import deque
+from dataclasses import dataclass, field
+from typing import Deque, Dict, Hashable, List, Optional, Sequence
+
+from ..cache import CacheManager
+from ..sampling.params import SamplingParams
+
+WAITING, RUNNING, FINISHED = "waiting", "running", "finished"
+
+
+@dataclass
+class Request:
+    req_id: Hashable
+    prompt: List[int]
+    params: SamplingParams
+    seed: int = 0
+    output: List[int] = field(default_factory=list)
+    num_computed: int = 0
+    status: str = WAITING
+    finish_reason: Optional[str] = None
+    preemptions: int = 0
+
+    @property
+    def tokens(self) -> List[int]:
+        return self.prompt + self.output
+
+    @property
+    def num_tokens(self) -> int:
+        return len(self.prompt) + len(self.output)
+
+    @property
+    def pending(self) -> int:
+        return self.num_tokens - self.num_computed
+
+
+@dataclass
+class Scheduled:
+    request: Request
+    start: int          # first token position fed this step
+    count: int          # number of tokens fed
+    samples: bool       # the portion reaches the end: its last logits are wanted
+
+
+@dataclass
+class StepPlan:
+    entries: List[Scheduled]
+    preempted: List[Request]
+    finished: List[Request]      # requests finished by the scheduler itself (reason "capacity")
+
+    @property
+    def num_tokens(self) -> int:
+        return sum(e.count for e in self.entries)
+
+
+class Scheduler:
+    def __init__(self, cache: CacheManager, max_num_seqs: int, max_num_batched_tokens: int, max_model_len: int,
+                 eos_token_id: Optional[int] = None):
+        self.cache = cache
+        self.max_num_seqs = int(max_num_seqs)
+        self.budget = int(max_num_batched_tokens)
+        self.max_model_len = int(max_model_len)
+        self.eos_token_id = eos_token_id
+        self.waiting: Deque[Request] = deque()
+        self.running: List[Request] = []       # in order of admission
+        self.finished: List[Request] = []
+
+    # ---------------------------------------------------------------- requests
+    def add(self, req: Request) -> None:
+        if not req.prompt:
+            raise ValueError("a request needs at least one prompt token")
+        if len(req.prompt) > self.max_model_len:
+            raise ValueError(f"prompt of {len(req.prompt)} tokens exceeds max_model_len {self.max_model_len}")
+        blocks_alone = -(-len(req.prompt) // self.cache.block_size)
+        if blocks_alone > self.cache.num_blocks:
+            raise ValueError(f"prompt of {len(req.prompt)} tokens cannot fit the cache "
+                             f"({self.cache.num_blocks} blocks of {self.cache.block_size})")
+        req.status = WAITING
+        self.waiting.append(req)
+
+    def has_work(self) -> bool:
+        return bool(self.waiting or self.running)
+
+    def abort(self, req_id) -> None:
+        for r in list(self.running):
+            if r.req_id == req_id:
+                self._finish(r, "abort")
+        for r in list(self.waiting):
+            if r.req_id == req_id:
+                self.waiting.remove(r)
+                r.status, r.finish_reason = FINISHED, "abort"
+                self.finished.append(r)
+
+    # ---------------------------------------------------------------- planning
+    def _needs(self, req: Request, count: int) -> List[int]:
+        return self.cache.blocks_needed(req.req_id, req.num_computed + count)
+
+    def _fits(self, need: Sequence[int], taken: Sequence[int]) -> bool:
+        free = self.cache.free_blocks()
+        return all(n + t <= f for n, t, f in zip(need, taken, free))
+
+    def _largest_fit(self, req: Request, want: int, taken: Sequence[int]) -> int:
+        """Largest portion <= want whose blocks are free now (0 if not even one token)."""
+        free = self.cache.free_blocks()
+        bs = self.cache.block_size
+        have = [len(self.cache.block_table(req.req_id, g)) if self.cache.has(req.req_id) else 0
+                for g in range(len(free))]
+        room = min((h + f - t) * bs for h, f, t in zip(have, free, taken)) if free else 1 << 60
+        return max(0, min(want, room - req.num_computed))
+
+    def _preempt(self, victim: Request) -> None:
+        if self.cache.has(victim.req_id):
+            self.cache.free_request(victim.req_id)
+        self.running.remove(victim)
+        victim.num_computed = 0
+        victim.status = WAITING
+        victim.preemptions += 1
+        self.waiting.appendleft(victim)
+
+    def _finish(self, req: Request, reason: str) -> None:
+        if self.cache.has(req.req_id):
+            self.cache.free_request(req.req_id)
+        if req in self.running:
+            self.running.remove(req)
+        req.status, req.finish_reason = FINISHED, reason
+        self.finished.append(req)
+
+    def schedule(self) -> StepPlan:
+        entries: List[Scheduled] = []
+        preempted: List[Request] = []
+        finished: List[Request] = []
+        taken = [0] * len(self.cache.groups)
+        budget = self.budget
+
+        order = [r for r in self.running if r.pending == 1] + [r for r in self.running if r.pending > 1]
+        scheduled_ids = set()
+        for req in order:
+            if req not in self.running or budget <= 0:   # preempted meanwhile / no budget left
+                continue
+            want = min(req.pending, budget)
+            while True:
+                count = self._largest_fit(req, want, taken)
+                if count >= 1 and (count == want or req.pending > 1):
+                    break
+                # not even the next token fits: take the blocks of the request admitted last
+                victims = [r for r in reversed(self.running) if r is not req and r.req_id not in scheduled_ids]
+                if not victims:
+                    count = 0
+                    break
+                self._preempt(victims[0])
+                preempted.append(victims[0])
+            if count == 0:
+                if not entries and len(self.running) == 1:
+                    # alone, nothing scheduled before it, and still no room: it can never go on
+                    self._finish(req, "capacity")
+                    finished.append(req)
+                continue
+            need = self._needs(req, count)
+            taken = [t + n for t, n in zip(taken, need)]
+            entries.append(Scheduled(req, req.num_computed, count, req.num_computed + count == req.num_tokens))
+            scheduled_ids.add(req.req_id)
+            budget -= count
+
+        slots_left = min(self.cache.free_slots, self.max_num_seqs - len(self.running))
+        while self.waiting and budget > 0 and slots_left > 0:
+            req = self.waiting[0]
+            want = min(req.pending, budget)
+            count = self._largest_fit(req, want, taken)
+            if count < 1:
+                if not self.running and not entries:
+                    self.waiting.popleft()
+                    req.status, req.finish_reason = FINISHED, "capacity"
+                    self.finished.append(req)
+                    finished.append(req)
+                    continue
+                break
+            self.waiting.popleft()
+            req.status = RUNNING
+            self.running.append(req)
+            need = self._needs(req, count)
+            taken = [t + n for t, n in zip(taken, need)]
+            entries.append(Scheduled(req, req.num_computed, count, req.num_computed + count == req.num_tokens))
+            scheduled_ids.add(req.req_id)
+            budget -= count
+            slots_left -= 1
+        return StepPlan(entries, preempted, finished)
+
+    # ------------------------------------------------------------------ results
+    def update(self, plan: StepPlan, sampled: Dict[Hashable, int]) -> List[Request]:
+        """After the step ran: advances every scheduled request, appends sampled tokens,
+        finishes and frees.  Returns the requests that finished now."""
+        done: List[Request] = []
+        for e in plan.entries:
+            req = e.request
+            req.num_computed = e.start + e.count
+            if not e.samples:
+                continue
+            tok = int(sampled[req.req_id])
+            req.output.append(tok)
+            reason = None
+            if self.eos_token_id is not None and tok == self.eos_token_id and not req.params.ignore_eos:
+                reason = "stop"
+            elif len(req.output) >= req.params.max_new_tokens:
+                reason = "length"
+            elif req.num_tokens >= self.max_model_len:
+                reason = "length"
+            if reason:
+                self._finish(req, reason)
+                done.append(req)
+        return done

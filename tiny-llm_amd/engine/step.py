@@ -109,26 +109,13 @@ class ModelRunner:
         if T > self.max_tokens:
             raise StepError(f"step brings {T} tokens, the budget is {self.max_tokens}")
 
-        new_reqs = [e.req_id for e in entries if not cm.has(e.req_id)]
-        if len(new_reqs) > cm.free_slots:
-            raise OutOfBlocks(f"{len(new_reqs)} new requests, {cm.free_slots} request slots are free")
-        ctx_lens, new_lens, needs = [], [], []
         for e in entries:
             c = cm.num_tokens(e.req_id) if cm.has(e.req_id) else 0
-            n = c + len(e.tokens)
-            if n > self.max_model_len:
-                raise StepError(f"request {e.req_id!r} would reach {n} tokens, the limit is {self.max_model_len}")
-            ctx_lens.append(c)
-            new_lens.append(n)
-            needs.append(cm.blocks_needed(e.req_id, n))
-        if not cm.can_grow(needs):
-            raise OutOfBlocks("the step needs more cache blocks than are free: "
-                              f"needs {[sum(n[g] for n in needs) for g in range(len(cm.groups))]}, "
-                              f"free {cm.free_blocks()}")
-        for rid in new_reqs:
-            cm.add_request(rid)
-        for e, n in zip(entries, new_lens):
-            cm.grow(e.req_id, n)
+            if c + len(e.tokens) > self.max_model_len:
+                raise StepError(f"request {e.req_id!r} would reach {c + len(e.tokens)} tokens, "
+                                f"the limit is {self.max_model_len}")
+        ctx_lens = cm.reserve_step([(e.req_id, len(e.tokens)) for e in entries])
+        new_lens = [c + len(e.tokens) for c, e in zip(ctx_lens, entries)]
 
         R, G = len(entries), len(cm.groups)
         max_blocks = max(1, max(-(-n // bs) for n in new_lens))
