@@ -1,0 +1,303 @@
+"""The cache manager and the scheduler's decisions, on the host only."""
+import random
+
+import pytest
+
+from tiny_llm_amd.cache import BlockPool, CacheError, CacheManager, NoFreeSlot, OutOfBlocks, RELEASED
+from tiny_llm_amd.engine.scheduler import Request, Scheduler
+from tiny_llm_amd.parts.base import CacheSpec, StateSpec
+from tiny_llm_amd.sampling import SamplingParams
+
+
+# ------------------------------------------------------------------ block pool
+def test_pool_reference_vectors():
+    # (ref) tests/runtime/test_page_pool.cpp:5-23: 10 pages, allocate(10) = 0..9, allocate(12) throws,
+    # freeing a free page throws
+    pool = BlockPool(10)
+    with pytest.raises(OutOfBlocks):
+        pool.allocate(12)
+    assert pool.free_count == 10            # a refused request takes nothing
+    assert pool.allocate(10) == list(range(10))
+    assert pool.free_count == 0
+    pool.free([3, 7])
+    with pytest.raises(CacheError):
+        pool.free([3])
+    with pytest.raises(CacheError):
+        pool.free([5, 5])
+    assert pool.allocate(2) == [7, 3]       # most recently freed first
+    with pytest.raises(CacheError):
+        pool.free([11])
+
+
+def full(n=1):
+    return [CacheSpec(2, 16)] * n
+
+
+def test_groups_by_need():
+    specs = [CacheSpec(2, 16), CacheSpec(2, 16, "window", 8), None, CacheSpec(2, 16), CacheSpec(2, 16, "window", 8),
+             CacheSpec(4, 16)]
+    cm = CacheManager(specs, [None] * 6, block_size=4, num_blocks=10, max_seqs=2)
+    assert [g.entries for g in cm.groups] == [[0, 3], [1, 4], [5]]
+    assert cm.group_of_entry == {0: 0, 3: 0, 1: 1, 4: 1, 5: 2}
+    assert cm.layer_cache(2) is None
+
+
+def test_grow_commit_free_and_reuse():
+    cm = CacheManager(full(2), [None, None], block_size=4, num_blocks=6, max_seqs=3)
+    assert cm.reserve_step([("a", 5)]) == [0]
+    assert cm.block_table("a", 0) == [0, 1]
+    cm.commit("a", 5)
+    assert cm.reserve_step([("a", 3), ("b", 9)]) == [5, 0]     # a: 5 -> 8 needs nothing new; b: 3 blocks
+    assert cm.block_table("a", 0) == [0, 1] and cm.block_table("b", 0) == [2, 3, 4]
+    cm.commit("a", 8)
+    cm.commit("b", 9)
+    with pytest.raises(OutOfBlocks):
+        cm.reserve_step([("a", 1), ("c", 5)])                  # needs 1 + 2, one is free
+    assert not cm.has("c") and cm.free_blocks() == [1] and cm.free_slots == 1   # nothing changed
+    cm.free_request("b")
+    assert cm.free_blocks() == [4]
+    cm.reserve_step([("c", 13)])
+    assert cm.block_table("c", 0) == [4, 3, 2, 5]              # b's pages are used again
+    cm.audit()
+    with pytest.raises(CacheError):
+        cm.free_request("b")
+    with pytest.raises(CacheError):
+        cm.commit("a", 3)                                       # cannot shrink
+    with pytest.raises(CacheError):
+        cm.commit("c", 99)                                      # no blocks for that
+
+
+def test_slots_run_out_and_come_back():
+    cm = CacheManager(full(), [StateSpec((3,))], block_size=4, num_blocks=50, max_seqs=2)
+    assert cm.add_request("a") == 0 and cm.add_request("b") == 1
+    with pytest.raises(NoFreeSlot):
+        cm.add_request("c")
+    with pytest.raises(NoFreeSlot):
+        cm.reserve_step([("c", 1)])
+    cm.free_request("a")
+    assert cm.add_request("c") == 0
+    with pytest.raises(CacheError):
+        cm.add_request("c")
+
+
+def test_window_gives_blocks_back_as_it_passes():
+    spec = [CacheSpec(1, 8), CacheSpec(1, 8, "window", 6)]
+    cm = CacheManager(spec, [None, None], block_size=4, num_blocks=8, max_seqs=2)
+    cm.reserve_step([("a", 10)])
+    cm.commit("a", 10)        # next query at >= 10 reads keys >= 5: block 0 (0..3) of the window group is done
+    assert cm.block_table("a", 0) == [0, 1, 2]
+    assert cm.block_table("a", 1) == [RELEASED, 1, 2]
+    assert cm.free_blocks() == [5, 6]
+    for n in range(11, 22):
+        cm.reserve_step([("a", 1)])
+        cm.commit("a", n)
+        cm.audit()
+    # at 21 tokens the window group holds keys 16.. only: logical blocks 4 and 5
+    assert [b != RELEASED for b in cm.block_table("a", 1)] == [False, False, False, False, True, True]
+    assert cm.free_blocks() == [8 - 6, 8 - 2]
+    cm.free_request("a")
+    assert cm.free_blocks() == [8, 8]
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_no_page_lost_held_twice_or_freed_twice_under_random_orders(seed):
+    rng = random.Random(seed)
+    spec = [CacheSpec(2, 16), CacheSpec(2, 16, "window", 11), CacheSpec(2, 16)]
+    cm = CacheManager(spec, [None, StateSpec((2,)), None], block_size=4, num_blocks=40, max_seqs=5)
+    live = {}
+    n_new = 0
+    for _ in range(600):
+        op = rng.random()
+        if op < 0.55 and (live or True):
+            batch = []
+            ids = list(live)
+            rng.shuffle(ids)
+            for rid in ids[:rng.randint(0, 3)]:
+                batch.append((rid, rng.choice([1, 1, 1, 2, 5, 9])))
+            if rng.random() < 0.4:
+                batch.append((f"n{n_new}", rng.randint(1, 30)))
+            if not batch:
+                continue
+            free_before, slots_before = cm.free_blocks(), cm.free_slots
+            try:
+                before = cm.reserve_step(batch)
+            except (OutOfBlocks, NoFreeSlot):
+                assert cm.free_blocks() == free_before and cm.free_slots == slots_before
+                continue
+            for (rid, n), c in zip(batch, before):
+                assert c == live.get(rid, 0)
+                live[rid] = c + n
+                cm.commit(rid, c + n)
+                for g in range(2):
+                    assert len(cm.block_table(rid, g)) == -(-live[rid] // 4)
+            if batch[-1][0].startswith("n") and batch[-1][0] == f"n{n_new}":
+                n_new += 1
+        elif live:
+            rid = rng.choice(list(live))
+            cm.free_request(rid)
+            del live[rid]
+        cm.audit()
+    for rid in list(live):
+        cm.free_request(rid)
+    assert cm.free_blocks() == [40, 40] and cm.free_slots == 5
+    cm.audit()
+
+
+# ------------------------------------------------------------------- scheduler
+def make_sched(num_blocks=64, block_size=4, max_seqs=4, budget=16, max_len=256, eos=None):
+    cm = CacheManager(full(), [None], block_size=block_size, num_blocks=num_blocks, max_seqs=max_seqs)
+    return cm, Scheduler(cm, max_seqs, budget, max_len, eos)
+
+
+def run_plan(cm, sched, plan, token=7):
+    """What the engine does with a plan, without a model: reserve, commit, 'sample' `token`."""
+    cm.reserve_step([(e.request.req_id, e.count) for e in plan.entries])
+    for e in plan.entries:
+        cm.commit(e.request.req_id, e.start + e.count)
+    tok = token if not callable(token) else None
+    sampled = {e.request.req_id: (token(e.request) if callable(token) else tok) for e in plan.entries if e.samples}
+    done = sched.update(plan, sampled)
+    cm.audit()
+    return done
+
+
+def req(rid, n_prompt, max_new=4, **kw):
+    return Request(rid, list(range(1, n_prompt + 1)), SamplingParams.greedy(max_new, **kw))
+
+
+def test_prompts_are_cut_under_the_token_budget():
+    cm, s = make_sched(budget=16)
+    s.add(req("a", 40))
+    s.add(req("b", 5))
+    p = s.schedule()
+    assert [(e.request.req_id, e.start, e.count, e.samples) for e in p.entries] == [("a", 0, 16, False)]
+    run_plan(cm, s, p)
+    p = s.schedule()
+    assert [(e.request.req_id, e.start, e.count) for e in p.entries] == [("a", 16, 16)]
+    run_plan(cm, s, p)
+    p = s.schedule()        # a's last 8 tokens, then b is admitted with what is left of the budget
+    assert [(e.request.req_id, e.start, e.count, e.samples) for e in p.entries] == [("a", 32, 8, True), ("b", 0, 5, True)]
+    assert p.num_tokens <= 16
+    run_plan(cm, s, p)
+    p = s.schedule()        # both decode: one token each, at position prompt_len + generated - 1
+    assert [(e.request.req_id, e.start, e.count, e.samples) for e in p.entries] == [("a", 40, 1, True), ("b", 5, 1, True)]
+
+
+def test_decoding_goes_before_prompt_portions():
+    cm, s = make_sched(budget=8)
+    s.add(req("a", 3))
+    run_plan(cm, s, s.schedule())
+    s.add(req("b", 20))
+    p = s.schedule()
+    assert [(e.request.req_id, e.count) for e in p.entries] == [("a", 1), ("b", 7)]
+    run_plan(cm, s, p)
+    p = s.schedule()
+    assert [(e.request.req_id, e.count) for e in p.entries] == [("a", 1), ("b", 7)]
+
+
+def test_finish_on_eos_length_and_model_len():
+    cm, s = make_sched(eos=9, max_len=12)
+    s.add(req("stop", 3, max_new=10))
+    s.add(req("len", 3, max_new=2))
+    s.add(req("ctx", 10, max_new=10))
+    s.add(req("ign", 3, max_new=3, ignore_eos=True))
+    run_plan(cm, s, s.schedule(), token=lambda r: 9 if r.req_id in ("stop", "ign") else 7)
+    by = {r.req_id: r for r in s.finished}
+    assert by["stop"].finish_reason == "stop" and by["stop"].output == [9]     # eos is part of the output
+    assert not cm.has("stop")                                                   # freed at once
+    run_plan(cm, s, s.schedule())
+    by = {r.req_id: r for r in s.finished}
+    assert by["len"].finish_reason == "length" and by["len"].output == [7, 7]
+    assert by["ctx"].finish_reason == "length" and len(by["ctx"].prompt) + len(by["ctx"].output) == 12
+    while s.has_work():     # "ign" was admitted a step later (the first step's budget was spent)
+        run_plan(cm, s, s.schedule(), token=lambda r: 9)
+    by = {r.req_id: r for r in s.finished}
+    assert by["ign"].finish_reason == "length" and by["ign"].output == [7, 9, 9]
+    assert {r.req_id for r in s.finished} == {"stop", "len", "ctx", "ign"}
+    assert cm.free_blocks() == [64] and cm.free_slots == 4 and not s.has_work()
+
+
+def test_admission_waits_for_slots_and_blocks():
+    cm, s = make_sched(num_blocks=6, block_size=4, max_seqs=2, budget=64)
+    for rid in "abc":
+        s.add(req(rid, 8, max_new=3))
+    p = s.schedule()
+    assert [e.request.req_id for e in p.entries] == ["a", "b"]      # two slots
+    run_plan(cm, s, p)
+    assert [r.req_id for r in s.waiting] == ["c"]
+    while s.running:
+        run_plan(cm, s, s.schedule())
+    assert [r.req_id for r in s.running + list(s.waiting)] == [] or s.has_work()
+    while s.has_work():
+        run_plan(cm, s, s.schedule())
+    assert sorted(r.req_id for r in s.finished) == ["a", "b", "c"]
+    assert all(len(r.output) == 3 for r in s.finished)
+
+
+def test_when_pages_run_out_the_newest_request_is_preempted_and_recomputed():
+    cm, s = make_sched(num_blocks=5, block_size=4, max_seqs=3, budget=64)
+    s.add(req("old", 8, max_new=12))
+    s.add(req("new", 8, max_new=12))
+    run_plan(cm, s, s.schedule())                 # 2 + 2 blocks, both sampled their first token
+    p = s.schedule()                              # both need a third block, one is free
+    assert [e.request.req_id for e in p.entries] == ["old"]
+    assert [r.req_id for r in p.preempted] == ["new"]
+    assert not cm.has("new") and s.waiting[0].req_id == "new" and s.waiting[0].num_computed == 0
+    assert s.waiting[0].output == [7]             # what it generated is kept and recomputed later
+    run_plan(cm, s, p)
+    steps = 0
+    while s.has_work():
+        plan = s.schedule()
+        assert plan.entries or plan.finished
+        run_plan(cm, s, plan)
+        steps += 1
+        assert steps < 200
+    by = {r.req_id: r for r in s.finished}
+    assert by["old"].finish_reason == "length" and len(by["old"].output) == 12
+    assert by["new"].finish_reason == "length" and len(by["new"].output) == 12 and by["new"].preemptions >= 1
+    assert cm.free_blocks() == [5] and cm.free_slots == 3
+
+
+def test_a_request_that_cannot_fit_alone_ends_with_capacity():
+    cm, s = make_sched(num_blocks=3, block_size=4, max_seqs=2, budget=64)
+    with pytest.raises(ValueError):
+        s.add(req("huge", 13))                    # the prompt alone needs 4 blocks of 3
+    s.add(req("grows", 10, max_new=50))
+    steps = 0
+    while s.has_work():
+        run_plan(cm, s, s.schedule())
+        steps += 1
+        assert steps < 100
+    r = s.finished[0]
+    assert r.finish_reason == "capacity" and len(r.prompt) + len(r.output) == 13   # 12 cached + the one in hand
+    assert cm.free_blocks() == [3]
+
+
+@pytest.mark.parametrize("seed", range(5))
+def test_scheduler_invariants_under_random_load(seed):
+    rng = random.Random(seed)
+    cm, s = make_sched(num_blocks=30, block_size=4, max_seqs=4, budget=24, max_len=80, eos=3)
+    added = 0
+    steps = 0
+    while added < 25 or s.has_work():
+        if added < 25 and rng.random() < 0.5:
+            s.add(req(f"r{added}", rng.randint(1, 40), max_new=rng.randint(1, 30)))
+            added += 1
+        if not s.has_work():
+            continue
+        plan = s.schedule()
+        assert plan.num_tokens <= 24
+        assert len(s.running) <= 4
+        ids = [e.request.req_id for e in plan.entries]
+        assert len(ids) == len(set(ids))
+        for e in plan.entries:
+            assert e.start == e.request.num_computed and e.count >= 1
+            assert e.samples == (e.start + e.count == e.request.num_tokens)
+        run_plan(cm, s, plan, token=lambda r: rng.choice([3, 5, 6, 8, 11, 12]))
+        steps += 1
+        assert steps < 3000
+    assert len(s.finished) == 25 and cm.free_blocks() == [30] and cm.free_slots == 4
+    for r in s.finished:
+        assert r.finish_reason in ("stop", "length", "capacity")
+        if r.finish_reason == "stop":
+            assert r.output[-1] == 3

@@ -1,0 +1,326 @@
+"""The engine above the step function: parts alone, generation through the entry points,
+seeded sampling, preemption, and a toy architecture with a stateful mixer that is
+registered here, in the test, without touching the framework's files."""
+import math
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import plain_llama as plain
+from util import CONFIGS, TINY_A, TINY_B, make_folder, random_tokens, read_weights, rel_err
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    out = {}
+    for name, (cfg, eng, init) in CONFIGS.items():
+        out[name] = make_folder(tmp_path_factory.mktemp(f"engine_{name}"), cfg, seed=11, **init)
+    return out
+
+
+def fake_ctx(lens, q_lens, block_size, n_groups=1, shuffle_seed=0):
+    """A StepContext for requests with lens[r] tokens of which the last q_lens[r] are new."""
+    from tiny_llm_amd.engine.step import StepContext
+    g = torch.Generator().manual_seed(shuffle_seed)
+    nb = sum(-(-l // block_size) for l in lens)
+    perm = torch.randperm(nb + 2, generator=g).tolist()
+    mb = max(-(-l // block_size) for l in lens)
+    bt = torch.zeros(len(lens), mb, dtype=torch.int32)
+    tok_pos, req_of, slots, cu = [], [], [], [0]
+    for r, (L, q) in enumerate(zip(lens, q_lens)):
+        for b in range(-(-L // block_size)):
+            bt[r, b] = perm.pop()
+        for p in range(L - q, L):
+            tok_pos.append(p)
+            req_of.append(r)
+            slots.append(int(bt[r, p // block_size]) * block_size + p % block_size)
+        cu.append(cu[-1] + q)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    T = len(tok_pos)
+    return StepContext(num_tokens=T, num_requests=len(lens), tokens=i32([0] * T), positions=i32(tok_pos),
+                       req_of_token=i32(req_of), cu_seqlens_q=i32(cu), seq_lens=i32(lens),
+                       state_slots=i32(list(range(len(lens)))), logit_rows=None, block_tables=[bt.to(DEV)],
+                       slot_mappings=[i32(slots)], q_lens=list(q_lens),
+                       context_lens=[l - q for l, q in zip(lens, q_lens)], slots_host=list(range(len(lens))),
+                       max_q_len=max(q_lens), max_seq_len=max(lens), block_size=block_size), nb + 2
+
+
+# ----------------------------------------------------------------- parts alone
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_ffn_embedding_head_parts(dtype):
+    from tiny_llm_amd.parts import FEED_FORWARDS, NORMS
+    from tiny_llm_amd.parts.embedding import LMHead, TokenEmbedding
+    g = torch.Generator().manual_seed(3)
+    H, I, V, T = 80, 136, 123, 19
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    x = torch.randn(T, H, generator=g)
+    norm = NORMS.get("rmsnorm")("n", dtype, DEV, hidden_size=H, eps=3e-6)
+    w = 1 + 0.2 * torch.randn(H, generator=g)
+    norm.bind({"n.weight": w.to(DEV)})
+    h = norm.forward(x.to(DEV))
+    assert h.dtype == dtype and rel_err(h, plain.rms_norm(x.double(), w.double(), 3e-6)) < tol
+
+    ffn = FEED_FORWARDS.get("swiglu")("f", dtype, DEV, hidden_size=H, intermediate_size=I)
+    ws = {n: (torch.randn(s, generator=g) / math.sqrt(s[1])).to(dtype) for n, s in
+          (("f.gate_proj.weight", (I, H)), ("f.up_proj.weight", (I, H)), ("f.down_proj.weight", (H, I)))}
+    ffn.bind({k: v.to(DEV) for k, v in ws.items()})
+    hin = torch.randn(T, H, generator=g).to(dtype)
+    res = torch.randn(T, H, generator=g)
+    out = ffn.forward(hin.to(DEV), None, res.clone().to(DEV))
+    act = None if dtype == torch.float32 else dtype
+    ref = res.double() + plain.swiglu(hin.double(), ws["f.gate_proj.weight"].double(), ws["f.up_proj.weight"].double(),
+                                      ws["f.down_proj.weight"].double(), act)
+    assert out.dtype == torch.float32 and rel_err(out, ref) < tol
+
+    emb = TokenEmbedding("e", dtype, DEV, vocab_size=V, hidden_size=H)
+    table = torch.randn(V, H, generator=g).to(dtype)
+    emb.bind({"e.weight": table.to(DEV)})
+    ids = [5, 0, V - 1, 5]
+    assert torch.equal(emb.forward(torch.tensor(ids, dtype=torch.int32, device=DEV)).cpu(), table.float()[ids])
+    head = LMHead("lm", dtype, DEV, vocab_size=V, hidden_size=H)
+    head.bind({"lm.weight": table.to(DEV)})
+    assert rel_err(head.forward(hin.to(DEV)), hin.double() @ table.double().T) < tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nq,nkv,hd,bs,window", [(6, 2, 48, 16, 0), (4, 4, 16, 8, 0), (5, 1, 80, 32, 0), (4, 2, 32, 8, 9)])
+def test_attention_part_alone(dtype, nq, nkv, hd, bs, window):
+    """Two steps through the part: a prefix of every request, then the rest (mixed lengths),
+    against the plain functions over the whole sequences."""
+    from tiny_llm_amd.parts import MIXERS, LayerCache
+    g = torch.Generator().manual_seed(hd + bs)
+    H = 72
+    lens, cut = [37, 9, 64, 1], [30, 8, 17, 0]
+    attn = MIXERS.get("attention")("a", dtype, DEV, hidden_size=H, num_heads=nq, num_kv_heads=nkv, head_dim=hd,
+                                   window=window, position={"kind": "rotary", "head_dim": hd, "theta": 777.0,
+                                                            "max_position": 128})
+    ws = {f"a.{n}_proj.weight": (torch.randn(s, generator=g) * f).to(dtype) for n, s, f in
+          (("q", (nq * hd, H), 0.3), ("k", (nkv * hd, H), 0.3), ("v", (nkv * hd, H), 0.1), ("o", (H, nq * hd), 0.1))}
+    attn.bind({k: v.to(DEV) for k, v in ws.items()})
+    hs = [torch.randn(L, H, generator=g).to(dtype) for L in lens]
+    act = None if dtype == torch.float32 else dtype
+    cos, sin = plain.rope_table(128, hd, 777.0)
+    refs = []
+    for h in hs:
+        L = h.shape[0]
+        rnd = (lambda t: t) if act is None else (lambda t: t.to(act).double())
+        q = rnd(plain.apply_rope(rnd(plain.linear(h.double(), ws["a.q_proj.weight"].double())).view(L, nq, hd), range(L), cos, sin))
+        k = rnd(plain.apply_rope(rnd(plain.linear(h.double(), ws["a.k_proj.weight"].double())).view(L, nkv, hd), range(L), cos, sin))
+        v = rnd(plain.linear(h.double(), ws["a.v_proj.weight"].double())).view(L, nkv, hd)
+        o = rnd(plain.attention_fast(q, k, v, range(L), window)).reshape(L, nq * hd)
+        refs.append(plain.linear(o, ws["a.o_proj.weight"].double()))
+    # step 1: prefixes; step 2: the rest.  Same physical blocks in both steps.
+    ctx2, nblocks = fake_ctx(lens, [l - c for l, c in zip(lens, cut)], bs)
+    kc = torch.full((nblocks, nkv, bs, hd), float("nan"), dtype=dtype, device=DEV)
+    vc = torch.full((nblocks, nkv, bs, hd), float("nan"), dtype=dtype, device=DEV)
+    cache = LayerCache(kc, vc, 0, True)
+    live = [r for r, c in enumerate(cut) if c > 0]
+    ctx1, _ = fake_ctx([cut[r] for r in live], [cut[r] for r in live], bs)
+    ctx1.block_tables = [ctx2.block_tables[0][live][:, :ctx1.block_tables[0].shape[1]].contiguous()]
+    slots = []
+    for i, r in enumerate(live):
+        slots += [int(ctx1.block_tables[0][i, p // bs]) * bs + p % bs for p in range(cut[r])]
+    ctx1.slot_mappings = [torch.tensor(slots, dtype=torch.int32, device=DEV)]
+    tol = 2e-5 if dtype == torch.float32 else 1.5e-2
+    h1 = torch.cat([hs[r][:cut[r]] for r in live]).to(DEV)
+    out1 = attn.forward(h1, ctx1, cache, None, torch.zeros(h1.shape[0], H, device=DEV))
+    assert rel_err(out1, torch.cat([refs[r][:cut[r]] for r in live])) < tol
+    h2 = torch.cat([hs[r][cut[r]:] for r in range(len(lens))]).to(DEV)
+    res = torch.randn(h2.shape[0], H, generator=g)
+    out2 = attn.forward(h2, ctx2, cache, None, res.clone().to(DEV))
+    ref2 = res.double() + torch.cat([refs[r][cut[r]:] for r in range(len(lens))])
+    assert rel_err(out2, ref2) < tol
+
+
+# ------------------------------------------------------------------ generation
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_through_the_entry_point(name, folders):
+    from tiny_llm_amd import Engine, SamplingParams
+    cfg, eng_kw, _ = CONFIGS[name]
+    w, c = read_weights(folders[name])
+    prompts = [random_tokens(n, cfg["vocab_size"], 50 + n) for n in ((5, 17, 31) if name == "A" else (1, 9, 40, 100))]
+    eng = Engine(folders[name], dtype="float32", max_num_seqs=4, max_num_batched_tokens=8 if name == "B" else 64, **eng_kw)
+    out = eng.generate(prompts, SamplingParams.greedy(16 if name == "A" else 6, ignore_eos=True))
+    for p, o in zip(prompts, out):
+        assert o == plain.greedy_generate(w, c, p, len(o))
+    assert eng.runner.cache.free_blocks() == [g.pool.num_blocks for g in eng.runner.cache.groups]
+    # eos ends a request and is part of its output
+    first = out[0][0]
+    eng.scheduler.eos_token_id = first
+    assert eng.generate([prompts[0]], SamplingParams.greedy(16))[0] == [first]
+
+
+def test_bfloat16_generation_follows_the_plain_model(folders):
+    from tiny_llm_amd import Engine, SamplingParams
+    cfg, eng_kw, _ = CONFIGS["A"]
+    w, c = read_weights(folders["A"], round_to=torch.bfloat16)
+    prompts = [random_tokens(n, cfg["vocab_size"], 70 + n) for n in (5, 17, 31)]
+    eng = Engine(folders["A"], dtype="bfloat16", max_num_seqs=4, **eng_kw)
+    out = eng.generate(prompts, SamplingParams.greedy(16, ignore_eos=True))
+    for p, o in zip(prompts, out):
+        ref = plain.llama_forward(w, c, p + o, act_dtype=torch.bfloat16)
+        for i, tok in enumerate(o):
+            row = ref[len(p) + i - 1]
+            # the chosen token is the plain model's argmax, or within rounding of it
+            assert float(row.max() - row[tok]) <= 2e-2 * float(row.abs().max())
+
+
+def test_seeded_sampling_does_not_depend_on_batching(folders):
+    """Temperature 0.8 with a fixed seed: the same tokens whether the request runs alone, beside
+    others, or with its prompt cut into portions of 8."""
+    from tiny_llm_amd import Engine, SamplingParams
+    cfg, eng_kw, _ = CONFIGS["B"]
+    prompts = [random_tokens(n, cfg["vocab_size"], 90 + n) for n in (1, 9, 40, 100)]
+    sp = [SamplingParams(max_new_tokens=24, temperature=0.8, top_k=50, top_p=0.95, seed=1234 + i, ignore_eos=True)
+          for i in range(4)]
+    together = Engine(folders["B"], dtype="float32", max_num_seqs=4, max_num_batched_tokens=8, **eng_kw).generate(prompts, sp)
+    alone_eng = Engine(folders["B"], dtype="float32", max_num_seqs=4, max_num_batched_tokens=512, **eng_kw)
+    for i in range(4):
+        assert alone_eng.generate([prompts[i]], sp[i])[0] == together[i]
+    assert len({tuple(t) for t in together}) == 4
+    # the plain chain, fed the engine's documented uniform numbers, draws the same tokens
+    w, c = read_weights(folders["B"])
+    toks = list(prompts[1])
+    for tok in together[1][:6]:
+        logits = plain.llama_forward(w, c, toks)[-1].float()
+        u = plain.uniform_for(sp[1].seed, len(toks))
+        assert plain.sample_token(logits, 0.8, 50, 0.95, u) == tok
+        toks.append(tok)
+
+
+def test_preemption_recomputes_and_gives_the_same_tokens(folders):
+    from tiny_llm_amd import Engine, SamplingParams
+    cfg, eng_kw, _ = CONFIGS["A"]
+    prompts = [random_tokens(n, cfg["vocab_size"], 130 + n) for n in (30, 28, 26)]
+    sp = SamplingParams.greedy(40, ignore_eos=True)
+    roomy = Engine(folders["A"], dtype="float32", max_num_seqs=4, kv_block_size=16).generate(prompts, sp)
+    tight = Engine(folders["A"], dtype="float32", max_num_seqs=4, kv_block_size=16, num_kv_blocks=9)
+    out = tight.generate(prompts, sp)            # 3 x 70 tokens need 15 blocks, 9 exist
+    assert out == roomy
+    assert sum(r.preemptions for r in tight.requests.values()) >= 1
+    assert all(r.finish_reason == "length" for r in tight.requests.values())
+    tight.runner.cache.audit()
+    assert tight.runner.cache.free_blocks() == [9]
+
+
+def test_command_line_generates_from_prompt_ids(folders):
+    cfg = CONFIGS["A"][0]
+    prompt = random_tokens(12, cfg["vocab_size"], 5)
+    w, c = read_weights(folders["A"])
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "tiny_llm"), "--model_path", folders["A"],
+                           "--nodo_sample", "--max_new_tokens=5", "--dtype", "float32", "--ignore_eos",
+                           "--prompt_ids", ",".join(map(str, prompt))], capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    got = [int(t) for t in proc.stdout.strip().splitlines()[-1].split()]
+    assert got == plain.greedy_generate(w, c, prompt, 5)
+    bad = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "tiny_llm"), "--model_path", "/nonexistent"],
+                         capture_output=True, text=True, timeout=120)
+    assert bad.returncode == 1 and "[Fatal]" in bad.stderr
+
+
+# ------------------------------------------------------ a toy architecture
+def test_toy_stateful_mixer_registers_builds_and_steps(tmp_path):
+    """A mixer with per-request state of fixed size (an exponential running mean), defined here.
+    The toy model mixes it with attention layers, runs one layer twice and lets one run read
+    another run's cache.  Cutting its input differently must not change its logits."""
+    from tiny_llm_amd.config import (EngineConfig, LayerSpec, ModelSpec, PartSpec, PlanEntry, register_architecture,
+                                     unregister_architecture)
+    from tiny_llm_amd.engine.loading import build_runner, random_model
+    from tiny_llm_amd.engine.step import StepEntry
+    from tiny_llm_amd.parts import MIXERS, Mixer, StateSpec, WeightSpec, add_to_residual, register_mixer
+
+    class DecayMixer(Mixer):
+        def __init__(self, prefix, dtype, device, *, hidden_size, decay):
+            super().__init__(prefix, dtype, device)
+            self.hidden_size, self.decay = hidden_size, decay
+
+        def weights(self):
+            return [WeightSpec(f"{self.prefix}.gain", (self.hidden_size,), role="vector", init="ones")]
+
+        def bind(self, tensors):
+            self.gain = tensors[f"{self.prefix}.gain"].float()
+
+        def state_spec(self):
+            return StateSpec((self.hidden_size,), torch.float32)
+
+        def forward(self, h, ctx, cache, state, residual):
+            out = torch.empty_like(h, dtype=torch.float32)
+            t = 0
+            for slot, n in zip(ctx.slots_host, ctx.q_lens):     # each request's tokens, in order, once
+                s = state[slot]
+                for i in range(n):
+                    s = self.decay * s + h[t + i].float()
+                    out[t + i] = s * self.gain
+                state[slot] = s
+                t += n
+            return add_to_residual(residual, out)
+
+    def read(raw):
+        return dict(raw)
+
+    def build(cfg):
+        H = cfg["hidden_size"]
+        norm = PartSpec("rmsnorm", {"hidden_size": H, "eps": 1e-5})
+        ffn = PartSpec("swiglu", {"hidden_size": H, "intermediate_size": cfg["intermediate_size"]})
+        attn = PartSpec("attention", {"hidden_size": H, "num_heads": 4, "num_kv_heads": 2, "head_dim": 16,
+                                      "position": {"kind": "rotary", "head_dim": 16, "theta": 100.0, "max_position": 256}})
+        win = PartSpec("attention", {"hidden_size": H, "num_heads": 4, "num_kv_heads": 2, "head_dim": 16, "window": 5,
+                                     "position": {"kind": "none"}})
+        toy = PartSpec("toy_decay", {"hidden_size": H, "decay": 0.5})
+        layers = tuple(LayerSpec(f"model.layers.{i}", "pre_norm", norm, m, norm, ffn) for i, m in enumerate([attn, toy, win]))
+        # layer 0, layer 1 (state), layer 2 (window), layer 0 again with a cache of its own,
+        # then layer 0 once more reading the first run's cache
+        plan = (PlanEntry(0), PlanEntry(1), PlanEntry(2), PlanEntry(0), PlanEntry(0, cache_of=0))
+        return ModelSpec("ToyForCausalLM", cfg["vocab_size"], H, 256, PartSpec("token_embedding", {
+            "vocab_size": cfg["vocab_size"], "hidden_size": H}), layers, plan, norm,
+            PartSpec("lm_head", {"vocab_size": cfg["vocab_size"], "hidden_size": H, "tied": True}))
+
+    register_mixer("toy_decay", DecayMixer)
+    register_architecture("ToyForCausalLM", read, build)
+    try:
+        raw = {"architectures": ["ToyForCausalLM"], "hidden_size": 64, "intermediate_size": 96, "vocab_size": 101}
+        engine = EngineConfig(dtype="float32", kv_block_size=4, max_cache_tokens=256, max_num_seqs=3,
+                              max_num_batched_tokens=256, use_graphs=False)
+        _, dec = random_model(raw, engine, seed=1, std=0.3)
+        runner = build_runner(dec, engine)
+        assert [g.entries for g in runner.cache.groups] == [[0, 3], [2]]       # full and windowed groups
+        assert runner.decoder.states[1].shape == (3, 64) and runner.decoder.states[0] is None
+        a, b = random_tokens(45, 101, 1), random_tokens(23, 101, 2)
+        whole = runner.step([StepEntry("a", a, list(range(45))), StepEntry("b", b, list(range(23)))]).cpu()
+        runner.finish("a")
+        runner.finish("b")
+        got_a, got_b = [], []
+        at_a = at_b = 0
+        for na, nb in [(7, 2), (2, 0), (19, 11), (1, 1), (16, 9)]:
+            ents = [StepEntry("a", a[at_a:at_a + na], list(range(na)))] if na else []
+            if nb:
+                ents.append(StepEntry("b", b[at_b:at_b + nb], list(range(nb))))
+            l = runner.step(ents).cpu()
+            got_a.append(l[:na])
+            got_b.append(l[na:])
+            at_a, at_b = at_a + na, at_b + nb
+            runner.cache.audit()
+        assert at_a == 45 and at_b == 23
+        assert rel_err(torch.cat(got_a), whole[:45]) < 1e-5 and rel_err(torch.cat(got_b), whole[45:]) < 1e-5
+        # the window group gave back what its window passed; the full group kept everything
+        assert sum(x >= 0 for x in runner.cache.block_table("a", 1)) <= 3
+        assert all(x >= 0 for x in runner.cache.block_table("a", 0))
+        # a slot is zeroed when a new request takes it
+        runner.finish("a")
+        again = runner.step([StepEntry("c", a, list(range(45)))]).cpu()
+        assert rel_err(again, whole[:45]) < 1e-5
+        # the state matters: another decay, other logits
+        dec.layers[1].mixer.decay = 0.9
+        runner.finish("c")
+        assert rel_err(runner.step([StepEntry("d", a, list(range(45)))]).cpu(), whole[:45]) > 1e-3
+    finally:
+        MIXERS.unregister("toy_decay")
+        unregister_architecture("ToyForCausalLM")

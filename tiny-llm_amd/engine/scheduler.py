@@ -18,12 +18,15 @@ Decisions (all host-side, testable without a GPU):
   token budget are left.
 * Budget: at most `max_num_batched_tokens` tokens per step; a prompt portion is
   `min(remaining, budget left, blocks that fit)`.
-* When pages run out for a running request, the request admitted last (other than
-  ones already scheduled this step) is preempted: its blocks and slot are given
-  back at once and it returns to the FRONT of the waiting queue with nothing
-  computed; prompt and output so far are recomputed when it is admitted again.  A
-  request that cannot fit even alone, with every other block free, is finished with
-  reason "capacity": the engine never deadlocks.
+* A waiting request is admitted only when the blocks for all its tokens are free
+  (its first portion may still be shorter: the token budget).
+* When pages run out for a running request, the request admitted last among those
+  not yet scheduled in the step (possibly the request itself) is preempted: its
+  blocks and slot are given back at once and it returns to the FRONT of the waiting
+  queue with nothing computed; prompt and output so far are recomputed when it is
+  admitted again.  No request is admitted in a step that preempted.  A request that
+  cannot go on even alone, with every other block free, is finished with reason
+  "capacity": the engine never deadlocks.
 """
 from __future__ import annotations
 
@@ -170,18 +173,21 @@ class Scheduler:
                 count = self._largest_fit(req, want, taken)
                 if count >= 1 and (count == want or req.pending > 1):
                     break
-                # not even the next token fits: take the blocks of the request admitted last
-                victims = [r for r in reversed(self.running) if r is not req and r.req_id not in scheduled_ids]
-                if not victims:
+                # Not even the next token fits.  The request admitted last among those not yet
+                # scheduled in this step gives its blocks back; that may be this request itself.
+                victim = next(r for r in reversed(self.running) if r.req_id not in scheduled_ids)
+                if victim is req:
                     count = 0
+                    if len(self.running) == 1 and not entries:
+                        self._finish(req, "capacity")      # alone, every other block free: it can never go on
+                        finished.append(req)
+                    else:
+                        self._preempt(req)
+                        preempted.append(req)
                     break
-                self._preempt(victims[0])
-                preempted.append(victims[0])
+                self._preempt(victim)
+                preempted.append(victim)
             if count == 0:
-                if not entries and len(self.running) == 1:
-                    # alone, nothing scheduled before it, and still no room: it can never go on
-                    self._finish(req, "capacity")
-                    finished.append(req)
                 continue
             need = self._needs(req, count)
             taken = [t + n for t, n in zip(taken, need)]
@@ -189,19 +195,21 @@ class Scheduler:
             scheduled_ids.add(req.req_id)
             budget -= count
 
+        # Admission, in arrival order, while a slot, the blocks for ALL the request's tokens and some
+        # budget are left; none in a step that preempted (the freed blocks are for those that run).
         slots_left = min(self.cache.free_slots, self.max_num_seqs - len(self.running))
-        while self.waiting and budget > 0 and slots_left > 0:
+        while self.waiting and budget > 0 and slots_left > 0 and not preempted:
             req = self.waiting[0]
-            want = min(req.pending, budget)
-            count = self._largest_fit(req, want, taken)
-            if count < 1:
-                if not self.running and not entries:
-                    self.waiting.popleft()
+            need_all = self.cache.blocks_needed(req.req_id, req.num_tokens)
+            if not self._fits(need_all, taken):
+                if any(n > self.cache.num_blocks for n in need_all):
+                    self.waiting.popleft()                 # more than the whole pool: it can never run
                     req.status, req.finish_reason = FINISHED, "capacity"
                     self.finished.append(req)
                     finished.append(req)
                     continue
                 break
+            count = min(req.pending, budget)
             self.waiting.popleft()
             req.status = RUNNING
             self.running.append(req)
