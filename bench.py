@@ -100,7 +100,10 @@ def run(args):
 
     # prefill of one 2,048-token prompt in one step, its last logits sampled
     pf_tokens = PREFILL_TOKENS
-    pf_s = prefill_run(3)
+    pf_s = prefill_run(3) if args.only in ("all", "prefill") else float("nan")
+    if args.only == "prefill":
+        print(json.dumps({"prefill_tok_s": round(pf_tokens / pf_s, 1), "ms": round(pf_s * 1e3, 3)}), flush=True)
+        return
     pf_flops = 2.0 * pf_tokens * matmul_params + L * nq * 2.0 * pf_tokens * pf_tokens * hd + 2.0 * V * H
     pf_frac = pf_flops / pf_s / (PEAK_TFLOPS[args.dtype] * 1e12)
 
@@ -111,7 +114,7 @@ def run(args):
     achieved = bytes_per_step / (dt / args.steps) / 1e9
 
     points = {}
-    for b in (1, 64):
+    for b in ((1, 64) if args.only == "all" else ()):
         d, _ = decode_run(b, args.steps, args.warmup)
         points[f"decode_b{b}"] = round(b * args.steps / d, 1)
 
@@ -142,6 +145,8 @@ def main():
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration (0: all)")
     ap.add_argument("--block-size", type=int, default=16)
+    ap.add_argument("--only", default="all", choices=["all", "decode", "prefill"],
+                    help="profiling aid: time only the decode batch or only the prefill")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         if int(os.environ.get("RANK", "0")) == 0:

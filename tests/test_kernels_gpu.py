@@ -234,7 +234,8 @@ def test_rope_invariants():
 
 
 # ------------------------------------------------------------- paged attention
-def _paged_case(dtype, lens, q_lens, nq, nkv, hd, bs, window=0, seed=0, boost=None, shuffle=True):
+def _paged_case(dtype, lens, q_lens, nq, nkv, hd, bs, window=0, seed=0, boost=None, shuffle=True,
+                impl="generic", n_splits=1):
     """Builds a batch: request r has lens[r] cached tokens, the last q_lens[r] are this step's
     queries.  Returns engine output and the plain result, both [T, nq, hd]."""
     g = torch.Generator().manual_seed(seed)
@@ -255,7 +256,7 @@ def _paged_case(dtype, lens, q_lens, nq, nkv, hd, bs, window=0, seed=0, boost=No
             k[far] = 0
             k[far, :, 0] = 6.0
             q[L - 1] = 0
-            q[L - 1, :, 0] = 6.0 * math.sqrt(hd) / 6.0 * 3
+            q[L - 1, :, 0] = 3.0 * math.sqrt(hd)          # score 18 against random ones of order 1
         for b in range(-(-L // bs)):
             blk = perm.pop()
             bt[r, b] = blk
@@ -269,10 +270,24 @@ def _paged_case(dtype, lens, q_lens, nq, nkv, hd, bs, window=0, seed=0, boost=No
         pos += list(range(L - ql, L))
     q = torch.cat(qs).reshape(-1, nq * hd).contiguous()
     out = torch.empty_like(q).to(DEV)
-    ops().paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), bt.to(DEV),
-                          torch.tensor(req_of, dtype=torch.int32, device=DEV),
-                          torch.tensor(pos, dtype=torch.int32, device=DEV), out, nq, nkv, hd,
-                          1.0 / math.sqrt(hd), window)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    if impl == "generic":
+        ops().paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), bt.to(DEV), i32(req_of), i32(pos), out, nq, nkv,
+                              hd, 1.0 / math.sqrt(hd), window)
+    else:
+        # query tiles of at most 16 // (nq / nkv) tokens, as the step context builds them
+        per = 16 // (nq // nkv)
+        t_req, t_tok0, t_ntok, t = [], [], [], 0
+        for r, ql in enumerate(q_lens):
+            for s0 in range(0, ql, per):
+                t_req.append(r)
+                t_tok0.append(t + s0)
+                t_ntok.append(min(per, ql - s0))
+            t += ql
+        T = q.shape[0]
+        scratch = torch.full((max(1, n_splits * T * nq * (hd + 2)),), float("nan"), device=DEV)
+        ops().flash_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), bt.to(DEV), (i32(t_req), i32(t_tok0), i32(t_ntok)),
+                              i32(pos), out, nq, nkv, hd, 1.0 / math.sqrt(hd), window, n_splits, scratch)
     return out.reshape(-1, nq, hd), torch.cat(refs)
 
 
@@ -302,6 +317,45 @@ def test_paged_attention_window_edge(dtype, window):
     out, ref = _paged_case(dtype, lens=[90, 40, 64], q_lens=[90, 1, 5], nq=4, nkv=2, hd=32, bs=8,
                            window=window, seed=window)
     assert rel(out, ref) < tol(dtype, 2e-6, 8e-3)
+
+
+FLASH_SHAPES = [(4, 2, 48, 32), (32, 4, 64, 16), (3, 1, 32, 8), (8, 8, 16, 16), (6, 2, 80, 16), (16, 1, 128, 64),
+                (5, 5, 112, 8), (12, 4, 96, 16)]
+
+
+@pytest.mark.parametrize("n_splits", [1, 3])
+@pytest.mark.parametrize("nq,nkv,hd,bs", FLASH_SHAPES)
+def test_flash_attention_mixed_batch(nq, nkv, hd, bs, n_splits):
+    out, ref = _paged_case(torch.bfloat16, lens=[123, 107, 65, 1, 300, 2], q_lens=[123, 40, 1, 1, 1, 2], nq=nq,
+                           nkv=nkv, hd=hd, bs=bs, seed=hd + bs, impl="flash", n_splits=n_splits)
+    assert not torch.isnan(out).any()
+    assert rel(out, ref) < 8e-3
+
+
+@pytest.mark.parametrize("n_splits", [1, 2, 7])
+def test_flash_attention_far_key_among_hundreds(n_splits):
+    for far in (0, 15, 16, 63, 64, 255, 256, 511, 699):
+        out, ref = _paged_case(torch.bfloat16, lens=[700], q_lens=[1], nq=8, nkv=1, hd=64, bs=16, seed=far,
+                               boost=far, impl="flash", n_splits=n_splits)
+        assert rel(out, ref) < 8e-3, far
+
+
+@pytest.mark.parametrize("window", [1, 7, 16, 33, 100])
+def test_flash_attention_window_edge(window):
+    for n_splits in (1, 2):
+        out, ref = _paged_case(torch.bfloat16, lens=[190, 40, 64, 130], q_lens=[190, 1, 5, 1], nq=4, nkv=2, hd=32,
+                               bs=8, window=window, seed=window, impl="flash", n_splits=n_splits)
+        assert not torch.isnan(out).any()
+        assert rel(out, ref) < 8e-3
+
+
+def test_flash_attention_decode_batch():
+    """Single decoded tokens of many requests of very different lengths, keys split over workgroups."""
+    lens = [1, 2, 63, 64, 65, 127, 128, 129, 500, 1000, 17, 256]
+    for n_splits in (1, 4):
+        out, ref = _paged_case(torch.bfloat16, lens=lens, q_lens=[1] * len(lens), nq=32, nkv=4, hd=64, bs=16,
+                               seed=5, impl="flash", n_splits=n_splits)
+        assert rel(out, ref) < 8e-3
 
 
 def test_paged_attention_reduces_to_library_routine():

@@ -87,6 +87,294 @@ __global__ __launch_bounds__(TL_WAVE) void paged_attention_kernel(
   }
 }
 
+
+// ============================================================== bfloat16 on MFMA
+// flash_attn_bf16_kernel: the same function on the matrix cores, for head sizes
+// that are multiples of 16 up to 128 and up to 16 query heads per kv head.
+//
+// A workgroup (four wave64) owns a tile of 16 query rows that share one request and
+// one kv head: `tile_ntok` consecutive tokens times the G query heads of the group,
+// row = token * G + head.  The four waves split the 64-key tiles of the request's
+// cache between them (and `n_splits` workgroups split them further for decoding
+// with few requests), each with a private LDS staging area, and merge their running
+// (max, sum, output) at the end.  Scores are computed transposed, S^T = K Q^T, with
+// v_mfma_f32_16x16x32_bf16: a lane then holds 16 scores of ONE query row, so the
+// online softmax is lane-local up to two shuffles, the probabilities are already in
+// the B-operand layout of the second product O^T = V^T P^T, and the output
+// accumulator of a lane belongs to that same row.  The probabilities enter the second
+// product as a sum of two bfloat16 terms, so no accuracy is lost against a float32
+// softmax times bfloat16 values.  V is transposed on its way into
+// LDS.  Rows of a tile outside [kv_begin, kv_end) are zero-filled instead of read:
+// stale pages may hold anything, and 0 * NaN is NaN.
+constexpr int FA_THREADS = 256, FA_WAVES = 4, FA_KT = 64, FA_VP = 68;
+
+template <int HDT>
+__global__ __launch_bounds__(FA_THREADS) void flash_attn_bf16_kernel(
+    const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_cache,
+    const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int max_blocks,
+    const int32_t* __restrict__ tile_req, const int32_t* __restrict__ tile_tok0,
+    const int32_t* __restrict__ tile_ntok, const int32_t* __restrict__ positions, bf16_t* __restrict__ out,
+    int64_t out_stride, float* __restrict__ part_o, float* __restrict__ part_ml, int nq, int nkv,
+    int block_size, float scale, int window, int n_splits, int n_tokens) {
+  constexpr int HD = HDT * 16;
+  constexpr int KS = (HD + 31) / 32;       // k-steps of the score product
+  constexpr int KP = KS * 32 + 8;          // LDS row stride of the K tile (elements)
+  constexpr int K_ELEMS = FA_KT * KP, V_ELEMS = HD * FA_VP;
+  constexpr int WAVE_ELEMS = K_ELEMS + V_ELEMS;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  bf16_t* smem = (bf16_t*)smem_raw;
+
+  const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
+  const int r16 = lane % 16, g = lane / 16;
+  const int tile = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
+  const int G = nq / nkv;
+  const int req = tile_req[tile], tok0 = tile_tok0[tile], ntok = tile_ntok[tile];
+  const int32_t* bt = block_tables + (int64_t)req * max_blocks;
+  bf16_t* Kl = smem + wave * WAVE_ELEMS;
+  bf16_t* Vl = Kl + K_ELEMS;
+
+  // this lane's query row
+  const int tok_local = r16 / G, hh = r16 % G;
+  const bool row_valid = tok_local < ntok;
+  const int tok = tok0 + (row_valid ? tok_local : 0);
+  const int head = kvh * G + hh;
+  const int pos = row_valid ? positions[tok] : -1;
+  const int row_lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
+
+  // key range of the tile: union over its rows
+  int hi = pos, lo = row_valid ? row_lo : 0x7fffffff;
+#pragma unroll
+  for (int off = 8; off > 0; off >>= 1) {
+    hi = max(hi, __shfl_xor(hi, off, TL_WAVE));
+    lo = min(lo, __shfl_xor(lo, off, TL_WAVE));
+  }
+  const int kv_end = hi + 1, kv_begin = lo;
+  const int first_tile = kv_begin / FA_KT, last_tile = (kv_end + FA_KT - 1) / FA_KT;
+  const int per_split = (last_tile - first_tile + n_splits - 1) / n_splits;
+  const int range_lo = first_tile + split * per_split;
+  const int range_hi = min(last_tile, range_lo + per_split);
+  const int iters = (max(range_hi - range_lo, 0) + FA_WAVES - 1) / FA_WAVES;
+
+  // query fragments (B operand): row r16, dims ks*32 + g*8 .. +8
+  bf16x8 qf[KS];
+  {
+    const bf16_t* qrow = q + (int64_t)tok * q_stride + (int64_t)head * HD;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d = ks * 32 + g * 8;
+      bf16x8 z = {};
+      qf[ks] = (row_valid && d < HD) ? *(const bf16x8*)(qrow + d) : z;
+    }
+  }
+
+  float m_run = -INFINITY, l_run = 0.f;
+  f32x4 o[HDT];
+#pragma unroll
+  for (int dt = 0; dt < HDT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int it = 0; it < iters; ++it) {
+    const int kt_idx = range_lo + it * FA_WAVES + wave;
+    const bool active = kt_idx < range_hi;
+    if (active) {
+      // stage this wave's tile: lane = key row
+      const int j = kt_idx * FA_KT + lane;
+      const bool in_range = j >= kv_begin && j < kv_end;
+      int64_t row_off = 0;
+      if (in_range) {
+        const int64_t blk = bt[j / block_size];
+        row_off = ((blk * nkv + kvh) * block_size + (j % block_size)) * HD;
+      }
+      const bf16_t* kp = k_cache + row_off;
+      const bf16_t* vp = v_cache + row_off;
+#pragma unroll
+      for (int c = 0; c < KS * 4; ++c) {
+        bf16x8 z = {};
+        const bf16x8 kv8 = (in_range && c * 8 < HD) ? *(const bf16x8*)(kp + c * 8) : z;
+        *(bf16x8*)(Kl + lane * KP + c * 8) = kv8;
+      }
+#pragma unroll
+      for (int c = 0; c < HD / 8; ++c) {
+        bf16x8 z = {};
+        const bf16x8 v8 = in_range ? *(const bf16x8*)(vp + c * 8) : z;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) Vl[(c * 8 + e) * FA_VP + lane] = v8[e];
+      }
+    }
+    __syncthreads();
+    if (active) {
+      // scores, transposed: acc[kt][r] = S^T[key kt*16 + g*4 + r][row r16]
+      f32x4 sc[4];
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt) {
+        sc[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const bf16x8 kf = *(const bf16x8*)(Kl + (kt * 16 + r16) * KP + ks * 32 + g * 8);
+          sc[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], sc[kt], 0, 0, 0);
+        }
+      }
+      float m_tile = -INFINITY;
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int j = kt_idx * FA_KT + kt * 16 + g * 4 + r;
+          const bool ok = row_valid && j <= pos && j >= row_lo;
+          const float sv = ok ? sc[kt][r] * scale : -INFINITY;
+          sc[kt][r] = sv;
+          m_tile = fmaxf(m_tile, sv);
+        }
+      m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, TL_WAVE));
+      m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, TL_WAVE));
+      const float m_new = fmaxf(m_run, m_tile);
+      const bool any = m_new > -INFINITY;
+      const float alpha = any ? expf(m_run - m_new) : 1.f;
+      float psum = 0.f;
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float p = any ? expf(sc[kt][r] - m_new) : 0.f;
+          sc[kt][r] = p;
+          psum += p;
+        }
+      psum += __shfl_xor(psum, 16, TL_WAVE);
+      psum += __shfl_xor(psum, 32, TL_WAVE);
+      l_run = l_run * alpha + psum;
+      m_run = m_new;
+#pragma unroll
+      for (int dt = 0; dt < HDT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[dt][r] *= alpha;
+      // O^T += V^T P^T; the k slots of a step are keys (2s)*16 + g*4 + 0..3 and (2s+1)*16 + g*4 + 0..3
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        // probabilities as two bfloat16 terms, p = hi + lo: the product then carries 16 bits of p
+        bf16x8 pb, pl;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float p0 = sc[2 * st][r], p1 = sc[2 * st + 1][r];
+          pb[r] = (bf16_t)p0;
+          pb[4 + r] = (bf16_t)p1;
+          pl[r] = (bf16_t)(p0 - (float)pb[r]);
+          pl[4 + r] = (bf16_t)(p1 - (float)pb[4 + r]);
+        }
+#pragma unroll
+        for (int dt = 0; dt < HDT; ++dt) {
+          const bf16_t* vrow = Vl + (dt * 16 + r16) * FA_VP + g * 4;
+          const bf16x4 lo4 = *(const bf16x4*)(vrow + (2 * st) * 16);
+          const bf16x4 hi4 = *(const bf16x4*)(vrow + (2 * st + 1) * 16);
+          bf16x8 vf;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            vf[r] = lo4[r];
+            vf[4 + r] = hi4[r];
+          }
+          o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb, o[dt], 0, 0, 0);
+          o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pl, o[dt], 0, 0, 0);
+        }
+      }
+    }
+    __syncthreads();
+  }
+
+  // merge the four waves: each leaves (m, l, O[16][HD]) as floats in its own LDS area
+  constexpr int MROW = HD + 2;
+  float* Mw = (float*)(smem + wave * WAVE_ELEMS);
+#pragma unroll
+  for (int dt = 0; dt < HDT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) Mw[r16 * MROW + dt * 16 + g * 4 + r] = o[dt][r];
+  if (g == 0) {
+    Mw[r16 * MROW + HD] = m_run;
+    Mw[r16 * MROW + HD + 1] = l_run;
+  }
+  __syncthreads();
+  {
+    const int row = tid / 16, dl = tid % 16;
+    const int t_local = row / G, h_local = row % G;
+    if (t_local < ntok) {
+      const int t = tok0 + t_local, h = kvh * G + h_local;
+      float mw[FA_WAVES], M = -INFINITY;
+#pragma unroll
+      for (int wv = 0; wv < FA_WAVES; ++wv) {
+        mw[wv] = ((const float*)(smem + wv * WAVE_ELEMS))[row * MROW + HD];
+        M = fmaxf(M, mw[wv]);
+      }
+      float L = 0.f, wgt[FA_WAVES];
+#pragma unroll
+      for (int wv = 0; wv < FA_WAVES; ++wv) {
+        wgt[wv] = mw[wv] > -INFINITY ? expf(mw[wv] - M) : 0.f;
+        L += wgt[wv] * ((const float*)(smem + wv * WAVE_ELEMS))[row * MROW + HD + 1];
+      }
+      for (int d = dl; d < HD; d += 16) {
+        float acc = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < FA_WAVES; ++wv)
+          acc += wgt[wv] * ((const float*)(smem + wv * WAVE_ELEMS))[row * MROW + d];
+        if (n_splits == 1) {
+          out[(int64_t)t * out_stride + (int64_t)h * HD + d] = (bf16_t)(L > 0.f ? acc / L : 0.f);
+        } else {
+          part_o[(((int64_t)split * n_tokens + t) * nq + h) * HD + d] = acc;
+        }
+      }
+      if (n_splits > 1 && dl == 0) {
+        float* ml = part_ml + (((int64_t)split * n_tokens + t) * nq + h) * 2;
+        ml[0] = M;
+        ml[1] = L;
+      }
+    }
+  }
+}
+
+// Merges the partial results of `n_splits` workgroups per (token, head).
+__global__ void flash_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                     bf16_t* __restrict__ out, int64_t out_stride, int n_tokens, int nq, int hd,
+                                     int n_splits) {
+  const int t = blockIdx.x, h = blockIdx.y;
+  float M = -INFINITY;
+  for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part_ml[(((int64_t)s * n_tokens + t) * nq + h) * 2]);
+  float L = 0.f;
+  for (int s = 0; s < n_splits; ++s) {
+    const float* ml = part_ml + (((int64_t)s * n_tokens + t) * nq + h) * 2;
+    if (ml[0] > -INFINITY) L += expf(ml[0] - M) * ml[1];
+  }
+  for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+    float acc = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+      const int64_t base = ((int64_t)s * n_tokens + t) * nq + h;
+      const float m = part_ml[base * 2];
+      if (m > -INFINITY) acc += expf(m - M) * part_o[base * hd + d];
+    }
+    out[(int64_t)t * out_stride + (int64_t)h * hd + d] = (bf16_t)(L > 0.f ? acc / L : 0.f);
+  }
+}
+
+template <int HDT>
+static int launch_flash(const bf16_t* q, int64_t q_stride, const bf16_t* k_cache, const bf16_t* v_cache,
+                        const int32_t* block_tables, int max_blocks, const int32_t* tile_req,
+                        const int32_t* tile_tok0, const int32_t* tile_ntok, const int32_t* positions, bf16_t* out,
+                        int64_t out_stride, float* part_o, float* part_ml, int n_tiles, int n_tokens, int nq, int nkv,
+                        int block_size, float scale, int window, int n_splits, hipStream_t stream) {
+  constexpr int HD = HDT * 16, KS = (HD + 31) / 32, KP = KS * 32 + 8;
+  constexpr size_t stage = (size_t)FA_WAVES * (FA_KT * KP + HD * FA_VP) * sizeof(bf16_t);
+  constexpr size_t merge = (size_t)FA_WAVES * 16 * (HD + 2) * sizeof(float);
+  static_assert((size_t)(FA_KT * KP + HD * FA_VP) * sizeof(bf16_t) >= 16 * (HD + 2) * sizeof(float),
+                "a wave's merge area must fit its staging area");
+  constexpr size_t smem = stage > merge ? stage : merge;
+  static bool configured = false;
+  if (!configured) {
+    if (hipFuncSetAttribute((const void*)flash_attn_bf16_kernel<HDT>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)smem) != hipSuccess)
+      return TL_ERR_LAUNCH;
+    configured = true;
+  }
+  hipLaunchKernelGGL(flash_attn_bf16_kernel<HDT>, dim3(n_tiles, nkv, n_splits), dim3(FA_THREADS), smem, stream, q,
+                     q_stride, k_cache, v_cache, block_tables, max_blocks, tile_req, tile_tok0, tile_ntok, positions,
+                     out, out_stride, part_o, part_ml, nq, nkv, block_size, scale, window, n_splits, n_tokens);
+  return TL_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -113,6 +401,40 @@ int tl_paged_attention(const void* q, int64_t q_stride, const void* k_cache, con
                        positions, (bf16_t*)out, out_stride, nq, nkv, hd, block_size, scale, window);
   else
     return TL_ERR_ARG;
+  return tl_launch_status();
+}
+
+// bfloat16 only.  Tiles: tile_req / tile_tok0 / tile_ntok [n_tiles] describe groups of at most
+// 16 / (nq / nkv) consecutive tokens of one request.  With n_splits > 1, part_o
+// [n_splits, n_tokens, nq, hd] and part_ml [n_splits, n_tokens, nq, 2] (float32) are scratch.
+int tl_flash_attention(const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
+                       const int32_t* block_tables, int max_blocks, const int32_t* tile_req,
+                       const int32_t* tile_tok0, const int32_t* tile_ntok, const int32_t* positions, void* out,
+                       int64_t out_stride, float* part_o, float* part_ml, int n_tiles, int n_tokens, int nq,
+                       int nkv, int hd, int block_size, float scale, int window, int n_splits,
+                       hipStream_t stream) {
+  if (n_tiles <= 0 || n_tokens <= 0) return TL_OK;
+  if (nq <= 0 || nkv <= 0 || nq % nkv || nq / nkv > 16 || hd <= 0 || hd % 16 || hd > 128 || block_size <= 0 ||
+      max_blocks <= 0 || window < 0 || n_splits < 1 || nkv > 65535 || n_splits > 65535 || q_stride % 8)
+    return TL_ERR_ARG;
+  if (n_splits > 1 && (!part_o || !part_ml)) return TL_ERR_ARG;
+  int rc = TL_ERR_ARG;
+#define TL_FLASH_CASE(HDT)                                                                                       \
+  case HDT:                                                                                                      \
+    rc = launch_flash<HDT>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,           \
+                           block_tables, max_blocks, tile_req, tile_tok0, tile_ntok, positions, (bf16_t*)out,    \
+                           out_stride, part_o, part_ml, n_tiles, n_tokens, nq, nkv, block_size, scale, window,   \
+                           n_splits, stream);                                                                    \
+    break;
+  switch (hd / 16) {
+    TL_FLASH_CASE(1) TL_FLASH_CASE(2) TL_FLASH_CASE(3) TL_FLASH_CASE(4)
+    TL_FLASH_CASE(5) TL_FLASH_CASE(6) TL_FLASH_CASE(7) TL_FLASH_CASE(8)
+  }
+#undef TL_FLASH_CASE
+  if (rc != TL_OK) return rc;
+  if (n_splits > 1)
+    hipLaunchKernelGGL(flash_combine_kernel, dim3(n_tokens, nq), dim3(64), 0, stream, part_o, part_ml, (bf16_t*)out,
+                       out_stride, n_tokens, nq, hd, n_splits);
   return tl_launch_status();
 }
 

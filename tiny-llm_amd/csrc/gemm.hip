@@ -184,6 +184,93 @@ __global__ __launch_bounds__(B_THREADS) void gemm_bf16_kernel(const bf16_t* __re
   }
 }
 
+
+// ============================================================ bfloat16, few rows
+// Decode-shaped products (M <= 64): the weight matrix is streamed once and is the
+// whole cost, so the kernel is built around keeping many 16-byte loads in flight.
+// A workgroup of eight wave64 owns 16 output columns (16 weight rows); the waves
+// split K in blocks of 128 and each accumulates a 16 x 16 tile per group of 16
+// activation rows with v_mfma_f32_16x16x32_bf16 (weight rows as the A operand read
+// straight from global memory, activations as the B operand).  A lane reads 64
+// contiguous bytes of its weight row per block; the k order inside an MFMA is
+// permuted accordingly on both operands, which a dot product does not notice.
+// Partial tiles meet in LDS and are added in a fixed order, so results are
+// deterministic; the residual add is folded into that epilogue.
+constexpr int S_WAVES = 8, S_THREADS = S_WAVES * TL_WAVE, S_COLS = 16, S_KBLK = 128;
+
+template <int MT, typename TO>
+__global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(
+    const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, TO* __restrict__ out,
+    const float* __restrict__ residual, int M, int N, int K, int64_t lda, int64_t ldo) {
+  __shared__ float part[S_WAVES][MT][16][17];
+  const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
+  const int n0 = blockIdx.x * S_COLS;
+  const int r16 = lane % 16, g = lane / 16;
+  const int n = n0 + r16;
+  const bf16_t* wrow = w + (int64_t)min(n, N - 1) * K;
+  const bool n_ok = n < N;
+
+  f32x4 acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const int nblk = (K + S_KBLK - 1) / S_KBLK;
+  for (int blk = wave; blk < nblk; blk += S_WAVES) {
+    const int kb = blk * S_KBLK + g * 32;   // this lane's 32 k of the block
+    bf16x8 fw[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int k = kb + i * 8;
+      bf16x8 z = {};
+      fw[i] = (n_ok && k < K) ? *(const bf16x8*)(wrow + k) : z;
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int m = mt * 16 + r16;
+      const bf16_t* arow = a + (int64_t)min(m, M - 1) * lda;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int k = kb + i * 8;
+        bf16x8 z = {};
+        const bf16x8 fa = (m < M && k < K) ? *(const bf16x8*)(arow + k) : z;
+        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[i], fa, acc[mt], 0, 0, 0);
+      }
+    }
+  }
+  // tile layout: lane holds rows (weight rows) g*4 + r, column (activation row) r16
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) part[wave][mt][g * 4 + r][r16] = acc[mt][r];
+  __syncthreads();
+  for (int e = tid; e < MT * 256; e += S_THREADS) {
+    const int mt = e / 256, m_local = (e % 256) / 16, nn = e % 16;
+    const int m = mt * 16 + m_local;
+    if (m >= M || n0 + nn >= N) continue;
+    float v = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < S_WAVES; ++wv) v += part[wv][mt][nn][m_local];
+    const int64_t o = (int64_t)m * ldo + n0 + nn;
+    if (residual) v += residual[o];
+    out[o] = from_f32<TO>(v);
+  }
+}
+
+template <typename TO>
+static void launch_skinny(const bf16_t* a, const bf16_t* w, TO* out, const float* residual, int M, int N, int K,
+                          int64_t lda, int64_t ldo, hipStream_t stream) {
+  dim3 g((N + S_COLS - 1) / S_COLS), b(S_THREADS);
+  const int mt = (M + 15) / 16;
+  if (mt == 1)
+    hipLaunchKernelGGL((gemm_skinny_bf16_kernel<1, TO>), g, b, 0, stream, a, w, out, residual, M, N, K, lda, ldo);
+  else if (mt == 2)
+    hipLaunchKernelGGL((gemm_skinny_bf16_kernel<2, TO>), g, b, 0, stream, a, w, out, residual, M, N, K, lda, ldo);
+  else if (mt == 3)
+    hipLaunchKernelGGL((gemm_skinny_bf16_kernel<3, TO>), g, b, 0, stream, a, w, out, residual, M, N, K, lda, ldo);
+  else
+    hipLaunchKernelGGL((gemm_skinny_bf16_kernel<4, TO>), g, b, 0, stream, a, w, out, residual, M, N, K, lda, ldo);
+}
+
 }  // namespace
 
 extern "C" {
@@ -202,7 +289,12 @@ int tl_linear(const void* a, const void* w, void* out, const float* residual, in
   } else if (dtype == 1) {
     if (K % 8 || lda % 8) return TL_ERR_ARG;
     dim3 g((N + B_BN - 1) / B_BN, (M + B_BM - 1) / B_BM);
-    if (out_dtype == 0)
+    if (M <= 64 && (out_dtype == 0 || out_dtype == 1)) {
+      if (out_dtype == 0)
+        launch_skinny<float>((const bf16_t*)a, (const bf16_t*)w, (float*)out, residual, M, N, K, lda, ldo, stream);
+      else
+        launch_skinny<bf16_t>((const bf16_t*)a, (const bf16_t*)w, (bf16_t*)out, residual, M, N, K, lda, ldo, stream);
+    } else if (out_dtype == 0)
       hipLaunchKernelGGL(gemm_bf16_kernel<float>, g, dim3(B_THREADS), 0, stream, (const bf16_t*)a,
                          (const bf16_t*)w, (float*)out, residual, M, N, K, lda, ldo);
     else if (out_dtype == 1)

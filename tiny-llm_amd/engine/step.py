@@ -52,9 +52,29 @@ class StepContext:
     max_seq_len: int = 0
     block_size: int = 0
 
+    _tiles: Dict[int, tuple] = field(default_factory=dict)
+
     @property
     def decode_only(self) -> bool:
         return self.max_q_len == 1
+
+    def attention_tiles(self, tokens_per_tile: int):
+        """(tile_req, tile_tok0, tile_ntok) int32 device tensors: every request's tokens of this
+        step cut into groups of at most `tokens_per_tile` (the query tiles of the MFMA attention
+        kernel).  Built once per width and step."""
+        if tokens_per_tile not in self._tiles:
+            req, tok0, ntok = [], [], []
+            t = 0
+            for r, n in enumerate(self.q_lens):
+                for s in range(0, n, tokens_per_tile):
+                    req.append(r)
+                    tok0.append(t + s)
+                    ntok.append(min(tokens_per_tile, n - s))
+                t += n
+            dev = self.tokens.device
+            packed = torch.tensor([req, tok0, ntok], dtype=torch.int32).to(dev, non_blocking=True)
+            self._tiles[tokens_per_tile] = (packed[0], packed[1], packed[2])
+        return self._tiles[tokens_per_tile]
 
 
 class StepError(ValueError):

@@ -70,10 +70,31 @@ class Attention(Mixer):
         ops.rope_store(qkv, ctx.positions, cos, sin, slots, cache.k if cache.write else None,
                        cache.v if cache.write else None, self.num_heads, self.num_kv_heads, self.head_dim, rot)
         attn = torch.empty((T, self.q_size), dtype=self.dtype, device=h.device)
-        ops.paged_attention(qkv[:, :self.q_size], cache.k, cache.v, ctx.block_tables[cache.group],
-                            ctx.req_of_token, ctx.positions, attn, self.num_heads, self.num_kv_heads,
-                            self.head_dim, self.scale, self.window)
+        q = qkv[:, :self.q_size]
+        if ops.flash_attention_supported(self.dtype, self.num_heads, self.num_kv_heads, self.head_dim):
+            group = self.num_heads // self.num_kv_heads
+            tiles = ctx.attention_tiles(16 // group)
+            n_splits, scratch = self._splits(ctx, tiles[0].numel(), T, h.device)
+            ops.flash_attention(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, attn,
+                                self.num_heads, self.num_kv_heads, self.head_dim, self.scale, self.window,
+                                n_splits, scratch)
+        else:
+            ops.paged_attention(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.req_of_token,
+                                ctx.positions, attn, self.num_heads, self.num_kv_heads, self.head_dim,
+                                self.scale, self.window)
         return ops.linear(attn, self.w_o, residual, residual)
+
+    def _splits(self, ctx, n_tiles: int, T: int, device):
+        """How many workgroups share one query tile's keys.  Prompt portions bring enough tiles
+        to fill the chip; a decode step with few requests does not, so its keys are split."""
+        want = 512                                   # workgroups that keep 256 CUs busy
+        have = n_tiles * self.num_kv_heads
+        key_tiles = max(1, -(-ctx.max_seq_len // 64) // 4)       # at least four 64-key tiles per split
+        n_splits = max(1, min(want // max(have, 1), key_tiles, 16))
+        if n_splits == 1:
+            return 1, None
+        return n_splits, torch.empty(n_splits * T * self.num_heads * (self.head_dim + 2), dtype=torch.float32,
+                                     device=device)
 
 
 register_mixer("attention", Attention)
