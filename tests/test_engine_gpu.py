@@ -211,6 +211,30 @@ def test_preemption_recomputes_and_gives_the_same_tokens(folders):
     assert tight.runner.cache.free_blocks() == [9]
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replays_equal_eager_steps(dtype, folders):
+    """Decode steps captured in a HIP graph: every replay, with eager work (prefill of new requests,
+    other batch sizes) between replays, gives the tokens of the eager path."""
+    from tiny_llm_amd import Engine, SamplingParams
+    cfg, eng_kw, _ = CONFIGS["A"]
+    prompts = [random_tokens(n, cfg["vocab_size"], 300 + n) for n in (40, 3, 17, 64, 9)]
+    sp = [SamplingParams.greedy(n, ignore_eos=True) for n in (50, 20, 35, 8, 44)]     # batch sizes change as they end
+    sp[2] = SamplingParams(max_new_tokens=35, temperature=0.9, top_k=20, top_p=0.9, seed=5, ignore_eos=True)
+    outs = {}
+    for graphs in (False, True):
+        eng = Engine(folders["A"], dtype=dtype, max_num_seqs=3, max_num_batched_tokens=32, use_graphs=graphs, **eng_kw)
+        outs[graphs] = eng.generate(prompts, sp)
+        if graphs:
+            assert any(g.graph is not None for g in eng.runner._graphs.values())
+            assert sum(g.runs for g in eng.runner._graphs.values()) > 60
+    if dtype == "float32":
+        assert outs[True] == outs[False]
+    else:
+        # bfloat16: key splits differ between the two paths, so sums round differently now and then
+        same = sum(a == b for x, y in zip(outs[True], outs[False]) for a, b in zip(x[:8], y[:8]))
+        assert same >= 0.8 * sum(min(len(x), 8) for x in outs[True])
+
+
 def test_command_line_generates_from_prompt_ids(folders):
     cfg = CONFIGS["A"][0]
     prompt = random_tokens(12, cfg["vocab_size"], 5)

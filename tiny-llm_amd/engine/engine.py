@@ -80,9 +80,19 @@ class Engine:
         done = list(plan.finished)
         if not plan.entries:
             return done
+        if all(e.count == 1 and e.samples for e in plan.entries):
+            # decode-only step: model and sampler run as one (captured) unit on the device
+            reqs = [e.request for e in plan.entries]
+            toks = self.runner.decode_step([r.req_id for r in reqs], [r.token_slice(e.start, 1)[0] for r, e in
+                                                                      zip(reqs, plan.entries)],
+                                           [r.params for r in reqs], [r.seed for r in reqs],
+                                           [r.num_tokens for r in reqs], use_graph=self.engine_config.use_graphs)
+            done += self.scheduler.update(plan, {r.req_id: t for r, t in zip(reqs, toks)})
+            self.steps_run += 1
+            return done
         entries, rows = [], []
         for e in plan.entries:
-            toks = e.request.tokens[e.start:e.start + e.count]
+            toks = e.request.token_slice(e.start, e.count)
             entries.append(StepEntry(e.request.req_id, toks, [e.count - 1] if e.samples else []))
             if e.samples:
                 rows.append(e.request)

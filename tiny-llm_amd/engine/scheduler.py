@@ -64,6 +64,15 @@ class Request:
     def pending(self) -> int:
         return self.num_tokens - self.num_computed
 
+    def token_slice(self, start: int, count: int) -> List[int]:
+        """tokens[start:start + count] without building the whole list."""
+        n = len(self.prompt)
+        if start >= n:
+            return self.output[start - n:start - n + count]
+        if start + count <= n:
+            return self.prompt[start:start + count]
+        return self.prompt[start:] + self.output[:start + count - n]
+
 
 @dataclass
 class Scheduled:

@@ -96,6 +96,7 @@ class ModelRunner:
             decoder.states[i] = cache.states[i]
         self._pinned: Optional[torch.Tensor] = None
         self._uploaded: Optional[torch.cuda.Event] = None
+        self._graphs: Dict[int, "DecodeGraph"] = {}
 
     # ----------------------------------------------------------------- metadata
     def _host_buffer(self, n: int) -> torch.Tensor:
@@ -201,7 +202,134 @@ class ModelRunner:
             self.cache.commit(e.req_id, c + n)
         return logits
 
+    # ------------------------------------------------------------ decode graphs
+    def decode_step(self, req_ids: Sequence[Hashable], tokens: Sequence[int], params, seeds: Sequence[int],
+                    counters: Sequence[int], use_graph: bool = True) -> List[int]:
+        """One decoded token for each request (its next input token given), sampled on the device.
+        With `use_graph` the whole step (model and sampler) is one HIP graph per batch size,
+        replayed on static buffers; only the metadata upload and the token download remain."""
+        R = len(req_ids)
+        cm = self.cache
+        for rid, t in zip(req_ids, tokens):
+            if not (0 <= int(t) < self.vocab_size):
+                raise StepError(f"token id {t} of request {rid!r} is outside the vocabulary")
+            if (cm.num_tokens(rid) if cm.has(rid) else 0) + 1 > self.max_model_len:
+                raise StepError(f"request {rid!r} would exceed {self.max_model_len} tokens")
+        ctx_lens = cm.reserve_step([(rid, 1) for rid in req_ids])
+        dg = self._graphs.get(R)
+        if dg is None:
+            dg = self._graphs[R] = DecodeGraph(self, R)
+        toks = dg.run(req_ids, tokens, ctx_lens, params, seeds, counters,
+                      capture=use_graph and self.decoder.graph_safe)
+        for rid, c in zip(req_ids, ctx_lens):
+            cm.commit(rid, c + 1)
+        return toks
+
     def finish(self, req_id) -> None:
         """The request is done: its blocks and its state slot are given back."""
         if self.cache.has(req_id):
             self.cache.free_request(req_id)
+
+
+class DecodeGraph:
+    """Static buffers and the captured HIP graph of a decode-only step of `R` requests.
+
+    Everything whose size depends on the step (block-table width, key splits of the attention
+    kernel) is fixed at its maximum, so one capture serves every step of that batch size.  The
+    first run of a size executes eagerly (kernels configure themselves, the allocator warms up);
+    the second is captured; later ones are replayed.  No memset node is recorded: buffers are
+    written by kernels and by the upload only."""
+
+    def __init__(self, runner: ModelRunner, R: int):
+        self.runner, self.R = runner, R
+        cm = runner.cache
+        dev = runner.device
+        bs = cm.block_size
+        self.G = len(cm.groups)
+        self.MB = -(-runner.max_model_len // bs)
+        G, MB = self.G, self.MB
+        # int32 sections: tokens, positions, req_of_token, cu_seqlens, seq_lens, state_slots, logit_rows,
+        # slot mappings, block tables, then sampling: temperature(f32) top_p(f32) top_k counters seeds(i64)
+        sizes = [R, R, R, R + 1, R, R, R] + [R] * G + [R * MB] * G + [R, R, R, R, 2 * R]
+        offs = [0]
+        for n in sizes:
+            offs.append(offs[-1] + ((n + 3) // 4) * 4)
+        self.offs = offs
+        self.host = torch.zeros(offs[-1], dtype=torch.int32, pin_memory=True)
+        self.dev = torch.zeros(offs[-1], dtype=torch.int32, device=dev)
+        self.np = self.host.numpy()
+        sec = lambda i, n: self.dev[offs[i]:offs[i] + n]
+        self.np[offs[2]:offs[2] + R] = np.arange(R)
+        self.np[offs[3]:offs[3] + R + 1] = np.arange(R + 1)
+        self.np[offs[6]:offs[6] + R] = np.arange(R)
+        self.ctx = StepContext(
+            num_tokens=R, num_requests=R, tokens=sec(0, R), positions=sec(1, R), req_of_token=sec(2, R),
+            cu_seqlens_q=sec(3, R + 1), seq_lens=sec(4, R), state_slots=sec(5, R), logit_rows=sec(6, R),
+            block_tables=[sec(7 + G + g, R * MB).view(R, MB) for g in range(G)],
+            slot_mappings=[sec(7 + g, R) for g in range(G)],
+            q_lens=[1] * R, context_lens=[0] * R, slots_host=[0] * R, max_q_len=1,
+            max_seq_len=runner.max_model_len, block_size=bs)
+        s0 = 7 + 2 * G
+        self.temperature = sec(s0, R).view(torch.float32)
+        self.top_p = sec(s0 + 1, R).view(torch.float32)
+        self.top_k = sec(s0 + 2, R)
+        self.counters = sec(s0 + 3, R)
+        self.seeds = sec(s0 + 4, 2 * R).view(torch.int64)
+        self.s0 = s0
+        self.out = torch.zeros(R, dtype=torch.int32, device=dev)
+        self.out_host = torch.zeros(R, dtype=torch.int32, pin_memory=True)
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.runs = 0
+        # the attention kernel's query tiles of a decode step never change: one token per request
+        ar = torch.arange(R, dtype=torch.int32, device=dev)
+        one = torch.ones(R, dtype=torch.int32, device=dev)
+        for width in range(1, 17):
+            self.ctx._tiles[width] = (ar, ar, one)
+
+    def _body(self):
+        from ..kernels import ops
+        logits = self.runner.decoder.forward(self.ctx)
+        ops.sample(logits, self.out, self.temperature, self.top_k, self.top_p, self.seeds, self.counters)
+
+    def run(self, req_ids, tokens, ctx_lens, params, seeds, counters, capture: bool) -> List[int]:
+        R, G, MB, offs, h = self.R, self.G, self.MB, self.offs, self.np
+        cm = self.runner.cache
+        bs = cm.block_size
+        h[offs[0]:offs[0] + R] = tokens
+        h[offs[1]:offs[1] + R] = ctx_lens
+        h[offs[4]:offs[4] + R] = np.asarray(ctx_lens, dtype=np.int32) + 1
+        slots = [cm.slot(rid) for rid in req_ids]
+        h[offs[5]:offs[5] + R] = slots
+        for g in range(G):
+            bt = h[offs[7 + G + g]:offs[7 + G + g] + R * MB].reshape(R, MB)
+            sm = h[offs[7 + g]:offs[7 + g] + R]
+            for r, (rid, c) in enumerate(zip(req_ids, ctx_lens)):
+                table = cm.block_table(rid, g)
+                tb = np.maximum(np.asarray(table, dtype=np.int32), 0)
+                bt[r, :len(table)] = tb
+                sm[r] = tb[c // bs] * bs + c % bs
+        s0 = self.s0
+        fview = self.host.view(torch.float32).numpy()
+        fview[offs[s0]:offs[s0] + R] = [p.temperature if p.do_sample else 0.0 for p in params]
+        fview[offs[s0 + 1]:offs[s0 + 1] + R] = [p.top_p for p in params]
+        h[offs[s0 + 2]:offs[s0 + 2] + R] = [p.top_k for p in params]
+        h[offs[s0 + 3]:offs[s0 + 3] + R] = counters
+        self.host.view(torch.int64).numpy()[offs[s0 + 4] // 2:offs[s0 + 4] // 2 + R] = \
+            [s & 0x7FFFFFFFFFFFFFFF for s in seeds]
+        self.ctx.context_lens = list(ctx_lens)
+        self.ctx.slots_host = slots
+        self.dev.copy_(self.host, non_blocking=True)
+        if not capture or self.runs == 0:
+            self._body()
+        elif self.graph is None:
+            torch.cuda.synchronize()
+            self.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self.graph):
+                self._body()
+            self.graph.replay()
+        else:
+            self.graph.replay()
+        self.runs += 1
+        self.out_host.copy_(self.out, non_blocking=True)
+        torch.cuda.current_stream().synchronize()
+        return self.out_host.tolist()

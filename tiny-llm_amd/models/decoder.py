@@ -59,6 +59,12 @@ class Decoder:
         out.extend([self.final_norm, self.lm_head])
         return out
 
+    @property
+    def graph_safe(self) -> bool:
+        """True if every part (and every mixer's position encoding) may be captured in a HIP graph."""
+        parts = self.parts() + [getattr(l.mixer, "position", None) for l in self.layers]
+        return all(p.graph_safe for p in parts if p is not None)
+
     def weight_specs(self) -> List[WeightSpec]:
         specs: List[WeightSpec] = []
         for p in self.parts():

@@ -22,6 +22,8 @@ from .base import (CacheSpec, LayerCache, Mixer, POSITION_ENCODINGS, WeightSpec,
 
 
 class Attention(Mixer):
+    graph_safe = True
+
     def __init__(self, prefix, dtype, device, *, hidden_size: int, num_heads: int, num_kv_heads: int,
                  head_dim: int, position: dict = None, window: int = 0, scale: float = None,
                  max_position: int = 0):

@@ -76,6 +76,11 @@ class LayerCache:
 class Part:
     """Base of every part: declares weights, receives them, computes."""
 
+    # True if `forward` only enqueues device work whose shape depends on nothing but the batch
+    # size (no host reads of step data, no host loops over requests): such a part may be
+    # captured in a HIP graph for decode steps.  Parts defined elsewhere default to False.
+    graph_safe = False
+
     def __init__(self, prefix: str, dtype: torch.dtype, device: torch.device):
         self.prefix = prefix
         self.dtype = dtype

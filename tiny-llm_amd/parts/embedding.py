@@ -13,6 +13,8 @@ from .base import Part, WeightSpec
 
 
 class TokenEmbedding(Part):
+    graph_safe = True
+
     def __init__(self, prefix, dtype, device, *, vocab_size: int, hidden_size: int):
         super().__init__(prefix, dtype, device)
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
@@ -30,6 +32,8 @@ class TokenEmbedding(Part):
 
 
 class LMHead(Part):
+    graph_safe = True
+
     def __init__(self, prefix, dtype, device, *, vocab_size: int, hidden_size: int, tied_to: str = None):
         super().__init__(prefix, dtype, device)
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)

@@ -15,6 +15,8 @@ from .base import FeedForward, WeightSpec, register_feed_forward
 
 
 class SwiGLU(FeedForward):
+    graph_safe = True
+
     def __init__(self, prefix, dtype, device, *, hidden_size: int, intermediate_size: int):
         super().__init__(prefix, dtype, device)
         self.hidden_size = int(hidden_size)

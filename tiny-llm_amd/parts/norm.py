@@ -15,6 +15,8 @@ from .base import Norm, WeightSpec, register_norm
 
 
 class RMSNorm(Norm):
+    graph_safe = True
+
     def __init__(self, prefix, dtype, device, *, hidden_size: int, eps: float, init: str = "ones"):
         super().__init__(prefix, dtype, device)
         self.hidden_size = int(hidden_size)

@@ -14,6 +14,8 @@ from .base import PositionEncoding, register_position_encoding
 
 
 class RotaryEmbedding(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, prefix, dtype, device, *, head_dim: int, theta: float, max_position: int,
                  rotary_dim: int = None):
         super().__init__(prefix, dtype, device)
@@ -35,6 +37,8 @@ class RotaryEmbedding(PositionEncoding):
 
 
 class NoPositionEncoding(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, prefix, dtype, device, **_):
         super().__init__(prefix, dtype, device)
 
