@@ -134,9 +134,9 @@ def attention_fast(q, k, v, positions, window: int = 0, scale: Optional[float] =
 def swiglu(h: torch.Tensor, Wg, Wu, Wd, act_dtype=None) -> torch.Tensor:
     """g = h Wg^T; g <- silu(g); u = h Wu^T; z = g * u; m = z Wd^T
     (tiny_llm/parser/llama_parser.cpp:225-249)."""
-    g = _rnd(linear(h, Wg), act_dtype)
-    u = _rnd(linear(h, Wu), act_dtype)
-    z = _rnd(silu(g) * u, act_dtype)
+    g = linear(h, Wg)
+    u = linear(h, Wu)
+    z = _rnd(silu(g) * u, act_dtype)      # the serving path stores only the gated product
     return linear(z, Wd)
 
 

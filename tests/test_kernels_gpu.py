@@ -122,6 +122,51 @@ def test_linear_sizes(dtype, M, K, N):
     assert rel(x, ref + res.double()) < 1e-5
 
 
+@pytest.mark.parametrize("M", [1, 5, 16, 17, 40, 64])
+@pytest.mark.parametrize("K,N", [(64, 251), (2048, 96), (176, 64), (5632, 40), (96, 517)])
+def test_linear_with_fused_norm_and_with_fused_swiglu(M, K, N):
+    """The few-row products with a prologue equal the separate kernels (norm, SiLU-gate, product)."""
+    g = torch.Generator().manual_seed(M * 7 + N)
+    x = torch.randn(M + 3, K, generator=g) * 2
+    nw = 1 + 0.1 * torch.randn(K, generator=g)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    res = torch.randn(M, N, generator=g)
+    rows = torch.randperm(M + 3, generator=g)[:M].to(torch.int32)
+    for nwt in (torch.float32, torch.bfloat16):
+        for use_rows in (False, True):
+            src = x[rows.long()] if use_rows else x[:M]
+            h = torch.empty(M, K, dtype=torch.bfloat16, device=DEV)
+            ops().rmsnorm(src.contiguous().to(DEV), nw.to(nwt).to(DEV), 1e-5, h)
+            ref = h.double().cpu() @ w.double().T + res.double()
+            out = torch.empty(M, N, dtype=torch.float32, device=DEV)
+            ops().linear_norm(x.to(DEV) if use_rows else x[:M].contiguous().to(DEV), nw.to(nwt).to(DEV), 1e-5,
+                              w.to(DEV), out, res.to(DEV), rows.to(DEV) if use_rows else None)
+            assert rel(out, ref) < 2e-3          # a norm statistic may round another way: one bf16 step on few inputs
+            plain_ref = plain.rms_norm(src.double(), nw.to(nwt).double(), 1e-5) @ w.double().T + res.double()
+            assert rel(out, plain_ref) < 1e-2
+    # norm prologue and SiLU-gate epilogue together: columns are interleaved (gate_j, up_j) pairs
+    if N % 2 == 0:
+        z = torch.empty(M, N // 2, dtype=torch.bfloat16, device=DEV)
+        ops().linear_norm(x[:M].contiguous().to(DEV), nw.to(DEV), 1e-5, w.to(DEV), z, epilogue="swiglu")
+        c = plain.rms_norm(x[:M].double(), nw.double(), 1e-5).to(torch.bfloat16).double() @ w.double().T
+        assert rel(z, plain.silu(c[:, 0::2]) * c[:, 1::2]) < 8e-3
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,K,N", [(1, 64, 352), (9, 96, 400), (64, 2048, 96), (65, 176, 128), (300, 256, 1030)])
+def test_linear_swiglu_epilogue(dtype, M, K, N):
+    g = torch.Generator().manual_seed(M + N)
+    a = torch.randn(M, K, generator=g).to(dtype)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K) * 2).to(dtype)
+    z = torch.empty(M, N // 2, dtype=dtype, device=DEV)
+    ops().linear(a.to(DEV), w.to(DEV), z, epilogue="swiglu")
+    c = a.double() @ w.double().T
+    assert rel(z, plain.silu(c[:, 0::2]) * c[:, 1::2]) < tol(dtype, 1e-5, 6e-3)
+    from tiny_llm_amd.kernels import KernelError
+    with pytest.raises(KernelError):
+        ops().linear(a.to(DEV), w.to(DEV), torch.empty(M, N, dtype=dtype, device=DEV), epilogue="swiglu")
+
+
 def test_linear_row_alone_equals_row_in_batch_fp32():
     g = torch.Generator().manual_seed(5)
     a = torch.randn(70, 200, generator=g).to(DEV)

@@ -17,7 +17,11 @@ namespace {
 // ===================================================================== float32
 constexpr int F_BM = 64, F_BN = 64, F_BK = 16, F_THREADS = 256;
 
-template <typename TO>
+// silu(g) * u of an interleaved gate|up pair of output columns, as the reference computes it
+// (tiny_llm/ops/cuda/silu.cu:10, arithmetic.cu:13), from the float32 accumulators.
+__device__ __forceinline__ float swiglu_pair(float g, float u) { return g / (1.f + expf(-g)) * u; }
+
+template <typename TO, bool SWIGLU>
 __global__ __launch_bounds__(F_THREADS) void gemm_f32_kernel(const float* __restrict__ a,
                                                              const float* __restrict__ w,
                                                              TO* __restrict__ out,
@@ -64,13 +68,22 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f32_kernel(const float* __rest
   for (int i = 0; i < 4; ++i) {
     const int m = m0 + ty * 4 + i;
     if (m >= M) continue;
+    if constexpr (SWIGLU) {   // columns (2j, 2j+1) = (gate_j, up_j); N is even
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int n = n0 + tx * 4 + j;
-      if (n >= N) continue;
-      float v = acc[i][j];
-      if (residual) v += residual[(int64_t)m * ldo + n];
-      out[(int64_t)m * ldo + n] = from_f32<TO>(v);
+      for (int j = 0; j < 4; j += 2) {
+        const int n = n0 + tx * 4 + j;
+        if (n >= N) continue;
+        out[(int64_t)m * ldo + n / 2] = from_f32<TO>(swiglu_pair(acc[i][j], acc[i][j + 1]));
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int n = n0 + tx * 4 + j;
+        if (n >= N) continue;
+        float v = acc[i][j];
+        if (residual) v += residual[(int64_t)m * ldo + n];
+        out[(int64_t)m * ldo + n] = from_f32<TO>(v);
+      }
     }
   }
 }
@@ -80,7 +93,7 @@ constexpr int B_BM = 128, B_BN = 128, B_BK = 32, B_THREADS = 256;
 constexpr int B_LD = B_BK + 8;  // LDS row stride in elements: 80 bytes, keeps 16-byte alignment
 
 // K must be a multiple of 8 (16-byte chunks of bf16 never straddle the end).
-template <typename TO>
+template <typename TO, bool SWIGLU>
 __global__ __launch_bounds__(B_THREADS) void gemm_bf16_kernel(const bf16_t* __restrict__ a,
                                                               const bf16_t* __restrict__ w,
                                                               TO* __restrict__ out,
@@ -159,6 +172,12 @@ __global__ __launch_bounds__(B_THREADS) void gemm_bf16_kernel(const bf16_t* __re
         const int n = n0 + wn * 64 + j * 32 + q * 8 + (lane / 32) * 4;
         if (n >= N) continue;
         float v[4] = {acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
+        if constexpr (SWIGLU) {   // (gate, up, gate, up) -> two outputs; N is even and n a multiple of 4
+          const int64_t oz = (int64_t)m * ldo + n / 2;
+          out[oz] = from_f32<TO>(swiglu_pair(v[0], v[1]));
+          if (n + 2 < N) out[oz + 1] = from_f32<TO>(swiglu_pair(v[2], v[3]));
+          continue;
+        }
         const int64_t o = (int64_t)m * ldo + n;
         if (vec_ok) {  // n + 3 < N because n and N are both multiples of 4
           if (residual) {
@@ -187,55 +206,162 @@ __global__ __launch_bounds__(B_THREADS) void gemm_bf16_kernel(const bf16_t* __re
 
 // ============================================================ bfloat16, few rows
 // Decode-shaped products (M <= 64): the weight matrix is streamed once and is the
-// whole cost, so the kernel is built around keeping many 16-byte loads in flight.
-// A workgroup of eight wave64 owns 16 output columns (16 weight rows); the waves
-// split K in blocks of 128 and each accumulates a 16 x 16 tile per group of 16
-// activation rows with v_mfma_f32_16x16x32_bf16 (weight rows as the A operand read
-// straight from global memory, activations as the B operand).  A lane reads 64
-// contiguous bytes of its weight row per block; the k order inside an MFMA is
-// permuted accordingly on both operands, which a dot product does not notice.
-// Partial tiles meet in LDS and are added in a fixed order, so results are
-// deterministic; the residual add is folded into that epilogue.
+// whole cost, and a step is a chain of such kernels, so the kernel is built around
+// (a) many 16-byte loads in flight and (b) as few dependent memory round trips and
+// as few launches as possible.  A workgroup of eight wave64 owns 16 output columns
+// (16 weight rows); the waves split K in blocks of 128 and each accumulates a
+// 16 x 16 tile per group of 16 activation rows with v_mfma_f32_16x16x32_bf16
+// (weight rows as the A operand read straight from global memory, activations as
+// the B operand).  A lane reads 64 contiguous bytes of its weight row per block; the
+// k order inside an MFMA is permuted accordingly on both operands, which a dot
+// product does not notice.  Partial tiles meet in LDS and are added in a fixed
+// order, so results are deterministic.
+//
+// Fused into it, to save launches: a prologue on the activations, either RMSNorm of
+// the float32 residual stream (statistics recomputed by every workgroup: a few KB
+// from L2) or SiLU-gate of a [M, 2K] gate|up matrix; an optional gather of input
+// rows; and the residual add in the epilogue, whose operand is fetched before the
+// main loop starts.
 constexpr int S_WAVES = 8, S_THREADS = S_WAVES * TL_WAVE, S_COLS = 16, S_KBLK = 128;
+enum { PRO_NONE = 0, PRO_NORM = 1 };
 
-template <int MT, typename TO>
-__global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(
-    const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, TO* __restrict__ out,
-    const float* __restrict__ residual, int M, int N, int K, int64_t lda, int64_t ldo) {
+struct SkinnyArgs {
+  const void* a;            // PRO_NONE: bf16 [M, K]; PRO_NORM: float [rows, K]
+  const bf16_t* w;          // [N, K]
+  void* out;                // [M, N]
+  const float* residual;    // [M, N] or null
+  const void* norm_w;       // PRO_NORM: [K], float or bf16
+  const int32_t* rows;      // optional gather of input rows
+  float eps;
+  int norm_w_is_f32;
+  int M, N, K;
+  int64_t lda, ldo;
+};
+
+template <int PRO>
+__device__ __forceinline__ bf16x8 skinny_fetch(const SkinnyArgs& p, int64_t row_off, int k, float rms) {
+  if constexpr (PRO == PRO_NONE) {
+    return *(const bf16x8*)((const bf16_t*)p.a + row_off + k);
+  } else if constexpr (PRO == PRO_NORM) {
+    const float* x = (const float*)p.a + row_off + k;
+    const f32x4 x0 = *(const f32x4*)x, x1 = *(const f32x4*)(x + 4);
+    float wv[8];
+    if (p.norm_w_is_f32) {
+      const f32x4 w0 = *(const f32x4*)((const float*)p.norm_w + k), w1 = *(const f32x4*)((const float*)p.norm_w + k + 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { wv[e] = w0[e]; wv[4 + e] = w1[e]; }
+    } else {
+      const bf16x8 w8 = *(const bf16x8*)((const bf16_t*)p.norm_w + k);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) wv[e] = (float)w8[e];
+    }
+    bf16x8 r;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      r[e] = (bf16_t)(wv[e] * x0[e] * rms);          // rms is the reciprocal here
+      r[4 + e] = (bf16_t)(wv[4 + e] * x1[e] * rms);
+    }
+    return r;
+  }
+}
+
+template <int MT, typename TO, int PRO, bool SWIGLU>
+__global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const SkinnyArgs p) {
   __shared__ float part[S_WAVES][MT][16][17];
+  __shared__ float rms_s[MT * 16];
   const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
+  const int M = p.M, N = p.N, K = p.K;
   const int n0 = blockIdx.x * S_COLS;
   const int r16 = lane % 16, g = lane / 16;
   const int n = n0 + r16;
-  const bf16_t* wrow = w + (int64_t)min(n, N - 1) * K;
+  const bf16_t* wrow = p.w + (int64_t)min(n, N - 1) * K;
   const bool n_ok = n < N;
+
+  // epilogue operands first: their latency hides behind the main loop
+  constexpr int EPT = (MT * 256 + S_THREADS - 1) / S_THREADS;
+  float res_v[EPT];
+#pragma unroll
+  for (int j = 0; j < EPT; ++j) {
+    const int e = tid + j * S_THREADS;
+    const int m = (e / 256) * 16 + (e % 256) / 16, nn = e % 16;
+    res_v[j] = (p.residual && e < MT * 256 && m < M && n0 + nn < N) ? p.residual[(int64_t)m * p.ldo + n0 + nn] : 0.f;
+  }
+
+  // input row of each activation row this lane feeds
+  int64_t row_off[MT];
+  bool m_ok[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = mt * 16 + r16;
+    m_ok[mt] = m < M;
+    const int src = p.rows ? p.rows[min(m, M - 1)] : min(m, M - 1);
+    row_off[mt] = (int64_t)src * p.lda;
+  }
+
+  constexpr int UN = MT == 1 ? 2 : 1;      // k blocks whose loads are issued together
+  const int nblk = (K + S_KBLK - 1) / S_KBLK;
+  bf16x8 fw[UN][4];
+  auto load_w = [&](int blk) {
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const int kb = (blk + u * S_WAVES) * S_KBLK + g * 32;   // this lane's 32 k of the block
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int k = kb + i * 8;
+        bf16x8 z = {};
+        fw[u][i] = (n_ok && k < K) ? *(const bf16x8*)(wrow + k) : z;
+      }
+    }
+  };
+  // the weight stream starts before anything that depends on the activations
+  load_w(wave);
+
+  float rms[MT];   // reciprocal of the row's root mean square
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) rms[mt] = 1.f;
+  if constexpr (PRO == PRO_NORM) {
+    for (int m = wave; m < M; m += S_WAVES) {
+      const int src = p.rows ? p.rows[m] : m;
+      const float* x = (const float*)p.a + (int64_t)src * p.lda;
+      float ss = 0.f;
+      for (int k = lane * 4; k < K; k += TL_WAVE * 4) {
+        const f32x4 v = *(const f32x4*)(x + k);
+        ss += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+      }
+      ss = wave_sum(ss);
+      if (lane == 0) rms_s[m] = 1.f / sqrtf(ss / (float)K + p.eps);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) rms[mt] = m_ok[mt] ? rms_s[mt * 16 + r16] : 1.f;
+  }
 
   f32x4 acc[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  const int nblk = (K + S_KBLK - 1) / S_KBLK;
-  for (int blk = wave; blk < nblk; blk += S_WAVES) {
-    const int kb = blk * S_KBLK + g * 32;   // this lane's 32 k of the block
-    bf16x8 fw[4];
+  for (int blk = wave; blk < nblk; blk += S_WAVES * UN) {
+    if (blk != wave) load_w(blk);
+    bf16x8 fa[UN][MT][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int k = kb + i * 8;
-      bf16x8 z = {};
-      fw[i] = (n_ok && k < K) ? *(const bf16x8*)(wrow + k) : z;
+    for (int u = 0; u < UN; ++u) {
+      const int kb = (blk + u * S_WAVES) * S_KBLK + g * 32;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int k = kb + i * 8;
+          bf16x8 z = {};
+          fa[u][mt][i] = (m_ok[mt] && k < K) ? skinny_fetch<PRO>(p, row_off[mt], k, rms[mt]) : z;
+        }
     }
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const int m = mt * 16 + r16;
-      const bf16_t* arow = a + (int64_t)min(m, M - 1) * lda;
+    for (int u = 0; u < UN; ++u)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int k = kb + i * 8;
-        bf16x8 z = {};
-        const bf16x8 fa = (m < M && k < K) ? *(const bf16x8*)(arow + k) : z;
-        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[i], fa, acc[mt], 0, 0, 0);
-      }
-    }
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[u][i], fa[u][mt][i], acc[mt], 0, 0, 0);
   }
   // tile layout: lane holds rows (weight rows) g*4 + r, column (activation row) r16
 #pragma unroll
@@ -243,68 +369,120 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(
 #pragma unroll
     for (int r = 0; r < 4; ++r) part[wave][mt][g * 4 + r][r16] = acc[mt][r];
   __syncthreads();
-  for (int e = tid; e < MT * 256; e += S_THREADS) {
+  TO* out = (TO*)p.out;
+#pragma unroll
+  for (int j = 0; j < EPT; ++j) {
+    const int e = tid + j * S_THREADS;
+    if (e >= MT * 256) continue;
     const int mt = e / 256, m_local = (e % 256) / 16, nn = e % 16;
     const int m = mt * 16 + m_local;
     if (m >= M || n0 + nn >= N) continue;
-    float v = 0.f;
+    if constexpr (SWIGLU) {   // columns (2j, 2j+1) = (gate_j, up_j): even threads make one output of a pair
+      if (nn & 1) continue;
+      float gv = 0.f, uv = 0.f;
 #pragma unroll
-    for (int wv = 0; wv < S_WAVES; ++wv) v += part[wv][mt][nn][m_local];
-    const int64_t o = (int64_t)m * ldo + n0 + nn;
-    if (residual) v += residual[o];
-    out[o] = from_f32<TO>(v);
+      for (int wv = 0; wv < S_WAVES; ++wv) {
+        gv += part[wv][mt][nn][m_local];
+        uv += part[wv][mt][nn + 1][m_local];
+      }
+      out[(int64_t)m * p.ldo + (n0 + nn) / 2] = from_f32<TO>(swiglu_pair(gv, uv));
+    } else {
+      float v = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < S_WAVES; ++wv) v += part[wv][mt][nn][m_local];
+      out[(int64_t)m * p.ldo + n0 + nn] = from_f32<TO>(v + res_v[j]);
+    }
   }
 }
 
-template <typename TO>
-static void launch_skinny(const bf16_t* a, const bf16_t* w, TO* out, const float* residual, int M, int N, int K,
-                          int64_t lda, int64_t ldo, hipStream_t stream) {
-  dim3 g((N + S_COLS - 1) / S_COLS), b(S_THREADS);
-  const int mt = (M + 15) / 16;
+template <typename TO, int PRO, bool SWIGLU>
+static void launch_skinny(const SkinnyArgs& p, hipStream_t stream) {
+  dim3 g((p.N + S_COLS - 1) / S_COLS), b(S_THREADS);
+  const int mt = (p.M + 15) / 16;
   if (mt == 1)
-    hipLaunchKernelGGL((gemm_skinny_bf16_kernel<1, TO>), g, b, 0, stream, a, w, out, residual, M, N, K, lda, ldo);
+    hipLaunchKernelGGL((gemm_skinny_bf16_kernel<1, TO, PRO, SWIGLU>), g, b, 0, stream, p);
   else if (mt == 2)
-    hipLaunchKernelGGL((gemm_skinny_bf16_kernel<2, TO>), g, b, 0, stream, a, w, out, residual, M, N, K, lda, ldo);
+    hipLaunchKernelGGL((gemm_skinny_bf16_kernel<2, TO, PRO, SWIGLU>), g, b, 0, stream, p);
   else if (mt == 3)
-    hipLaunchKernelGGL((gemm_skinny_bf16_kernel<3, TO>), g, b, 0, stream, a, w, out, residual, M, N, K, lda, ldo);
+    hipLaunchKernelGGL((gemm_skinny_bf16_kernel<3, TO, PRO, SWIGLU>), g, b, 0, stream, p);
   else
-    hipLaunchKernelGGL((gemm_skinny_bf16_kernel<4, TO>), g, b, 0, stream, a, w, out, residual, M, N, K, lda, ldo);
+    hipLaunchKernelGGL((gemm_skinny_bf16_kernel<4, TO, PRO, SWIGLU>), g, b, 0, stream, p);
+}
+
+template <int PRO>
+static int launch_skinny_out(const SkinnyArgs& p, int out_dtype, bool swiglu, hipStream_t stream) {
+  if (out_dtype == 0 && !swiglu)
+    launch_skinny<float, PRO, false>(p, stream);
+  else if (out_dtype == 1 && !swiglu)
+    launch_skinny<bf16_t, PRO, false>(p, stream);
+  else if (out_dtype == 1 && swiglu)
+    launch_skinny<bf16_t, PRO, true>(p, stream);
+  else
+    return TL_ERR_ARG;
+  return TL_OK;
 }
 
 }  // namespace
 
 extern "C" {
 
-// dtype: element type of a and w (0 float32, 1 bfloat16); out_dtype: of out.
-// lda: row stride of a in elements; ldo: row stride of out and residual.
+// out = a @ w.T, then an epilogue.  dtype: element type of a and w (0 float32, 1 bfloat16);
+// out_dtype: of out.  lda: row stride of a in elements; ldo: row stride of out and residual.
+// epilogue 0: (+ residual[m, n]), out is [M, N].
+// epilogue 1: SiLU-gate of interleaved columns, out[m, j] = silu(c[m, 2j]) * c[m, 2j+1], out is
+//             [M, N/2] of the input's type; N must be even; no residual.
 int tl_linear(const void* a, const void* w, void* out, const float* residual, int M, int N, int K,
-              int64_t lda, int64_t ldo, int dtype, int out_dtype, hipStream_t stream) {
+              int64_t lda, int64_t ldo, int dtype, int out_dtype, int epilogue, hipStream_t stream) {
   if (M <= 0) return TL_OK;
-  if (N <= 0 || K <= 0 || lda < K || ldo < N) return TL_ERR_ARG;
+  const bool swiglu = epilogue == 1;
+  if (N <= 0 || K <= 0 || lda < K || ldo < (swiglu ? N / 2 : N) || epilogue < 0 || epilogue > 1) return TL_ERR_ARG;
+  if (swiglu && ((N & 1) || residual || out_dtype != dtype)) return TL_ERR_ARG;
   if (dtype == 0) {
     if (out_dtype != 0) return TL_ERR_ARG;
     dim3 g((N + F_BN - 1) / F_BN, (M + F_BM - 1) / F_BM);
-    hipLaunchKernelGGL(gemm_f32_kernel<float>, g, dim3(F_THREADS), 0, stream, (const float*)a, (const float*)w,
-                       (float*)out, residual, M, N, K, lda, ldo);
+    if (swiglu)
+      hipLaunchKernelGGL((gemm_f32_kernel<float, true>), g, dim3(F_THREADS), 0, stream, (const float*)a,
+                         (const float*)w, (float*)out, residual, M, N, K, lda, ldo);
+    else
+      hipLaunchKernelGGL((gemm_f32_kernel<float, false>), g, dim3(F_THREADS), 0, stream, (const float*)a,
+                         (const float*)w, (float*)out, residual, M, N, K, lda, ldo);
   } else if (dtype == 1) {
     if (K % 8 || lda % 8) return TL_ERR_ARG;
+    if (out_dtype != 0 && out_dtype != 1) return TL_ERR_ARG;
     dim3 g((N + B_BN - 1) / B_BN, (M + B_BM - 1) / B_BM);
-    if (M <= 64 && (out_dtype == 0 || out_dtype == 1)) {
-      if (out_dtype == 0)
-        launch_skinny<float>((const bf16_t*)a, (const bf16_t*)w, (float*)out, residual, M, N, K, lda, ldo, stream);
-      else
-        launch_skinny<bf16_t>((const bf16_t*)a, (const bf16_t*)w, (bf16_t*)out, residual, M, N, K, lda, ldo, stream);
-    } else if (out_dtype == 0)
-      hipLaunchKernelGGL(gemm_bf16_kernel<float>, g, dim3(B_THREADS), 0, stream, (const bf16_t*)a,
-                         (const bf16_t*)w, (float*)out, residual, M, N, K, lda, ldo);
-    else if (out_dtype == 1)
-      hipLaunchKernelGGL(gemm_bf16_kernel<bf16_t>, g, dim3(B_THREADS), 0, stream, (const bf16_t*)a,
+    if (M <= 64) {
+      SkinnyArgs p{a, (const bf16_t*)w, out, residual, nullptr, nullptr, 0.f, 0, M, N, K, lda, ldo};
+      if (launch_skinny_out<PRO_NONE>(p, out_dtype, swiglu, stream) != TL_OK) return TL_ERR_ARG;
+    } else if (swiglu) {
+      hipLaunchKernelGGL((gemm_bf16_kernel<bf16_t, true>), g, dim3(B_THREADS), 0, stream, (const bf16_t*)a,
                          (const bf16_t*)w, (bf16_t*)out, residual, M, N, K, lda, ldo);
-    else
-      return TL_ERR_ARG;
+    } else if (out_dtype == 0) {
+      hipLaunchKernelGGL((gemm_bf16_kernel<float, false>), g, dim3(B_THREADS), 0, stream, (const bf16_t*)a,
+                         (const bf16_t*)w, (float*)out, residual, M, N, K, lda, ldo);
+    } else {
+      hipLaunchKernelGGL((gemm_bf16_kernel<bf16_t, false>), g, dim3(B_THREADS), 0, stream, (const bf16_t*)a,
+                         (const bf16_t*)w, (bf16_t*)out, residual, M, N, K, lda, ldo);
+    }
   } else {
     return TL_ERR_ARG;
   }
+  return tl_launch_status();
+}
+
+// Few-row (M <= 64) bfloat16 product whose input is the float32 residual stream: the rows of a
+// (gathered through `rows` if given) are RMS-normalised with norm_w (float32 or bfloat16) and eps
+// inside the kernel.  Epilogues as in tl_linear.
+int tl_linear_norm(const void* a, const void* w, void* out, const float* residual, const void* norm_w,
+                   const int32_t* rows, float eps, int norm_w_dtype, int M, int N, int K, int64_t lda,
+                   int64_t ldo, int out_dtype, int epilogue, hipStream_t stream) {
+  if (M <= 0) return TL_OK;
+  const bool swiglu = epilogue == 1;
+  if (M > 64 || N <= 0 || K <= 0 || K % 8 || lda % 8 || lda < K || ldo < (swiglu ? N / 2 : N) || !norm_w ||
+      (norm_w_dtype != 0 && norm_w_dtype != 1) || epilogue < 0 || epilogue > 1)
+    return TL_ERR_ARG;
+  if (swiglu && ((N & 1) || residual)) return TL_ERR_ARG;
+  SkinnyArgs p{a, (const bf16_t*)w, out, residual, norm_w, rows, eps, norm_w_dtype == 0 ? 1 : 0, M, N, K, lda, ldo};
+  if (launch_skinny_out<PRO_NORM>(p, out_dtype, swiglu, stream) != TL_OK) return TL_ERR_ARG;
   return tl_launch_status();
 }
 

@@ -105,20 +105,27 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor
     return out
 
 
-def linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor,
-           residual: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out = a @ w.T (+ residual).  a [M, K], w [N, K] share an element type;
-    out [M, N] is that type or float32; residual float32 with out's strides."""
+def linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, residual: Optional[torch.Tensor] = None,
+           epilogue: Optional[str] = None) -> torch.Tensor:
+    """out = a @ w.T (+ residual).  a [M, K], w [N, K] share an element type; out [M, N] is that
+    type or float32; residual float32 with out's strides.  epilogue="swiglu": the N columns are
+    interleaved (gate_j, up_j) pairs and out [M, N/2] = silu(gate) * up, computed from the float32
+    accumulators."""
     _dev(a, w, out, residual)
     _rows_2d(a, "linear input")
     _rows_2d(out, "linear output")
     M, K = a.shape
     N = w.shape[0]
+    swiglu = _epilogue(epilogue)
     _need(w.dim() == 2 and w.is_contiguous() and w.shape[1] == K, f"weight must be contiguous [N, {K}]")
     _need(a.dtype == w.dtype, "input and weight must share an element type")
-    _need(tuple(out.shape) == (M, N), f"linear output must be [{M}, {N}]")
     dt, odt = _dt(a), _dt(out)
-    _need(odt == dt or odt == 0, "linear output must have the input's type or float32")
+    if swiglu:
+        _need(N % 2 == 0 and tuple(out.shape) == (M, N // 2) and odt == dt and residual is None,
+              f"the SiLU-gate epilogue writes [{M}, {N // 2}] of the input's type and takes no residual")
+    else:
+        _need(tuple(out.shape) == (M, N), f"linear output must be [{M}, {N}]")
+        _need(odt == dt or odt == 0, "linear output must have the input's type or float32")
     if residual is not None:
         _need(residual.dtype == torch.float32 and residual.shape == out.shape
               and residual.stride() == out.stride(), "residual must be float32 with the output's layout")
@@ -126,11 +133,55 @@ def linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor,
         _need(K % 8 == 0 and a.stride(0) % 8 == 0,
               f"bfloat16 linear needs an inner size that is a multiple of 8, got K={K}")
     al = 16 if dt == 1 else 4      # the bfloat16 kernel moves 16-byte vectors
-    _check(_lib().tl_linear(_ptr(a, al), _ptr(w, al), _ptr(out, al), _ptr(residual, al), c_int(M), c_int(N),
+    ao = 16 if (dt == 1 and not swiglu and M > 64) else 4
+    _check(_lib().tl_linear(_ptr(a, al), _ptr(w, al), _ptr(out, ao), _ptr(residual, ao), c_int(M), c_int(N),
                             c_int(K), c_int64(a.stride(0)), c_int64(out.stride(0)), c_int(dt), c_int(odt),
-                            _stream()), "linear")
+                            c_int(swiglu), _stream()), "linear")
     return out
 
+
+def _epilogue(name: Optional[str]) -> int:
+    if name is None:
+        return 0
+    _need(name == "swiglu", f"unknown epilogue {name!r}")
+    return 1
+
+FUSED_ROWS = 16     # most rows for which a fused prologue pays (every workgroup repeats it)
+FUSED_MAX_ROWS = 64  # most rows the kernel takes
+
+
+def linear_norm(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: torch.Tensor, out: torch.Tensor,
+                residual: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None,
+                epilogue: Optional[str] = None) -> torch.Tensor:
+    """out = rmsnorm(x[rows] or x; norm_weight, eps) @ w.T, then the epilogue of `linear`, in one
+    kernel: at most FUSED_MAX_ROWS rows of float32 x, bfloat16 w."""
+    _dev(x, norm_weight, w, out, residual, rows)
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.stride(1) == 1, "norm input must be float32 [T, K]")
+    K = x.shape[1]
+    M = x.shape[0] if rows is None else rows.numel()
+    N = w.shape[0]
+    swiglu = _epilogue(epilogue)
+    _need(0 < M <= FUSED_MAX_ROWS, f"the fused product takes at most {FUSED_MAX_ROWS} rows, got {M}")
+    _need(w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_contiguous() and w.shape[1] == K,
+          f"weight must be contiguous bfloat16 [N, {K}]")
+    _need(norm_weight.is_contiguous() and norm_weight.numel() == K, f"norm weight must have {K} elements")
+    _need(K % 8 == 0 and x.stride(0) % 8 == 0, "inner size must be a multiple of 8")
+    _rows_2d(out, "linear output")
+    if swiglu:
+        _need(N % 2 == 0 and tuple(out.shape) == (M, N // 2) and out.dtype == torch.bfloat16 and residual is None,
+              f"the SiLU-gate epilogue writes bfloat16 [{M}, {N // 2}] and takes no residual")
+    else:
+        _need(tuple(out.shape) == (M, N), f"linear output must be [{M}, {N}]")
+    if rows is not None:
+        _need(rows.dtype == torch.int32 and rows.is_contiguous(), "row index must be contiguous int32")
+    if residual is not None:
+        _need(residual.dtype == torch.float32 and residual.shape == out.shape
+              and residual.stride() == out.stride(), "residual must be float32 with the output's layout")
+    _check(_lib().tl_linear_norm(_ptr(x, 16), _ptr(w, 16), _ptr(out), _ptr(residual), _ptr(norm_weight, 16),
+                                 _ptr(rows), c_float(eps), c_int(_dt(norm_weight)), c_int(M), c_int(N), c_int(K),
+                                 c_int64(x.stride(0)), c_int64(out.stride(0)), c_int(_dt(out)), c_int(swiglu),
+                                 _stream()), "linear_norm")
+    return out
 
 def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     """out[t, j] = silu(gate_up[t, j]) * gate_up[t, I + j]."""

@@ -89,5 +89,6 @@ class Decoder:
             x = self.layers[e.layer].block.forward(x, ctx, self.caches[i], self.states[i])
         if ctx.logit_rows is None or ctx.logit_rows.numel() == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=x.device)
-        h = self.final_norm.forward(x, ctx.logit_rows)
+        norm = self.final_norm
+        h = norm.lazy(x, ctx.logit_rows) if hasattr(norm, "lazy") else norm.forward(x, ctx.logit_rows)
         return self.lm_head.forward(h)

@@ -18,11 +18,13 @@ from typing import Dict, List, Optional
 import torch
 
 from ..kernels import ops
+from .norm import LazyNorm
 from .base import (CacheSpec, LayerCache, Mixer, POSITION_ENCODINGS, WeightSpec, register_mixer)
 
 
 class Attention(Mixer):
     graph_safe = True
+    accepts_lazy_norm = True
 
     def __init__(self, prefix, dtype, device, *, hidden_size: int, num_heads: int, num_kv_heads: int,
                  head_dim: int, position: dict = None, window: int = 0, scale: float = None,
@@ -63,20 +65,23 @@ class Attention(Mixer):
 
     # --------------------------------------------------------------------- compute
     def forward(self, h, ctx, cache: LayerCache, state, residual):
-        T = h.shape[0]
-        qkv = torch.empty((T, self.q_size + 2 * self.kv_size), dtype=self.dtype, device=h.device)
-        ops.linear(h, self.w_qkv, qkv)
+        T = residual.shape[0]
+        qkv = torch.empty((T, self.q_size + 2 * self.kv_size), dtype=self.dtype, device=residual.device)
+        if isinstance(h, LazyNorm):
+            ops.linear_norm(h.x, h.weight, h.eps, self.w_qkv, qkv, rows=h.rows)
+        else:
+            ops.linear(h, self.w_qkv, qkv)
         tables = self.position.rotary_tables()
         cos, sin, rot = tables if tables is not None else (None, None, 0)
         slots = ctx.slot_mappings[cache.group] if cache.write else None
         ops.rope_store(qkv, ctx.positions, cos, sin, slots, cache.k if cache.write else None,
                        cache.v if cache.write else None, self.num_heads, self.num_kv_heads, self.head_dim, rot)
-        attn = torch.empty((T, self.q_size), dtype=self.dtype, device=h.device)
+        attn = torch.empty((T, self.q_size), dtype=self.dtype, device=residual.device)
         q = qkv[:, :self.q_size]
         if ops.flash_attention_supported(self.dtype, self.num_heads, self.num_kv_heads, self.head_dim):
             group = self.num_heads // self.num_kv_heads
             tiles = ctx.attention_tiles(16 // group)
-            n_splits, scratch = self._splits(ctx, tiles[0].numel(), T, h.device)
+            n_splits, scratch = self._splits(ctx, tiles[0].numel(), T, residual.device)
             ops.flash_attention(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, attn,
                                 self.num_heads, self.num_kv_heads, self.head_dim, self.scale, self.window,
                                 n_splits, scratch)

@@ -10,6 +10,7 @@ import torch
 
 from ..kernels import ops
 from .base import Part, WeightSpec
+from .norm import LazyNorm
 
 
 class TokenEmbedding(Part):
@@ -47,6 +48,10 @@ class LMHead(Part):
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.weight = tensors[f"{self.prefix}.weight"].contiguous()
 
-    def forward(self, h: torch.Tensor) -> torch.Tensor:
+    def forward(self, h) -> torch.Tensor:
+        """h: activations [n, H], or a LazyNorm whose norm rides in the product."""
+        if isinstance(h, LazyNorm):
+            out = torch.empty((h.num_rows, self.vocab_size), dtype=torch.float32, device=h.x.device)
+            return ops.linear_norm(h.x, h.weight, h.eps, self.weight, out, rows=h.rows)
         out = torch.empty((h.shape[0], self.vocab_size), dtype=torch.float32, device=h.device)
         return ops.linear(h, self.weight, out)

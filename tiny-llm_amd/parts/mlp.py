@@ -2,7 +2,9 @@
 
 Reference: tiny_llm/parser/llama_parser.cpp:225-255 (gate, SiLU in place, up,
 multiply, down, add), tiny_llm/ops/cuda/silu.cu:10 (x / (1 + exp(-x))).  Gate and
-up weights are concatenated on load into one [2I, H] matrix.
+up weights are interleaved row by row on load into one [2I, H] matrix, and the
+SiLU-gate runs in the epilogue of that one product on its float32 accumulators:
+the [T, 2I] intermediate of the reference's four kernels is never written.
 """
 from __future__ import annotations
 
@@ -11,11 +13,13 @@ from typing import Dict, List, Optional
 import torch
 
 from ..kernels import ops
+from .norm import LazyNorm
 from .base import FeedForward, WeightSpec, register_feed_forward
 
 
 class SwiGLU(FeedForward):
     graph_safe = True
+    accepts_lazy_norm = True
 
     def __init__(self, prefix, dtype, device, *, hidden_size: int, intermediate_size: int):
         super().__init__(prefix, dtype, device)
@@ -31,16 +35,20 @@ class SwiGLU(FeedForward):
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         p = self.prefix
-        self.w_gate_up = torch.cat([tensors[f"{p}.gate_proj.weight"], tensors[f"{p}.up_proj.weight"]],
-                                   dim=0).contiguous()
+        gate, up = tensors[f"{p}.gate_proj.weight"], tensors[f"{p}.up_proj.weight"]
+        # rows interleaved (gate_0, up_0, gate_1, up_1, ...): a product's epilogue then sees each
+        # pair side by side and writes silu(gate) * up directly
+        self.w_gate_up = torch.stack([gate, up], dim=1).reshape(2 * self.intermediate_size,
+                                                                self.hidden_size).contiguous()
         self.w_down = tensors[f"{p}.down_proj.weight"].contiguous()
 
     def forward(self, h, ctx, residual):
-        T = h.shape[0]
-        gate_up = torch.empty((T, 2 * self.intermediate_size), dtype=self.dtype, device=h.device)
-        ops.linear(h, self.w_gate_up, gate_up)
-        z = torch.empty((T, self.intermediate_size), dtype=self.dtype, device=h.device)
-        ops.silu_mul(gate_up, z)
+        T, dev = residual.shape[0], residual.device
+        z = torch.empty((T, self.intermediate_size), dtype=self.dtype, device=dev)
+        if isinstance(h, LazyNorm):
+            ops.linear_norm(h.x, h.weight, h.eps, self.w_gate_up, z, rows=h.rows, epilogue="swiglu")
+        else:
+            ops.linear(h, self.w_gate_up, z, epilogue="swiglu")
         return ops.linear(z, self.w_down, residual, residual)
 
 

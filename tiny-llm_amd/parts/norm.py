@@ -14,6 +14,22 @@ from ..kernels import ops
 from .base import Norm, WeightSpec, register_norm
 
 
+class LazyNorm:
+    """A norm that has not run yet: (x, weight, eps).  A consumer that can fuse the norm into its
+    first product takes the fields; any other calls `materialize()`."""
+
+    def __init__(self, norm: "RMSNorm", x: torch.Tensor, rows: Optional[torch.Tensor] = None):
+        self.norm, self.x, self.rows = norm, x, rows
+        self.weight, self.eps = norm.weight, norm.eps
+
+    @property
+    def num_rows(self) -> int:
+        return self.x.shape[0] if self.rows is None else self.rows.numel()
+
+    def materialize(self) -> torch.Tensor:
+        return self.norm.forward(self.x, self.rows)
+
+
 class RMSNorm(Norm):
     graph_safe = True
 
@@ -29,6 +45,13 @@ class RMSNorm(Norm):
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.weight = tensors[f"{self.prefix}.weight"].contiguous()
+
+    def lazy(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None):
+        """For few rows in bfloat16 the norm can ride in the consumer's first product."""
+        n = x.shape[0] if rows is None else rows.numel()
+        if self.dtype == torch.bfloat16 and 0 < n <= ops.FUSED_ROWS and self.hidden_size % 8 == 0:
+            return LazyNorm(self, x, rows)
+        return self.forward(x, rows)
 
     def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         n = x.shape[0] if rows is None else rows.numel()
