@@ -131,13 +131,26 @@ def attention_fast(q, k, v, positions, window: int = 0, scale: Optional[float] =
     return out
 
 
-def swiglu(h: torch.Tensor, Wg, Wu, Wd, act_dtype=None) -> torch.Tensor:
+def swiglu(h: torch.Tensor, Wg, Wu, Wd, act_dtype=None, row_scale=None) -> torch.Tensor:
     """g = h Wg^T; g <- silu(g); u = h Wu^T; z = g * u; m = z Wd^T
-    (tiny_llm/parser/llama_parser.cpp:225-249)."""
+    (tiny_llm/parser/llama_parser.cpp:225-249).  `row_scale` multiplies g and u (see normed_linear)."""
     g = linear(h, Wg)
     u = linear(h, Wu)
+    if row_scale is not None:
+        g, u = g * row_scale, u * row_scale
     z = _rnd(silu(g) * u, act_dtype)      # the serving path stores only the gated product
     return linear(z, Wd)
+
+
+def norm_operand(x: torch.Tensor, w: torch.Tensor, eps: float, act_dtype):
+    """(h, row_scale) with rms_norm(x) W^T == (h W^T) * row_scale.  In float64 h is the norm itself.
+    With act_dtype the serving path's rounding is followed: it feeds bf16(w * x) to the product and
+    applies 1 / rms to the result."""
+    if act_dtype is None:
+        return rms_norm(x, w, eps), None
+    H = x.shape[-1]
+    r = torch.sqrt((x * x / H).sum(dim=-1, keepdim=True) + eps)
+    return _rnd(w.to(x.dtype) * x, act_dtype), 1.0 / r
 
 
 # ------------------------------------------------------------------------- model
@@ -156,20 +169,22 @@ def llama_forward(w: Dict[str, torch.Tensor], cfg: dict, tokens: Sequence[int],
     x = embedding(tokens, w["model.embed_tokens.weight"])
     for i in range(cfg["num_hidden_layers"]):
         p = f"model.layers.{i}"
-        h = _rnd(rms_norm(x, w[f"{p}.input_layernorm.weight"], eps), act_dtype)
-        q = _rnd(linear(h, w[f"{p}.self_attn.q_proj.weight"]), act_dtype).view(T, nq, hd)
-        k = _rnd(linear(h, w[f"{p}.self_attn.k_proj.weight"]), act_dtype).view(T, nkv, hd)
-        v = _rnd(linear(h, w[f"{p}.self_attn.v_proj.weight"]), act_dtype).view(T, nkv, hd)
+        h, rs = norm_operand(x, w[f"{p}.input_layernorm.weight"], eps, act_dtype)
+        sc = (lambda t: t) if rs is None else (lambda t: t * rs)
+        q = _rnd(sc(linear(h, w[f"{p}.self_attn.q_proj.weight"])), act_dtype).view(T, nq, hd)
+        k = _rnd(sc(linear(h, w[f"{p}.self_attn.k_proj.weight"])), act_dtype).view(T, nkv, hd)
+        v = _rnd(sc(linear(h, w[f"{p}.self_attn.v_proj.weight"])), act_dtype).view(T, nkv, hd)
         q = _rnd(apply_rope(q, positions, cos, sin), act_dtype)
         k = _rnd(apply_rope(k, positions, cos, sin), act_dtype)
         o = _rnd(attention_fast(q, k, v, positions, window), act_dtype).reshape(T, nq * hd)
         x = x + linear(o, w[f"{p}.self_attn.o_proj.weight"])
-        h2 = _rnd(rms_norm(x, w[f"{p}.post_attention_layernorm.weight"], eps), act_dtype)
+        h2, rs2 = norm_operand(x, w[f"{p}.post_attention_layernorm.weight"], eps, act_dtype)
         x = x + swiglu(h2, w[f"{p}.mlp.gate_proj.weight"], w[f"{p}.mlp.up_proj.weight"],
-                       w[f"{p}.mlp.down_proj.weight"], act_dtype)
-    xn = _rnd(rms_norm(x, w["model.norm.weight"], eps), act_dtype)
+                       w[f"{p}.mlp.down_proj.weight"], act_dtype, rs2)
+    xn, rsn = norm_operand(x, w["model.norm.weight"], eps, act_dtype)
     head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", False) else w["lm_head.weight"]
-    return linear(xn, head)
+    logits = linear(xn, head)
+    return logits if rsn is None else logits * rsn
 
 
 def greedy_generate(w, cfg, prompt: Sequence[int], n_new: int, act_dtype=None) -> List[int]:

@@ -49,6 +49,27 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const TW* __restrict
   for (int j = threadIdx.x; j < hidden; j += kThreads) dst[j] = from_f32<TO>(to_f32(w[j]) * src[j] / r);
 }
 
+// --------------------------------------------------- RMSNorm, scale left out
+// out = bf16(w * x) and inv_rms = 1 / sqrt(mean(x^2) + eps) per row: the operand of a product that
+// applies the row factor to its result (the few-row product does the same inside its kernel).
+template <typename TW>
+__global__ void norm_prescale_kernel(const float* __restrict__ x, const TW* __restrict__ w,
+                                     const int32_t* __restrict__ rows, bf16_t* __restrict__ out,
+                                     float* __restrict__ inv_rms, int hidden, float eps) {
+  __shared__ float red[kWaves];
+  const int64_t in_row = rows ? rows[blockIdx.x] : blockIdx.x;
+  const float* src = x + in_row * hidden;
+  bf16_t* dst = out + (int64_t)blockIdx.x * hidden;
+  float ss = 0.f;
+  for (int j = threadIdx.x; j < hidden; j += kThreads) {
+    const float v = src[j];
+    ss += v * v;
+    dst[j] = (bf16_t)(to_f32(w[j]) * v);
+  }
+  ss = block_sum<kWaves>(ss, red);
+  if (threadIdx.x == 0) inv_rms[blockIdx.x] = 1.f / sqrtf(ss / (float)hidden + eps);
+}
+
 // ------------------------------------------------------------------ SiLU-gate
 // z[t, j] = silu(gate_up[t, j]) * gate_up[t, I + j]
 template <typename T>
@@ -154,6 +175,22 @@ int tl_rmsnorm(const float* x, const void* w, const int32_t* rows, void* out, in
     hipLaunchKernelGGL((rmsnorm_kernel<float, bf16_t>), g, b, 0, stream, x, (const float*)w, rows, (bf16_t*)out, hidden, eps);
   else if (w_dtype == 1 && out_dtype == 1)
     hipLaunchKernelGGL((rmsnorm_kernel<bf16_t, bf16_t>), g, b, 0, stream, x, (const bf16_t*)w, rows, (bf16_t*)out, hidden, eps);
+  else
+    return TL_ERR_ARG;
+  return tl_launch_status();
+}
+
+int tl_norm_prescale(const float* x, const void* w, const int32_t* rows, void* out, float* inv_rms, int n_rows,
+                      int hidden, float eps, int w_dtype, hipStream_t stream) {
+  if (n_rows <= 0) return TL_OK;
+  if (hidden <= 0) return TL_ERR_ARG;
+  dim3 g(n_rows), b(kThreads);
+  if (w_dtype == 0)
+    hipLaunchKernelGGL(norm_prescale_kernel<float>, g, b, 0, stream, x, (const float*)w, rows, (bf16_t*)out, inv_rms,
+                       hidden, eps);
+  else if (w_dtype == 1)
+    hipLaunchKernelGGL(norm_prescale_kernel<bf16_t>, g, b, 0, stream, x, (const bf16_t*)w, rows, (bf16_t*)out,
+                       inv_rms, hidden, eps);
   else
     return TL_ERR_ARG;
   return tl_launch_status();

@@ -97,7 +97,8 @@ template <typename TO, bool SWIGLU>
 __global__ __launch_bounds__(B_THREADS) void gemm_bf16_kernel(const bf16_t* __restrict__ a,
                                                               const bf16_t* __restrict__ w,
                                                               TO* __restrict__ out,
-                                                              const float* __restrict__ residual, int M,
+                                                              const float* __restrict__ residual,
+                                                              const float* __restrict__ row_scale, int M,
                                                               int N, int K, int64_t lda, int64_t ldo) {
   __shared__ __attribute__((aligned(16))) bf16_t As[B_BM * B_LD];
   __shared__ __attribute__((aligned(16))) bf16_t Ws[B_BN * B_LD];
@@ -165,13 +166,15 @@ __global__ __launch_bounds__(B_THREADS) void gemm_bf16_kernel(const bf16_t* __re
   for (int i = 0; i < 2; ++i) {
     const int m = m0 + wm * 64 + i * 32 + lane % 32;
     if (m >= M) continue;
+    const float rs = row_scale ? row_scale[m] : 1.f;   // e.g. 1 / rms of a norm left out of the operand
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int n = n0 + wn * 64 + j * 32 + q * 8 + (lane / 32) * 4;
         if (n >= N) continue;
-        float v[4] = {acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
+        float v[4] = {acc[i][j][q * 4 + 0] * rs, acc[i][j][q * 4 + 1] * rs, acc[i][j][q * 4 + 2] * rs,
+                      acc[i][j][q * 4 + 3] * rs};
         if constexpr (SWIGLU) {   // (gate, up, gate, up) -> two outputs; N is even and n a multiple of 4
           const int64_t oz = (int64_t)m * ldo + n / 2;
           out[oz] = from_f32<TO>(swiglu_pair(v[0], v[1]));
@@ -212,10 +215,8 @@ __global__ __launch_bounds__(B_THREADS) void gemm_bf16_kernel(const bf16_t* __re
 // (16 weight rows); the waves split K in blocks of 128 and each accumulates a
 // 16 x 16 tile per group of 16 activation rows with v_mfma_f32_16x16x32_bf16
 // (weight rows as the A operand read straight from global memory, activations as
-// the B operand).  A lane reads 64 contiguous bytes of its weight row per block; the
-// k order inside an MFMA is permuted accordingly on both operands, which a dot
-// product does not notice.  Partial tiles meet in LDS and are added in a fixed
-// order, so results are deterministic.
+// the B operand).  Partial tiles meet in LDS and are added in a fixed order, so
+// results are deterministic.
 //
 // Fused into it, to save launches: a prologue on the activations, either RMSNorm of
 // the float32 residual stream (statistics recomputed by every workgroup: a few KB
@@ -232,17 +233,22 @@ struct SkinnyArgs {
   const float* residual;    // [M, N] or null
   const void* norm_w;       // PRO_NORM: [K], float or bf16
   const int32_t* rows;      // optional gather of input rows
+  const float* row_scale;   // optional factor of each output row (a norm applied by an earlier kernel)
   float eps;
   int norm_w_is_f32;
   int M, N, K;
   int64_t lda, ldo;
 };
 
+// One 8-wide k chunk of an activation row as an MFMA operand.  With the norm prologue the chunk
+// is w * x of the float32 residual stream (rounded to bfloat16) and `ss` collects x^2: the row's
+// 1 / rms is a common factor of the whole dot product and is applied to the result instead, so
+// nothing has to wait for the row statistics.
 template <int PRO>
-__device__ __forceinline__ bf16x8 skinny_fetch(const SkinnyArgs& p, int64_t row_off, int k, float rms) {
+__device__ __forceinline__ bf16x8 skinny_fetch(const SkinnyArgs& p, int64_t row_off, int k, float& ss) {
   if constexpr (PRO == PRO_NONE) {
     return *(const bf16x8*)((const bf16_t*)p.a + row_off + k);
-  } else if constexpr (PRO == PRO_NORM) {
+  } else {
     const float* x = (const float*)p.a + row_off + k;
     const f32x4 x0 = *(const f32x4*)x, x1 = *(const f32x4*)(x + 4);
     float wv[8];
@@ -258,8 +264,9 @@ __device__ __forceinline__ bf16x8 skinny_fetch(const SkinnyArgs& p, int64_t row_
     bf16x8 r;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      r[e] = (bf16_t)(wv[e] * x0[e] * rms);          // rms is the reciprocal here
-      r[4 + e] = (bf16_t)(wv[4 + e] * x1[e] * rms);
+      r[e] = (bf16_t)(wv[e] * x0[e]);
+      r[4 + e] = (bf16_t)(wv[4 + e] * x1[e]);
+      ss += x0[e] * x0[e] + x1[e] * x1[e];
     }
     return r;
   }
@@ -268,7 +275,7 @@ __device__ __forceinline__ bf16x8 skinny_fetch(const SkinnyArgs& p, int64_t row_
 template <int MT, typename TO, int PRO, bool SWIGLU>
 __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const SkinnyArgs p) {
   __shared__ float part[S_WAVES][MT][16][17];
-  __shared__ float rms_s[MT * 16];
+  __shared__ float ss_part[S_WAVES][MT * 16];
   const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
   const int M = p.M, N = p.N, K = p.K;
   const int n0 = blockIdx.x * S_COLS;
@@ -300,59 +307,37 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
 
   constexpr int UN = MT == 1 ? 2 : 1;      // k blocks whose loads are issued together
   const int nblk = (K + S_KBLK - 1) / S_KBLK;
-  bf16x8 fw[UN][4];
-  auto load_w = [&](int blk) {
+  f32x4 acc[MT];
+  float ss[MT];                            // this lane's share of sum x^2 of its rows (norm prologue)
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    ss[mt] = 0.f;
+  }
+  for (int blk = wave; blk < nblk; blk += S_WAVES * UN) {
+    bf16x8 fw[UN][4], fa[UN][MT][4];
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
-      const int kb = (blk + u * S_WAVES) * S_KBLK + g * 32;   // this lane's 32 k of the block
+      // MFMA i of the block covers k = i*32 .. i*32+31, lane group g its 8 k from g*8: one load
+      // instruction then reads 64 contiguous bytes of each of the 16 weight rows
+      const int kb = (blk + u * S_WAVES) * S_KBLK + g * 8;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int k = kb + i * 8;
+        const int k = kb + i * 32;
         bf16x8 z = {};
         fw[u][i] = (n_ok && k < K) ? *(const bf16x8*)(wrow + k) : z;
       }
     }
-  };
-  // the weight stream starts before anything that depends on the activations
-  load_w(wave);
-
-  float rms[MT];   // reciprocal of the row's root mean square
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) rms[mt] = 1.f;
-  if constexpr (PRO == PRO_NORM) {
-    for (int m = wave; m < M; m += S_WAVES) {
-      const int src = p.rows ? p.rows[m] : m;
-      const float* x = (const float*)p.a + (int64_t)src * p.lda;
-      float ss = 0.f;
-      for (int k = lane * 4; k < K; k += TL_WAVE * 4) {
-        const f32x4 v = *(const f32x4*)(x + k);
-        ss += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
-      }
-      ss = wave_sum(ss);
-      if (lane == 0) rms_s[m] = 1.f / sqrtf(ss / (float)K + p.eps);
-    }
-    __syncthreads();
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) rms[mt] = m_ok[mt] ? rms_s[mt * 16 + r16] : 1.f;
-  }
-
-  f32x4 acc[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-  for (int blk = wave; blk < nblk; blk += S_WAVES * UN) {
-    if (blk != wave) load_w(blk);
-    bf16x8 fa[UN][MT][4];
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
-      const int kb = (blk + u * S_WAVES) * S_KBLK + g * 32;
+      const int kb = (blk + u * S_WAVES) * S_KBLK + g * 8;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int k = kb + i * 8;
+          const int k = kb + i * 32;
           bf16x8 z = {};
-          fa[u][mt][i] = (m_ok[mt] && k < K) ? skinny_fetch<PRO>(p, row_off[mt], k, rms[mt]) : z;
+          fa[u][mt][i] = (m_ok[mt] && k < K) ? skinny_fetch<PRO>(p, row_off[mt], k, ss[mt]) : z;
         }
     }
 #pragma unroll
@@ -368,6 +353,15 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int r = 0; r < 4; ++r) part[wave][mt][g * 4 + r][r16] = acc[mt][r];
+  if constexpr (PRO == PRO_NORM) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      float t = ss[mt];
+      t += __shfl_xor(t, 16, TL_WAVE);
+      t += __shfl_xor(t, 32, TL_WAVE);
+      if (g == 0) ss_part[wave][mt * 16 + r16] = t;
+    }
+  }
   __syncthreads();
   TO* out = (TO*)p.out;
 #pragma unroll
@@ -377,6 +371,13 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
     const int mt = e / 256, m_local = (e % 256) / 16, nn = e % 16;
     const int m = mt * 16 + m_local;
     if (m >= M || n0 + nn >= N) continue;
+    float scale = p.row_scale ? p.row_scale[m] : 1.f;   // the row factor left out of the operands
+    if constexpr (PRO == PRO_NORM) {
+      float t = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < S_WAVES; ++wv) t += ss_part[wv][m];
+      scale = 1.f / sqrtf(t / (float)K + p.eps);
+    }
     if constexpr (SWIGLU) {   // columns (2j, 2j+1) = (gate_j, up_j): even threads make one output of a pair
       if (nn & 1) continue;
       float gv = 0.f, uv = 0.f;
@@ -385,12 +386,12 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
         gv += part[wv][mt][nn][m_local];
         uv += part[wv][mt][nn + 1][m_local];
       }
-      out[(int64_t)m * p.ldo + (n0 + nn) / 2] = from_f32<TO>(swiglu_pair(gv, uv));
+      out[(int64_t)m * p.ldo + (n0 + nn) / 2] = from_f32<TO>(swiglu_pair(gv * scale, uv * scale));
     } else {
       float v = 0.f;
 #pragma unroll
       for (int wv = 0; wv < S_WAVES; ++wv) v += part[wv][mt][nn][m_local];
-      out[(int64_t)m * p.ldo + n0 + nn] = from_f32<TO>(v + res_v[j]);
+      out[(int64_t)m * p.ldo + n0 + nn] = from_f32<TO>(v * scale + res_v[j]);
     }
   }
 }
@@ -428,12 +429,16 @@ extern "C" {
 
 // out = a @ w.T, then an epilogue.  dtype: element type of a and w (0 float32, 1 bfloat16);
 // out_dtype: of out.  lda: row stride of a in elements; ldo: row stride of out and residual.
+// row_scale (optional, bfloat16 only): every row m of the product is multiplied by row_scale[m]
+// before the epilogue.
 // epilogue 0: (+ residual[m, n]), out is [M, N].
 // epilogue 1: SiLU-gate of interleaved columns, out[m, j] = silu(c[m, 2j]) * c[m, 2j+1], out is
 //             [M, N/2] of the input's type; N must be even; no residual.
-int tl_linear(const void* a, const void* w, void* out, const float* residual, int M, int N, int K,
-              int64_t lda, int64_t ldo, int dtype, int out_dtype, int epilogue, hipStream_t stream) {
+int tl_linear(const void* a, const void* w, void* out, const float* residual, const float* row_scale, int M,
+              int N, int K, int64_t lda, int64_t ldo, int dtype, int out_dtype, int epilogue,
+              hipStream_t stream) {
   if (M <= 0) return TL_OK;
+  if (row_scale && dtype != 1) return TL_ERR_ARG;   // only the bfloat16 kernels scale rows
   const bool swiglu = epilogue == 1;
   if (N <= 0 || K <= 0 || lda < K || ldo < (swiglu ? N / 2 : N) || epilogue < 0 || epilogue > 1) return TL_ERR_ARG;
   if (swiglu && ((N & 1) || residual || out_dtype != dtype)) return TL_ERR_ARG;
@@ -451,17 +456,17 @@ int tl_linear(const void* a, const void* w, void* out, const float* residual, in
     if (out_dtype != 0 && out_dtype != 1) return TL_ERR_ARG;
     dim3 g((N + B_BN - 1) / B_BN, (M + B_BM - 1) / B_BM);
     if (M <= 64) {
-      SkinnyArgs p{a, (const bf16_t*)w, out, residual, nullptr, nullptr, 0.f, 0, M, N, K, lda, ldo};
+      SkinnyArgs p{a, (const bf16_t*)w, out, residual, nullptr, nullptr, row_scale, 0.f, 0, M, N, K, lda, ldo};
       if (launch_skinny_out<PRO_NONE>(p, out_dtype, swiglu, stream) != TL_OK) return TL_ERR_ARG;
     } else if (swiglu) {
       hipLaunchKernelGGL((gemm_bf16_kernel<bf16_t, true>), g, dim3(B_THREADS), 0, stream, (const bf16_t*)a,
-                         (const bf16_t*)w, (bf16_t*)out, residual, M, N, K, lda, ldo);
+                         (const bf16_t*)w, (bf16_t*)out, residual, row_scale, M, N, K, lda, ldo);
     } else if (out_dtype == 0) {
       hipLaunchKernelGGL((gemm_bf16_kernel<float, false>), g, dim3(B_THREADS), 0, stream, (const bf16_t*)a,
-                         (const bf16_t*)w, (float*)out, residual, M, N, K, lda, ldo);
+                         (const bf16_t*)w, (float*)out, residual, row_scale, M, N, K, lda, ldo);
     } else {
       hipLaunchKernelGGL((gemm_bf16_kernel<bf16_t, false>), g, dim3(B_THREADS), 0, stream, (const bf16_t*)a,
-                         (const bf16_t*)w, (bf16_t*)out, residual, M, N, K, lda, ldo);
+                         (const bf16_t*)w, (bf16_t*)out, residual, row_scale, M, N, K, lda, ldo);
     }
   } else {
     return TL_ERR_ARG;
@@ -481,7 +486,7 @@ int tl_linear_norm(const void* a, const void* w, void* out, const float* residua
       (norm_w_dtype != 0 && norm_w_dtype != 1) || epilogue < 0 || epilogue > 1)
     return TL_ERR_ARG;
   if (swiglu && ((N & 1) || residual)) return TL_ERR_ARG;
-  SkinnyArgs p{a, (const bf16_t*)w, out, residual, norm_w, rows, eps, norm_w_dtype == 0 ? 1 : 0, M, N, K, lda, ldo};
+  SkinnyArgs p{a, (const bf16_t*)w, out, residual, norm_w, rows, nullptr, eps, norm_w_dtype == 0 ? 1 : 0, M, N, K, lda, ldo};
   if (launch_skinny_out<PRO_NORM>(p, out_dtype, swiglu, stream) != TL_OK) return TL_ERR_ARG;
   return tl_launch_status();
 }

@@ -106,11 +106,11 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor
 
 
 def linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, residual: Optional[torch.Tensor] = None,
-           epilogue: Optional[str] = None) -> torch.Tensor:
+           epilogue: Optional[str] = None, row_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out = a @ w.T (+ residual).  a [M, K], w [N, K] share an element type; out [M, N] is that
     type or float32; residual float32 with out's strides.  epilogue="swiglu": the N columns are
     interleaved (gate_j, up_j) pairs and out [M, N/2] = silu(gate) * up, computed from the float32
-    accumulators."""
+    accumulators.  row_scale [M] multiplies the rows of the product first (bfloat16 only)."""
     _dev(a, w, out, residual)
     _rows_2d(a, "linear input")
     _rows_2d(out, "linear output")
@@ -134,8 +134,11 @@ def linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, residual: Option
               f"bfloat16 linear needs an inner size that is a multiple of 8, got K={K}")
     al = 16 if dt == 1 else 4      # the bfloat16 kernel moves 16-byte vectors
     ao = 16 if (dt == 1 and not swiglu and M > 64) else 4
-    _check(_lib().tl_linear(_ptr(a, al), _ptr(w, al), _ptr(out, ao), _ptr(residual, ao), c_int(M), c_int(N),
-                            c_int(K), c_int64(a.stride(0)), c_int64(out.stride(0)), c_int(dt), c_int(odt),
+    if row_scale is not None:
+        _need(dt == 1 and row_scale.dtype == torch.float32 and row_scale.is_contiguous()
+              and row_scale.numel() == M, "row scales go with the bfloat16 product: float32, one per row")
+    _check(_lib().tl_linear(_ptr(a, al), _ptr(w, al), _ptr(out, ao), _ptr(residual, ao), _ptr(row_scale), c_int(M),
+                            c_int(N), c_int(K), c_int64(a.stride(0)), c_int64(out.stride(0)), c_int(dt), c_int(odt),
                             c_int(swiglu), _stream()), "linear")
     return out
 
@@ -146,34 +149,45 @@ def _epilogue(name: Optional[str]) -> int:
     _need(name == "swiglu", f"unknown epilogue {name!r}")
     return 1
 
-FUSED_ROWS = 16     # most rows for which a fused prologue pays (every workgroup repeats it)
-FUSED_MAX_ROWS = 64  # most rows the kernel takes
+FUSED_MAX_ROWS = 64    # most rows the few-row product kernel takes
+FUSED_MAX_COLS = 4096  # most columns for which the fused norm prologue pays
 
 
 def linear_norm(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: torch.Tensor, out: torch.Tensor,
                 residual: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None,
                 epilogue: Optional[str] = None) -> torch.Tensor:
-    """out = rmsnorm(x[rows] or x; norm_weight, eps) @ w.T, then the epilogue of `linear`, in one
-    kernel: at most FUSED_MAX_ROWS rows of float32 x, bfloat16 w."""
+    """out = rmsnorm(x[rows] or x; norm_weight, eps) @ w.T, then the epilogue of `linear`, for float32
+    x and bfloat16 w.  The norm is evaluated as (bf16(norm_weight * x) @ w.T) / rms: the row factor
+    1 / rms is applied to the product, so the operand does not wait for the row statistics.  Few
+    rows and few columns run in ONE kernel (every workgroup prepares the operand itself, which pays
+    while one round of workgroups covers the columns); otherwise a pre-scale kernel writes the
+    operand and the row factors once and the plain product applies them."""
     _dev(x, norm_weight, w, out, residual, rows)
     _need(x.dtype == torch.float32 and x.dim() == 2 and x.stride(1) == 1, "norm input must be float32 [T, K]")
     K = x.shape[1]
     M = x.shape[0] if rows is None else rows.numel()
     N = w.shape[0]
     swiglu = _epilogue(epilogue)
-    _need(0 < M <= FUSED_MAX_ROWS, f"the fused product takes at most {FUSED_MAX_ROWS} rows, got {M}")
+    _need(M > 0, "the product needs at least one row")
     _need(w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_contiguous() and w.shape[1] == K,
           f"weight must be contiguous bfloat16 [N, {K}]")
     _need(norm_weight.is_contiguous() and norm_weight.numel() == K, f"norm weight must have {K} elements")
     _need(K % 8 == 0 and x.stride(0) % 8 == 0, "inner size must be a multiple of 8")
+    if rows is not None:
+        _need(rows.dtype == torch.int32 and rows.is_contiguous(), "row index must be contiguous int32")
+    if M > FUSED_MAX_ROWS or N > FUSED_MAX_COLS:
+        _need(x.is_contiguous(), "norm input must be contiguous")
+        h = torch.empty((M, K), dtype=torch.bfloat16, device=x.device)
+        inv_rms = torch.empty(M, dtype=torch.float32, device=x.device)
+        _check(_lib().tl_norm_prescale(_ptr(x), _ptr(norm_weight), _ptr(rows), _ptr(h), _ptr(inv_rms), c_int(M),
+                                       c_int(K), c_float(eps), c_int(_dt(norm_weight)), _stream()), "norm_prescale")
+        return linear(h, w, out, residual, epilogue, row_scale=inv_rms)
     _rows_2d(out, "linear output")
     if swiglu:
         _need(N % 2 == 0 and tuple(out.shape) == (M, N // 2) and out.dtype == torch.bfloat16 and residual is None,
               f"the SiLU-gate epilogue writes bfloat16 [{M}, {N // 2}] and takes no residual")
     else:
         _need(tuple(out.shape) == (M, N), f"linear output must be [{M}, {N}]")
-    if rows is not None:
-        _need(rows.dtype == torch.int32 and rows.is_contiguous(), "row index must be contiguous int32")
     if residual is not None:
         _need(residual.dtype == torch.float32 and residual.shape == out.shape
               and residual.stride() == out.stride(), "residual must be float32 with the output's layout")

@@ -47,9 +47,8 @@ class RMSNorm(Norm):
         self.weight = tensors[f"{self.prefix}.weight"].contiguous()
 
     def lazy(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None):
-        """For few rows in bfloat16 the norm can ride in the consumer's first product."""
-        n = x.shape[0] if rows is None else rows.numel()
-        if self.dtype == torch.bfloat16 and 0 < n <= ops.FUSED_ROWS and self.hidden_size % 8 == 0:
+        """In bfloat16 the norm rides in the consumer's first product (`ops.linear_norm`)."""
+        if self.dtype == torch.bfloat16 and self.hidden_size % 8 == 0:
             return LazyNorm(self, x, rows)
         return self.forward(x, rows)
 
