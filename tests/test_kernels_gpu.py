@@ -326,7 +326,7 @@ def _paged_case(dtype, lens, q_lens, nq, nkv, hd, bs, window=0, seed=0, boost=No
                               hd, 1.0 / math.sqrt(hd), window)
     else:
         # query tiles of at most 16 // (nq / nkv) tokens, as the step context builds them
-        per = 16 // (nq // nkv)
+        per = (16 // (nq // nkv)) * (8 if impl == "prefill" else 1)
         t_req, t_tok0, t_ntok, t = [], [], [], 0
         for r, ql in enumerate(q_lens):
             for s0 in range(0, ql, per):
@@ -335,6 +335,10 @@ def _paged_case(dtype, lens, q_lens, nq, nkv, hd, bs, window=0, seed=0, boost=No
                 t_ntok.append(min(per, ql - s0))
             t += ql
         T = q.shape[0]
+        if impl == "prefill":
+            ops().flash_prefill(q.to(DEV), kc.to(DEV), vc.to(DEV), bt.to(DEV), (i32(t_req), i32(t_tok0), i32(t_ntok)),
+                                i32(pos), out, nq, nkv, hd, 1.0 / math.sqrt(hd), window)
+            return out.reshape(-1, nq, hd), torch.cat(refs)
         scratch = torch.full((max(1, n_splits * T * nq * (hd + 2)),), float("nan"), device=DEV)
         ops().flash_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), bt.to(DEV), (i32(t_req), i32(t_tok0), i32(t_ntok)),
                               i32(pos), out, nq, nkv, hd, 1.0 / math.sqrt(hd), window, n_splits, scratch)
@@ -380,6 +384,29 @@ def test_flash_attention_mixed_batch(nq, nkv, hd, bs, n_splits):
                            nkv=nkv, hd=hd, bs=bs, seed=hd + bs, impl="flash", n_splits=n_splits)
     assert not torch.isnan(out).any()
     assert rel(out, ref) < 8e-3
+
+
+@pytest.mark.parametrize("nq,nkv,hd,bs", FLASH_SHAPES)
+def test_flash_prefill_mixed_batch(nq, nkv, hd, bs):
+    out, ref = _paged_case(torch.bfloat16, lens=[123, 107, 65, 1, 300, 2, 513], q_lens=[123, 40, 1, 1, 1, 2, 257],
+                           nq=nq, nkv=nkv, hd=hd, bs=bs, seed=hd + bs, impl="prefill")
+    assert not torch.isnan(out).any()
+    assert rel(out, ref) < 8e-3
+
+
+@pytest.mark.parametrize("window", [1, 7, 16, 33, 100])
+def test_flash_prefill_window_edge(window):
+    out, ref = _paged_case(torch.bfloat16, lens=[190, 40, 64, 130], q_lens=[190, 1, 5, 70], nq=4, nkv=2, hd=32,
+                           bs=8, window=window, seed=window, impl="prefill")
+    assert not torch.isnan(out).any()
+    assert rel(out, ref) < 8e-3
+
+
+def test_flash_prefill_far_key_among_hundreds():
+    for far in (0, 15, 16, 63, 64, 255, 256, 511, 699):
+        out, ref = _paged_case(torch.bfloat16, lens=[700], q_lens=[30], nq=8, nkv=1, hd=64, bs=16, seed=far,
+                               boost=far, impl="prefill")
+        assert rel(out, ref) < 8e-3, far
 
 
 @pytest.mark.parametrize("n_splits", [1, 2, 7])

@@ -327,6 +327,207 @@ __global__ __launch_bounds__(FA_THREADS) void flash_attn_bf16_kernel(
   }
 }
 
+// flash_prefill_bf16_kernel: the same mathematics arranged for prompt portions.  A workgroup
+// owns up to 8 query tiles (two per wave, 128 rows: for 8 heads per kv head that is 16 tokens) of
+// consecutive tokens of one request, and all four waves work on the SAME 64-key tile, staged and
+// transposed once per workgroup; so a key or value row is fetched once per 128 query rows.  There
+// is nothing to merge at the end: every row lives in one lane group of one wave.
+constexpr int FP_RT = 2;                      // query tiles (of 16 rows) per wave
+constexpr int FP_TILES = FA_WAVES * FP_RT;    // query tiles per workgroup
+
+template <int HDT>
+__global__ __launch_bounds__(FA_THREADS) void flash_prefill_bf16_kernel(
+    const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_cache,
+    const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int max_blocks,
+    const int32_t* __restrict__ tile_req, const int32_t* __restrict__ tile_tok0,
+    const int32_t* __restrict__ tile_ntok, const int32_t* __restrict__ positions, bf16_t* __restrict__ out,
+    int64_t out_stride, int nq, int nkv, int block_size, float scale, int window) {
+  constexpr int HD = HDT * 16;
+  constexpr int KS = (HD + 31) / 32;
+  constexpr int KP = KS * 32 + 8;
+  __shared__ __attribute__((aligned(16))) bf16_t Kl[FA_KT * KP];
+  __shared__ __attribute__((aligned(16))) bf16_t Vl[HD * FA_VP];
+
+  const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
+  const int r16 = lane % 16, g = lane / 16;
+  const int tile = blockIdx.x, kvh = blockIdx.y;
+  const int G = nq / nkv, TW = 16 / G;
+  const int req = tile_req[tile], tok0 = tile_tok0[tile], ntok = tile_ntok[tile];
+  const int32_t* bt = block_tables + (int64_t)req * max_blocks;
+
+  // the tokens of a tile are consecutive tokens of one request, so their positions are consecutive
+  const int pos_first = positions[tok0], pos_last = pos_first + ntok - 1;
+  const int kv_end = pos_last + 1;
+  const int kv_begin = (window > 0 && pos_first + 1 > window) ? pos_first + 1 - window : 0;
+  const int first_tile = kv_begin / FA_KT, last_tile = (kv_end + FA_KT - 1) / FA_KT;
+
+  // this lane's query rows, one per query tile of its wave
+  bool row_valid[FP_RT];
+  int pos[FP_RT], row_lo[FP_RT], tok[FP_RT];
+  const int head = kvh * G + r16 % G;
+  bf16x8 qf[FP_RT][KS];
+#pragma unroll
+  for (int rt = 0; rt < FP_RT; ++rt) {
+    const int tok_local = (wave * FP_RT + rt) * TW + r16 / G;
+    row_valid[rt] = r16 / G < TW && tok_local < ntok;
+    tok[rt] = tok0 + (row_valid[rt] ? tok_local : 0);
+    pos[rt] = row_valid[rt] ? pos_first + tok_local : -1;
+    row_lo[rt] = (window > 0 && pos[rt] + 1 > window) ? pos[rt] + 1 - window : 0;
+    const bf16_t* qrow = q + (int64_t)tok[rt] * q_stride + (int64_t)head * HD;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d = ks * 32 + g * 8;
+      bf16x8 z = {};
+      qf[rt][ks] = (row_valid[rt] && d < HD) ? *(const bf16x8*)(qrow + d) : z;
+    }
+  }
+  // a wave whose rows all end before a key tile begins has nothing to do in it
+  int wave_hi = max(pos[0], pos[1]);
+#pragma unroll
+  for (int off = 8; off > 0; off >>= 1) wave_hi = max(wave_hi, __shfl_xor(wave_hi, off, TL_WAVE));
+
+  float m_run[FP_RT], l_run[FP_RT];
+  f32x4 o[FP_RT][HDT];
+#pragma unroll
+  for (int rt = 0; rt < FP_RT; ++rt) {
+    m_run[rt] = -INFINITY;
+    l_run[rt] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < HDT; ++dt) o[rt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const float c_log2 = scale * 1.44269504088896341f;     // scores are kept in units of log2 e
+
+  for (int kt_idx = first_tile; kt_idx < last_tile; ++kt_idx) {
+    {
+      // stage the tile: thread = (key row lane, chunk group wave); V is transposed on the way
+      const int j = kt_idx * FA_KT + lane;
+      const bool in_range = j >= kv_begin && j < kv_end;
+      int64_t row_off = 0;
+      if (in_range) {
+        const int64_t blk = bt[j / block_size];
+        row_off = ((blk * nkv + kvh) * block_size + (j % block_size)) * HD;
+      }
+      const bf16_t* kp = k_cache + row_off;
+      const bf16_t* vp = v_cache + row_off;
+#pragma unroll
+      for (int c0 = 0; c0 < KS * 4; c0 += FA_WAVES) {
+        const int c = c0 + wave;
+        if (c < KS * 4) {
+          bf16x8 z = {};
+          const bf16x8 k8 = (in_range && c * 8 < HD) ? *(const bf16x8*)(kp + c * 8) : z;
+          *(bf16x8*)(Kl + lane * KP + c * 8) = k8;
+        }
+      }
+#pragma unroll
+      for (int c0 = 0; c0 < HD / 8; c0 += FA_WAVES) {
+        const int c = c0 + wave;
+        if (c < HD / 8) {
+          bf16x8 z = {};
+          const bf16x8 v8 = in_range ? *(const bf16x8*)(vp + c * 8) : z;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) Vl[(c * 8 + e) * FA_VP + lane] = v8[e];
+        }
+      }
+    }
+    __syncthreads();
+    if (kt_idx * FA_KT <= wave_hi) {
+      f32x4 sc[FP_RT][4];
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt) {
+#pragma unroll
+        for (int rt = 0; rt < FP_RT; ++rt) sc[rt][kt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const bf16x8 kf = *(const bf16x8*)(Kl + (kt * 16 + r16) * KP + ks * 32 + g * 8);
+#pragma unroll
+          for (int rt = 0; rt < FP_RT; ++rt)
+            sc[rt][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[rt][ks], sc[rt][kt], 0, 0, 0);
+        }
+      }
+      bf16x8 pb[FP_RT][2], pl[FP_RT][2];
+#pragma unroll
+      for (int rt = 0; rt < FP_RT; ++rt) {
+        float m_tile = -INFINITY;
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int j = kt_idx * FA_KT + kt * 16 + g * 4 + r;
+            const bool ok = row_valid[rt] && j <= pos[rt] && j >= row_lo[rt];
+            const float sv = ok ? sc[rt][kt][r] * c_log2 : -INFINITY;
+            sc[rt][kt][r] = sv;
+            m_tile = fmaxf(m_tile, sv);
+          }
+        m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, TL_WAVE));
+        m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, TL_WAVE));
+        const float m_new = fmaxf(m_run[rt], m_tile);
+        const bool any = m_new > -INFINITY;
+        const float alpha = any ? exp2f(m_run[rt] - m_new) : 1.f;
+        float psum = 0.f;
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float p = any ? exp2f(sc[rt][kt][r] - m_new) : 0.f;
+            sc[rt][kt][r] = p;
+            psum += p;
+          }
+        psum += __shfl_xor(psum, 16, TL_WAVE);
+        psum += __shfl_xor(psum, 32, TL_WAVE);
+        l_run[rt] = l_run[rt] * alpha + psum;
+        m_run[rt] = m_new;
+#pragma unroll
+        for (int dt = 0; dt < HDT; ++dt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) o[rt][dt][r] *= alpha;
+#pragma unroll
+        for (int st = 0; st < 2; ++st)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float p0 = sc[rt][2 * st][r], p1 = sc[rt][2 * st + 1][r];
+            pb[rt][st][r] = (bf16_t)p0;
+            pb[rt][st][4 + r] = (bf16_t)p1;
+            pl[rt][st][r] = (bf16_t)(p0 - (float)pb[rt][st][r]);
+            pl[rt][st][4 + r] = (bf16_t)(p1 - (float)pb[rt][st][4 + r]);
+          }
+      }
+#pragma unroll
+      for (int st = 0; st < 2; ++st)
+#pragma unroll
+        for (int dt = 0; dt < HDT; ++dt) {
+          const bf16_t* vrow = Vl + (dt * 16 + r16) * FA_VP + g * 4;
+          const bf16x4 lo4 = *(const bf16x4*)(vrow + (2 * st) * 16);
+          const bf16x4 hi4 = *(const bf16x4*)(vrow + (2 * st + 1) * 16);
+          bf16x8 vf;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            vf[r] = lo4[r];
+            vf[4 + r] = hi4[r];
+          }
+#pragma unroll
+          for (int rt = 0; rt < FP_RT; ++rt) {
+            o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb[rt][st], o[rt][dt], 0, 0, 0);
+            o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pl[rt][st], o[rt][dt], 0, 0, 0);
+          }
+        }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int rt = 0; rt < FP_RT; ++rt) {
+    if (!row_valid[rt]) continue;
+    const float inv = l_run[rt] > 0.f ? 1.f / l_run[rt] : 0.f;
+    bf16_t* orow = out + (int64_t)tok[rt] * out_stride + (int64_t)head * HD + g * 4;
+#pragma unroll
+    for (int dt = 0; dt < HDT; ++dt) {
+      bf16x4 v4;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) v4[r] = (bf16_t)(o[rt][dt][r] * inv);
+      *(bf16x4*)(orow + dt * 16) = v4;
+    }
+  }
+}
+
 // Merges the partial results of `n_splits` workgroups per (token, head).
 __global__ void flash_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                      bf16_t* __restrict__ out, int64_t out_stride, int n_tokens, int nq, int hd,
@@ -401,6 +602,32 @@ int tl_paged_attention(const void* q, int64_t q_stride, const void* k_cache, con
                        positions, (bf16_t*)out, out_stride, nq, nkv, hd, block_size, scale, window);
   else
     return TL_ERR_ARG;
+  return tl_launch_status();
+}
+
+// bfloat16 only, for steps that hold prompt portions.  Tiles describe groups of at most
+// 8 * (16 / (nq / nkv)) consecutive tokens of one request.
+int tl_flash_prefill(const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
+                     const int32_t* block_tables, int max_blocks, const int32_t* tile_req,
+                     const int32_t* tile_tok0, const int32_t* tile_ntok, const int32_t* positions, void* out,
+                     int64_t out_stride, int n_tiles, int nq, int nkv, int hd, int block_size, float scale,
+                     int window, hipStream_t stream) {
+  if (n_tiles <= 0) return TL_OK;
+  if (nq <= 0 || nkv <= 0 || nq % nkv || nq / nkv > 16 || hd <= 0 || hd % 16 || hd > 128 || block_size <= 0 ||
+      max_blocks <= 0 || window < 0 || nkv > 65535 || q_stride % 8 || out_stride % 4)
+    return TL_ERR_ARG;
+#define TL_PREFILL_CASE(HDT)                                                                                      \
+  case HDT:                                                                                                       \
+    hipLaunchKernelGGL(flash_prefill_bf16_kernel<HDT>, dim3(n_tiles, nkv), dim3(FA_THREADS), 0, stream,           \
+                       (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,  \
+                       max_blocks, tile_req, tile_tok0, tile_ntok, positions, (bf16_t*)out, out_stride, nq, nkv,  \
+                       block_size, scale, window);                                                                \
+    break;
+  switch (hd / 16) {
+    TL_PREFILL_CASE(1) TL_PREFILL_CASE(2) TL_PREFILL_CASE(3) TL_PREFILL_CASE(4)
+    TL_PREFILL_CASE(5) TL_PREFILL_CASE(6) TL_PREFILL_CASE(7) TL_PREFILL_CASE(8)
+  }
+#undef TL_PREFILL_CASE
   return tl_launch_status();
 }
 

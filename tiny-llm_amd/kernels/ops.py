@@ -333,6 +333,44 @@ def flash_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     return out
 
 
+PREFILL_TILES = 8     # query tiles (of 16 rows) one workgroup of the prefill attention kernel owns
+
+
+def flash_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                  tiles, positions: torch.Tensor, out: torch.Tensor, num_heads: int, num_kv_heads: int,
+                  head_dim: int, scale: float, window: int = 0) -> torch.Tensor:
+    """`flash_attention` arranged for prompt portions: `tiles` are groups of at most
+    PREFILL_TILES * (16 // (heads / kv_heads)) consecutive tokens of one request, and a key or value
+    row is staged once per such group."""
+    tile_req, tile_tok0, tile_ntok = tiles
+    _dev(q, k_cache, v_cache, block_tables, tile_req, tile_tok0, tile_ntok, positions, out)
+    _rows_2d(q, "q")
+    _rows_2d(out, "attention output")
+    T = q.shape[0]
+    _need(flash_attention_supported(q.dtype, num_heads, num_kv_heads, head_dim),
+          "the MFMA attention kernel takes bfloat16, head sizes in steps of 16 up to 128, up to 16 heads per kv head")
+    _need(q.shape[1] == num_heads * head_dim and tuple(out.shape) == (T, num_heads * head_dim),
+          "q and the attention output must be [T, heads * head_dim]")
+    _need(q.dtype == k_cache.dtype == v_cache.dtype == out.dtype, "q, caches and output must share an element type")
+    _need(k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dim() == 4
+          and k_cache.shape == v_cache.shape and k_cache.shape[1] == num_kv_heads
+          and k_cache.shape[3] == head_dim, "cache must be contiguous [blocks, kv_heads, block, head_dim]")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(),
+          "block tables must be contiguous int32 [requests, max_blocks]")
+    _need(positions.dtype == torch.int32 and positions.is_contiguous() and positions.numel() == T,
+          "positions must be contiguous int32, one per row")
+    n_tiles = tile_req.numel()
+    for t in (tile_req, tile_tok0, tile_ntok):
+        _need(t.dtype == torch.int32 and t.is_contiguous() and t.numel() == n_tiles, "tile arrays must be int32 [tiles]")
+    _need(q.stride(0) % 8 == 0 and out.stride(0) % 4 == 0, "q and output rows must be vector aligned")
+    _check(_lib().tl_flash_prefill(
+        _ptr(q, 16), c_int64(q.stride(0)), _ptr(k_cache, 16), _ptr(v_cache, 16), _ptr(block_tables),
+        c_int(block_tables.shape[1]), _ptr(tile_req), _ptr(tile_tok0), _ptr(tile_ntok), _ptr(positions),
+        _ptr(out, 8), c_int64(out.stride(0)), c_int(n_tiles), c_int(num_heads), c_int(num_kv_heads),
+        c_int(head_dim), c_int(k_cache.shape[2]), c_float(scale), c_int(window), _stream()), "flash_prefill")
+    return out
+
+
 def sample(logits: torch.Tensor, out: torch.Tensor, temperature: Optional[torch.Tensor] = None,
            top_k: Optional[torch.Tensor] = None, top_p: Optional[torch.Tensor] = None,
            seeds: Optional[torch.Tensor] = None, counters: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -80,11 +80,18 @@ class Attention(Mixer):
         q = qkv[:, :self.q_size]
         if ops.flash_attention_supported(self.dtype, self.num_heads, self.num_kv_heads, self.head_dim):
             group = self.num_heads // self.num_kv_heads
-            tiles = ctx.attention_tiles(16 // group)
-            n_splits, scratch = self._splits(ctx, tiles[0].numel(), T, residual.device)
-            ops.flash_attention(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, attn,
-                                self.num_heads, self.num_kv_heads, self.head_dim, self.scale, self.window,
-                                n_splits, scratch)
+            if ctx.max_q_len > 1:
+                # prompt portions: many query rows share each staged key tile
+                tiles = ctx.attention_tiles(ops.PREFILL_TILES * (16 // group))
+                ops.flash_prefill(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, attn,
+                                  self.num_heads, self.num_kv_heads, self.head_dim, self.scale, self.window)
+            else:
+                # decoding: one token per request, its keys split over waves and workgroups
+                tiles = ctx.attention_tiles(16 // group)
+                n_splits, scratch = self._splits(ctx, tiles[0].numel(), T, residual.device)
+                ops.flash_attention(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, attn,
+                                    self.num_heads, self.num_kv_heads, self.head_dim, self.scale, self.window,
+                                    n_splits, scratch)
         else:
             ops.paged_attention(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.req_of_token,
                                 ctx.positions, attn, self.num_heads, self.num_kv_heads, self.head_dim,
