@@ -350,7 +350,8 @@ __global__ __launch_bounds__(FA_THREADS) void flash_prefill_bf16_kernel(
 
   const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
   const int r16 = lane % 16, g = lane / 16;
-  const int tile = blockIdx.x, kvh = blockIdx.y;
+  // later tiles of a prompt have more keys to go through: they are started first
+  const int tile = gridDim.x - 1 - blockIdx.x, kvh = blockIdx.y;
   const int G = nq / nkv, TW = 16 / G;
   const int req = tile_req[tile], tok0 = tile_tok0[tile], ntok = tile_ntok[tile];
   const int32_t* bt = block_tables + (int64_t)req * max_blocks;
@@ -386,50 +387,82 @@ __global__ __launch_bounds__(FA_THREADS) void flash_prefill_bf16_kernel(
 #pragma unroll
   for (int off = 8; off > 0; off >>= 1) wave_hi = max(wave_hi, __shfl_xor(wave_hi, off, TL_WAVE));
 
+  // The running maximum starts at a large negative FINITE number, so exp2(m - m') is never
+  // exp2(-inf + inf); a masked score is -inf and its probability exp2(-inf) = 0.
+  constexpr float kNegBig = -1.0e30f;
   float m_run[FP_RT], l_run[FP_RT];
   f32x4 o[FP_RT][HDT];
 #pragma unroll
   for (int rt = 0; rt < FP_RT; ++rt) {
-    m_run[rt] = -INFINITY;
+    m_run[rt] = kNegBig;
     l_run[rt] = 0.f;
 #pragma unroll
     for (int dt = 0; dt < HDT; ++dt) o[rt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
   const float c_log2 = scale * 1.44269504088896341f;     // scores are kept in units of log2 e
+  // smallest position and largest window start among this wave's valid rows: a key tile that lies
+  // wholly between them is visible to every row and needs no mask
+  int wave_lo_pos = 0x7fffffff, wave_hi_lo = 0;
+#pragma unroll
+  for (int rt = 0; rt < FP_RT; ++rt)
+    if (row_valid[rt]) {
+      wave_lo_pos = min(wave_lo_pos, pos[rt]);
+      wave_hi_lo = max(wave_hi_lo, row_lo[rt]);
+    }
+#pragma unroll
+  for (int off = 8; off > 0; off >>= 1) {
+    wave_lo_pos = min(wave_lo_pos, __shfl_xor(wave_lo_pos, off, TL_WAVE));
+    wave_hi_lo = max(wave_hi_lo, __shfl_xor(wave_hi_lo, off, TL_WAVE));
+  }
+  bool all_valid = row_valid[0] && row_valid[1];
+  all_valid = __all(all_valid);
+
+  // staging registers: thread = (key row `lane`, chunk group `wave`); the rows of the next tile are
+  // requested while the current tile is being worked on
+  constexpr int KC = (KS * 4 + FA_WAVES - 1) / FA_WAVES, VC = (HD / 8 + FA_WAVES - 1) / FA_WAVES;
+  bf16x8 k_stage[KC], v_stage[VC];
+  auto fetch_tile = [&](int kt_idx) {
+    const int j = kt_idx * FA_KT + lane;
+    const bool in_range = j >= kv_begin && j < kv_end;
+    int64_t row_off = 0;
+    if (in_range) {
+      const int64_t blk = bt[j / block_size];
+      row_off = ((blk * nkv + kvh) * block_size + (j % block_size)) * HD;
+    }
+    const bf16_t* kp = k_cache + row_off;
+    const bf16_t* vp = v_cache + row_off;
+#pragma unroll
+    for (int ci = 0; ci < KC; ++ci) {
+      const int c = ci * FA_WAVES + wave;
+      bf16x8 z = {};
+      k_stage[ci] = (in_range && c * 8 < HD) ? *(const bf16x8*)(kp + c * 8) : z;
+    }
+#pragma unroll
+    for (int ci = 0; ci < VC; ++ci) {
+      const int c = ci * FA_WAVES + wave;
+      bf16x8 z = {};
+      v_stage[ci] = (in_range && c < HD / 8) ? *(const bf16x8*)(vp + c * 8) : z;
+    }
+  };
+  if (first_tile < last_tile) fetch_tile(first_tile);
 
   for (int kt_idx = first_tile; kt_idx < last_tile; ++kt_idx) {
-    {
-      // stage the tile: thread = (key row lane, chunk group wave); V is transposed on the way
-      const int j = kt_idx * FA_KT + lane;
-      const bool in_range = j >= kv_begin && j < kv_end;
-      int64_t row_off = 0;
-      if (in_range) {
-        const int64_t blk = bt[j / block_size];
-        row_off = ((blk * nkv + kvh) * block_size + (j % block_size)) * HD;
-      }
-      const bf16_t* kp = k_cache + row_off;
-      const bf16_t* vp = v_cache + row_off;
+    // registers -> LDS; V is transposed on the way
 #pragma unroll
-      for (int c0 = 0; c0 < KS * 4; c0 += FA_WAVES) {
-        const int c = c0 + wave;
-        if (c < KS * 4) {
-          bf16x8 z = {};
-          const bf16x8 k8 = (in_range && c * 8 < HD) ? *(const bf16x8*)(kp + c * 8) : z;
-          *(bf16x8*)(Kl + lane * KP + c * 8) = k8;
-        }
-      }
+    for (int ci = 0; ci < KC; ++ci) {
+      const int c = ci * FA_WAVES + wave;
+      if (c < KS * 4) *(bf16x8*)(Kl + lane * KP + c * 8) = k_stage[ci];
+    }
 #pragma unroll
-      for (int c0 = 0; c0 < HD / 8; c0 += FA_WAVES) {
-        const int c = c0 + wave;
-        if (c < HD / 8) {
-          bf16x8 z = {};
-          const bf16x8 v8 = in_range ? *(const bf16x8*)(vp + c * 8) : z;
+    for (int ci = 0; ci < VC; ++ci) {
+      const int c = ci * FA_WAVES + wave;
+      if (c < HD / 8) {
 #pragma unroll
-          for (int e = 0; e < 8; ++e) Vl[(c * 8 + e) * FA_VP + lane] = v8[e];
-        }
+        for (int e = 0; e < 8; ++e) Vl[(c * 8 + e) * FA_VP + lane] = v_stage[ci][e];
       }
     }
     __syncthreads();
+    if (kt_idx + 1 < last_tile) fetch_tile(kt_idx + 1);
     if (kt_idx * FA_KT <= wave_hi) {
       f32x4 sc[FP_RT][4];
 #pragma unroll
@@ -445,30 +478,39 @@ __global__ __launch_bounds__(FA_THREADS) void flash_prefill_bf16_kernel(
         }
       }
       bf16x8 pb[FP_RT][2], pl[FP_RT][2];
+      const int tile_j0 = kt_idx * FA_KT;
+      const bool no_mask = all_valid && tile_j0 + FA_KT - 1 <= wave_lo_pos && tile_j0 >= wave_hi_lo;
 #pragma unroll
       for (int rt = 0; rt < FP_RT; ++rt) {
-        float m_tile = -INFINITY;
+        float m_tile = kNegBig;
+        if (no_mask) {
 #pragma unroll
-        for (int kt = 0; kt < 4; ++kt)
+          for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int j = kt_idx * FA_KT + kt * 16 + g * 4 + r;
-            const bool ok = row_valid[rt] && j <= pos[rt] && j >= row_lo[rt];
-            const float sv = ok ? sc[rt][kt][r] * c_log2 : -INFINITY;
-            sc[rt][kt][r] = sv;
-            m_tile = fmaxf(m_tile, sv);
-          }
+            for (int r = 0; r < 4; ++r) m_tile = fmaxf(m_tile, sc[rt][kt][r]);
+        } else {
+#pragma unroll
+          for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int j = tile_j0 + kt * 16 + g * 4 + r;
+              const bool ok = row_valid[rt] && j <= pos[rt] && j >= row_lo[rt];
+              const float sv = ok ? sc[rt][kt][r] : -INFINITY;
+              sc[rt][kt][r] = sv;
+              m_tile = fmaxf(m_tile, sv);
+            }
+        }
         m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, TL_WAVE));
         m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, TL_WAVE));
-        const float m_new = fmaxf(m_run[rt], m_tile);
-        const bool any = m_new > -INFINITY;
-        const float alpha = any ? exp2f(m_run[rt] - m_new) : 1.f;
+        // the maximum is taken over raw scores (the scale is positive) and scaled once
+        const float m_new = fmaxf(m_run[rt], m_tile * c_log2);
+        const float alpha = __builtin_amdgcn_exp2f(m_run[rt] - m_new);
         float psum = 0.f;
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            const float p = any ? exp2f(sc[rt][kt][r] - m_new) : 0.f;
+            const float p = __builtin_amdgcn_exp2f(fmaf(sc[rt][kt][r], c_log2, -m_new));
             sc[rt][kt][r] = p;
             psum += p;
           }
@@ -476,10 +518,12 @@ __global__ __launch_bounds__(FA_THREADS) void flash_prefill_bf16_kernel(
         psum += __shfl_xor(psum, 32, TL_WAVE);
         l_run[rt] = l_run[rt] * alpha + psum;
         m_run[rt] = m_new;
+        if (__any(alpha != 1.f)) {
 #pragma unroll
-        for (int dt = 0; dt < HDT; ++dt)
+          for (int dt = 0; dt < HDT; ++dt)
 #pragma unroll
-          for (int r = 0; r < 4; ++r) o[rt][dt][r] *= alpha;
+            for (int r = 0; r < 4; ++r) o[rt][dt][r] *= alpha;
+        }
 #pragma unroll
         for (int st = 0; st < 2; ++st)
 #pragma unroll

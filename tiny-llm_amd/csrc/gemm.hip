@@ -8,8 +8,8 @@
 //    matrix mode.  The k order of the accumulation does not depend on M, so a row
 //    gives the same bits whether it is computed alone or in a batch.
 //  * gemm_bf16_kernel: bf16 inputs on the MFMA matrix cores
-//    (v_mfma_f32_32x32x16_bf16), float32 accumulation, 128x128x32 tiles staged
-//    through LDS, four wave64 per workgroup.
+//    (v_mfma_f32_32x32x16_bf16), float32 accumulation, 128x128x64 (or 64x128x64) tiles
+//    staged through double-buffered LDS, four wave64 per workgroup.
 #include "common.h"
 
 namespace {
@@ -89,82 +89,116 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f32_kernel(const float* __rest
 }
 
 // ==================================================================== bfloat16
-constexpr int B_BM = 128, B_BN = 128, B_BK = 32, B_THREADS = 256;
-constexpr int B_LD = B_BK + 8;  // LDS row stride in elements: 80 bytes, keeps 16-byte alignment
+// Tiles of BM x 128 outputs (BM = 128, or 64 where that is needed to fill the chip), k in steps
+// of 64, four wave64 as 2 x 2, each owning (BM/2) x 64 outputs as 32x32x16 MFMA tiles.  Operand
+// tiles go global -> registers -> LDS; LDS is double-buffered so an iteration needs one barrier,
+// and the global loads of the next k step are in flight while the current one is multiplied.
+constexpr int B_BN = 128, B_BK = 64, B_THREADS = 256;
+constexpr int B_LD = B_BK + 8;  // LDS row stride in elements: 144 bytes, keeps 16-byte alignment
+
+template <int BM>
+struct GemmStage {                       // one k step of both operand tiles, spread over the threads
+  static constexpr int AC = BM * (B_BK / 8) / B_THREADS, WC = B_BN * (B_BK / 8) / B_THREADS;
+  bf16x8 a[AC], w[WC];
+};
 
 // K must be a multiple of 8 (16-byte chunks of bf16 never straddle the end).
-template <typename TO, bool SWIGLU>
+template <int BM, typename TO, bool SWIGLU, bool FULL>
 __global__ __launch_bounds__(B_THREADS) void gemm_bf16_kernel(const bf16_t* __restrict__ a,
                                                               const bf16_t* __restrict__ w,
                                                               TO* __restrict__ out,
                                                               const float* __restrict__ residual,
                                                               const float* __restrict__ row_scale, int M,
                                                               int N, int K, int64_t lda, int64_t ldo) {
-  __shared__ __attribute__((aligned(16))) bf16_t As[B_BM * B_LD];
-  __shared__ __attribute__((aligned(16))) bf16_t Ws[B_BN * B_LD];
+  constexpr int MI = BM / 64;            // 32-row MFMA tiles per wave along m
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  bf16_t* As = (bf16_t*)smem_raw;                       // [2][BM][B_LD]
+  bf16_t* Ws = As + 2 * BM * B_LD;                      // [2][B_BN][B_LD]
   const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
   const int wm = wave / 2, wn = wave % 2;
-  const int m0 = blockIdx.y * B_BM, n0 = blockIdx.x * B_BN;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * B_BN;
 
-  f32x16 acc[2][2];
+  f32x16 acc[MI][2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < MI; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  // staging: 512 16-byte chunks per operand tile, two per thread
-  bf16x8 ra[2], rw[2];
-  auto load_tiles = [&](int k0) {
+  using Stage = GemmStage<BM>;
+  // Loads are unconditional (addresses clamped into the matrix; a chunk that lies outside is zeroed
+  // when it is written to LDS): a predicated load becomes a branch, and then the outstanding-load
+  // counter cannot be used to wait for one stage while the next stays in flight.
+  auto load_stage = [&](Stage& st, int k0) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < Stage::AC; ++i) {
       const int c = tid + i * B_THREADS;
-      const int row = c / 4, kc = (c % 4) * 8;
-      const int k = k0 + kc;
-      bf16x8 z = {};
-      ra[i] = (m0 + row < M && k < K) ? *(const bf16x8*)(a + (int64_t)(m0 + row) * lda + k) : z;
-      rw[i] = (n0 + row < N && k < K) ? *(const bf16x8*)(w + (int64_t)(n0 + row) * K + k) : z;
+      const int row = m0 + c / 8, k = k0 + (c % 8) * 8;
+      st.a[i] = *(const bf16x8*)(a + (int64_t)min(row, M - 1) * lda + min(k, K - 8));
+    }
+#pragma unroll
+    for (int i = 0; i < Stage::WC; ++i) {
+      const int c = tid + i * B_THREADS;
+      const int row = n0 + c / 8, k = k0 + (c % 8) * 8;
+      st.w[i] = *(const bf16x8*)(w + (int64_t)min(row, N - 1) * K + min(k, K - 8));
     }
   };
-  auto store_tiles = [&]() {
+  // FULL: M, N and K are multiples of the tile, so no chunk lies outside and nothing is zeroed
+  auto store_stage = [&](const Stage& st, int buf, int k0) {
+    bf16x8 z = {};
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < Stage::AC; ++i) {
       const int c = tid + i * B_THREADS;
-      const int row = c / 4, kc = (c % 4) * 8;
-      *(bf16x8*)(As + row * B_LD + kc) = ra[i];
-      *(bf16x8*)(Ws + row * B_LD + kc) = rw[i];
+      const bool ok = FULL || (m0 + c / 8 < M && k0 + (c % 8) * 8 < K);
+      *(bf16x8*)(As + (buf * BM + c / 8) * B_LD + (c % 8) * 8) = ok ? st.a[i] : z;
+    }
+#pragma unroll
+    for (int i = 0; i < Stage::WC; ++i) {
+      const int c = tid + i * B_THREADS;
+      const bool ok = FULL || (n0 + c / 8 < N && k0 + (c % 8) * 8 < K);
+      *(bf16x8*)(Ws + (buf * B_BN + c / 8) * B_LD + (c % 8) * 8) = ok ? st.w[i] : z;
     }
   };
-
-  load_tiles(0);
-  for (int k0 = 0; k0 < K; k0 += B_BK) {
-    __syncthreads();
-    store_tiles();
-    __syncthreads();
-    if (k0 + B_BK < K) load_tiles(k0 + B_BK);
+  auto compute = [&](int buf) {
 #pragma unroll
     for (int ks = 0; ks < B_BK; ks += 16) {
-      bf16x8 fa[2], fw[2];
+      bf16x8 fa[MI], fw[2];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        fa[i] = *(const bf16x8*)(As + (wm * 64 + i * 32 + lane % 32) * B_LD + ks + (lane / 32) * 8);
-        fw[i] = *(const bf16x8*)(Ws + (wn * 64 + i * 32 + lane % 32) * B_LD + ks + (lane / 32) * 8);
-      }
+      for (int i = 0; i < MI; ++i)
+        fa[i] = *(const bf16x8*)(As + (buf * BM + wm * (BM / 2) + i * 32 + lane % 32) * B_LD + ks + (lane / 32) * 8);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        fw[j] = *(const bf16x8*)(Ws + (buf * B_BN + wn * 64 + j * 32 + lane % 32) * B_LD + ks + (lane / 32) * 8);
       // result tile is transposed (rows = n, columns = m) so that a lane holds four
       // consecutive n of one output row and can store them as one vector
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[j], fa[i], acc[i][j], 0, 0, 0);
     }
+  };
+
+  const int nk = (K + B_BK - 1) / B_BK;
+  Stage st;
+  load_stage(st, 0);
+  store_stage(st, 0, 0);
+  __syncthreads();
+  // iteration kt: the loads of step kt + 1 are in flight while step kt is multiplied out of
+  // LDS[kt & 1]; they land in the other LDS buffer before the iteration's one barrier
+  for (int kt = 0; kt < nk; ++kt) {
+    const int cur = kt & 1;
+    if (kt + 1 < nk) load_stage(st, (kt + 1) * B_BK);
+    compute(cur);
+    if (kt + 1 < nk) store_stage(st, cur ^ 1, (kt + 1) * B_BK);
+    __syncthreads();
   }
 
   const bool vec_ok = (N % 4 == 0) && (ldo % 4 == 0);
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int m = m0 + wm * 64 + i * 32 + lane % 32;
+  for (int i = 0; i < MI; ++i) {
+    const int m = m0 + wm * (BM / 2) + i * 32 + lane % 32;
     if (m >= M) continue;
     const float rs = row_scale ? row_scale[m] : 1.f;   // e.g. 1 / rms of a norm left out of the operand
 #pragma unroll
@@ -188,11 +222,11 @@ __global__ __launch_bounds__(B_THREADS) void gemm_bf16_kernel(const bf16_t* __re
             v[0] += r[0]; v[1] += r[1]; v[2] += r[2]; v[3] += r[3];
           }
           if constexpr (sizeof(TO) == 4) {
-            f32x4 s = {v[0], v[1], v[2], v[3]};
-            *(f32x4*)((float*)out + o) = s;
+            f32x4 sv = {v[0], v[1], v[2], v[3]};
+            *(f32x4*)((float*)out + o) = sv;
           } else {
-            bf16x4 s = {(bf16_t)v[0], (bf16_t)v[1], (bf16_t)v[2], (bf16_t)v[3]};
-            *(bf16x4*)((bf16_t*)out + o) = s;
+            bf16x4 sv = {(bf16_t)v[0], (bf16_t)v[1], (bf16_t)v[2], (bf16_t)v[3]};
+            *(bf16x4*)((bf16_t*)out + o) = sv;
           }
         } else {
           for (int e = 0; e < 4 && n + e < N; ++e) {
@@ -206,6 +240,42 @@ __global__ __launch_bounds__(B_THREADS) void gemm_bf16_kernel(const bf16_t* __re
   }
 }
 
+template <int BM, typename TO, bool SWIGLU, bool FULL>
+static int launch_gemm_bf16_full(const bf16_t* a, const bf16_t* w, TO* out, const float* residual,
+                                 const float* row_scale, int M, int N, int K, int64_t lda, int64_t ldo,
+                                 hipStream_t stream) {
+  constexpr size_t smem = (size_t)2 * (BM + B_BN) * B_LD * sizeof(bf16_t);
+  static bool configured = false;
+  if (!configured) {
+    if (hipFuncSetAttribute((const void*)gemm_bf16_kernel<BM, TO, SWIGLU, FULL>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+      return TL_ERR_LAUNCH;
+    configured = true;
+  }
+  dim3 g((N + B_BN - 1) / B_BN, (M + BM - 1) / BM);
+  hipLaunchKernelGGL((gemm_bf16_kernel<BM, TO, SWIGLU, FULL>), g, dim3(B_THREADS), smem, stream, a, w, out, residual,
+                     row_scale, M, N, K, lda, ldo);
+  return TL_OK;
+}
+
+template <int BM, typename TO, bool SWIGLU>
+static int launch_gemm_bf16(const bf16_t* a, const bf16_t* w, TO* out, const float* residual, const float* row_scale,
+                            int M, int N, int K, int64_t lda, int64_t ldo, hipStream_t stream) {
+  if (M % BM == 0 && N % B_BN == 0 && K % B_BK == 0)
+    return launch_gemm_bf16_full<BM, TO, SWIGLU, true>(a, w, out, residual, row_scale, M, N, K, lda, ldo, stream);
+  return launch_gemm_bf16_full<BM, TO, SWIGLU, false>(a, w, out, residual, row_scale, M, N, K, lda, ldo, stream);
+}
+
+// Tiles of 128 rows unless that leaves compute units without a workgroup.
+template <typename TO, bool SWIGLU>
+static int launch_gemm_bf16_any(const bf16_t* a, const bf16_t* w, TO* out, const float* residual,
+                                const float* row_scale, int M, int N, int K, int64_t lda, int64_t ldo,
+                                hipStream_t stream) {
+  const int64_t wgs128 = (int64_t)((N + B_BN - 1) / B_BN) * ((M + 127) / 128);
+  if (wgs128 >= 512)
+    return launch_gemm_bf16<128, TO, SWIGLU>(a, w, out, residual, row_scale, M, N, K, lda, ldo, stream);
+  return launch_gemm_bf16<64, TO, SWIGLU>(a, w, out, residual, row_scale, M, N, K, lda, ldo, stream);
+}
 
 // ============================================================ bfloat16, few rows
 // Decode-shaped products (M <= 64): the weight matrix is streamed once and is the
@@ -454,19 +524,21 @@ int tl_linear(const void* a, const void* w, void* out, const float* residual, co
   } else if (dtype == 1) {
     if (K % 8 || lda % 8) return TL_ERR_ARG;
     if (out_dtype != 0 && out_dtype != 1) return TL_ERR_ARG;
-    dim3 g((N + B_BN - 1) / B_BN, (M + B_BM - 1) / B_BM);
     if (M <= 64) {
       SkinnyArgs p{a, (const bf16_t*)w, out, residual, nullptr, nullptr, row_scale, 0.f, 0, M, N, K, lda, ldo};
       if (launch_skinny_out<PRO_NONE>(p, out_dtype, swiglu, stream) != TL_OK) return TL_ERR_ARG;
-    } else if (swiglu) {
-      hipLaunchKernelGGL((gemm_bf16_kernel<bf16_t, true>), g, dim3(B_THREADS), 0, stream, (const bf16_t*)a,
-                         (const bf16_t*)w, (bf16_t*)out, residual, row_scale, M, N, K, lda, ldo);
-    } else if (out_dtype == 0) {
-      hipLaunchKernelGGL((gemm_bf16_kernel<float, false>), g, dim3(B_THREADS), 0, stream, (const bf16_t*)a,
-                         (const bf16_t*)w, (float*)out, residual, row_scale, M, N, K, lda, ldo);
     } else {
-      hipLaunchKernelGGL((gemm_bf16_kernel<bf16_t, false>), g, dim3(B_THREADS), 0, stream, (const bf16_t*)a,
-                         (const bf16_t*)w, (bf16_t*)out, residual, row_scale, M, N, K, lda, ldo);
+      int rc;
+      if (swiglu)
+        rc = launch_gemm_bf16_any<bf16_t, true>((const bf16_t*)a, (const bf16_t*)w, (bf16_t*)out, residual, row_scale,
+                                                M, N, K, lda, ldo, stream);
+      else if (out_dtype == 0)
+        rc = launch_gemm_bf16_any<float, false>((const bf16_t*)a, (const bf16_t*)w, (float*)out, residual, row_scale,
+                                                M, N, K, lda, ldo, stream);
+      else
+        rc = launch_gemm_bf16_any<bf16_t, false>((const bf16_t*)a, (const bf16_t*)w, (bf16_t*)out, residual,
+                                                 row_scale, M, N, K, lda, ldo, stream);
+      if (rc != TL_OK) return rc;
     }
   } else {
     return TL_ERR_ARG;
