@@ -435,6 +435,48 @@ def test_flash_attention_decode_batch():
         assert rel(out, ref) < 8e-3
 
 
+@pytest.mark.parametrize("nq,nkv,hd,bs", [(32, 4, 64, 16), (3, 1, 32, 8), (8, 8, 16, 16), (16, 2, 128, 32), (6, 2, 80, 16)])
+@pytest.mark.parametrize("n_splits", [1, 3])
+def test_flash_attention_fused_rotation_and_cache_write(nq, nkv, hd, bs, n_splits):
+    """Decode step with rotation and cache write inside the attention kernel == rope_store + attention."""
+    from tiny_llm_amd.parts.rotary import RotaryEmbedding
+    g = torch.Generator().manual_seed(nq + hd)
+    lens = [1, 2, 63, 64, 65, 129, 300, 17]
+    R = len(lens)
+    rot = RotaryEmbedding("r", torch.bfloat16, DEV, head_dim=hd, theta=10000.0, max_position=512)
+    cos, sin, rd = rot.rotary_tables()
+    nblocks = sum(-(-l // bs) for l in lens) + 2
+    perm = torch.randperm(nblocks, generator=g).tolist()
+    mb = max(-(-l // bs) for l in lens)
+    bt = torch.zeros(R, mb, dtype=torch.int32)
+    kc = (torch.randn(nblocks, nkv, bs, hd, generator=g)).to(torch.bfloat16)
+    vc = (torch.randn(nblocks, nkv, bs, hd, generator=g)).to(torch.bfloat16)
+    slots = []
+    for r, L in enumerate(lens):
+        for b in range(-(-L // bs)):
+            bt[r, b] = perm.pop()
+        slots.append(int(bt[r, (L - 1) // bs]) * bs + (L - 1) % bs)
+    qkv = torch.randn(R, (nq + 2 * nkv) * hd, generator=g).to(torch.bfloat16)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    pos = i32([l - 1 for l in lens])
+    tiles = (i32(list(range(R))), i32(list(range(R))), i32([1] * R))
+    scratch = torch.full((n_splits * R * nq * (hd + 2),), float("nan"), device=DEV)
+    # separate kernels
+    kc1, vc1, qkv1 = kc.clone().to(DEV), vc.clone().to(DEV), qkv.clone().to(DEV)
+    ops().rope_store(qkv1, pos, cos, sin, i32(slots), kc1, vc1, nq, nkv, hd, rd)
+    out1 = torch.empty(R, nq * hd, dtype=torch.bfloat16, device=DEV)
+    ops().flash_attention(qkv1[:, :nq * hd], kc1, vc1, bt.to(DEV), tiles, pos, out1, nq, nkv, hd, hd ** -0.5, 0,
+                          n_splits, scratch)
+    # fused
+    kc2, vc2, qkv2 = kc.clone().to(DEV), vc.clone().to(DEV), qkv.clone().to(DEV)
+    out2 = torch.empty(R, nq * hd, dtype=torch.bfloat16, device=DEV)
+    ops().flash_attention(qkv2[:, :nq * hd], kc2, vc2, bt.to(DEV), tiles, pos, out2, nq, nkv, hd, hd ** -0.5, 0,
+                          n_splits, scratch, fused_rope=(cos, sin))
+    assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2)      # the same rows, the same bits
+    assert torch.equal(qkv2.cpu(), qkv)                          # the input rows are left as they were
+    assert rel(out2, out1.double()) < 1e-6
+
+
 def test_paged_attention_reduces_to_library_routine():
     """One request, whole prompt, identity block table: plain causal attention."""
     nq = nkv = 2

@@ -92,9 +92,9 @@ __global__ __launch_bounds__(TL_WAVE) void paged_attention_kernel(
 // flash_attn_bf16_kernel: the same function on the matrix cores, for head sizes
 // that are multiples of 16 up to 128 and up to 16 query heads per kv head.
 //
-// A workgroup (four wave64) owns a tile of 16 query rows that share one request and
-// one kv head: `tile_ntok` consecutive tokens times the G query heads of the group,
-// row = token * G + head.  The four waves split the 64-key tiles of the request's
+// A workgroup (eight wave64, four for wide heads) owns a tile of 16 query rows that share one
+// request and one kv head: `tile_ntok` consecutive tokens times the G query heads of the group,
+// row = token * G + head.  The waves split the 64-key tiles of the request's
 // cache between them (and `n_splits` workgroups split them further for decoding
 // with few requests), each with a private LDS staging area, and merge their running
 // (max, sum, output) at the end.  Scores are computed transposed, S^T = K Q^T, with
@@ -107,15 +107,46 @@ __global__ __launch_bounds__(TL_WAVE) void paged_attention_kernel(
 // LDS.  Rows of a tile outside [kv_begin, kv_end) are zero-filled instead of read:
 // stale pages may hold anything, and 0 * NaN is NaN.
 constexpr int FA_THREADS = 256, FA_WAVES = 4, FA_KT = 64, FA_VP = 68;
+constexpr float kNegBig = -1.0e30f;   // "no key yet": finite, so exp2(m - m') never sees inf - inf
 
-template <int HDT>
-__global__ __launch_bounds__(FA_THREADS) void flash_attn_bf16_kernel(
+// Optional fusion for decode steps (every tile is ONE new token): the query and the new key are
+// rotated here and the new key and value are written to the cache here, instead of by a kernel of
+// their own (rope_store_kernel) before this one.  q then points at the token's unrotated qkv row.
+struct FusedRope {
+  const float* cos_t;      // [positions, HD / 2]; null: nothing is fused
+  const float* sin_t;
+  bf16_t* k_cache_w;       // the caches, writable
+  bf16_t* v_cache_w;
+  int k_off, v_off;        // element offsets of this row's k and v heads from its q heads
+};
+
+// Rotate-half of 8 dims starting at d0 (a multiple of 8): own chunk x, partner chunk y = the dims
+// d0 +- HD/2; the expressions are rope_store_kernel's.
+template <int HD>
+__device__ __forceinline__ bf16x8 rotate_chunk(const bf16x8 x, const bf16x8 y, int d0, const float* cs,
+                                               const float* sn) {
+  constexpr int HALF = HD / 2;
+  bf16x8 r;
+  const bool first = d0 < HALF;
+  const int j0 = first ? d0 : d0 - HALF;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float c = cs[j0 + e], sv = sn[j0 + e];
+    const float a = first ? (float)x[e] : (float)y[e];     // the pair's first-half value
+    const float b = first ? (float)y[e] : (float)x[e];     // and its second-half value
+    r[e] = (bf16_t)(first ? c * a - sv * b : sv * a + c * b);
+  }
+  return r;
+}
+
+template <int HDT, int WAVES>
+__global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
     const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ tile_req, const int32_t* __restrict__ tile_tok0,
     const int32_t* __restrict__ tile_ntok, const int32_t* __restrict__ positions, bf16_t* __restrict__ out,
     int64_t out_stride, float* __restrict__ part_o, float* __restrict__ part_ml, int nq, int nkv,
-    int block_size, float scale, int window, int n_splits, int n_tokens) {
+    int block_size, float scale, int window, int n_splits, int n_tokens, const FusedRope fused) {
   constexpr int HD = HDT * 16;
   constexpr int KS = (HD + 31) / 32;       // k-steps of the score product
   constexpr int KP = KS * 32 + 8;          // LDS row stride of the K tile (elements)
@@ -132,6 +163,7 @@ __global__ __launch_bounds__(FA_THREADS) void flash_attn_bf16_kernel(
   const int32_t* bt = block_tables + (int64_t)req * max_blocks;
   bf16_t* Kl = smem + wave * WAVE_ELEMS;
   bf16_t* Vl = Kl + K_ELEMS;
+  const bool do_rope = fused.cos_t != nullptr;
 
   // this lane's query row
   const int tok_local = r16 / G, hh = r16 % G;
@@ -153,7 +185,11 @@ __global__ __launch_bounds__(FA_THREADS) void flash_attn_bf16_kernel(
   const int per_split = (last_tile - first_tile + n_splits - 1) / n_splits;
   const int range_lo = first_tile + split * per_split;
   const int range_hi = min(last_tile, range_lo + per_split);
-  const int iters = (max(range_hi - range_lo, 0) + FA_WAVES - 1) / FA_WAVES;
+  const int iters = (max(range_hi - range_lo, 0) + WAVES - 1) / WAVES;
+  // fused mode: the one new token of the tile, at position kv_end - 1
+  const int new_pos = kv_end - 1;
+  const float* cs = do_rope ? fused.cos_t + (int64_t)new_pos * (HD / 2) : nullptr;
+  const float* sn = do_rope ? fused.sin_t + (int64_t)new_pos * (HD / 2) : nullptr;
 
   // query fragments (B operand): row r16, dims ks*32 + g*8 .. +8
   bf16x8 qf[KS];
@@ -163,17 +199,22 @@ __global__ __launch_bounds__(FA_THREADS) void flash_attn_bf16_kernel(
     for (int ks = 0; ks < KS; ++ks) {
       const int d = ks * 32 + g * 8;
       bf16x8 z = {};
-      qf[ks] = (row_valid && d < HD) ? *(const bf16x8*)(qrow + d) : z;
+      qf[ks] = z;
+      if (row_valid && d < HD) {
+        const bf16x8 x = *(const bf16x8*)(qrow + d);
+        qf[ks] = do_rope ? rotate_chunk<HD>(x, *(const bf16x8*)(qrow + (d + HD / 2) % HD), d, cs, sn) : x;
+      }
     }
   }
 
-  float m_run = -INFINITY, l_run = 0.f;
+  float m_run = kNegBig, l_run = 0.f;
   f32x4 o[HDT];
 #pragma unroll
   for (int dt = 0; dt < HDT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const float c_log2 = scale * 1.44269504088896341f;     // scores are kept in units of log2 e
 
   for (int it = 0; it < iters; ++it) {
-    const int kt_idx = range_lo + it * FA_WAVES + wave;
+    const int kt_idx = range_lo + it * WAVES + wave;
     const bool active = kt_idx < range_hi;
     if (active) {
       // stage this wave's tile: lane = key row
@@ -184,20 +225,43 @@ __global__ __launch_bounds__(FA_THREADS) void flash_attn_bf16_kernel(
         const int64_t blk = bt[j / block_size];
         row_off = ((blk * nkv + kvh) * block_size + (j % block_size)) * HD;
       }
-      const bf16_t* kp = k_cache + row_off;
-      const bf16_t* vp = v_cache + row_off;
+      if (do_rope && j == new_pos) {
+        // the new token's own key and value: made here from its qkv row, and written to the cache
+        const bf16_t* krow = q + (int64_t)tok0 * q_stride + fused.k_off + (int64_t)kvh * HD;
+        const bf16_t* vrow = q + (int64_t)tok0 * q_stride + fused.v_off + (int64_t)kvh * HD;
 #pragma unroll
-      for (int c = 0; c < KS * 4; ++c) {
-        bf16x8 z = {};
-        const bf16x8 kv8 = (in_range && c * 8 < HD) ? *(const bf16x8*)(kp + c * 8) : z;
-        *(bf16x8*)(Kl + lane * KP + c * 8) = kv8;
-      }
+        for (int c = 0; c < KS * 4; ++c) {
+          bf16x8 k8 = {};
+          if (c * 8 < HD) {
+            k8 = rotate_chunk<HD>(*(const bf16x8*)(krow + c * 8), *(const bf16x8*)(krow + (c * 8 + HD / 2) % HD),
+                                  c * 8, cs, sn);
+            *(bf16x8*)(fused.k_cache_w + row_off + c * 8) = k8;
+          }
+          *(bf16x8*)(Kl + lane * KP + c * 8) = k8;
+        }
 #pragma unroll
-      for (int c = 0; c < HD / 8; ++c) {
-        bf16x8 z = {};
-        const bf16x8 v8 = in_range ? *(const bf16x8*)(vp + c * 8) : z;
+        for (int c = 0; c < HD / 8; ++c) {
+          const bf16x8 v8 = *(const bf16x8*)(vrow + c * 8);
+          *(bf16x8*)(fused.v_cache_w + row_off + c * 8) = v8;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) Vl[(c * 8 + e) * FA_VP + lane] = v8[e];
+          for (int e = 0; e < 8; ++e) Vl[(c * 8 + e) * FA_VP + lane] = v8[e];
+        }
+      } else {
+        const bf16_t* kp = k_cache + row_off;
+        const bf16_t* vp = v_cache + row_off;
+#pragma unroll
+        for (int c = 0; c < KS * 4; ++c) {
+          bf16x8 z = {};
+          const bf16x8 kv8 = (in_range && c * 8 < HD) ? *(const bf16x8*)(kp + c * 8) : z;
+          *(bf16x8*)(Kl + lane * KP + c * 8) = kv8;
+        }
+#pragma unroll
+        for (int c = 0; c < HD / 8; ++c) {
+          bf16x8 z = {};
+          const bf16x8 v8 = in_range ? *(const bf16x8*)(vp + c * 8) : z;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) Vl[(c * 8 + e) * FA_VP + lane] = v8[e];
+        }
       }
     }
     __syncthreads();
@@ -213,28 +277,27 @@ __global__ __launch_bounds__(FA_THREADS) void flash_attn_bf16_kernel(
           sc[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], sc[kt], 0, 0, 0);
         }
       }
-      float m_tile = -INFINITY;
+      float m_tile = kNegBig;
 #pragma unroll
       for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int j = kt_idx * FA_KT + kt * 16 + g * 4 + r;
           const bool ok = row_valid && j <= pos && j >= row_lo;
-          const float sv = ok ? sc[kt][r] * scale : -INFINITY;
+          const float sv = ok ? sc[kt][r] : -INFINITY;
           sc[kt][r] = sv;
           m_tile = fmaxf(m_tile, sv);
         }
       m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, TL_WAVE));
       m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, TL_WAVE));
-      const float m_new = fmaxf(m_run, m_tile);
-      const bool any = m_new > -INFINITY;
-      const float alpha = any ? expf(m_run - m_new) : 1.f;
+      const float m_new = fmaxf(m_run, m_tile * c_log2);   // the scale is positive: the maximum commutes
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
       float psum = 0.f;
 #pragma unroll
       for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const float p = any ? expf(sc[kt][r] - m_new) : 0.f;
+          const float p = __builtin_amdgcn_exp2f(fmaf(sc[kt][r], c_log2, -m_new));
           sc[kt][r] = p;
           psum += p;
         }
@@ -278,7 +341,7 @@ __global__ __launch_bounds__(FA_THREADS) void flash_attn_bf16_kernel(
     __syncthreads();
   }
 
-  // merge the four waves: each leaves (m, l, O[16][HD]) as floats in its own LDS area
+  // merge the waves: each leaves (m, l, O[16][HD]) as floats in its own LDS area
   constexpr int MROW = HD + 2;
   float* Mw = (float*)(smem + wave * WAVE_ELEMS);
 #pragma unroll
@@ -290,39 +353,38 @@ __global__ __launch_bounds__(FA_THREADS) void flash_attn_bf16_kernel(
     Mw[r16 * MROW + HD + 1] = l_run;
   }
   __syncthreads();
-  {
-    const int row = tid / 16, dl = tid % 16;
+  for (int e = tid; e < 16 * 16; e += WAVES * TL_WAVE) {
+    const int row = e / 16, dl = e % 16;
     const int t_local = row / G, h_local = row % G;
-    if (t_local < ntok) {
-      const int t = tok0 + t_local, h = kvh * G + h_local;
-      float mw[FA_WAVES], M = -INFINITY;
+    if (t_local >= ntok) continue;
+    const int t = tok0 + t_local, h = kvh * G + h_local;
+    float mw[WAVES], M = kNegBig;
 #pragma unroll
-      for (int wv = 0; wv < FA_WAVES; ++wv) {
-        mw[wv] = ((const float*)(smem + wv * WAVE_ELEMS))[row * MROW + HD];
-        M = fmaxf(M, mw[wv]);
-      }
-      float L = 0.f, wgt[FA_WAVES];
+    for (int wv = 0; wv < WAVES; ++wv) {
+      mw[wv] = ((const float*)(smem + wv * WAVE_ELEMS))[row * MROW + HD];
+      M = fmaxf(M, mw[wv]);
+    }
+    float L = 0.f, wgt[WAVES];
 #pragma unroll
-      for (int wv = 0; wv < FA_WAVES; ++wv) {
-        wgt[wv] = mw[wv] > -INFINITY ? expf(mw[wv] - M) : 0.f;
-        L += wgt[wv] * ((const float*)(smem + wv * WAVE_ELEMS))[row * MROW + HD + 1];
-      }
-      for (int d = dl; d < HD; d += 16) {
-        float acc = 0.f;
+    for (int wv = 0; wv < WAVES; ++wv) {
+      wgt[wv] = __builtin_amdgcn_exp2f(mw[wv] - M);      // a wave without keys has l = 0 and O = 0
+      L += wgt[wv] * ((const float*)(smem + wv * WAVE_ELEMS))[row * MROW + HD + 1];
+    }
+    for (int d = dl; d < HD; d += 16) {
+      float acc = 0.f;
 #pragma unroll
-        for (int wv = 0; wv < FA_WAVES; ++wv)
-          acc += wgt[wv] * ((const float*)(smem + wv * WAVE_ELEMS))[row * MROW + d];
-        if (n_splits == 1) {
-          out[(int64_t)t * out_stride + (int64_t)h * HD + d] = (bf16_t)(L > 0.f ? acc / L : 0.f);
-        } else {
-          part_o[(((int64_t)split * n_tokens + t) * nq + h) * HD + d] = acc;
-        }
+      for (int wv = 0; wv < WAVES; ++wv)
+        acc += wgt[wv] * ((const float*)(smem + wv * WAVE_ELEMS))[row * MROW + d];
+      if (n_splits == 1) {
+        out[(int64_t)t * out_stride + (int64_t)h * HD + d] = (bf16_t)(L > 0.f ? acc / L : 0.f);
+      } else {
+        part_o[(((int64_t)split * n_tokens + t) * nq + h) * HD + d] = acc;
       }
-      if (n_splits > 1 && dl == 0) {
-        float* ml = part_ml + (((int64_t)split * n_tokens + t) * nq + h) * 2;
-        ml[0] = M;
-        ml[1] = L;
-      }
+    }
+    if (n_splits > 1 && dl == 0) {
+      float* ml = part_ml + (((int64_t)split * n_tokens + t) * nq + h) * 2;
+      ml[0] = M;       // in units of log2 e
+      ml[1] = L;
     }
   }
 }
@@ -389,7 +451,6 @@ __global__ __launch_bounds__(FA_THREADS) void flash_prefill_bf16_kernel(
 
   // The running maximum starts at a large negative FINITE number, so exp2(m - m') is never
   // exp2(-inf + inf); a masked score is -inf and its probability exp2(-inf) = 0.
-  constexpr float kNegBig = -1.0e30f;
   float m_run[FP_RT], l_run[FP_RT];
   f32x4 o[FP_RT][HDT];
 #pragma unroll
@@ -577,47 +638,66 @@ __global__ void flash_combine_kernel(const float* __restrict__ part_o, const flo
                                      bf16_t* __restrict__ out, int64_t out_stride, int n_tokens, int nq, int hd,
                                      int n_splits) {
   const int t = blockIdx.x, h = blockIdx.y;
-  float M = -INFINITY;
+  float M = kNegBig;       // maxima are in units of log2 e; a split without keys has l = 0 and O = 0
   for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part_ml[(((int64_t)s * n_tokens + t) * nq + h) * 2]);
   float L = 0.f;
   for (int s = 0; s < n_splits; ++s) {
     const float* ml = part_ml + (((int64_t)s * n_tokens + t) * nq + h) * 2;
-    if (ml[0] > -INFINITY) L += expf(ml[0] - M) * ml[1];
+    L += __builtin_amdgcn_exp2f(ml[0] - M) * ml[1];
   }
   for (int d = threadIdx.x; d < hd; d += blockDim.x) {
     float acc = 0.f;
     for (int s = 0; s < n_splits; ++s) {
       const int64_t base = ((int64_t)s * n_tokens + t) * nq + h;
-      const float m = part_ml[base * 2];
-      if (m > -INFINITY) acc += expf(m - M) * part_o[base * hd + d];
+      acc += __builtin_amdgcn_exp2f(part_ml[base * 2] - M) * part_o[base * hd + d];
     }
     out[(int64_t)t * out_stride + (int64_t)h * hd + d] = (bf16_t)(L > 0.f ? acc / L : 0.f);
   }
 }
 
+template <int HDT, int WAVES>
+static int launch_flash_w(const bf16_t* q, int64_t q_stride, const bf16_t* k_cache, const bf16_t* v_cache,
+                          const int32_t* block_tables, int max_blocks, const int32_t* tile_req,
+                          const int32_t* tile_tok0, const int32_t* tile_ntok, const int32_t* positions, bf16_t* out,
+                          int64_t out_stride, float* part_o, float* part_ml, int n_tiles, int n_tokens, int nq,
+                          int nkv, int block_size, float scale, int window, int n_splits, const FusedRope& fused,
+                          hipStream_t stream) {
+  constexpr int HD = HDT * 16, KS = (HD + 31) / 32, KP = KS * 32 + 8;
+  constexpr size_t stage = (size_t)WAVES * (FA_KT * KP + HD * FA_VP) * sizeof(bf16_t);
+  static_assert((size_t)(FA_KT * KP + HD * FA_VP) * sizeof(bf16_t) >= 16 * (HD + 2) * sizeof(float),
+                "a wave's merge area must fit its staging area");
+  static bool configured = false;
+  if (!configured) {
+    if (hipFuncSetAttribute((const void*)flash_attn_bf16_kernel<HDT, WAVES>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)stage) != hipSuccess)
+      return TL_ERR_LAUNCH;
+    configured = true;
+  }
+  hipLaunchKernelGGL((flash_attn_bf16_kernel<HDT, WAVES>), dim3(n_tiles, nkv, n_splits), dim3(WAVES * TL_WAVE), stage,
+                     stream, q, q_stride, k_cache, v_cache, block_tables, max_blocks, tile_req, tile_tok0, tile_ntok,
+                     positions, out, out_stride, part_o, part_ml, nq, nkv, block_size, scale, window, n_splits,
+                     n_tokens, fused);
+  return TL_OK;
+}
+
+// Eight waves share a query tile where their staging areas fit the 160 KB of LDS, else four.
 template <int HDT>
 static int launch_flash(const bf16_t* q, int64_t q_stride, const bf16_t* k_cache, const bf16_t* v_cache,
                         const int32_t* block_tables, int max_blocks, const int32_t* tile_req,
                         const int32_t* tile_tok0, const int32_t* tile_ntok, const int32_t* positions, bf16_t* out,
                         int64_t out_stride, float* part_o, float* part_ml, int n_tiles, int n_tokens, int nq, int nkv,
-                        int block_size, float scale, int window, int n_splits, hipStream_t stream) {
+                        int block_size, float scale, int window, int n_splits, const FusedRope& fused,
+                        hipStream_t stream) {
   constexpr int HD = HDT * 16, KS = (HD + 31) / 32, KP = KS * 32 + 8;
-  constexpr size_t stage = (size_t)FA_WAVES * (FA_KT * KP + HD * FA_VP) * sizeof(bf16_t);
-  constexpr size_t merge = (size_t)FA_WAVES * 16 * (HD + 2) * sizeof(float);
-  static_assert((size_t)(FA_KT * KP + HD * FA_VP) * sizeof(bf16_t) >= 16 * (HD + 2) * sizeof(float),
-                "a wave's merge area must fit its staging area");
-  constexpr size_t smem = stage > merge ? stage : merge;
-  static bool configured = false;
-  if (!configured) {
-    if (hipFuncSetAttribute((const void*)flash_attn_bf16_kernel<HDT>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)smem) != hipSuccess)
-      return TL_ERR_LAUNCH;
-    configured = true;
-  }
-  hipLaunchKernelGGL(flash_attn_bf16_kernel<HDT>, dim3(n_tiles, nkv, n_splits), dim3(FA_THREADS), smem, stream, q,
-                     q_stride, k_cache, v_cache, block_tables, max_blocks, tile_req, tile_tok0, tile_ntok, positions,
-                     out, out_stride, part_o, part_ml, nq, nkv, block_size, scale, window, n_splits, n_tokens);
-  return TL_OK;
+  constexpr size_t per_wave = (size_t)(FA_KT * KP + HD * FA_VP) * sizeof(bf16_t);
+  if constexpr (8 * per_wave <= 150 * 1024)
+    return launch_flash_w<HDT, 8>(q, q_stride, k_cache, v_cache, block_tables, max_blocks, tile_req, tile_tok0,
+                                  tile_ntok, positions, out, out_stride, part_o, part_ml, n_tiles, n_tokens, nq, nkv,
+                                  block_size, scale, window, n_splits, fused, stream);
+  else
+    return launch_flash_w<HDT, 4>(q, q_stride, k_cache, v_cache, block_tables, max_blocks, tile_req, tile_tok0,
+                                  tile_ntok, positions, out, out_stride, part_o, part_ml, n_tiles, n_tokens, nq, nkv,
+                                  block_size, scale, window, n_splits, fused, stream);
 }
 
 }  // namespace
@@ -683,19 +763,24 @@ int tl_flash_attention(const void* q, int64_t q_stride, const void* k_cache, con
                        const int32_t* tile_tok0, const int32_t* tile_ntok, const int32_t* positions, void* out,
                        int64_t out_stride, float* part_o, float* part_ml, int n_tiles, int n_tokens, int nq,
                        int nkv, int hd, int block_size, float scale, int window, int n_splits,
-                       hipStream_t stream) {
+                       const float* rope_cos, const float* rope_sin, int fuse_store, hipStream_t stream) {
   if (n_tiles <= 0 || n_tokens <= 0) return TL_OK;
   if (nq <= 0 || nkv <= 0 || nq % nkv || nq / nkv > 16 || hd <= 0 || hd % 16 || hd > 128 || block_size <= 0 ||
       max_blocks <= 0 || window < 0 || n_splits < 1 || nkv > 65535 || n_splits > 65535 || q_stride % 8)
     return TL_ERR_ARG;
   if (n_splits > 1 && (!part_o || !part_ml)) return TL_ERR_ARG;
+  // fused rotation and cache write: q is the first slice of rows [q heads | k heads | v heads], every
+  // tile is one token, the whole head is rotated
+  if (fuse_store && (!rope_cos || !rope_sin || n_tiles != n_tokens)) return TL_ERR_ARG;
+  FusedRope fused{fuse_store ? rope_cos : nullptr, fuse_store ? rope_sin : nullptr, (bf16_t*)k_cache, (bf16_t*)v_cache,
+                  nq * hd, (nq + nkv) * hd};
   int rc = TL_ERR_ARG;
 #define TL_FLASH_CASE(HDT)                                                                                       \
   case HDT:                                                                                                      \
     rc = launch_flash<HDT>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,           \
                            block_tables, max_blocks, tile_req, tile_tok0, tile_ntok, positions, (bf16_t*)out,    \
                            out_stride, part_o, part_ml, n_tiles, n_tokens, nq, nkv, block_size, scale, window,   \
-                           n_splits, stream);                                                                    \
+                           n_splits, fused, stream);                                                             \
     break;
   switch (hd / 16) {
     TL_FLASH_CASE(1) TL_FLASH_CASE(2) TL_FLASH_CASE(3) TL_FLASH_CASE(4)

@@ -291,11 +291,15 @@ def flash_attention_supported(dtype: torch.dtype, num_heads: int, num_kv_heads: 
 def flash_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                     tiles, positions: torch.Tensor, out: torch.Tensor, num_heads: int, num_kv_heads: int,
                     head_dim: int, scale: float, window: int = 0, n_splits: int = 1,
-                    scratch: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    scratch: Optional[torch.Tensor] = None, fused_rope=None) -> torch.Tensor:
     """The same function as `paged_attention` on the matrix cores (bfloat16).  `tiles` =
     (tile_req, tile_tok0, tile_ntok): groups of at most 16 // (heads / kv_heads) consecutive
     tokens of one request.  n_splits > 1 needs float32 `scratch` of at least
-    n_splits * T * heads * (head_dim + 2) elements."""
+    n_splits * T * heads * (head_dim + 2) elements.
+
+    fused_rope=(cos, sin), for steps of ONE new token per request: `q` is the first slice of the
+    unrotated rows [q heads | k heads | v heads]; the kernel rotates q and the new key over the
+    whole head and writes the new key and value into the caches itself (no `rope_store` before)."""
     tile_req, tile_tok0, tile_ntok = tiles
     _dev(q, k_cache, v_cache, block_tables, tile_req, tile_tok0, tile_ntok, positions, out, scratch)
     _rows_2d(q, "q")
@@ -324,12 +328,23 @@ def flash_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
               and scratch.numel() >= need, f"split attention needs {need} float32 of scratch")
         part_o = scratch[:n_splits * T * num_heads * head_dim]
         part_ml = scratch[n_splits * T * num_heads * head_dim:]
+    cos = sin = None
+    if fused_rope is not None:
+        cos, sin = fused_rope
+        _dev(cos, sin)
+        _need(n_tiles == T, "the fused rotation and cache write take one token per tile")
+        _need(cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.is_contiguous() and sin.is_contiguous()
+              and cos.shape == sin.shape and cos.shape[1] == head_dim // 2,
+              "angle tables must be float32 [positions, head_dim / 2]")
+        # q must be the head of a [q | k | v] row
+        _need(q.stride(0) >= (num_heads + 2 * num_kv_heads) * head_dim, "fused mode needs q inside its qkv rows")
     _check(_lib().tl_flash_attention(
         _ptr(q, 16), c_int64(q.stride(0)), _ptr(k_cache, 16), _ptr(v_cache, 16), _ptr(block_tables),
         c_int(block_tables.shape[1]), _ptr(tile_req), _ptr(tile_tok0), _ptr(tile_ntok), _ptr(positions),
         _ptr(out, 8), c_int64(out.stride(0)), _ptr(part_o), _ptr(part_ml), c_int(n_tiles), c_int(T),
         c_int(num_heads), c_int(num_kv_heads), c_int(head_dim), c_int(k_cache.shape[2]), c_float(scale),
-        c_int(window), c_int(n_splits), _stream()), "flash_attention")
+        c_int(window), c_int(n_splits), _ptr(cos), _ptr(sin), c_int(1 if fused_rope is not None else 0),
+        _stream()), "flash_attention")
     return out
 
 

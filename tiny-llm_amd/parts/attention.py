@@ -73,38 +73,40 @@ class Attention(Mixer):
             ops.linear(h, self.w_qkv, qkv)
         tables = self.position.rotary_tables()
         cos, sin, rot = tables if tables is not None else (None, None, 0)
-        slots = ctx.slot_mappings[cache.group] if cache.write else None
-        ops.rope_store(qkv, ctx.positions, cos, sin, slots, cache.k if cache.write else None,
-                       cache.v if cache.write else None, self.num_heads, self.num_kv_heads, self.head_dim, rot)
         attn = torch.empty((T, self.q_size), dtype=self.dtype, device=residual.device)
         q = qkv[:, :self.q_size]
-        if ops.flash_attention_supported(self.dtype, self.num_heads, self.num_kv_heads, self.head_dim):
-            group = self.num_heads // self.num_kv_heads
-            if ctx.max_q_len > 1:
-                # prompt portions: many query rows share each staged key tile
-                tiles = ctx.attention_tiles(ops.PREFILL_TILES * (16 // group))
-                ops.flash_prefill(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, attn,
-                                  self.num_heads, self.num_kv_heads, self.head_dim, self.scale, self.window)
-            else:
-                # decoding: one token per request, its keys split over waves and workgroups
-                tiles = ctx.attention_tiles(16 // group)
-                n_splits, scratch = self._splits(ctx, tiles[0].numel(), T, residual.device)
-                ops.flash_attention(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, attn,
-                                    self.num_heads, self.num_kv_heads, self.head_dim, self.scale, self.window,
-                                    n_splits, scratch)
+        flash = ops.flash_attention_supported(self.dtype, self.num_heads, self.num_kv_heads, self.head_dim)
+        group = self.num_heads // self.num_kv_heads
+        # decode steps: rotation and cache write ride in the attention kernel
+        fuse = flash and ctx.max_q_len == 1 and cache.write and rot == self.head_dim
+        if not fuse:
+            slots = ctx.slot_mappings[cache.group] if cache.write else None
+            ops.rope_store(qkv, ctx.positions, cos, sin, slots, cache.k if cache.write else None,
+                           cache.v if cache.write else None, self.num_heads, self.num_kv_heads, self.head_dim, rot)
+        if flash and ctx.max_q_len > 1:
+            # prompt portions: many query rows share each staged key tile
+            tiles = ctx.attention_tiles(ops.PREFILL_TILES * (16 // group))
+            ops.flash_prefill(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, attn,
+                              self.num_heads, self.num_kv_heads, self.head_dim, self.scale, self.window)
+        elif flash:
+            # decoding: one token per request, its keys split over the waves of a workgroup (and over
+            # workgroups when the context is long)
+            tiles = ctx.attention_tiles(16 // group)
+            n_splits, scratch = self._splits(ctx, T, residual.device)
+            ops.flash_attention(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, attn,
+                                self.num_heads, self.num_kv_heads, self.head_dim, self.scale, self.window,
+                                n_splits, scratch, fused_rope=(cos, sin) if fuse else None)
         else:
             ops.paged_attention(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.req_of_token,
                                 ctx.positions, attn, self.num_heads, self.num_kv_heads, self.head_dim,
                                 self.scale, self.window)
         return ops.linear(attn, self.w_o, residual, residual)
 
-    def _splits(self, ctx, n_tiles: int, T: int, device):
-        """How many workgroups share one query tile's keys.  Prompt portions bring enough tiles
-        to fill the chip; a decode step with few requests does not, so its keys are split."""
-        want = 512                                   # workgroups that keep 256 CUs busy
-        have = n_tiles * self.num_kv_heads
-        key_tiles = max(1, -(-ctx.max_seq_len // 64) // 4)       # at least four 64-key tiles per split
-        n_splits = max(1, min(want // max(have, 1), key_tiles, 16))
+    def _splits(self, ctx, T: int, device):
+        """How many workgroups share one query tile's keys.  Eight waves of one workgroup take up to
+        about 4096 keys between them without help; longer contexts are split further."""
+        key_tiles = -(-ctx.max_seq_len // 64)
+        n_splits = max(1, min(-(-key_tiles // 64), 16))
         if n_splits == 1:
             return 1, None
         return n_splits, torch.empty(n_splits * T * self.num_heads * (self.head_dim + 2), dtype=torch.float32,
