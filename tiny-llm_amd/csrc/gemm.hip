@@ -8,8 +8,10 @@
 //    matrix mode.  The k order of the accumulation does not depend on M, so a row
 //    gives the same bits whether it is computed alone or in a batch.
 //  * gemm_bf16_kernel: bf16 inputs on the MFMA matrix cores
-//    (v_mfma_f32_32x32x16_bf16), float32 accumulation, 128x128x64 (or 64x128x64) tiles
-//    staged through double-buffered LDS, four wave64 per workgroup.
+//    (v_mfma_f32_32x32x16_bf16), float32 accumulation, 256x256, 128x128 or 64x128 tiles with
+//    k steps of 64 staged through double-buffered LDS.
+#include <type_traits>
+
 #include "common.h"
 
 namespace {
@@ -89,130 +91,201 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f32_kernel(const float* __rest
 }
 
 // ==================================================================== bfloat16
-// Tiles of BM x 128 outputs (BM = 128, or 64 where that is needed to fill the chip), k in steps
-// of 64, four wave64 as 2 x 2, each owning (BM/2) x 64 outputs as 32x32x16 MFMA tiles.  Operand
-// tiles go global -> registers -> LDS; LDS is double-buffered so an iteration needs one barrier,
-// and the global loads of the next k step are in flight while the current one is multiplied.
-constexpr int B_BN = 128, B_BK = 64, B_THREADS = 256;
+// Tiles of BM x BN outputs, k in steps of 64, WM x WN wave64, each owning (BM/WM) x (BN/WN)
+// outputs as 32x32x16 MFMA tiles.  Operand tiles go global -> registers -> LDS; LDS is
+// double-buffered so an iteration needs one barrier, and the global loads of the next k step are
+// in flight while the current one is multiplied.
+//
+// Tile shapes: 256 x 256 (eight waves of 128 x 64), 256 x 128, 128 x 128 and 64 x 128.  The larger
+// the tile, the fewer operand bytes and LDS reads per flop and the higher the rate on a full chip;
+// small products take small tiles all the same, because 256 compute units want at least that many
+// workgroups (launch_gemm_bf16_any estimates the time of each shape and takes the best).
+//
+// Workgroups are handed to the eight XCDs in turn, each with an L2 of its own.  The tile index is
+// therefore remapped so that an XCD owns a contiguous run of tiles in column-major order: it then
+// reads only its own share of the weight matrix (plus the activations), instead of all of it.
+constexpr int B_BK = 64;
 constexpr int B_LD = B_BK + 8;  // LDS row stride in elements: 144 bytes, keeps 16-byte alignment
+constexpr int B_XCDS = 8;
 
-template <int BM>
-struct GemmStage {                       // one k step of both operand tiles, spread over the threads
-  static constexpr int AC = BM * (B_BK / 8) / B_THREADS, WC = B_BN * (B_BK / 8) / B_THREADS;
-  bf16x8 a[AC], w[WC];
+template <int BM, int BN, int WM, int WN>
+struct GemmShape {
+  static constexpr int THREADS = WM * WN * TL_WAVE;
+  static constexpr int TM = BM / WM, TN = BN / WN;        // a wave's outputs
+  static constexpr int MI = TM / 32, NJ = TN / 32;        // as 32 x 32 MFMA tiles
+  static constexpr int AC = BM * (B_BK / 8) / THREADS, WC = BN * (B_BK / 8) / THREADS;
+  static constexpr size_t SMEM = (size_t)2 * (BM + BN) * B_LD * sizeof(bf16_t);
+  static_assert(TM % 32 == 0 && TN % 32 == 0 && AC >= 1 && WC >= 1, "tile does not divide");
 };
 
 // K must be a multiple of 8 (16-byte chunks of bf16 never straddle the end).
-template <int BM, typename TO, bool SWIGLU, bool FULL>
-__global__ __launch_bounds__(B_THREADS) void gemm_bf16_kernel(const bf16_t* __restrict__ a,
-                                                              const bf16_t* __restrict__ w,
-                                                              TO* __restrict__ out,
-                                                              const float* __restrict__ residual,
-                                                              const float* __restrict__ row_scale, int M,
-                                                              int N, int K, int64_t lda, int64_t ldo) {
-  constexpr int MI = BM / 64;            // 32-row MFMA tiles per wave along m
+template <int BM, int BN, int WM, int WN, typename TO, bool SWIGLU, bool FULL>
+__global__ __launch_bounds__(WM * WN * TL_WAVE) void gemm_bf16_kernel(const bf16_t* __restrict__ a,
+                                                                      const bf16_t* __restrict__ w,
+                                                                      TO* __restrict__ out,
+                                                                      const float* __restrict__ residual,
+                                                                      const float* __restrict__ row_scale, int M,
+                                                                      int N, int K, int64_t lda, int64_t ldo) {
+  using S = GemmShape<BM, BN, WM, WN>;
+  constexpr int MI = S::MI, NJ = S::NJ, THREADS = S::THREADS;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   bf16_t* As = (bf16_t*)smem_raw;                       // [2][BM][B_LD]
-  bf16_t* Ws = As + 2 * BM * B_LD;                      // [2][B_BN][B_LD]
+  bf16_t* Ws = As + 2 * BM * B_LD;                      // [2][BN][B_LD]
   const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
-  const int wm = wave / 2, wn = wave % 2;
-  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * B_BN;
+  const int wm = wave / WN, wn = wave % WN;
+  const int tiles_m = (M + BM - 1) / BM, total = tiles_m * ((N + BN - 1) / BN);
+  const int per_xcd = (total + B_XCDS - 1) / B_XCDS;
+  const int t = (blockIdx.x % B_XCDS) * per_xcd + blockIdx.x / B_XCDS;
+  if (t >= total) return;                               // the grid is padded to a multiple of 8
+  const int m0 = (t % tiles_m) * BM, n0 = (t / tiles_m) * BN;
 
-  f32x16 acc[MI][2];
+  f32x16 acc[MI][NJ];
 #pragma unroll
   for (int i = 0; i < MI; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < NJ; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  using Stage = GemmStage<BM>;
-  // Loads are unconditional (addresses clamped into the matrix; a chunk that lies outside is zeroed
-  // when it is written to LDS): a predicated load becomes a branch, and then the outstanding-load
-  // counter cannot be used to wait for one stage while the next stays in flight.
-  auto load_stage = [&](Stage& st, int k0) {
-#pragma unroll
-    for (int i = 0; i < Stage::AC; ++i) {
-      const int c = tid + i * B_THREADS;
-      const int row = m0 + c / 8, k = k0 + (c % 8) * 8;
-      st.a[i] = *(const bf16x8*)(a + (int64_t)min(row, M - 1) * lda + min(k, K - 8));
-    }
-#pragma unroll
-    for (int i = 0; i < Stage::WC; ++i) {
-      const int c = tid + i * B_THREADS;
-      const int row = n0 + c / 8, k = k0 + (c % 8) * 8;
-      st.w[i] = *(const bf16x8*)(w + (int64_t)min(row, N - 1) * K + min(k, K - 8));
-    }
+  // One k step of both operand tiles is AC + WC 16-byte pieces per thread.  Global loads are
+  // unconditional (addresses clamped into the matrix; a piece that lies outside is zeroed when it
+  // is written to LDS): a predicated load becomes a branch, and then the outstanding-load counter
+  // cannot be used to wait for one piece while the next stays in flight.
+  constexpr int PIECES = S::AC + S::WC;
+  bf16x8 stage[PIECES];
+  const int prow = tid / 8, pk = (tid % 8) * 8;            // this thread's row within a pass, k offset
+  constexpr int PASS = THREADS / 8;                        // rows per pass
+  auto gload1 = [&](int k0, int p) {
+    const bool is_a = p < S::AC;
+    const int row = (is_a ? m0 + p * PASS : n0 + (p - S::AC) * PASS) + prow, k = k0 + pk;
+    const bf16_t* base = is_a ? a : w;
+    const int64_t ld = is_a ? lda : (int64_t)K;
+    const int lim = is_a ? M : N;
+    stage[p] = *(const bf16x8*)(base + (int64_t)(FULL ? row : min(row, lim - 1)) * ld + (FULL ? k : min(k, K - 8)));
   };
-  // FULL: M, N and K are multiples of the tile, so no chunk lies outside and nothing is zeroed
-  auto store_stage = [&](const Stage& st, int buf, int k0) {
+  // FULL: M, N and K are multiples of the tile, so no piece lies outside and nothing is zeroed
+  auto lds_write1 = [&](int buf, int k0, int p) {
+    const bool is_a = p < S::AC;
+    const int r = (is_a ? p : p - S::AC) * PASS + prow;
+    const bool ok = FULL || ((is_a ? m0 + r < M : n0 + r < N) && k0 + pk < K);
     bf16x8 z = {};
+    bf16_t* dst = is_a ? As + (buf * BM + r) * B_LD + pk : Ws + (buf * BN + r) * B_LD + pk;
+    *(bf16x8*)dst = ok ? stage[p] : z;
+  };
+  // MFMA operands of one k16 step: NJ weight pieces, then MI activation pieces, in the order of use
+  struct Frag {
+    bf16x8 w[NJ], a[MI];
+  };
+  constexpr int FRAG = NJ + MI;
+  const bf16_t* ra = As + (wm * S::TM + lane % 32) * B_LD + (lane / 32) * 8;
+  const bf16_t* rw = Ws + (wn * S::TN + lane % 32) * B_LD + (lane / 32) * 8;
+  auto lds_read1 = [&](Frag& f, int buf, int ks, int p) {
+    if (p < NJ) f.w[p] = *(const bf16x8*)(rw + (buf * BN + p * 32) * B_LD + ks * 16);
+    else f.a[p - NJ] = *(const bf16x8*)(ra + (buf * BM + (p - NJ) * 32) * B_LD + ks * 16);
+  };
+  // The MFMAs of one k16 step, with memory operations issued between them: slot(n) comes after the
+  // n-th MFMA.  The result tile is transposed (rows = n, columns = m) so that a lane holds four
+  // consecutive n of one output row and can store them as one vector.  The scheduling barriers
+  // keep the compiler from gathering the memory operations back into one place.
+  constexpr int SLOTS = MI * NJ;
+  auto group = [&](const Frag& f, auto&& slot) {
 #pragma unroll
-    for (int i = 0; i < Stage::AC; ++i) {
-      const int c = tid + i * B_THREADS;
-      const bool ok = FULL || (m0 + c / 8 < M && k0 + (c % 8) * 8 < K);
-      *(bf16x8*)(As + (buf * BM + c / 8) * B_LD + (c % 8) * 8) = ok ? st.a[i] : z;
-    }
-#pragma unroll
-    for (int i = 0; i < Stage::WC; ++i) {
-      const int c = tid + i * B_THREADS;
-      const bool ok = FULL || (n0 + c / 8 < N && k0 + (c % 8) * 8 < K);
-      *(bf16x8*)(Ws + (buf * B_BN + c / 8) * B_LD + (c % 8) * 8) = ok ? st.w[i] : z;
+    for (int n = 0; n < SLOTS; ++n) {
+      acc[n / NJ][n % NJ] =
+          __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.w[n % NJ], f.a[n / NJ], acc[n / NJ][n % NJ], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      slot(n);
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
-  auto compute = [&](int buf) {
+  // pieces [n * per, (n + 1) * per) of `total`, for spreading `total` operations over slots
+  auto spread = [](int n, int total, int slots, auto&& op) {
+    const int per = (total + slots - 1) / slots;
 #pragma unroll
-    for (int ks = 0; ks < B_BK; ks += 16) {
-      bf16x8 fa[MI], fw[2];
-#pragma unroll
-      for (int i = 0; i < MI; ++i)
-        fa[i] = *(const bf16x8*)(As + (buf * BM + wm * (BM / 2) + i * 32 + lane % 32) * B_LD + ks + (lane / 32) * 8);
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-        fw[j] = *(const bf16x8*)(Ws + (buf * B_BN + wn * 64 + j * 32 + lane % 32) * B_LD + ks + (lane / 32) * 8);
-      // result tile is transposed (rows = n, columns = m) so that a lane holds four
-      // consecutive n of one output row and can store them as one vector
-#pragma unroll
-      for (int i = 0; i < MI; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[j], fa[i], acc[i][j], 0, 0, 0);
-    }
+    for (int p = n * per; p < (n + 1) * per; ++p)
+      if (p < total) op(p);
   };
 
+  // The loop is software-pipelined by hand, because all waves of a workgroup meet at the barrier
+  // of every k step and so cannot cover for each other: while the MFMAs of one k16 step run, the
+  // fragments of the next are read; the tile of step kt + 1 (loaded into registers during step
+  // kt - 1) is written to the other LDS buffer in the middle of step kt, and the loads of tile
+  // kt + 2 are issued right after; the last k16 step of a tile is multiplied after the barrier,
+  // while the first fragments of the next tile are on their way.
   const int nk = (K + B_BK - 1) / B_BK;
-  Stage st;
-  load_stage(st, 0);
-  store_stage(st, 0, 0);
+#pragma unroll
+  for (int p = 0; p < PIECES; ++p) gload1(0, p);
+#pragma unroll
+  for (int p = 0; p < PIECES; ++p) lds_write1(0, 0, p);
+  if (nk > 1) {
+#pragma unroll
+    for (int p = 0; p < PIECES; ++p) gload1(B_BK, p);
+  }
   __syncthreads();
-  // iteration kt: the loads of step kt + 1 are in flight while step kt is multiplied out of
-  // LDS[kt & 1]; they land in the other LDS buffer before the iteration's one barrier
-  for (int kt = 0; kt < nk; ++kt) {
-    const int cur = kt & 1;
-    if (kt + 1 < nk) load_stage(st, (kt + 1) * B_BK);
-    compute(cur);
-    if (kt + 1 < nk) store_stage(st, cur ^ 1, (kt + 1) * B_BK);
+  Frag f0, f1;
+#pragma unroll
+  for (int p = 0; p < FRAG; ++p) lds_read1(f0, 0, 0, p);
+  static_assert(SLOTS >= 2, "a wave owns at least two MFMA tiles");
+  constexpr int HALF = SLOTS / 2;
+  auto step = [&](auto has_next, auto has_next2, int kt) {
+    constexpr bool NX = decltype(has_next)::value, NX2 = decltype(has_next2)::value;
+    const int cur = kt & 1, nxt = cur ^ 1, k1 = (kt + 1) * B_BK, k2 = (kt + 2) * B_BK;
+    group(f0, [&](int n) { spread(n, FRAG, SLOTS, [&](int p) { lds_read1(f1, cur, 1, p); }); });
+    group(f1, [&](int n) {
+      spread(n, FRAG, SLOTS, [&](int p) { lds_read1(f0, cur, 2, p); });
+      if constexpr (NX)
+        if (n >= SLOTS - HALF) spread(n - (SLOTS - HALF), PIECES / 2, HALF, [&](int p) { lds_write1(nxt, k1, p); });
+    });
+    group(f0, [&](int n) {
+      spread(n, FRAG, SLOTS, [&](int p) { lds_read1(f1, cur, 3, p); });
+      if constexpr (NX)
+        if (n < HALF) spread(n, PIECES - PIECES / 2, HALF, [&](int p) { lds_write1(nxt, k1, PIECES / 2 + p); });
+      if constexpr (NX2)
+        if (n >= SLOTS - HALF) spread(n - (SLOTS - HALF), PIECES, HALF, [&](int p) { gload1(k2, p); });
+    });
     __syncthreads();
+    group(f1, [&](int n) {
+      if constexpr (NX) spread(n, FRAG, SLOTS, [&](int p) { lds_read1(f0, nxt, 0, p); });
+    });
+  };
+  {
+    int kt = 0;
+    for (; kt + 2 < nk; ++kt) step(std::true_type{}, std::true_type{}, kt);
+    if (kt + 1 < nk) {
+      step(std::true_type{}, std::false_type{}, kt);
+      ++kt;
+    }
+    step(std::false_type{}, std::false_type{}, kt);
   }
 
   const bool vec_ok = (N % 4 == 0) && (ldo % 4 == 0);
 #pragma unroll
   for (int i = 0; i < MI; ++i) {
-    const int m = m0 + wm * (BM / 2) + i * 32 + lane % 32;
+    const int m = m0 + wm * S::TM + i * 32 + lane % 32;
     if (m >= M) continue;
     const float rs = row_scale ? row_scale[m] : 1.f;   // e.g. 1 / rms of a norm left out of the operand
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < NJ; ++j) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int n = n0 + wn * 64 + j * 32 + q * 8 + (lane / 32) * 4;
+        const int n = n0 + wn * S::TN + j * 32 + q * 8 + (lane / 32) * 4;
         if (n >= N) continue;
         float v[4] = {acc[i][j][q * 4 + 0] * rs, acc[i][j][q * 4 + 1] * rs, acc[i][j][q * 4 + 2] * rs,
                       acc[i][j][q * 4 + 3] * rs};
         if constexpr (SWIGLU) {   // (gate, up, gate, up) -> two outputs; N is even and n a multiple of 4
           const int64_t oz = (int64_t)m * ldo + n / 2;
-          out[oz] = from_f32<TO>(swiglu_pair(v[0], v[1]));
-          if (n + 2 < N) out[oz + 1] = from_f32<TO>(swiglu_pair(v[2], v[3]));
+          if (n + 2 < N) {
+            typedef TO to2 __attribute__((ext_vector_type(2)));
+            to2 sv = {from_f32<TO>(swiglu_pair(v[0], v[1])), from_f32<TO>(swiglu_pair(v[2], v[3]))};
+            if (ldo % 2 == 0) {
+              *(to2*)(out + oz) = sv;
+            } else {
+              out[oz] = sv[0];
+              out[oz + 1] = sv[1];
+            }
+          } else {
+            out[oz] = from_f32<TO>(swiglu_pair(v[0], v[1]));
+          }
           continue;
         }
         const int64_t o = (int64_t)m * ldo + n;
@@ -240,41 +313,68 @@ __global__ __launch_bounds__(B_THREADS) void gemm_bf16_kernel(const bf16_t* __re
   }
 }
 
-template <int BM, typename TO, bool SWIGLU, bool FULL>
+template <int BM, int BN, int WM, int WN, typename TO, bool SWIGLU, bool FULL>
 static int launch_gemm_bf16_full(const bf16_t* a, const bf16_t* w, TO* out, const float* residual,
                                  const float* row_scale, int M, int N, int K, int64_t lda, int64_t ldo,
                                  hipStream_t stream) {
-  constexpr size_t smem = (size_t)2 * (BM + B_BN) * B_LD * sizeof(bf16_t);
+  using S = GemmShape<BM, BN, WM, WN>;
   static bool configured = false;
   if (!configured) {
-    if (hipFuncSetAttribute((const void*)gemm_bf16_kernel<BM, TO, SWIGLU, FULL>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+    if (hipFuncSetAttribute((const void*)gemm_bf16_kernel<BM, BN, WM, WN, TO, SWIGLU, FULL>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::SMEM) != hipSuccess)
       return TL_ERR_LAUNCH;
     configured = true;
   }
-  dim3 g((N + B_BN - 1) / B_BN, (M + BM - 1) / BM);
-  hipLaunchKernelGGL((gemm_bf16_kernel<BM, TO, SWIGLU, FULL>), g, dim3(B_THREADS), smem, stream, a, w, out, residual,
-                     row_scale, M, N, K, lda, ldo);
+  const int64_t total = (int64_t)((N + BN - 1) / BN) * ((M + BM - 1) / BM);
+  const int64_t grid = (total + B_XCDS - 1) / B_XCDS * B_XCDS;
+  if (grid > 0x7fffffff) return TL_ERR_ARG;
+  hipLaunchKernelGGL((gemm_bf16_kernel<BM, BN, WM, WN, TO, SWIGLU, FULL>), dim3((unsigned)grid), dim3(S::THREADS),
+                     S::SMEM, stream, a, w, out, residual, row_scale, M, N, K, lda, ldo);
   return TL_OK;
 }
 
-template <int BM, typename TO, bool SWIGLU>
+template <int BM, int BN, int WM, int WN, typename TO, bool SWIGLU>
 static int launch_gemm_bf16(const bf16_t* a, const bf16_t* w, TO* out, const float* residual, const float* row_scale,
                             int M, int N, int K, int64_t lda, int64_t ldo, hipStream_t stream) {
-  if (M % BM == 0 && N % B_BN == 0 && K % B_BK == 0)
-    return launch_gemm_bf16_full<BM, TO, SWIGLU, true>(a, w, out, residual, row_scale, M, N, K, lda, ldo, stream);
-  return launch_gemm_bf16_full<BM, TO, SWIGLU, false>(a, w, out, residual, row_scale, M, N, K, lda, ldo, stream);
+  if (M % BM == 0 && N % BN == 0 && K % B_BK == 0)
+    return launch_gemm_bf16_full<BM, BN, WM, WN, TO, SWIGLU, true>(a, w, out, residual, row_scale, M, N, K, lda, ldo,
+                                                                   stream);
+  return launch_gemm_bf16_full<BM, BN, WM, WN, TO, SWIGLU, false>(a, w, out, residual, row_scale, M, N, K, lda, ldo,
+                                                                  stream);
 }
 
-// Tiles of 128 rows unless that leaves compute units without a workgroup.
+// Which tile: the one with the smallest estimated time.  A compute unit works through
+// ceil(workgroups / 256) tiles one after the other, each at the rate that its tile shape reaches
+// on a full chip (measured, TFLOP/s: the larger the tile, the fewer operand bytes per flop).
 template <typename TO, bool SWIGLU>
 static int launch_gemm_bf16_any(const bf16_t* a, const bf16_t* w, TO* out, const float* residual,
                                 const float* row_scale, int M, int N, int K, int64_t lda, int64_t ldo,
                                 hipStream_t stream) {
-  const int64_t wgs128 = (int64_t)((N + B_BN - 1) / B_BN) * ((M + 127) / 128);
-  if (wgs128 >= 512)
-    return launch_gemm_bf16<128, TO, SWIGLU>(a, w, out, residual, row_scale, M, N, K, lda, ldo, stream);
-  return launch_gemm_bf16<64, TO, SWIGLU>(a, w, out, residual, row_scale, M, N, K, lda, ldo, stream);
+  struct Choice {
+    int bm, bn;
+    double rate;
+  };
+  static const Choice choices[4] = {{256, 256, 1060.}, {256, 128, 900.}, {128, 128, 760.}, {64, 128, 640.}};
+  int best = 0;
+  double best_cost = 0.;
+  for (int c = 0; c < 4; ++c) {
+    const int64_t wgs = (int64_t)((M + choices[c].bm - 1) / choices[c].bm) * ((N + choices[c].bn - 1) / choices[c].bn);
+    const double cost = (double)((wgs + 255) / 256) * choices[c].bm * choices[c].bn / choices[c].rate;
+    if (c == 0 || cost < best_cost) {
+      best = c;
+      best_cost = cost;
+    }
+  }
+  switch (best) {
+    case 0:
+      return launch_gemm_bf16<256, 256, 2, 4, TO, SWIGLU>(a, w, out, residual, row_scale, M, N, K, lda, ldo, stream);
+    case 1:
+      return launch_gemm_bf16<256, 128, 4, 2, TO, SWIGLU>(a, w, out, residual, row_scale, M, N, K, lda, ldo, stream);
+    case 2:
+      return launch_gemm_bf16<128, 128, 2, 2, TO, SWIGLU>(a, w, out, residual, row_scale, M, N, K, lda, ldo, stream);
+    default:
+      return launch_gemm_bf16<64, 128, 2, 2, TO, SWIGLU>(a, w, out, residual, row_scale, M, N, K, lda, ldo, stream);
+  }
 }
 
 // ============================================================ bfloat16, few rows
