@@ -390,20 +390,23 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
 }
 
 // flash_prefill_bf16_kernel: the same mathematics arranged for prompt portions.  A workgroup
-// owns up to 8 query tiles (two per wave, 128 rows: for 8 heads per kv head that is 16 tokens) of
-// consecutive tokens of one request, and all four waves work on the SAME 64-key tile, staged and
+// owns up to 8 query tiles (one per wave, 128 rows: for 8 heads per kv head that is 16 tokens) of
+// consecutive tokens of one request, and all eight waves work on the SAME 64-key tile, staged and
 // transposed once per workgroup; so a key or value row is fetched once per 128 query rows.  There
-// is nothing to merge at the end: every row lives in one lane group of one wave.
-constexpr int FP_RT = 2;                      // query tiles (of 16 rows) per wave
-constexpr int FP_TILES = FA_WAVES * FP_RT;    // query tiles per workgroup
+// is nothing to merge at the end: every row lives in one lane group of one wave.  Eight waves
+// with one query tile each rather than four with two: the workgroup with the most keys sets the
+// kernel's duration, and its time per key tile is the work of one wave.
+constexpr int FP_RT = 1;                      // query tiles (of 16 rows) per wave
+constexpr int FP_WAVES = 8, FP_THREADS = FP_WAVES * TL_WAVE;
+constexpr int FP_TILES = FP_WAVES * FP_RT;    // query tiles per workgroup
 
 template <int HDT>
-__global__ __launch_bounds__(FA_THREADS) void flash_prefill_bf16_kernel(
+__global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
     const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ tile_req, const int32_t* __restrict__ tile_tok0,
     const int32_t* __restrict__ tile_ntok, const int32_t* __restrict__ positions, bf16_t* __restrict__ out,
-    int64_t out_stride, int nq, int nkv, int block_size, float scale, int window) {
+    int64_t out_stride, int n_tiles, int nq, int nkv, int block_size, float scale, int window) {
   constexpr int HD = HDT * 16;
   constexpr int KS = (HD + 31) / 32;
   constexpr int KP = KS * 32 + 8;
@@ -412,8 +415,14 @@ __global__ __launch_bounds__(FA_THREADS) void flash_prefill_bf16_kernel(
 
   const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
   const int r16 = lane % 16, g = lane / 16;
-  // later tiles of a prompt have more keys to go through: they are started first
-  const int tile = gridDim.x - 1 - blockIdx.x, kvh = blockIdx.y;
+  // Later tiles of a prompt have more keys to go through.  The first half of the workgroups takes
+  // the items (tile, kv head) from the heaviest down, the second half from the lightest up: all
+  // of them are resident at once when they fit, workgroup i beside workgroup i + half on the same
+  // compute unit, and so every compute unit gets about the same number of key tiles.
+  const int total = n_tiles * nkv, half = total / 2;
+  const int L = blockIdx.x;
+  const int item = L < half ? L : total - 1 - (L - half);
+  const int tile = n_tiles - 1 - item / nkv, kvh = item % nkv;
   const int G = nq / nkv, TW = 16 / G;
   const int req = tile_req[tile], tok0 = tile_tok0[tile], ntok = tile_ntok[tile];
   const int32_t* bt = block_tables + (int64_t)req * max_blocks;
@@ -445,7 +454,9 @@ __global__ __launch_bounds__(FA_THREADS) void flash_prefill_bf16_kernel(
     }
   }
   // a wave whose rows all end before a key tile begins has nothing to do in it
-  int wave_hi = max(pos[0], pos[1]);
+  int wave_hi = pos[0];
+#pragma unroll
+  for (int rt = 1; rt < FP_RT; ++rt) wave_hi = max(wave_hi, pos[rt]);
 #pragma unroll
   for (int off = 8; off > 0; off >>= 1) wave_hi = max(wave_hi, __shfl_xor(wave_hi, off, TL_WAVE));
 
@@ -475,12 +486,14 @@ __global__ __launch_bounds__(FA_THREADS) void flash_prefill_bf16_kernel(
     wave_lo_pos = min(wave_lo_pos, __shfl_xor(wave_lo_pos, off, TL_WAVE));
     wave_hi_lo = max(wave_hi_lo, __shfl_xor(wave_hi_lo, off, TL_WAVE));
   }
-  bool all_valid = row_valid[0] && row_valid[1];
+  bool all_valid = true;
+#pragma unroll
+  for (int rt = 0; rt < FP_RT; ++rt) all_valid = all_valid && row_valid[rt];
   all_valid = __all(all_valid);
 
   // staging registers: thread = (key row `lane`, chunk group `wave`); the rows of the next tile are
   // requested while the current tile is being worked on
-  constexpr int KC = (KS * 4 + FA_WAVES - 1) / FA_WAVES, VC = (HD / 8 + FA_WAVES - 1) / FA_WAVES;
+  constexpr int KC = (KS * 4 + FP_WAVES - 1) / FP_WAVES, VC = (HD / 8 + FP_WAVES - 1) / FP_WAVES;
   bf16x8 k_stage[KC], v_stage[VC];
   auto fetch_tile = [&](int kt_idx) {
     const int j = kt_idx * FA_KT + lane;
@@ -494,13 +507,13 @@ __global__ __launch_bounds__(FA_THREADS) void flash_prefill_bf16_kernel(
     const bf16_t* vp = v_cache + row_off;
 #pragma unroll
     for (int ci = 0; ci < KC; ++ci) {
-      const int c = ci * FA_WAVES + wave;
+      const int c = ci * FP_WAVES + wave;
       bf16x8 z = {};
       k_stage[ci] = (in_range && c * 8 < HD) ? *(const bf16x8*)(kp + c * 8) : z;
     }
 #pragma unroll
     for (int ci = 0; ci < VC; ++ci) {
-      const int c = ci * FA_WAVES + wave;
+      const int c = ci * FP_WAVES + wave;
       bf16x8 z = {};
       v_stage[ci] = (in_range && c < HD / 8) ? *(const bf16x8*)(vp + c * 8) : z;
     }
@@ -511,12 +524,12 @@ __global__ __launch_bounds__(FA_THREADS) void flash_prefill_bf16_kernel(
     // registers -> LDS; V is transposed on the way
 #pragma unroll
     for (int ci = 0; ci < KC; ++ci) {
-      const int c = ci * FA_WAVES + wave;
+      const int c = ci * FP_WAVES + wave;
       if (c < KS * 4) *(bf16x8*)(Kl + lane * KP + c * 8) = k_stage[ci];
     }
 #pragma unroll
     for (int ci = 0; ci < VC; ++ci) {
-      const int c = ci * FA_WAVES + wave;
+      const int c = ci * FP_WAVES + wave;
       if (c < HD / 8) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) Vl[(c * 8 + e) * FA_VP + lane] = v_stage[ci][e];
@@ -738,14 +751,15 @@ int tl_flash_prefill(const void* q, int64_t q_stride, const void* k_cache, const
                      int window, hipStream_t stream) {
   if (n_tiles <= 0) return TL_OK;
   if (nq <= 0 || nkv <= 0 || nq % nkv || nq / nkv > 16 || hd <= 0 || hd % 16 || hd > 128 || block_size <= 0 ||
-      max_blocks <= 0 || window < 0 || nkv > 65535 || q_stride % 8 || out_stride % 4)
+      max_blocks <= 0 || window < 0 || nkv > 65535 || (int64_t)n_tiles * nkv > 0x7fffffff || q_stride % 8 ||
+      out_stride % 4)
     return TL_ERR_ARG;
 #define TL_PREFILL_CASE(HDT)                                                                                      \
   case HDT:                                                                                                       \
-    hipLaunchKernelGGL(flash_prefill_bf16_kernel<HDT>, dim3(n_tiles, nkv), dim3(FA_THREADS), 0, stream,           \
+    hipLaunchKernelGGL(flash_prefill_bf16_kernel<HDT>, dim3(n_tiles * nkv), dim3(FP_THREADS), 0, stream,          \
                        (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,  \
-                       max_blocks, tile_req, tile_tok0, tile_ntok, positions, (bf16_t*)out, out_stride, nq, nkv,  \
-                       block_size, scale, window);                                                                \
+                       max_blocks, tile_req, tile_tok0, tile_ntok, positions, (bf16_t*)out, out_stride, n_tiles,  \
+                       nq, nkv, block_size, scale, window);                                                       \
     break;
   switch (hd / 16) {
     TL_PREFILL_CASE(1) TL_PREFILL_CASE(2) TL_PREFILL_CASE(3) TL_PREFILL_CASE(4)
