@@ -406,12 +406,14 @@ __global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
     const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ tile_req, const int32_t* __restrict__ tile_tok0,
     const int32_t* __restrict__ tile_ntok, const int32_t* __restrict__ positions, bf16_t* __restrict__ out,
-    int64_t out_stride, int n_tiles, int nq, int nkv, int block_size, float scale, int window) {
+    int64_t out_stride, int n_tiles, int nq, int nkv, int block_size, int bs_shift, float scale, int window) {
   constexpr int HD = HDT * 16;
   constexpr int KS = (HD + 31) / 32;
   constexpr int KP = KS * 32 + 8;
-  __shared__ __attribute__((aligned(16))) bf16_t Kl[FA_KT * KP];
-  __shared__ __attribute__((aligned(16))) bf16_t Vl[HD * FA_VP];
+  // two staging buffers: the next key tile is written while the current one is worked on, so a
+  // key tile costs one barrier
+  __shared__ __attribute__((aligned(16))) bf16_t Kbuf[2][FA_KT * KP];
+  __shared__ __attribute__((aligned(16))) bf16_t Vbuf[2][HD * FA_VP];
 
   const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
   const int r16 = lane % 16, g = lane / 16;
@@ -500,8 +502,9 @@ __global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
     const bool in_range = j >= kv_begin && j < kv_end;
     int64_t row_off = 0;
     if (in_range) {
-      const int64_t blk = bt[j / block_size];
-      row_off = ((blk * nkv + kvh) * block_size + (j % block_size)) * HD;
+      const int jb = bs_shift >= 0 ? j >> bs_shift : j / block_size;     // uniform choice: no division
+      const int64_t blk = bt[jb];
+      row_off = ((blk * nkv + kvh) * block_size + (j - jb * block_size)) * HD;
     }
     const bf16_t* kp = k_cache + row_off;
     const bf16_t* vp = v_cache + row_off;
@@ -518,10 +521,10 @@ __global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
       v_stage[ci] = (in_range && c < HD / 8) ? *(const bf16x8*)(vp + c * 8) : z;
     }
   };
-  if (first_tile < last_tile) fetch_tile(first_tile);
-
-  for (int kt_idx = first_tile; kt_idx < last_tile; ++kt_idx) {
-    // registers -> LDS; V is transposed on the way
+  // registers -> LDS; V is transposed on the way
+  auto store_tile = [&](int buf) {
+    bf16_t* Kl = Kbuf[buf];
+    bf16_t* Vl = Vbuf[buf];
 #pragma unroll
     for (int ci = 0; ci < KC; ++ci) {
       const int c = ci * FP_WAVES + wave;
@@ -535,8 +538,24 @@ __global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
         for (int e = 0; e < 8; ++e) Vl[(c * 8 + e) * FA_VP + lane] = v_stage[ci][e];
       }
     }
-    __syncthreads();
-    if (kt_idx + 1 < last_tile) fetch_tile(kt_idx + 1);
+  };
+  if (first_tile < last_tile) {
+    fetch_tile(first_tile);
+    store_tile(0);
+    if (first_tile + 1 < last_tile) fetch_tile(first_tile + 1);
+  }
+  __syncthreads();
+
+  for (int kt_idx = first_tile; kt_idx < last_tile; ++kt_idx) {
+    const int cur = (kt_idx - first_tile) & 1;
+    // the next tile (requested one iteration ago) goes into the other buffer, which every wave
+    // has finished reading before the last barrier; then the tile after it is requested
+    if (kt_idx + 1 < last_tile) {
+      store_tile(cur ^ 1);
+      if (kt_idx + 2 < last_tile) fetch_tile(kt_idx + 2);
+    }
+    const bf16_t* Kl = Kbuf[cur];
+    const bf16_t* Vl = Vbuf[cur];
     if (kt_idx * FA_KT <= wave_hi) {
       f32x4 sc[FP_RT][4];
 #pragma unroll
@@ -754,12 +773,15 @@ int tl_flash_prefill(const void* q, int64_t q_stride, const void* k_cache, const
       max_blocks <= 0 || window < 0 || nkv > 65535 || (int64_t)n_tiles * nkv > 0x7fffffff || q_stride % 8 ||
       out_stride % 4)
     return TL_ERR_ARG;
+  int bs_shift = -1;      // log2 of the page size where it is a power of two
+  for (int sh = 0; sh < 31; ++sh)
+    if ((1 << sh) == block_size) bs_shift = sh;
 #define TL_PREFILL_CASE(HDT)                                                                                      \
   case HDT:                                                                                                       \
     hipLaunchKernelGGL(flash_prefill_bf16_kernel<HDT>, dim3(n_tiles * nkv), dim3(FP_THREADS), 0, stream,          \
                        (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,  \
                        max_blocks, tile_req, tile_tok0, tile_ntok, positions, (bf16_t*)out, out_stride, n_tiles,  \
-                       nq, nkv, block_size, scale, window);                                                       \
+                       nq, nkv, block_size, bs_shift, scale, window);                                             \
     break;
   switch (hd / 16) {
     TL_PREFILL_CASE(1) TL_PREFILL_CASE(2) TL_PREFILL_CASE(3) TL_PREFILL_CASE(4)
