@@ -164,6 +164,10 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
   bf16_t* Kl = smem + wave * WAVE_ELEMS;
   bf16_t* Vl = Kl + K_ELEMS;
   const bool do_rope = fused.cos_t != nullptr;
+  // Key tiles are dealt out in turn (see below), so without a window this wave's first tile is
+  // known here: the page of this lane's row in it is requested together with the position.  The
+  // index is clamped into the table; an entry that belongs to no key of the request is not used.
+  const int spec_blk = max(bt[min(((split * WAVES + wave) * FA_KT + lane) / block_size, max_blocks - 1)], 0);
 
   // this lane's query row
   const int tok_local = r16 / G, hh = r16 % G;
@@ -182,10 +186,12 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
   }
   const int kv_end = hi + 1, kv_begin = lo;
   const int first_tile = kv_begin / FA_KT, last_tile = (kv_end + FA_KT - 1) / FA_KT;
-  const int per_split = (last_tile - first_tile + n_splits - 1) / n_splits;
-  const int range_lo = first_tile + split * per_split;
-  const int range_hi = min(last_tile, range_lo + per_split);
-  const int iters = (max(range_hi - range_lo, 0) + WAVES - 1) / WAVES;
+  // Key tiles are dealt out in turn: tile (it0 + it) * stride + split * WAVES + wave belongs to
+  // iteration `it` of this wave.  Which tiles a wave gets then does not depend on the positions,
+  // so the page of its first tile can be looked up before the positions have arrived.
+  const int stride = WAVES * n_splits, mine = split * WAVES + wave;
+  const int it0 = first_tile / stride;
+  const int iters = (last_tile - mine + stride - 1) / stride - it0;      // may be <= 0: no tile
   // fused mode: the one new token of the tile, at position kv_end - 1
   const int new_pos = kv_end - 1;
   const float* cs = do_rope ? fused.cos_t + (int64_t)new_pos * (HD / 2) : nullptr;
@@ -213,59 +219,70 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
   for (int dt = 0; dt < HDT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   const float c_log2 = scale * 1.44269504088896341f;     // scores are kept in units of log2 e
 
+  // A wave stages its tile in an LDS area of its own (lane = key row), so nothing in this loop
+  // waits for another wave.  The rows of the next tile are requested before the current tile is
+  // worked on.
+  constexpr int KCH = KS * 4, VCH = HD / 8;
+  bf16x8 k_stage[KCH], v_stage[VCH];
+  int64_t stage_off = 0;        // element offset of this lane's row in the caches
+  bool stage_in = false;        // the row is a key of this tile's range
+  auto fetch = [&](int it, int spec_blk) {
+    const int j = ((it0 + it) * stride + mine) * FA_KT + lane;
+    stage_in = j >= kv_begin && j < kv_end;
+    stage_off = 0;
+    if (stage_in) {
+      const int jb = j / block_size;
+      const int64_t blk = spec_blk >= 0 ? spec_blk : bt[jb];
+      stage_off = ((blk * nkv + kvh) * block_size + (j - jb * block_size)) * HD;
+    }
+    const bf16_t* kp = k_cache + stage_off;
+    const bf16_t* vp = v_cache + stage_off;
+    bf16x8 z = {};
+#pragma unroll
+    for (int c = 0; c < KCH; ++c) k_stage[c] = (stage_in && c * 8 < HD) ? *(const bf16x8*)(kp + c * 8) : z;
+#pragma unroll
+    for (int c = 0; c < VCH; ++c) v_stage[c] = stage_in ? *(const bf16x8*)(vp + c * 8) : z;
+  };
+  if (iters > 0) fetch(0, it0 == 0 ? spec_blk : -1);
+
   for (int it = 0; it < iters; ++it) {
-    const int kt_idx = range_lo + it * WAVES + wave;
-    const bool active = kt_idx < range_hi;
-    if (active) {
-      // stage this wave's tile: lane = key row
+    const int kt_idx = (it0 + it) * stride + mine;
+    {
       const int j = kt_idx * FA_KT + lane;
-      const bool in_range = j >= kv_begin && j < kv_end;
-      int64_t row_off = 0;
-      if (in_range) {
-        const int64_t blk = bt[j / block_size];
-        row_off = ((blk * nkv + kvh) * block_size + (j % block_size)) * HD;
-      }
       if (do_rope && j == new_pos) {
         // the new token's own key and value: made here from its qkv row, and written to the cache
         const bf16_t* krow = q + (int64_t)tok0 * q_stride + fused.k_off + (int64_t)kvh * HD;
         const bf16_t* vrow = q + (int64_t)tok0 * q_stride + fused.v_off + (int64_t)kvh * HD;
 #pragma unroll
-        for (int c = 0; c < KS * 4; ++c) {
-          bf16x8 k8 = {};
+        for (int c = 0; c < KCH; ++c) {
           if (c * 8 < HD) {
-            k8 = rotate_chunk<HD>(*(const bf16x8*)(krow + c * 8), *(const bf16x8*)(krow + (c * 8 + HD / 2) % HD),
-                                  c * 8, cs, sn);
-            *(bf16x8*)(fused.k_cache_w + row_off + c * 8) = k8;
+            k_stage[c] = rotate_chunk<HD>(*(const bf16x8*)(krow + c * 8),
+                                          *(const bf16x8*)(krow + (c * 8 + HD / 2) % HD), c * 8, cs, sn);
+            *(bf16x8*)(fused.k_cache_w + stage_off + c * 8) = k_stage[c];
           }
-          *(bf16x8*)(Kl + lane * KP + c * 8) = k8;
         }
 #pragma unroll
-        for (int c = 0; c < HD / 8; ++c) {
-          const bf16x8 v8 = *(const bf16x8*)(vrow + c * 8);
-          *(bf16x8*)(fused.v_cache_w + row_off + c * 8) = v8;
-#pragma unroll
-          for (int e = 0; e < 8; ++e) Vl[(c * 8 + e) * FA_VP + lane] = v8[e];
-        }
-      } else {
-        const bf16_t* kp = k_cache + row_off;
-        const bf16_t* vp = v_cache + row_off;
-#pragma unroll
-        for (int c = 0; c < KS * 4; ++c) {
-          bf16x8 z = {};
-          const bf16x8 kv8 = (in_range && c * 8 < HD) ? *(const bf16x8*)(kp + c * 8) : z;
-          *(bf16x8*)(Kl + lane * KP + c * 8) = kv8;
-        }
-#pragma unroll
-        for (int c = 0; c < HD / 8; ++c) {
-          bf16x8 z = {};
-          const bf16x8 v8 = in_range ? *(const bf16x8*)(vp + c * 8) : z;
-#pragma unroll
-          for (int e = 0; e < 8; ++e) Vl[(c * 8 + e) * FA_VP + lane] = v8[e];
+        for (int c = 0; c < VCH; ++c) {
+          v_stage[c] = *(const bf16x8*)(vrow + c * 8);
+          *(bf16x8*)(fused.v_cache_w + stage_off + c * 8) = v_stage[c];
         }
       }
+      // registers -> this wave's LDS area; V is transposed on the way
+#pragma unroll
+      for (int c = 0; c < KCH; ++c) *(bf16x8*)(Kl + lane * KP + c * 8) = k_stage[c];
+#pragma unroll
+      for (int c = 0; c < VCH; ++c) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) Vl[(c * 8 + e) * FA_VP + lane] = v_stage[c][e];
+      }
     }
-    __syncthreads();
-    if (active) {
+    if (it + 1 < iters) fetch(it + 1, -1);
+    // the LDS operations of one wave are carried out in order; the fences keep the compiler from
+    // moving the reads of other lanes' rows above the writes
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    {
       // scores, transposed: acc[kt][r] = S^T[key kt*16 + g*4 + r][row r16]
       f32x4 sc[4];
 #pragma unroll
@@ -338,8 +355,12 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
         }
       }
     }
-    __syncthreads();
+    // this wave's reads of its area are done before the next tile is written over it
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
+  __syncthreads();      // the merge below writes over the staging areas
 
   // merge the waves: each leaves (m, l, O[16][HD]) as floats in its own LDS area
   constexpr int MROW = HD + 2;
