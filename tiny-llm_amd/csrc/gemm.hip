@@ -410,36 +410,61 @@ struct SkinnyArgs {
   int64_t lda, ldo;
 };
 
-// One 8-wide k chunk of an activation row as an MFMA operand.  With the norm prologue the chunk
-// is w * x of the float32 residual stream (rounded to bfloat16) and `ss` collects x^2: the row's
-// 1 / rms is a common factor of the whole dot product and is applied to the result instead, so
-// nothing has to wait for the row statistics.
+// One 8-wide k chunk of an activation row, as loaded (Raw) and as an MFMA operand.  With the norm
+// prologue the operand is w * x of the float32 residual stream (rounded to bfloat16) and `ss`
+// collects x^2: the row's 1 / rms is a common factor of the whole dot product and is applied to
+// the result instead, so nothing has to wait for the row statistics.  Loading and converting are
+// separate steps so that the loads of the next k block can be in flight while this one is used.
 template <int PRO>
-__device__ __forceinline__ bf16x8 skinny_fetch(const SkinnyArgs& p, int64_t row_off, int k, float& ss) {
-  if constexpr (PRO == PRO_NONE) {
-    return *(const bf16x8*)((const bf16_t*)p.a + row_off + k);
-  } else {
-    const float* x = (const float*)p.a + row_off + k;
-    const f32x4 x0 = *(const f32x4*)x, x1 = *(const f32x4*)(x + 4);
-    float wv[8];
+struct SkinnyChunk;
+template <>
+struct SkinnyChunk<PRO_NONE> {
+  bf16x8 v;
+  __device__ __forceinline__ void load(const SkinnyArgs& p, int64_t off) { v = *(const bf16x8*)((const bf16_t*)p.a + off); }
+};
+template <>
+struct SkinnyChunk<PRO_NORM> {
+  f32x4 x0, x1;
+  __device__ __forceinline__ void load(const SkinnyArgs& p, int64_t off) {
+    const float* x = (const float*)p.a + off;
+    x0 = *(const f32x4*)x;
+    x1 = *(const f32x4*)(x + 4);
+  }
+};
+// the norm weights of one k chunk, as floats
+struct NormChunk {
+  f32x4 w0, w1;
+  __device__ __forceinline__ void load(const SkinnyArgs& p, int k) {
     if (p.norm_w_is_f32) {
-      const f32x4 w0 = *(const f32x4*)((const float*)p.norm_w + k), w1 = *(const f32x4*)((const float*)p.norm_w + k + 4);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) { wv[e] = w0[e]; wv[4 + e] = w1[e]; }
+      w0 = *(const f32x4*)((const float*)p.norm_w + k);
+      w1 = *(const f32x4*)((const float*)p.norm_w + k + 4);
     } else {
       const bf16x8 w8 = *(const bf16x8*)((const bf16_t*)p.norm_w + k);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) wv[e] = (float)w8[e];
+      for (int e = 0; e < 4; ++e) {
+        w0[e] = (float)w8[e];
+        w1[e] = (float)w8[4 + e];
+      }
     }
-    bf16x8 r;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      r[e] = (bf16_t)(wv[e] * x0[e]);
-      r[4 + e] = (bf16_t)(wv[4 + e] * x1[e]);
-      ss += x0[e] * x0[e] + x1[e] * x1[e];
-    }
-    return r;
   }
+};
+// `k_ok`: the chunk lies inside the row (it counts towards the sum of squares); the product itself
+// is protected by zeroing the weight chunk instead.
+__device__ __forceinline__ bf16x8 skinny_operand(const SkinnyChunk<PRO_NONE>& c, const NormChunk&, bool, float&) {
+  return c.v;
+}
+__device__ __forceinline__ bf16x8 skinny_operand(const SkinnyChunk<PRO_NORM>& c, const NormChunk& nw, bool k_ok,
+                                                 float& ss) {
+  bf16x8 r;
+  float q = 0.f;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    r[e] = (bf16_t)(nw.w0[e] * c.x0[e]);
+    r[4 + e] = (bf16_t)(nw.w1[e] * c.x1[e]);
+    q += c.x0[e] * c.x0[e] + c.x1[e] * c.x1[e];
+  }
+  ss += k_ok ? q : 0.f;
+  return r;
 }
 
 template <int MT, typename TO, int PRO, bool SWIGLU>
@@ -452,7 +477,6 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
   const int r16 = lane % 16, g = lane / 16;
   const int n = n0 + r16;
   const bf16_t* wrow = p.w + (int64_t)min(n, N - 1) * K;
-  const bool n_ok = n < N;
 
   // epilogue operands first: their latency hides behind the main loop
   constexpr int EPT = (MT * 256 + S_THREADS - 1) / S_THREADS;
@@ -466,17 +490,48 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
 
   // input row of each activation row this lane feeds
   int64_t row_off[MT];
-  bool m_ok[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int m = mt * 16 + r16;
-    m_ok[mt] = m < M;
     const int src = p.rows ? p.rows[min(m, M - 1)] : min(m, M - 1);
     row_off[mt] = (int64_t)src * p.lda;
   }
 
-  constexpr int UN = MT == 1 ? 2 : 1;      // k blocks whose loads are issued together
+  // A stage is UN k blocks of 128 (all loads of a stage are issued together).  With more than one
+  // row tile two stages take turns, so the loads of the next stage are in flight while this one
+  // is multiplied; with one row tile the registers are better spent on a second resident
+  // workgroup.  Loads are unconditional with the address clamped into the matrix: a predicated
+  // load would become a branch and the stages could not overlap.  Rows beyond M or N only feed
+  // outputs that are never written; a chunk beyond K is zeroed on the weight side when it is used.
+  constexpr int UN = MT == 1 ? 2 : 1;
+  constexpr bool TWO_STAGES = MT > 1;
+  struct Stage {
+    bf16x8 fw[UN][4];
+    SkinnyChunk<PRO> fa[UN][MT][4];
+    NormChunk nw[PRO == PRO_NORM ? UN : 1][PRO == PRO_NORM ? 4 : 1];
+  };
   const int nblk = (K + S_KBLK - 1) / S_KBLK;
+  auto load = [&](Stage& st, int blk) {
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      // MFMA i of the block covers k = i*32 .. i*32+31, lane group g its 8 k from g*8: one load
+      // instruction then reads 64 contiguous bytes of each of the 16 weight rows
+      const int kb = (blk + u * S_WAVES) * S_KBLK + g * 8;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) st.fw[u][i] = *(const bf16x8*)(wrow + min(kb + i * 32, K - 8));
+    }
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const int kb = (blk + u * S_WAVES) * S_KBLK + g * 8;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int k = min(kb + i * 32, K - 8);
+        if constexpr (PRO == PRO_NORM) st.nw[u][i].load(p, k);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) st.fa[u][mt][i].load(p, row_off[mt] + k);
+      }
+    }
+  };
   f32x4 acc[MT];
   float ss[MT];                            // this lane's share of sum x^2 of its rows (norm prologue)
 #pragma unroll
@@ -484,39 +539,48 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
     acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
     ss[mt] = 0.f;
   }
-  for (int blk = wave; blk < nblk; blk += S_WAVES * UN) {
-    bf16x8 fw[UN][4], fa[UN][MT][4];
+  auto multiply = [&](const Stage& st, int blk) {
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
-      // MFMA i of the block covers k = i*32 .. i*32+31, lane group g its 8 k from g*8: one load
-      // instruction then reads 64 contiguous bytes of each of the 16 weight rows
       const int kb = (blk + u * S_WAVES) * S_KBLK + g * 8;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int k = kb + i * 32;
+        const bool k_ok = kb + i * 32 < K;
         bf16x8 z = {};
-        fw[u][i] = (n_ok && k < K) ? *(const bf16x8*)(wrow + k) : z;
+        const bf16x8 fw = k_ok ? st.fw[u][i] : z;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          const bf16x8 fa = skinny_operand(st.fa[u][mt][i], st.nw[PRO == PRO_NORM ? u : 0][PRO == PRO_NORM ? i : 0],
+                                           k_ok, ss[mt]);
+          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw, fa, acc[mt], 0, 0, 0);
+        }
       }
     }
-#pragma unroll
-    for (int u = 0; u < UN; ++u) {
-      const int kb = (blk + u * S_WAVES) * S_KBLK + g * 8;
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int k = kb + i * 32;
-          bf16x8 z = {};
-          fa[u][mt][i] = (m_ok[mt] && k < K) ? skinny_fetch<PRO>(p, row_off[mt], k, ss[mt]) : z;
-        }
+  };
+  constexpr int STEP = S_WAVES * UN;
+  if constexpr (TWO_STAGES) {
+    Stage s0, s1;
+    int blk = wave;
+    if (blk < nblk) {
+      load(s0, blk);
+      while (true) {
+        const int b1 = blk + STEP;
+        if (b1 < nblk) load(s1, b1);
+        multiply(s0, blk);
+        if (b1 >= nblk) break;
+        const int b2 = b1 + STEP;
+        if (b2 < nblk) load(s0, b2);
+        multiply(s1, b1);
+        if (b2 >= nblk) break;
+        blk = b2;
+      }
     }
-#pragma unroll
-    for (int u = 0; u < UN; ++u)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[u][i], fa[u][mt][i], acc[mt], 0, 0, 0);
+  } else {
+    Stage s0;
+    for (int blk = wave; blk < nblk; blk += STEP) {
+      load(s0, blk);
+      multiply(s0, blk);
+    }
   }
   // tile layout: lane holds rows (weight rows) g*4 + r, column (activation row) r16
 #pragma unroll
@@ -570,14 +634,18 @@ template <typename TO, int PRO, bool SWIGLU>
 static void launch_skinny(const SkinnyArgs& p, hipStream_t stream) {
   dim3 g((p.N + S_COLS - 1) / S_COLS), b(S_THREADS);
   const int mt = (p.M + 15) / 16;
-  if (mt == 1)
+  if (mt == 1) {
     hipLaunchKernelGGL((gemm_skinny_bf16_kernel<1, TO, PRO, SWIGLU>), g, b, 0, stream, p);
-  else if (mt == 2)
-    hipLaunchKernelGGL((gemm_skinny_bf16_kernel<2, TO, PRO, SWIGLU>), g, b, 0, stream, p);
-  else if (mt == 3)
-    hipLaunchKernelGGL((gemm_skinny_bf16_kernel<3, TO, PRO, SWIGLU>), g, b, 0, stream, p);
-  else
-    hipLaunchKernelGGL((gemm_skinny_bf16_kernel<4, TO, PRO, SWIGLU>), g, b, 0, stream, p);
+    return;
+  }
+  if constexpr (PRO == PRO_NONE) {       // the norm prologue exists for one row tile only
+    if (mt == 2)
+      hipLaunchKernelGGL((gemm_skinny_bf16_kernel<2, TO, PRO, SWIGLU>), g, b, 0, stream, p);
+    else if (mt == 3)
+      hipLaunchKernelGGL((gemm_skinny_bf16_kernel<3, TO, PRO, SWIGLU>), g, b, 0, stream, p);
+    else
+      hipLaunchKernelGGL((gemm_skinny_bf16_kernel<4, TO, PRO, SWIGLU>), g, b, 0, stream, p);
+  }
 }
 
 template <int PRO>
@@ -646,7 +714,7 @@ int tl_linear(const void* a, const void* w, void* out, const float* residual, co
   return tl_launch_status();
 }
 
-// Few-row (M <= 64) bfloat16 product whose input is the float32 residual stream: the rows of a
+// Few-row (M <= 16) bfloat16 product whose input is the float32 residual stream: the rows of a
 // (gathered through `rows` if given) are RMS-normalised with norm_w (float32 or bfloat16) and eps
 // inside the kernel.  Epilogues as in tl_linear.
 int tl_linear_norm(const void* a, const void* w, void* out, const float* residual, const void* norm_w,
@@ -654,7 +722,7 @@ int tl_linear_norm(const void* a, const void* w, void* out, const float* residua
                    int64_t ldo, int out_dtype, int epilogue, hipStream_t stream) {
   if (M <= 0) return TL_OK;
   const bool swiglu = epilogue == 1;
-  if (M > 64 || N <= 0 || K <= 0 || K % 8 || lda % 8 || lda < K || ldo < (swiglu ? N / 2 : N) || !norm_w ||
+  if (M > 16 || N <= 0 || K <= 0 || K % 8 || lda % 8 || lda < K || ldo < (swiglu ? N / 2 : N) || !norm_w ||
       (norm_w_dtype != 0 && norm_w_dtype != 1) || epilogue < 0 || epilogue > 1)
     return TL_ERR_ARG;
   if (swiglu && ((N & 1) || residual)) return TL_ERR_ARG;

@@ -149,7 +149,7 @@ def _epilogue(name: Optional[str]) -> int:
     _need(name == "swiglu", f"unknown epilogue {name!r}")
     return 1
 
-FUSED_MAX_ROWS = 64    # most rows the few-row product kernel takes
+FUSED_MAX_ROWS = 16    # most rows for which the few-row product kernel normalises its input itself
 FUSED_MAX_COLS = 4096  # most columns for which the fused norm prologue pays
 
 
