@@ -382,8 +382,9 @@ static int launch_gemm_bf16_any(const bf16_t* a, const bf16_t* w, TO* out, const
 // whole cost, and a step is a chain of such kernels, so the kernel is built around
 // (a) many 16-byte loads in flight and (b) as few dependent memory round trips and
 // as few launches as possible.  A workgroup of eight wave64 owns 16 output columns
-// (16 weight rows); the waves split K in blocks of 128 and each accumulates a
-// 16 x 16 tile per group of 16 activation rows with v_mfma_f32_16x16x32_bf16
+// (16 weight rows; 32 or 64 when there are more than 16 activation rows); the waves split K in
+// blocks of 128 and each accumulates a
+// 16 x 16 tile per group of 16 activation rows and 16 columns with v_mfma_f32_16x16x32_bf16
 // (weight rows as the A operand read straight from global memory, activations as
 // the B operand).  Partial tiles meet in LDS and are added in a fixed order, so
 // results are deterministic.
@@ -467,25 +468,29 @@ __device__ __forceinline__ bf16x8 skinny_operand(const SkinnyChunk<PRO_NORM>& c,
   return r;
 }
 
-template <int MT, typename TO, int PRO, bool SWIGLU>
+template <int MT, int CT, typename TO, int PRO, bool SWIGLU>
 __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const SkinnyArgs p) {
-  __shared__ float part[S_WAVES][MT][16][17];
-  __shared__ float ss_part[S_WAVES][MT * 16];
+  extern __shared__ __attribute__((aligned(16))) unsigned char skinny_smem[];
+  typedef float Tile[16][17];
+  Tile* part = (Tile*)skinny_smem;                                  // [S_WAVES][MT * CT]
+  float* ss_part = (float*)(part + S_WAVES * MT * CT);              // [S_WAVES][MT * 16]
   const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
   const int M = p.M, N = p.N, K = p.K;
-  const int n0 = blockIdx.x * S_COLS;
+  const int n0 = blockIdx.x * (S_COLS * CT);
   const int r16 = lane % 16, g = lane / 16;
-  const int n = n0 + r16;
-  const bf16_t* wrow = p.w + (int64_t)min(n, N - 1) * K;
+  const bf16_t* wrow[CT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) wrow[ct] = p.w + (int64_t)min(n0 + ct * 16 + r16, N - 1) * K;
 
   // epilogue operands first: their latency hides behind the main loop
-  constexpr int EPT = (MT * 256 + S_THREADS - 1) / S_THREADS;
+  constexpr int TILES = MT * CT;
+  constexpr int EPT = (TILES * 256 + S_THREADS - 1) / S_THREADS;
   float res_v[EPT];
 #pragma unroll
   for (int j = 0; j < EPT; ++j) {
     const int e = tid + j * S_THREADS;
-    const int m = (e / 256) * 16 + (e % 256) / 16, nn = e % 16;
-    res_v[j] = (p.residual && e < MT * 256 && m < M && n0 + nn < N) ? p.residual[(int64_t)m * p.ldo + n0 + nn] : 0.f;
+    const int tile = e / 256, m = (tile / CT) * 16 + (e % 256) / 16, n = n0 + (tile % CT) * 16 + e % 16;
+    res_v[j] = (p.residual && e < TILES * 256 && m < M && n < N) ? p.residual[(int64_t)m * p.ldo + n] : 0.f;
   }
 
   // input row of each activation row this lane feeds
@@ -497,16 +502,16 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
     row_off[mt] = (int64_t)src * p.lda;
   }
 
-  // A stage is UN k blocks of 128 (all loads of a stage are issued together).  With more than one
-  // row tile two stages take turns, so the loads of the next stage are in flight while this one
-  // is multiplied; with one row tile the registers are better spent on a second resident
+  // A stage is UN k blocks of 128 (all loads of a stage are issued together).  Where the
+  // registers allow, two stages take turns, so the loads of the next stage are in flight while
+  // this one is multiplied; with one tile the registers are better spent on a second resident
   // workgroup.  Loads are unconditional with the address clamped into the matrix: a predicated
   // load would become a branch and the stages could not overlap.  Rows beyond M or N only feed
   // outputs that are never written; a chunk beyond K is zeroed on the weight side when it is used.
-  constexpr int UN = MT == 1 ? 2 : 1;
-  constexpr bool TWO_STAGES = MT > 1;
+  constexpr int UN = TILES == 1 ? 2 : 1;
+  constexpr bool TWO_STAGES = TILES > 1 && MT + CT <= 5;
   struct Stage {
-    bf16x8 fw[UN][4];
+    bf16x8 fw[UN][CT][4];
     SkinnyChunk<PRO> fa[UN][MT][4];
     NormChunk nw[PRO == PRO_NORM ? UN : 1][PRO == PRO_NORM ? 4 : 1];
   };
@@ -518,7 +523,9 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
       // instruction then reads 64 contiguous bytes of each of the 16 weight rows
       const int kb = (blk + u * S_WAVES) * S_KBLK + g * 8;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) st.fw[u][i] = *(const bf16x8*)(wrow + min(kb + i * 32, K - 8));
+      for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) st.fw[u][ct][i] = *(const bf16x8*)(wrow[ct] + min(kb + i * 32, K - 8));
     }
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
@@ -532,12 +539,13 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
       }
     }
   };
-  f32x4 acc[MT];
+  f32x4 acc[MT][CT];
   float ss[MT];                            // this lane's share of sum x^2 of its rows (norm prologue)
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
     ss[mt] = 0.f;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) acc[mt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
   auto multiply = [&](const Stage& st, int blk) {
 #pragma unroll
@@ -547,12 +555,17 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
       for (int i = 0; i < 4; ++i) {
         const bool k_ok = kb + i * 32 < K;
         bf16x8 z = {};
-        const bf16x8 fw = k_ok ? st.fw[u][i] : z;
+        bf16x8 fa[MT];
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          const bf16x8 fa = skinny_operand(st.fa[u][mt][i], st.nw[PRO == PRO_NORM ? u : 0][PRO == PRO_NORM ? i : 0],
-                                           k_ok, ss[mt]);
-          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw, fa, acc[mt], 0, 0, 0);
+        for (int mt = 0; mt < MT; ++mt)
+          fa[mt] = skinny_operand(st.fa[u][mt][i], st.nw[PRO == PRO_NORM ? u : 0][PRO == PRO_NORM ? i : 0], k_ok,
+                                  ss[mt]);
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+          const bf16x8 fw = k_ok ? st.fw[u][ct][i] : z;
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            acc[mt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw, fa[mt], acc[mt][ct], 0, 0, 0);
         }
       }
     }
@@ -586,14 +599,16 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) part[wave][mt][g * 4 + r][r16] = acc[mt][r];
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) part[wave * TILES + mt * CT + ct][g * 4 + r][r16] = acc[mt][ct][r];
   if constexpr (PRO == PRO_NORM) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       float t = ss[mt];
       t += __shfl_xor(t, 16, TL_WAVE);
       t += __shfl_xor(t, 32, TL_WAVE);
-      if (g == 0) ss_part[wave][mt * 16 + r16] = t;
+      if (g == 0) ss_part[wave * (MT * 16) + mt * 16 + r16] = t;
     }
   }
   __syncthreads();
@@ -601,15 +616,15 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
 #pragma unroll
   for (int j = 0; j < EPT; ++j) {
     const int e = tid + j * S_THREADS;
-    if (e >= MT * 256) continue;
-    const int mt = e / 256, m_local = (e % 256) / 16, nn = e % 16;
-    const int m = mt * 16 + m_local;
-    if (m >= M || n0 + nn >= N) continue;
+    if (e >= TILES * 256) continue;
+    const int tile = e / 256, m_local = (e % 256) / 16, nn = e % 16;
+    const int m = (tile / CT) * 16 + m_local, n = n0 + (tile % CT) * 16 + nn;
+    if (m >= M || n >= N) continue;
     float scale = p.row_scale ? p.row_scale[m] : 1.f;   // the row factor left out of the operands
     if constexpr (PRO == PRO_NORM) {
       float t = 0.f;
 #pragma unroll
-      for (int wv = 0; wv < S_WAVES; ++wv) t += ss_part[wv][m];
+      for (int wv = 0; wv < S_WAVES; ++wv) t += ss_part[wv * (MT * 16) + m];
       scale = 1.f / sqrtf(t / (float)K + p.eps);
     }
     if constexpr (SWIGLU) {   // columns (2j, 2j+1) = (gate_j, up_j): even threads make one output of a pair
@@ -617,48 +632,63 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
       float gv = 0.f, uv = 0.f;
 #pragma unroll
       for (int wv = 0; wv < S_WAVES; ++wv) {
-        gv += part[wv][mt][nn][m_local];
-        uv += part[wv][mt][nn + 1][m_local];
+        gv += part[wv * TILES + tile][nn][m_local];
+        uv += part[wv * TILES + tile][nn + 1][m_local];
       }
-      out[(int64_t)m * p.ldo + (n0 + nn) / 2] = from_f32<TO>(swiglu_pair(gv * scale, uv * scale));
+      out[(int64_t)m * p.ldo + n / 2] = from_f32<TO>(swiglu_pair(gv * scale, uv * scale));
     } else {
       float v = 0.f;
 #pragma unroll
-      for (int wv = 0; wv < S_WAVES; ++wv) v += part[wv][mt][nn][m_local];
-      out[(int64_t)m * p.ldo + n0 + nn] = from_f32<TO>(v * scale + res_v[j]);
+      for (int wv = 0; wv < S_WAVES; ++wv) v += part[wv * TILES + tile][nn][m_local];
+      out[(int64_t)m * p.ldo + n] = from_f32<TO>(v * scale + res_v[j]);
     }
   }
 }
 
+// Column tiles per workgroup: every workgroup reads all M activation rows, so with more rows it
+// should own more columns, or the activations are read more often than the weights.
+template <int MT, int CT, typename TO, int PRO, bool SWIGLU>
+static int launch_skinny_tile(const SkinnyArgs& p, hipStream_t stream) {
+  constexpr size_t smem = (size_t)S_WAVES * MT * CT * 16 * 17 * sizeof(float) + (size_t)S_WAVES * MT * 16 * sizeof(float);
+  static bool configured = false;
+  if (!configured) {
+    if (hipFuncSetAttribute((const void*)gemm_skinny_bf16_kernel<MT, CT, TO, PRO, SWIGLU>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+      return TL_ERR_LAUNCH;
+    configured = true;
+  }
+  dim3 g((p.N + S_COLS * CT - 1) / (S_COLS * CT)), b(S_THREADS);
+  hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, CT, TO, PRO, SWIGLU>), g, b, smem, stream, p);
+  return TL_OK;
+}
+
+// More column tiles only while at least 256 workgroups remain: fewer cannot pull the weights
+// through fast enough.
+template <int MT, typename TO, bool SWIGLU>
+static int launch_skinny_rows(const SkinnyArgs& p, hipStream_t stream) {
+  if (p.N >= 256 * 64) return launch_skinny_tile<MT, 4, TO, PRO_NONE, SWIGLU>(p, stream);
+  if (p.N >= 256 * 32) return launch_skinny_tile<MT, 2, TO, PRO_NONE, SWIGLU>(p, stream);
+  return launch_skinny_tile<MT, 1, TO, PRO_NONE, SWIGLU>(p, stream);
+}
+
 template <typename TO, int PRO, bool SWIGLU>
-static void launch_skinny(const SkinnyArgs& p, hipStream_t stream) {
-  dim3 g((p.N + S_COLS - 1) / S_COLS), b(S_THREADS);
+static int launch_skinny(const SkinnyArgs& p, hipStream_t stream) {
   const int mt = (p.M + 15) / 16;
-  if (mt == 1) {
-    hipLaunchKernelGGL((gemm_skinny_bf16_kernel<1, TO, PRO, SWIGLU>), g, b, 0, stream, p);
-    return;
-  }
+  if (mt == 1) return launch_skinny_tile<1, 1, TO, PRO, SWIGLU>(p, stream);
   if constexpr (PRO == PRO_NONE) {       // the norm prologue exists for one row tile only
-    if (mt == 2)
-      hipLaunchKernelGGL((gemm_skinny_bf16_kernel<2, TO, PRO, SWIGLU>), g, b, 0, stream, p);
-    else if (mt == 3)
-      hipLaunchKernelGGL((gemm_skinny_bf16_kernel<3, TO, PRO, SWIGLU>), g, b, 0, stream, p);
-    else
-      hipLaunchKernelGGL((gemm_skinny_bf16_kernel<4, TO, PRO, SWIGLU>), g, b, 0, stream, p);
+    if (mt == 2) return launch_skinny_rows<2, TO, SWIGLU>(p, stream);
+    if (mt == 3) return launch_skinny_rows<3, TO, SWIGLU>(p, stream);
+    return launch_skinny_rows<4, TO, SWIGLU>(p, stream);
   }
+  return TL_ERR_ARG;
 }
 
 template <int PRO>
 static int launch_skinny_out(const SkinnyArgs& p, int out_dtype, bool swiglu, hipStream_t stream) {
-  if (out_dtype == 0 && !swiglu)
-    launch_skinny<float, PRO, false>(p, stream);
-  else if (out_dtype == 1 && !swiglu)
-    launch_skinny<bf16_t, PRO, false>(p, stream);
-  else if (out_dtype == 1 && swiglu)
-    launch_skinny<bf16_t, PRO, true>(p, stream);
-  else
-    return TL_ERR_ARG;
-  return TL_OK;
+  if (out_dtype == 0 && !swiglu) return launch_skinny<float, PRO, false>(p, stream);
+  if (out_dtype == 1 && !swiglu) return launch_skinny<bf16_t, PRO, false>(p, stream);
+  if (out_dtype == 1 && swiglu) return launch_skinny<bf16_t, PRO, true>(p, stream);
+  return TL_ERR_ARG;
 }
 
 }  // namespace
@@ -694,7 +724,8 @@ int tl_linear(const void* a, const void* w, void* out, const float* residual, co
     if (out_dtype != 0 && out_dtype != 1) return TL_ERR_ARG;
     if (M <= 64) {
       SkinnyArgs p{a, (const bf16_t*)w, out, residual, nullptr, nullptr, row_scale, 0.f, 0, M, N, K, lda, ldo};
-      if (launch_skinny_out<PRO_NONE>(p, out_dtype, swiglu, stream) != TL_OK) return TL_ERR_ARG;
+      const int rc = launch_skinny_out<PRO_NONE>(p, out_dtype, swiglu, stream);
+      if (rc != TL_OK) return rc;
     } else {
       int rc;
       if (swiglu)
@@ -727,7 +758,8 @@ int tl_linear_norm(const void* a, const void* w, void* out, const float* residua
     return TL_ERR_ARG;
   if (swiglu && ((N & 1) || residual)) return TL_ERR_ARG;
   SkinnyArgs p{a, (const bf16_t*)w, out, residual, norm_w, rows, nullptr, eps, norm_w_dtype == 0 ? 1 : 0, M, N, K, lda, ldo};
-  if (launch_skinny_out<PRO_NORM>(p, out_dtype, swiglu, stream) != TL_OK) return TL_ERR_ARG;
+  const int rc = launch_skinny_out<PRO_NORM>(p, out_dtype, swiglu, stream);
+  if (rc != TL_OK) return rc;
   return tl_launch_status();
 }
 
