@@ -157,6 +157,48 @@ def test_linear_norm(M, K, N):
     assert rel(ob, c) < 6e-3
 
 
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 40, 64])
+@pytest.mark.parametrize("K,N,N2", [(64, 248, 96), (5632, 2048, 516), (176, 64, 40), (96, 520, 1030)])
+def test_linear_handoff(M, K, N, N2):
+    """A norm handed from the product that writes the residual stream to the product that reads
+    it: the first also writes bf16(w * x) and partial sums of x^2, the second applies 1 / rms."""
+    g = torch.Generator().manual_seed(M * 11 + N)
+    z = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w1 = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    res = torch.randn(M, N, generator=g)
+    w2 = (torch.randn(N2, N, generator=g) / math.sqrt(N)).to(torch.bfloat16)
+    x_ref = z.double() @ w1.double().T + res.double()
+    for nwt in (torch.float32, torch.bfloat16):
+        nw = (1 + 0.1 * torch.randn(N, generator=g)).to(nwt)
+        x = res.clone().to(DEV)
+        operand = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+        sumsq = torch.full((M, (N + 15) // 16), float("nan"), dtype=torch.float32, device=DEV)
+        ops().linear_handoff(z.to(DEV), w1.to(DEV), x, x, emit=(nw.to(DEV), operand, sumsq))
+        assert rel(x, x_ref) < 1e-5
+        xs = x.cpu().double()
+        # the operand is the rounded product of the weight and the float32 result, element by element
+        assert torch.equal(operand.cpu(), (nw.float() * x.cpu()).to(torch.bfloat16))
+        assert rel(sumsq.sum(dim=1), (xs * xs).sum(dim=1)) < 1e-6
+        inv = 1.0 / torch.sqrt((xs * xs).mean(dim=-1, keepdim=True) + 1e-5)
+        c = (operand.cpu().double() @ w2.double().T) * inv
+        out = torch.empty(M, N2, dtype=torch.float32, device=DEV)
+        ops().linear_handoff(operand, w2.to(DEV), out, prepared=(sumsq, 1e-5, N))
+        assert rel(out, c) < 1e-5
+        assert rel(out, plain.rms_norm(xs, nw.double(), 1e-5) @ w2.double().T) < 1e-2
+        # with a gather of rows, as the output head takes the wanted positions
+        rows = torch.randperm(M, generator=g)[:max(1, M // 2)].to(torch.int32)
+        outg = torch.empty(rows.numel(), N2, dtype=torch.float32, device=DEV)
+        ops().linear_handoff(operand, w2.to(DEV), outg, rows=rows.to(DEV), prepared=(sumsq, 1e-5, N))
+        assert rel(outg, c[rows.long()]) < 1e-5
+        # with the SiLU-gate epilogue, as the feed-forward's first product
+        zz = torch.empty(M, N2 // 2, dtype=torch.bfloat16, device=DEV)
+        ops().linear_handoff(operand, w2.to(DEV), zz, epilogue="swiglu", prepared=(sumsq, 1e-5, N))
+        assert rel(zz, plain.silu(c[:, 0::2]) * c[:, 1::2]) < 6e-3
+    with pytest.raises(Exception):
+        ops().linear_handoff(torch.zeros(65, K, dtype=torch.bfloat16, device=DEV), w1.to(DEV),
+                             torch.empty(65, N, dtype=torch.float32, device=DEV))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,K,N", [(1, 64, 352), (9, 96, 400), (64, 2048, 96), (65, 176, 128), (300, 256, 1030)])
 def test_linear_swiglu_epilogue(dtype, M, K, N):

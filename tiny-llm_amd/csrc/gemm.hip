@@ -409,6 +409,17 @@ struct SkinnyArgs {
   int norm_w_is_f32;
   int M, N, K;
   int64_t lda, ldo;
+  // A norm handed from producer to consumer.  The producer (float32 output, no SiLU-gate) also
+  // writes emit_operand[m, n] = bf16(emit_w[n] * out[m, n]) and, per group of 16 columns, the sum
+  // of out^2 into emit_sumsq[m, group] (ceil(N / 16) groups).  The consumer takes such an operand
+  // as `a` and turns in_sumsq [rows, in_parts] into its row factor 1 / sqrt(sum / in_width + in_eps).
+  const void* emit_w = nullptr;
+  int emit_w_is_f32 = 0;
+  bf16_t* emit_operand = nullptr;
+  float* emit_sumsq = nullptr;
+  const float* in_sumsq = nullptr;
+  int in_parts = 0, in_width = 0;
+  float in_eps = 0.f;
 };
 
 // One 8-wide k chunk of an activation row, as loaded (Raw) and as an MFMA operand.  With the norm
@@ -500,6 +511,19 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
     const int m = mt * 16 + r16;
     const int src = p.rows ? p.rows[min(m, M - 1)] : min(m, M - 1);
     row_off[mt] = (int64_t)src * p.lda;
+  }
+
+  // row factors of a norm whose sums of squares arrive in parts: one wave per row, fixed order
+  float* scale_s = ss_part + S_WAVES * MT * 16;                      // [MT * 16]
+  if (p.in_sumsq) {
+    for (int r = wave; r < MT * 16; r += S_WAVES) {
+      const int m = min(r, M - 1);
+      const int64_t src = p.rows ? p.rows[m] : m;
+      float t = 0.f;
+      for (int q = lane; q < p.in_parts; q += TL_WAVE) t += p.in_sumsq[src * p.in_parts + q];
+      t = wave_sum(t);
+      if (lane == 0) scale_s[r] = 1.f / sqrtf(t / (float)p.in_width + p.in_eps);
+    }
   }
 
   // A stage is UN k blocks of 128 (all loads of a stage are issued together).  Where the
@@ -616,19 +640,21 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
 #pragma unroll
   for (int j = 0; j < EPT; ++j) {
     const int e = tid + j * S_THREADS;
-    if (e >= TILES * 256) continue;
+    if (e >= TILES * 256) continue;       // whole waves: 256 elements are four waves
     const int tile = e / 256, m_local = (e % 256) / 16, nn = e % 16;
     const int m = (tile / CT) * 16 + m_local, n = n0 + (tile % CT) * 16 + nn;
-    if (m >= M || n >= N) continue;
-    float scale = p.row_scale ? p.row_scale[m] : 1.f;   // the row factor left out of the operands
+    const bool valid = m < M && n < N;
+    float scale = 1.f;                    // the row factor left out of the operands
+    if (p.row_scale) scale = p.row_scale[min(m, M - 1)];
+    if (p.in_sumsq) scale = scale_s[(tile / CT) * 16 + m_local];
     if constexpr (PRO == PRO_NORM) {
       float t = 0.f;
 #pragma unroll
-      for (int wv = 0; wv < S_WAVES; ++wv) t += ss_part[wv * (MT * 16) + m];
+      for (int wv = 0; wv < S_WAVES; ++wv) t += ss_part[wv * (MT * 16) + (tile / CT) * 16 + m_local];
       scale = 1.f / sqrtf(t / (float)K + p.eps);
     }
     if constexpr (SWIGLU) {   // columns (2j, 2j+1) = (gate_j, up_j): even threads make one output of a pair
-      if (nn & 1) continue;
+      if ((nn & 1) || !valid) continue;
       float gv = 0.f, uv = 0.f;
 #pragma unroll
       for (int wv = 0; wv < S_WAVES; ++wv) {
@@ -640,7 +666,20 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
       float v = 0.f;
 #pragma unroll
       for (int wv = 0; wv < S_WAVES; ++wv) v += part[wv * TILES + tile][nn][m_local];
-      out[(int64_t)m * p.ldo + n] = from_f32<TO>(v * scale + res_v[j]);
+      v = v * scale + res_v[j];
+      if (valid) out[(int64_t)m * p.ldo + n] = from_f32<TO>(v);
+      if constexpr (sizeof(TO) == 4) {
+        if (p.emit_operand) {             // uniform: the 16 lanes of a row group stay together
+          if (valid) {
+            const float wn = p.emit_w_is_f32 ? ((const float*)p.emit_w)[n] : (float)((const bf16_t*)p.emit_w)[n];
+            p.emit_operand[(int64_t)m * N + n] = (bf16_t)(wn * v);
+          }
+          float sq = valid ? v * v : 0.f;
+#pragma unroll
+          for (int off = 1; off < 16; off <<= 1) sq += __shfl_xor(sq, off, TL_WAVE);
+          if (nn == 0 && m < M) p.emit_sumsq[(int64_t)m * ((N + 15) / 16) + (n0 / 16 + tile % CT)] = sq;
+        }
+      }
     }
   }
 }
@@ -649,7 +688,7 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
 // should own more columns, or the activations are read more often than the weights.
 template <int MT, int CT, typename TO, int PRO, bool SWIGLU>
 static int launch_skinny_tile(const SkinnyArgs& p, hipStream_t stream) {
-  constexpr size_t smem = (size_t)S_WAVES * MT * CT * 16 * 17 * sizeof(float) + (size_t)S_WAVES * MT * 16 * sizeof(float);
+  constexpr size_t smem = (size_t)S_WAVES * MT * CT * 16 * 17 * sizeof(float) + (size_t)(S_WAVES + 1) * MT * 16 * sizeof(float);
   static bool configured = false;
   if (!configured) {
     if (hipFuncSetAttribute((const void*)gemm_skinny_bf16_kernel<MT, CT, TO, PRO, SWIGLU>,
@@ -742,6 +781,43 @@ int tl_linear(const void* a, const void* w, void* out, const float* residual, co
   } else {
     return TL_ERR_ARG;
   }
+  return tl_launch_status();
+}
+
+// Few-row (M <= 64) bfloat16 product that takes part in handing a norm from one product to the
+// next (see SkinnyArgs).  Consumer side: in_sumsq [rows of a, in_parts] (a is then the operand a
+// producer wrote; `rows` gathers rows of both).  Producer side (out_dtype 0, epilogue 0): emit_w
+// [N] (element type emit_w_dtype), emit_operand bf16 [M, N], emit_sumsq float [M, ceil(N / 16)].
+// Either side may be absent.
+int tl_linear_handoff(const void* a, const void* w, void* out, const float* residual, const int32_t* rows,
+                      const float* in_sumsq, int in_parts, float in_eps, int in_width, const void* emit_w,
+                      int emit_w_dtype, void* emit_operand, float* emit_sumsq, int M, int N, int K, int64_t lda,
+                      int64_t ldo, int out_dtype, int epilogue, hipStream_t stream) {
+  if (M <= 0) return TL_OK;
+  const bool swiglu = epilogue == 1;
+  if (M > 64 || N <= 0 || K <= 0 || K % 8 || lda % 8 || lda < K || ldo < (swiglu ? N / 2 : N) || epilogue < 0 ||
+      epilogue > 1 || (out_dtype != 0 && out_dtype != 1))
+    return TL_ERR_ARG;
+  if (swiglu && ((N & 1) || residual || out_dtype != 1)) return TL_ERR_ARG;
+  if (in_sumsq && (in_parts <= 0 || in_width <= 0)) return TL_ERR_ARG;
+  const bool emit = emit_operand != nullptr;
+  if (emit && (!emit_w || !emit_sumsq || swiglu || out_dtype != 0 || (emit_w_dtype != 0 && emit_w_dtype != 1)))
+    return TL_ERR_ARG;
+  SkinnyArgs p{a, (const bf16_t*)w, out, residual, nullptr, rows, nullptr, 0.f, 0, M, N, K, lda, ldo};
+  if (emit) {
+    p.emit_w = emit_w;
+    p.emit_w_is_f32 = emit_w_dtype == 0 ? 1 : 0;
+    p.emit_operand = (bf16_t*)emit_operand;
+    p.emit_sumsq = emit_sumsq;
+  }
+  if (in_sumsq) {
+    p.in_sumsq = in_sumsq;
+    p.in_parts = in_parts;
+    p.in_width = in_width;
+    p.in_eps = in_eps;
+  }
+  const int rc = launch_skinny_out<PRO_NONE>(p, out_dtype, swiglu, stream);
+  if (rc != TL_OK) return rc;
   return tl_launch_status();
 }
 

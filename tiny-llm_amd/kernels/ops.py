@@ -197,6 +197,73 @@ def linear_norm(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: torch
                                  _stream()), "linear_norm")
     return out
 
+HANDOFF_MAX_ROWS = 64   # most rows for which a product can hand a norm to the next one
+
+
+def can_hand_off(rows: int, width: int, dtype: torch.dtype) -> bool:
+    """Whether `linear_handoff` can prepare a norm over `width` columns for `rows` rows."""
+    return dtype == torch.bfloat16 and 0 < rows <= HANDOFF_MAX_ROWS and width % 8 == 0
+
+
+def linear_handoff(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, residual: Optional[torch.Tensor] = None,
+                   epilogue: Optional[str] = None, rows: Optional[torch.Tensor] = None, prepared=None,
+                   emit=None) -> torch.Tensor:
+    """The few-row bfloat16 product with a norm handed over between products, in one launch each.
+
+    emit = (norm_weight [N], operand [M, N] bfloat16, sumsq [M, ceil(N / 16)] float32): besides
+    out = a @ w.T + residual (float32) the kernel writes operand = bf16(norm_weight * out) and the
+    sums of out^2 over groups of 16 columns.  prepared = (sumsq [R, P], eps, width): `a` is such an
+    operand ([R, K]; `rows` picks rows of both) and the product is multiplied by
+    1 / sqrt(sum(sumsq[row]) / width + eps): together the two are rmsnorm(out) @ w.T."""
+    _dev(a, w, out, residual, rows)
+    _rows_2d(a, "linear input")
+    _rows_2d(out, "linear output")
+    K = a.shape[1]
+    M = a.shape[0] if rows is None else rows.numel()
+    N = w.shape[0]
+    swiglu = _epilogue(epilogue)
+    _need(0 < M <= HANDOFF_MAX_ROWS, f"a norm is handed over for at most {HANDOFF_MAX_ROWS} rows")
+    _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_contiguous()
+          and w.shape[1] == K, f"input and weight must be bfloat16, weight contiguous [N, {K}]")
+    _need(K % 8 == 0 and a.stride(0) % 8 == 0, "inner size must be a multiple of 8")
+    if rows is not None:
+        _need(rows.dtype == torch.int32 and rows.is_contiguous(), "row index must be contiguous int32")
+    if swiglu:
+        _need(N % 2 == 0 and tuple(out.shape) == (M, N // 2) and out.dtype == torch.bfloat16 and residual is None,
+              f"the SiLU-gate epilogue writes bfloat16 [{M}, {N // 2}] and takes no residual")
+    else:
+        _need(tuple(out.shape) == (M, N) and out.dtype in (torch.float32, torch.bfloat16),
+              f"linear output must be [{M}, {N}], float32 or bfloat16")
+    if residual is not None:
+        _need(residual.dtype == torch.float32 and residual.shape == out.shape
+              and residual.stride() == out.stride(), "residual must be float32 with the output's layout")
+    sumsq_in, parts, eps, width = None, 0, 0.0, 0
+    if prepared is not None:
+        sumsq_in, eps, width = prepared
+        _dev(sumsq_in)
+        _need(sumsq_in.dtype == torch.float32 and sumsq_in.dim() == 2 and sumsq_in.is_contiguous()
+              and sumsq_in.shape[0] == a.shape[0] and width > 0,
+              "sums of squares must be contiguous float32 [rows of the input, parts]")
+        parts = sumsq_in.shape[1]
+    emit_w = emit_op = emit_sq = None
+    if emit is not None:
+        emit_w, emit_op, emit_sq = emit
+        _dev(emit_w, emit_op, emit_sq)
+        _need(not swiglu and out.dtype == torch.float32, "only a float32 product without SiLU-gate prepares a norm")
+        _need(emit_w.is_contiguous() and emit_w.numel() == N and emit_w.dtype in (torch.float32, torch.bfloat16),
+              f"norm weight must have {N} elements, float32 or bfloat16")
+        _need(emit_op.dtype == torch.bfloat16 and emit_op.is_contiguous() and tuple(emit_op.shape) == (M, N),
+              f"operand must be contiguous bfloat16 [{M}, {N}]")
+        _need(emit_sq.dtype == torch.float32 and emit_sq.is_contiguous()
+              and tuple(emit_sq.shape) == (M, (N + 15) // 16), f"sums of squares must be float32 [{M}, {(N + 15) // 16}]")
+    _check(_lib().tl_linear_handoff(
+        _ptr(a, 16), _ptr(w, 16), _ptr(out), _ptr(residual), _ptr(rows), _ptr(sumsq_in), c_int(parts), c_float(eps),
+        c_int(width), _ptr(emit_w), c_int(_dt(emit_w) if emit_w is not None else 0), _ptr(emit_op), _ptr(emit_sq),
+        c_int(M), c_int(N), c_int(K), c_int64(a.stride(0)), c_int64(out.stride(0)), c_int(_dt(out)), c_int(swiglu),
+        _stream()), "linear_handoff")
+    return out
+
+
 def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     """out[t, j] = silu(gate_up[t, j]) * gate_up[t, I + j]."""
     _dev(gate_up, out)

@@ -85,10 +85,27 @@ class Decoder:
     def forward(self, ctx) -> torch.Tensor:
         """Runs the tokens of `ctx` through the plan; float32 logits at ctx.logit_rows."""
         x = self.embedding.forward(ctx.tokens)
-        for i, e in enumerate(self.spec.plan):
-            x = self.layers[e.layer].block.forward(x, ctx, self.caches[i], self.states[i])
-        if ctx.logit_rows is None or ctx.logit_rows.numel() == 0:
+        wants_logits = ctx.logit_rows is not None and ctx.logit_rows.numel() > 0
+        plan = self.spec.plan
+        # A block may prepare the norm that reads its result (the next block's first norm, or the
+        # final norm) in its last product; `prepared` carries that from one block to the next.
+        prepared = None
+        for i, e in enumerate(plan):
+            block = self.layers[e.layer].block
+            if not hasattr(block, "forward_chained"):
+                x, prepared = block.forward(x, ctx, self.caches[i], self.states[i]), None
+                continue
+            if i + 1 < len(plan):
+                nxt = self.layers[plan[i + 1].layer].block
+                next_norm = getattr(nxt, "first_norm", None) if hasattr(nxt, "forward_chained") else None
+            else:
+                next_norm = self.final_norm if wants_logits and hasattr(self.final_norm, "lazy") else None
+            x, prepared = block.forward_chained(x, ctx, self.caches[i], self.states[i], prepared, next_norm)
+        if not wants_logits:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=x.device)
         norm = self.final_norm
-        h = norm.lazy(x, ctx.logit_rows) if hasattr(norm, "lazy") else norm.forward(x, ctx.logit_rows)
+        if hasattr(norm, "lazy"):
+            h = norm.lazy(x, ctx.logit_rows, prepared=prepared) if prepared is not None else norm.lazy(x, ctx.logit_rows)
+        else:
+            h = norm.forward(x, ctx.logit_rows)
         return self.lm_head.forward(h)

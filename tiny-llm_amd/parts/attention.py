@@ -19,12 +19,14 @@ import torch
 
 from ..kernels import ops
 from .norm import LazyNorm
-from .base import (CacheSpec, LayerCache, Mixer, POSITION_ENCODINGS, WeightSpec, register_mixer)
+from .base import (CacheSpec, LayerCache, Mixer, POSITION_ENCODINGS, WeightSpec, project_into_residual,
+                   register_mixer)
 
 
 class Attention(Mixer):
     graph_safe = True
     accepts_lazy_norm = True
+    prepares_next_norm = True
 
     def __init__(self, prefix, dtype, device, *, hidden_size: int, num_heads: int, num_kv_heads: int,
                  head_dim: int, position: dict = None, window: int = 0, scale: float = None,
@@ -64,11 +66,11 @@ class Attention(Mixer):
         return CacheSpec(self.num_kv_heads, self.head_dim, "window" if self.window else "full", self.window)
 
     # --------------------------------------------------------------------- compute
-    def forward(self, h, ctx, cache: LayerCache, state, residual):
+    def forward(self, h, ctx, cache: LayerCache, state, residual, next_norm=None):
         T = residual.shape[0]
         qkv = torch.empty((T, self.q_size + 2 * self.kv_size), dtype=self.dtype, device=residual.device)
         if isinstance(h, LazyNorm):
-            ops.linear_norm(h.x, h.weight, h.eps, self.w_qkv, qkv, rows=h.rows)
+            h.linear(self.w_qkv, qkv)
         else:
             ops.linear(h, self.w_qkv, qkv)
         tables = self.position.rotary_tables()
@@ -100,7 +102,8 @@ class Attention(Mixer):
             ops.paged_attention(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.req_of_token,
                                 ctx.positions, attn, self.num_heads, self.num_kv_heads, self.head_dim,
                                 self.scale, self.window)
-        return ops.linear(attn, self.w_o, residual, residual)
+        out, prepared = project_into_residual(attn, self.w_o, residual, next_norm)
+        return out if next_norm is None else (out, prepared)
 
     def _splits(self, ctx, T: int, device):
         """How many workgroups share one query tile's keys.  Eight waves of one workgroup take up to

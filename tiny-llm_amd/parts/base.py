@@ -13,6 +13,9 @@ Calling conventions
 * A mixer and a feed-forward receive the normed activations `h` and the
   residual, and return `residual + f(h)` as float32 (writing into `residual`
   is allowed); `add_to_residual` does that for parts that do not fuse it.
+* A part with `prepares_next_norm = True` also takes `next_norm=` (the norm that will read its
+  result, or None) and may return `(residual, prepared)`: it has prepared that norm in its last
+  product (`project_into_residual`).  Nothing else has to know about this.
 * A mixer additionally receives the step context (who is in the batch, where
   each token sits), its view of the paged cache (or None) and its per-request
   state tensor [slots, ...] (or None).
@@ -134,6 +137,20 @@ class Block:
 
     def forward(self, x, ctx, cache, state):
         raise NotImplementedError
+
+
+def project_into_residual(z: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, next_norm=None):
+    """residual += z @ w.T, the last product of a mixer or feed-forward.  Returns
+    (residual, prepared): when `next_norm` (the norm that will read the result) can be prepared by
+    this very product (few rows, bfloat16), `prepared` is what its `lazy()` takes; else None."""
+    from ..kernels import ops
+    bufs = None
+    if next_norm is not None and hasattr(next_norm, "hand_off_buffers") and residual.is_contiguous():
+        bufs = next_norm.hand_off_buffers(residual.shape[0], residual.device)
+    if bufs is not None and z.dtype == torch.bfloat16 and bufs[1].shape == residual.shape:
+        ops.linear_handoff(z, w, residual, residual, emit=bufs)
+        return residual, (bufs[1], bufs[2])
+    return ops.linear(z, w, residual, residual), None
 
 
 def add_to_residual(residual: torch.Tensor, y: torch.Tensor) -> torch.Tensor:

@@ -7,16 +7,35 @@ from .base import Block, register_block
 
 class PreNormBlock(Block):
     def forward(self, x, ctx, cache, state):
-        h = self._normed(self.mixer_norm, self.mixer, x)
-        x = self.mixer.forward(h, ctx, cache, state, x)
-        h = self._normed(self.ffn_norm, self.ffn, x)
-        return self.ffn.forward(h, ctx, x)
+        return self.forward_chained(x, ctx, cache, state)[0]
+
+    @property
+    def first_norm(self):
+        """The norm that reads this block's input, for whoever writes that input."""
+        return self.mixer_norm if getattr(self.mixer, "accepts_lazy_norm", False) else None
+
+    def forward_chained(self, x, ctx, cache, state, prepared=None, next_norm=None):
+        """As `forward`, between neighbours: `prepared` is this block's first norm as prepared by the
+        product that wrote x (or None); `next_norm` is the norm that will read this block's result
+        (or None).  Returns (x, that norm prepared or None)."""
+        h = self._normed(self.mixer_norm, self.mixer, x, prepared)
+        ffn_norm = self.ffn_norm if getattr(self.ffn, "accepts_lazy_norm", False) else None
+        x, prep = self._run(self.mixer, (h, ctx, cache, state, x), ffn_norm)
+        h = self._normed(self.ffn_norm, self.ffn, x, prep)
+        return self._run(self.ffn, (h, ctx, x), next_norm)
 
     @staticmethod
-    def _normed(norm, consumer, x):
+    def _run(part, args, next_norm):
+        if next_norm is not None and getattr(part, "prepares_next_norm", False):
+            out = part.forward(*args, next_norm=next_norm)
+            return out if isinstance(out, tuple) else (out, None)
+        return part.forward(*args), None
+
+    @staticmethod
+    def _normed(norm, consumer, x, prepared=None):
         # a consumer that says so may receive the norm unevaluated and fuse it into its first product
         if getattr(consumer, "accepts_lazy_norm", False) and hasattr(norm, "lazy"):
-            return norm.lazy(x)
+            return norm.lazy(x, prepared=prepared) if prepared is not None else norm.lazy(x)
         return norm.forward(x)
 
 

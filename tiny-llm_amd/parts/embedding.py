@@ -52,6 +52,6 @@ class LMHead(Part):
         """h: activations [n, H], or a LazyNorm whose norm rides in the product."""
         if isinstance(h, LazyNorm):
             out = torch.empty((h.num_rows, self.vocab_size), dtype=torch.float32, device=h.x.device)
-            return ops.linear_norm(h.x, h.weight, h.eps, self.weight, out, rows=h.rows)
+            return h.linear(self.weight, out)
         out = torch.empty((h.shape[0], self.vocab_size), dtype=torch.float32, device=h.device)
         return ops.linear(h, self.weight, out)

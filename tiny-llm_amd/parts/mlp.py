@@ -14,12 +14,13 @@ import torch
 
 from ..kernels import ops
 from .norm import LazyNorm
-from .base import FeedForward, WeightSpec, register_feed_forward
+from .base import FeedForward, WeightSpec, project_into_residual, register_feed_forward
 
 
 class SwiGLU(FeedForward):
     graph_safe = True
     accepts_lazy_norm = True
+    prepares_next_norm = True
 
     def __init__(self, prefix, dtype, device, *, hidden_size: int, intermediate_size: int):
         super().__init__(prefix, dtype, device)
@@ -42,14 +43,15 @@ class SwiGLU(FeedForward):
                                                                 self.hidden_size).contiguous()
         self.w_down = tensors[f"{p}.down_proj.weight"].contiguous()
 
-    def forward(self, h, ctx, residual):
+    def forward(self, h, ctx, residual, next_norm=None):
         T, dev = residual.shape[0], residual.device
         z = torch.empty((T, self.intermediate_size), dtype=self.dtype, device=dev)
         if isinstance(h, LazyNorm):
-            ops.linear_norm(h.x, h.weight, h.eps, self.w_gate_up, z, rows=h.rows, epilogue="swiglu")
+            h.linear(self.w_gate_up, z, epilogue="swiglu")
         else:
             ops.linear(h, self.w_gate_up, z, epilogue="swiglu")
-        return ops.linear(z, self.w_down, residual, residual)
+        out, prepared = project_into_residual(z, self.w_down, residual, next_norm)
+        return out if next_norm is None else (out, prepared)
 
 
 register_feed_forward("swiglu", SwiGLU)

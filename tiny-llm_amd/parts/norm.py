@@ -16,11 +16,24 @@ from .base import Norm, WeightSpec, register_norm
 
 class LazyNorm:
     """A norm that has not run yet: (x, weight, eps).  A consumer that can fuse the norm into its
-    first product takes the fields; any other calls `materialize()`."""
+    first product takes the fields; any other calls `materialize()`.
 
-    def __init__(self, norm: "RMSNorm", x: torch.Tensor, rows: Optional[torch.Tensor] = None):
+    `prepared` = (operand, sumsq): the product that wrote x has already written
+    operand = bf16(weight * x) and the sums of x^2 over groups of columns
+    (`ops.linear_handoff`), so the consumer's product needs no pass over x at all."""
+
+    def __init__(self, norm: "RMSNorm", x: torch.Tensor, rows: Optional[torch.Tensor] = None, prepared=None):
         self.norm, self.x, self.rows = norm, x, rows
         self.weight, self.eps = norm.weight, norm.eps
+        self.prepared = prepared
+
+    def linear(self, w: torch.Tensor, out: torch.Tensor, epilogue: Optional[str] = None) -> torch.Tensor:
+        """out = norm(x)[rows] @ w.T (then the epilogue), by the cheapest route there is."""
+        if self.prepared is not None and self.num_rows <= ops.HANDOFF_MAX_ROWS:
+            operand, sumsq = self.prepared
+            return ops.linear_handoff(operand, w, out, epilogue=epilogue, rows=self.rows,
+                                      prepared=(sumsq, self.eps, self.x.shape[1]))
+        return ops.linear_norm(self.x, self.weight, self.eps, w, out, rows=self.rows, epilogue=epilogue)
 
     @property
     def num_rows(self) -> int:
@@ -46,11 +59,20 @@ class RMSNorm(Norm):
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.weight = tensors[f"{self.prefix}.weight"].contiguous()
 
-    def lazy(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None):
+    def lazy(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None, prepared=None):
         """In bfloat16 the norm rides in the consumer's first product (`ops.linear_norm`)."""
         if self.dtype == torch.bfloat16 and self.hidden_size % 8 == 0:
-            return LazyNorm(self, x, rows)
+            return LazyNorm(self, x, rows, prepared)
         return self.forward(x, rows)
+
+    def hand_off_buffers(self, n_rows: int, device):
+        """(weight, operand, sumsq) for a product that writes this norm's input and can prepare the
+        norm on the way (`ops.linear_handoff`), or None where that does not apply."""
+        if not ops.can_hand_off(n_rows, self.hidden_size, self.dtype):
+            return None
+        operand = torch.empty((n_rows, self.hidden_size), dtype=torch.bfloat16, device=device)
+        sumsq = torch.empty((n_rows, (self.hidden_size + 15) // 16), dtype=torch.float32, device=device)
+        return self.weight, operand, sumsq
 
     def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         n = x.shape[0] if rows is None else rows.numel()
