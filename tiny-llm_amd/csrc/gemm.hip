@@ -513,9 +513,12 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
     row_off[mt] = (int64_t)src * p.lda;
   }
 
-  // row factors of a norm whose sums of squares arrive in parts: one wave per row, fixed order
+  // Row factors of a norm whose sums of squares arrive in parts: one wave per row, fixed order.
+  // Called after the first stage's loads have been issued, so that its own loads queue behind
+  // them instead of holding them up.
   float* scale_s = ss_part + S_WAVES * MT * 16;                      // [MT * 16]
-  if (p.in_sumsq) {
+  auto row_factors = [&]() {
+    if (!p.in_sumsq) return;
     for (int r = wave; r < MT * 16; r += S_WAVES) {
       const int m = min(r, M - 1);
       const int64_t src = p.rows ? p.rows[m] : m;
@@ -524,7 +527,7 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
       t = wave_sum(t);
       if (lane == 0) scale_s[r] = 1.f / sqrtf(t / (float)p.in_width + p.in_eps);
     }
-  }
+  };
 
   // A stage is UN k blocks of 128 (all loads of a stage are issued together).  Where the
   // registers allow, two stages take turns, so the loads of the next stage are in flight while
@@ -595,11 +598,13 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
     }
   };
   constexpr int STEP = S_WAVES * UN;
+  if (wave >= nblk) row_factors();        // a wave without a k block
   if constexpr (TWO_STAGES) {
     Stage s0, s1;
     int blk = wave;
     if (blk < nblk) {
       load(s0, blk);
+      row_factors();
       while (true) {
         const int b1 = blk + STEP;
         if (b1 < nblk) load(s1, b1);
@@ -616,6 +621,7 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
     Stage s0;
     for (int blk = wave; blk < nblk; blk += STEP) {
       load(s0, blk);
+      if (blk == wave) row_factors();
       multiply(s0, blk);
     }
   }
