@@ -258,58 +258,78 @@ __global__ __launch_bounds__(WM * WN * TL_WAVE) void gemm_bf16_kernel(const bf16
     step(std::false_type{}, std::false_type{}, kt);
   }
 
+  // Epilogue.  A lane's accumulators hold four consecutive n of 32 different rows, so stored from
+  // there a row would go out in 16-byte pieces.  Each wave therefore passes its result, 32 rows x
+  // 64 columns at a time, through an LDS area of its own (the operand tiles are no longer read:
+  // the last fragments were fetched before the loop's last barrier) and reads it back row by
+  // row: 16 lanes then cover 256 contiguous bytes of one row, and so do the residual reads.
+  static_assert(S::TN == 64, "the epilogue stages 64 columns per wave");
+  constexpr int E_LD = 68;                 // floats per staged row: 16-byte aligned, conflict-free
+  static_assert((size_t)WM * WN * 32 * E_LD * sizeof(float) <= S::SMEM, "staging areas fit the tile buffers");
+  float* cstage = (float*)smem_raw + wave * (32 * E_LD);
   const bool vec_ok = (N % 4 == 0) && (ldo % 4 == 0);
 #pragma unroll
   for (int i = 0; i < MI; ++i) {
-    const int m = m0 + wm * S::TM + i * 32 + lane % 32;
-    if (m >= M) continue;
-    const float rs = row_scale ? row_scale[m] : 1.f;   // e.g. 1 / rms of a norm left out of the operand
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
+    for (int j = 0; j < NJ; ++j)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int n = n0 + wn * S::TN + j * 32 + q * 8 + (lane / 32) * 4;
-        if (n >= N) continue;
-        float v[4] = {acc[i][j][q * 4 + 0] * rs, acc[i][j][q * 4 + 1] * rs, acc[i][j][q * 4 + 2] * rs,
-                      acc[i][j][q * 4 + 3] * rs};
-        if constexpr (SWIGLU) {   // (gate, up, gate, up) -> two outputs; N is even and n a multiple of 4
-          const int64_t oz = (int64_t)m * ldo + n / 2;
-          if (n + 2 < N) {
-            typedef TO to2 __attribute__((ext_vector_type(2)));
-            to2 sv = {from_f32<TO>(swiglu_pair(v[0], v[1])), from_f32<TO>(swiglu_pair(v[2], v[3]))};
-            if (ldo % 2 == 0) {
-              *(to2*)(out + oz) = sv;
-            } else {
-              out[oz] = sv[0];
-              out[oz + 1] = sv[1];
-            }
+        f32x4 v4 = {acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
+        *(f32x4*)(cstage + (lane % 32) * E_LD + j * 32 + q * 8 + (lane / 32) * 4) = v4;
+      }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int c8 = 0; c8 < 8; ++c8) {
+      const int c = c8 * TL_WAVE + lane;
+      const int r = c / 16, col = (c % 16) * 4;
+      const int m = m0 + wm * S::TM + i * 32 + r, n = n0 + wn * S::TN + col;
+      if (m >= M || n >= N) continue;
+      const f32x4 s4 = *(const f32x4*)(cstage + r * E_LD + col);
+      const float rs = row_scale ? row_scale[m] : 1.f;   // e.g. 1 / rms of a norm left out of the operand
+      float v[4] = {s4[0] * rs, s4[1] * rs, s4[2] * rs, s4[3] * rs};
+      if constexpr (SWIGLU) {   // (gate, up, gate, up) -> two outputs; N is even and n a multiple of 4
+        const int64_t oz = (int64_t)m * ldo + n / 2;
+        if (n + 2 < N) {
+          typedef TO to2 __attribute__((ext_vector_type(2)));
+          to2 sv = {from_f32<TO>(swiglu_pair(v[0], v[1])), from_f32<TO>(swiglu_pair(v[2], v[3]))};
+          if (ldo % 2 == 0) {
+            *(to2*)(out + oz) = sv;
           } else {
-            out[oz] = from_f32<TO>(swiglu_pair(v[0], v[1]));
-          }
-          continue;
-        }
-        const int64_t o = (int64_t)m * ldo + n;
-        if (vec_ok) {  // n + 3 < N because n and N are both multiples of 4
-          if (residual) {
-            const f32x4 r = *(const f32x4*)(residual + o);
-            v[0] += r[0]; v[1] += r[1]; v[2] += r[2]; v[3] += r[3];
-          }
-          if constexpr (sizeof(TO) == 4) {
-            f32x4 sv = {v[0], v[1], v[2], v[3]};
-            *(f32x4*)((float*)out + o) = sv;
-          } else {
-            bf16x4 sv = {(bf16_t)v[0], (bf16_t)v[1], (bf16_t)v[2], (bf16_t)v[3]};
-            *(bf16x4*)((bf16_t*)out + o) = sv;
+            out[oz] = sv[0];
+            out[oz + 1] = sv[1];
           }
         } else {
-          for (int e = 0; e < 4 && n + e < N; ++e) {
-            float x = v[e];
-            if (residual) x += residual[o + e];
-            out[o + e] = from_f32<TO>(x);
-          }
+          out[oz] = from_f32<TO>(swiglu_pair(v[0], v[1]));
+        }
+        continue;
+      }
+      const int64_t o = (int64_t)m * ldo + n;
+      if (vec_ok) {  // n + 3 < N because n and N are both multiples of 4
+        if (residual) {
+          const f32x4 rv = *(const f32x4*)(residual + o);
+          v[0] += rv[0]; v[1] += rv[1]; v[2] += rv[2]; v[3] += rv[3];
+        }
+        if constexpr (sizeof(TO) == 4) {
+          f32x4 sv = {v[0], v[1], v[2], v[3]};
+          *(f32x4*)((float*)out + o) = sv;
+        } else {
+          bf16x4 sv = {(bf16_t)v[0], (bf16_t)v[1], (bf16_t)v[2], (bf16_t)v[3]};
+          *(bf16x4*)((bf16_t*)out + o) = sv;
+        }
+      } else {
+        for (int e = 0; e < 4 && n + e < N; ++e) {
+          float x = v[e];
+          if (residual) x += residual[o + e];
+          out[o + e] = from_f32<TO>(x);
         }
       }
     }
+    // the area is written again for the next 32 rows
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
 }
 
