@@ -580,17 +580,20 @@ __global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
     if (kt_idx * FA_KT <= wave_hi) {
       f32x4 sc[FP_RT][4];
 #pragma unroll
-      for (int kt = 0; kt < 4; ++kt) {
+      for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
         for (int rt = 0; rt < FP_RT; ++rt) sc[rt][kt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      // k steps outermost: consecutive MFMAs then write different accumulators and need not wait
+      // for each other
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
+      for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) {
           const bf16x8 kf = *(const bf16x8*)(Kl + (kt * 16 + r16) * KP + ks * 32 + g * 8);
 #pragma unroll
           for (int rt = 0; rt < FP_RT; ++rt)
             sc[rt][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[rt][ks], sc[rt][kt], 0, 0, 0);
         }
-      }
       bf16x8 pb[FP_RT][2], pl[FP_RT][2];
       const int tile_j0 = kt_idx * FA_KT;
       const bool no_mask = all_valid && tile_j0 + FA_KT - 1 <= wave_lo_pos && tile_j0 >= wave_hi_lo;
@@ -649,6 +652,7 @@ __global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
             pl[rt][st][4 + r] = (bf16_t)(p1 - (float)pb[rt][st][4 + r]);
           }
       }
+      bf16x8 vfr[2][HDT];
 #pragma unroll
       for (int st = 0; st < 2; ++st)
 #pragma unroll
@@ -662,12 +666,19 @@ __global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
             vf[r] = lo4[r];
             vf[4 + r] = hi4[r];
           }
-#pragma unroll
-          for (int rt = 0; rt < FP_RT; ++rt) {
-            o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb[rt][st], o[rt][dt], 0, 0, 0);
-            o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pl[rt][st], o[rt][dt], 0, 0, 0);
-          }
+          vfr[st][dt] = vf;
         }
+      // the four products into one accumulator are kept four MFMAs apart
+#pragma unroll
+      for (int st = 0; st < 2; ++st)
+#pragma unroll
+        for (int lo = 0; lo < 2; ++lo)
+#pragma unroll
+          for (int dt = 0; dt < HDT; ++dt)
+#pragma unroll
+            for (int rt = 0; rt < FP_RT; ++rt)
+              o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vfr[st][dt], lo ? pl[rt][st] : pb[rt][st], o[rt][dt],
+                                                                  0, 0, 0);
     }
     __syncthreads();
   }
