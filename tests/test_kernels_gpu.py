@@ -122,6 +122,35 @@ def test_linear_sizes(dtype, M, K, N):
     assert rel(x, ref + res.double()) < 1e-5
 
 
+@pytest.mark.parametrize("tile", [1, 2, 3, 4])
+@pytest.mark.parametrize("M,K,N", [(65, 64, 2), (257, 200, 258), (300, 72, 516), (513, 136, 130), (256, 128, 512),
+                                   (130, 1096, 700)])
+def test_linear_every_tile(tile, M, K, N):
+    """Each tile shape of the bfloat16 product on sizes that end inside a tile (rows, columns and
+    inner size), with every epilogue: by size alone the large tiles are only chosen for large,
+    regular products."""
+    g = torch.Generator().manual_seed(tile * 100 + M + N)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    res = torch.randn(M, N, generator=g)
+    scale = torch.rand(M, generator=g) + 0.5
+    ref = a.double() @ w.double().T
+    out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops().linear(a.to(DEV), w.to(DEV), out, tile=tile)
+    assert rel(out, ref) < 6e-3
+    x = res.clone().to(DEV)
+    ops().linear(a.to(DEV), w.to(DEV), x, x, row_scale=scale.to(DEV), tile=tile)
+    assert rel(x, ref * scale.double()[:, None] + res.double()) < 1e-5
+    z = torch.full((M, N // 2), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops().linear(a.to(DEV), w[:N // 2 * 2].contiguous().to(DEV), z, epilogue="swiglu", tile=tile)
+    assert rel(z, plain.silu(ref[:, 0:N // 2 * 2:2]) * ref[:, 1:N // 2 * 2:2]) < 6e-3
+    # a view with a row stride of its own, as the q columns of a qkv buffer
+    wide = torch.zeros(M, N + 24, dtype=torch.bfloat16, device=DEV)
+    ops().linear(a.to(DEV), w.to(DEV), wide[:, 8:8 + N] if N % 8 == 0 else wide[:, :N], tile=tile)
+    assert rel(wide[:, 8:8 + N] if N % 8 == 0 else wide[:, :N], ref) < 6e-3
+    assert float(wide[:, N + 8:].abs().sum()) == 0.0
+
+
 @pytest.mark.parametrize("M", [1, 5, 16, 17, 40, 64, 65, 200])
 @pytest.mark.parametrize("K,N", [(64, 251), (2048, 96), (176, 64), (5632, 40), (96, 516)])
 def test_linear_norm(M, K, N):

@@ -369,7 +369,7 @@ static int launch_gemm_bf16(const bf16_t* a, const bf16_t* w, TO* out, const flo
 template <typename TO, bool SWIGLU>
 static int launch_gemm_bf16_any(const bf16_t* a, const bf16_t* w, TO* out, const float* residual,
                                 const float* row_scale, int M, int N, int K, int64_t lda, int64_t ldo,
-                                hipStream_t stream) {
+                                int tile, hipStream_t stream) {
   struct Choice {
     int bm, bn;
     double rate;
@@ -385,6 +385,7 @@ static int launch_gemm_bf16_any(const bf16_t* a, const bf16_t* w, TO* out, const
       best_cost = cost;
     }
   }
+  if (tile >= 1 && tile <= 4) best = tile - 1;     // the caller's choice (tests, tuning)
   switch (best) {
     case 0:
       return launch_gemm_bf16<256, 256, 2, 4, TO, SWIGLU>(a, w, out, residual, row_scale, M, N, K, lda, ldo, stream);
@@ -767,13 +768,16 @@ extern "C" {
 // epilogue 0: (+ residual[m, n]), out is [M, N].
 // epilogue 1: SiLU-gate of interleaved columns, out[m, j] = silu(c[m, 2j]) * c[m, 2j+1], out is
 //             [M, N/2] of the input's type; N must be even; no residual.
-int tl_linear(const void* a, const void* w, void* out, const float* residual, const float* row_scale, int M,
-              int N, int K, int64_t lda, int64_t ldo, int dtype, int out_dtype, int epilogue,
-              hipStream_t stream) {
+// tile (bfloat16, M > 64): 0 lets the size decide; 1..4 force 256x256, 256x128, 128x128, 64x128.
+int tl_linear_tile(const void* a, const void* w, void* out, const float* residual, const float* row_scale, int M,
+                   int N, int K, int64_t lda, int64_t ldo, int dtype, int out_dtype, int epilogue, int tile,
+                   hipStream_t stream) {
   if (M <= 0) return TL_OK;
   if (row_scale && dtype != 1) return TL_ERR_ARG;   // only the bfloat16 kernels scale rows
   const bool swiglu = epilogue == 1;
-  if (N <= 0 || K <= 0 || lda < K || ldo < (swiglu ? N / 2 : N) || epilogue < 0 || epilogue > 1) return TL_ERR_ARG;
+  if (N <= 0 || K <= 0 || lda < K || ldo < (swiglu ? N / 2 : N) || epilogue < 0 || epilogue > 1 || tile < 0 ||
+      tile > 4)
+    return TL_ERR_ARG;
   if (swiglu && ((N & 1) || residual || out_dtype != dtype)) return TL_ERR_ARG;
   if (dtype == 0) {
     if (out_dtype != 0) return TL_ERR_ARG;
@@ -795,19 +799,25 @@ int tl_linear(const void* a, const void* w, void* out, const float* residual, co
       int rc;
       if (swiglu)
         rc = launch_gemm_bf16_any<bf16_t, true>((const bf16_t*)a, (const bf16_t*)w, (bf16_t*)out, residual, row_scale,
-                                                M, N, K, lda, ldo, stream);
+                                                M, N, K, lda, ldo, tile, stream);
       else if (out_dtype == 0)
         rc = launch_gemm_bf16_any<float, false>((const bf16_t*)a, (const bf16_t*)w, (float*)out, residual, row_scale,
-                                                M, N, K, lda, ldo, stream);
+                                                M, N, K, lda, ldo, tile, stream);
       else
         rc = launch_gemm_bf16_any<bf16_t, false>((const bf16_t*)a, (const bf16_t*)w, (bf16_t*)out, residual,
-                                                 row_scale, M, N, K, lda, ldo, stream);
+                                                 row_scale, M, N, K, lda, ldo, tile, stream);
       if (rc != TL_OK) return rc;
     }
   } else {
     return TL_ERR_ARG;
   }
   return tl_launch_status();
+}
+
+int tl_linear(const void* a, const void* w, void* out, const float* residual, const float* row_scale, int M,
+              int N, int K, int64_t lda, int64_t ldo, int dtype, int out_dtype, int epilogue,
+              hipStream_t stream) {
+  return tl_linear_tile(a, w, out, residual, row_scale, M, N, K, lda, ldo, dtype, out_dtype, epilogue, 0, stream);
 }
 
 // Few-row (M <= 64) bfloat16 product that takes part in handing a norm from one product to the

@@ -106,11 +106,13 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor
 
 
 def linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, residual: Optional[torch.Tensor] = None,
-           epilogue: Optional[str] = None, row_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+           epilogue: Optional[str] = None, row_scale: Optional[torch.Tensor] = None, tile: int = 0) -> torch.Tensor:
     """out = a @ w.T (+ residual).  a [M, K], w [N, K] share an element type; out [M, N] is that
     type or float32; residual float32 with out's strides.  epilogue="swiglu": the N columns are
     interleaved (gate_j, up_j) pairs and out [M, N/2] = silu(gate) * up, computed from the float32
-    accumulators.  row_scale [M] multiplies the rows of the product first (bfloat16 only)."""
+    accumulators.  row_scale [M] multiplies the rows of the product first (bfloat16 only).
+    tile: 0 lets the sizes choose the tile of the bfloat16 product for more than 64 rows; 1 to 4
+    force 256x256, 256x128, 128x128, 64x128 (tests and tuning)."""
     _dev(a, w, out, residual)
     _rows_2d(a, "linear input")
     _rows_2d(out, "linear output")
@@ -137,9 +139,10 @@ def linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, residual: Option
     if row_scale is not None:
         _need(dt == 1 and row_scale.dtype == torch.float32 and row_scale.is_contiguous()
               and row_scale.numel() == M, "row scales go with the bfloat16 product: float32, one per row")
-    _check(_lib().tl_linear(_ptr(a, al), _ptr(w, al), _ptr(out, ao), _ptr(residual, ao), _ptr(row_scale), c_int(M),
-                            c_int(N), c_int(K), c_int64(a.stride(0)), c_int64(out.stride(0)), c_int(dt), c_int(odt),
-                            c_int(swiglu), _stream()), "linear")
+    _need(0 <= tile <= 4, "tile is 0 (by size) or 1 to 4")
+    _check(_lib().tl_linear_tile(_ptr(a, al), _ptr(w, al), _ptr(out, ao), _ptr(residual, ao), _ptr(row_scale),
+                                 c_int(M), c_int(N), c_int(K), c_int64(a.stride(0)), c_int64(out.stride(0)), c_int(dt),
+                                 c_int(odt), c_int(swiglu), c_int(tile), _stream()), "linear")
     return out
 
 
