@@ -201,7 +201,7 @@ def test_linear_handoff(M, K, N, N2):
         nw = (1 + 0.1 * torch.randn(N, generator=g)).to(nwt)
         x = res.clone().to(DEV)
         operand = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
-        sumsq = torch.full((M, (N + 15) // 16), float("nan"), dtype=torch.float32, device=DEV)
+        sumsq = torch.full((M, ops().handoff_parts(M, N, K)), float("nan"), dtype=torch.float32, device=DEV)
         ops().linear_handoff(z.to(DEV), w1.to(DEV), x, x, emit=(nw.to(DEV), operand, sumsq))
         assert rel(x, x_ref) < 1e-5
         xs = x.cpu().double()
@@ -223,9 +223,60 @@ def test_linear_handoff(M, K, N, N2):
         zz = torch.empty(M, N2 // 2, dtype=torch.bfloat16, device=DEV)
         ops().linear_handoff(operand, w2.to(DEV), zz, epilogue="swiglu", prepared=(sumsq, 1e-5, N))
         assert rel(zz, plain.silu(c[:, 0::2]) * c[:, 1::2]) < 6e-3
-    with pytest.raises(Exception):
-        ops().linear_handoff(torch.zeros(65, K, dtype=torch.bfloat16, device=DEV), w1.to(DEV),
-                             torch.empty(65, N, dtype=torch.float32, device=DEV))
+    with pytest.raises(Exception):      # a gather of more rows than the few-row product takes
+        ops().linear_handoff(torch.zeros(80, K, dtype=torch.bfloat16, device=DEV), w1.to(DEV),
+                             torch.empty(65, N, dtype=torch.float32, device=DEV),
+                             rows=torch.arange(65, dtype=torch.int32, device=DEV))
+
+
+@pytest.mark.parametrize("M", [17, 64, 65, 200, 512])
+@pytest.mark.parametrize("K,N", [(5632, 2048), (2048, 4100), (1096, 518)])
+def test_linear_split_k(M, K, N):
+    """Products with few output tiles split their inner size over workgroups and add the parts up
+    in a second kernel, which also applies every epilogue and both sides of the norm hand-off."""
+    g = torch.Generator().manual_seed(M + K + N)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    res = torch.randn(M, N, generator=g)
+    scale = torch.rand(M, generator=g) + 0.5
+    ref = a.double() @ w.double().T
+    splits = ops().split_k(M, N, K)
+    if M > 64 or N * K >= (8 << 20):
+        assert splits > 1                     # these sizes are here because they are split
+    out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops().linear(a.to(DEV), w.to(DEV), out)
+    assert rel(out, ref) < 6e-3
+    x = res.clone().to(DEV)
+    ops().linear(a.to(DEV), w.to(DEV), x, x, row_scale=scale.to(DEV))
+    assert rel(x, ref * scale.double()[:, None] + res.double()) < 1e-5
+    z = torch.full((M, N // 2), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops().linear(a.to(DEV), w.to(DEV), z, epilogue="swiglu")
+    assert rel(z, plain.silu(ref[:, 0::2]) * ref[:, 1::2]) < 6e-3
+    y = torch.empty(M, N, dtype=torch.float32, device=DEV)
+    ops().linear(a.to(DEV), w.to(DEV), y)
+    assert rel(y, ref) < 1e-5
+    y2 = torch.empty(M, N, dtype=torch.float32, device=DEV)
+    ops().linear(a.to(DEV), w.to(DEV), y2)
+    assert torch.equal(y, y2)                 # the parts are added in a fixed order
+    if not ops().can_hand_off(M, N, K, torch.bfloat16) or N % 8:
+        return
+    # producer side of the norm hand-off, then a consumer
+    nw = 1 + 0.1 * torch.randn(N, generator=g)
+    x = res.clone().to(DEV)
+    operand = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    sumsq = torch.full((M, ops().handoff_parts(M, N, K)), float("nan"), dtype=torch.float32, device=DEV)
+    ops().linear_handoff(a.to(DEV), w.to(DEV), x, x, emit=(nw.to(DEV), operand, sumsq))
+    assert rel(x, ref + res.double()) < 1e-5
+    xs = x.cpu().double()
+    assert torch.equal(operand.cpu(), (nw * x.cpu()).to(torch.bfloat16))
+    assert rel(sumsq.sum(dim=1), (xs * xs).sum(dim=1)) < 1e-6
+    w2 = (torch.randn(5000, N, generator=g) / math.sqrt(N)).to(torch.bfloat16)
+    inv = 1.0 / torch.sqrt((xs * xs).mean(dim=-1, keepdim=True) + 1e-5)
+    c = (operand.cpu().double() @ w2.double().T) * inv
+    if M <= 64 or ops().split_k(M, 5000, N) > 1:
+        zz = torch.empty(M, 2500, dtype=torch.bfloat16, device=DEV)
+        ops().linear_handoff(operand, w2.to(DEV), zz, epilogue="swiglu", prepared=(sumsq, 1e-5, N))
+        assert rel(zz, plain.silu(c[:, 0::2]) * c[:, 1::2]) < 6e-3
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

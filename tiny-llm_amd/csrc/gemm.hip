@@ -125,7 +125,8 @@ __global__ __launch_bounds__(WM * WN * TL_WAVE) void gemm_bf16_kernel(const bf16
                                                                       TO* __restrict__ out,
                                                                       const float* __restrict__ residual,
                                                                       const float* __restrict__ row_scale, int M,
-                                                                      int N, int K, int64_t lda, int64_t ldo) {
+                                                                      int N, int K, int64_t lda, int64_t ldo,
+                                                                      int k_per_split) {
   using S = GemmShape<BM, BN, WM, WN>;
   constexpr int MI = S::MI, NJ = S::NJ, THREADS = S::THREADS;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -133,11 +134,19 @@ __global__ __launch_bounds__(WM * WN * TL_WAVE) void gemm_bf16_kernel(const bf16
   bf16_t* Ws = As + 2 * BM * B_LD;                      // [2][BN][B_LD]
   const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
   const int wm = wave / WN, wn = wave % WN;
-  const int tiles_m = (M + BM - 1) / BM, total = tiles_m * ((N + BN - 1) / BN);
+  // k_per_split > 0 (a multiple of the k step): the inner size is split over workgroups, each
+  // writing its float32 partial product [M, N] behind `out` (no epilogue); a second kernel adds
+  // them up.  That is how products with few output tiles still fill the chip.
+  const int splits = k_per_split > 0 ? (K + k_per_split - 1) / k_per_split : 1;
+  const int tiles_m = (M + BM - 1) / BM, tiles = tiles_m * ((N + BN - 1) / BN), total = tiles * splits;
   const int per_xcd = (total + B_XCDS - 1) / B_XCDS;
-  const int t = (blockIdx.x % B_XCDS) * per_xcd + blockIdx.x / B_XCDS;
-  if (t >= total) return;                               // the grid is padded to a multiple of 8
+  const int t_all = (blockIdx.x % B_XCDS) * per_xcd + blockIdx.x / B_XCDS;
+  if (t_all >= total) return;                           // the grid is padded to a multiple of 8
+  const int split = t_all / tiles, t = t_all % tiles;
   const int m0 = (t % tiles_m) * BM, n0 = (t / tiles_m) * BN;
+  const int kbase = split * k_per_split;
+  const int kend = k_per_split > 0 ? min(K, kbase + k_per_split) : K;
+  if (k_per_split > 0) out += (int64_t)split * M * ldo;
 
   f32x16 acc[MI][NJ];
 #pragma unroll
@@ -212,14 +221,14 @@ __global__ __launch_bounds__(WM * WN * TL_WAVE) void gemm_bf16_kernel(const bf16
   // kt - 1) is written to the other LDS buffer in the middle of step kt, and the loads of tile
   // kt + 2 are issued right after; the last k16 step of a tile is multiplied after the barrier,
   // while the first fragments of the next tile are on their way.
-  const int nk = (K + B_BK - 1) / B_BK;
+  const int nk = (kend - kbase + B_BK - 1) / B_BK;
 #pragma unroll
-  for (int p = 0; p < PIECES; ++p) gload1(0, p);
+  for (int p = 0; p < PIECES; ++p) gload1(kbase, p);
 #pragma unroll
-  for (int p = 0; p < PIECES; ++p) lds_write1(0, 0, p);
+  for (int p = 0; p < PIECES; ++p) lds_write1(0, kbase, p);
   if (nk > 1) {
 #pragma unroll
-    for (int p = 0; p < PIECES; ++p) gload1(B_BK, p);
+    for (int p = 0; p < PIECES; ++p) gload1(kbase + B_BK, p);
   }
   __syncthreads();
   Frag f0, f1;
@@ -229,7 +238,7 @@ __global__ __launch_bounds__(WM * WN * TL_WAVE) void gemm_bf16_kernel(const bf16
   constexpr int HALF = SLOTS / 2;
   auto step = [&](auto has_next, auto has_next2, int kt) {
     constexpr bool NX = decltype(has_next)::value, NX2 = decltype(has_next2)::value;
-    const int cur = kt & 1, nxt = cur ^ 1, k1 = (kt + 1) * B_BK, k2 = (kt + 2) * B_BK;
+    const int cur = kt & 1, nxt = cur ^ 1, k1 = kbase + (kt + 1) * B_BK, k2 = kbase + (kt + 2) * B_BK;
     group(f0, [&](int n) { spread(n, FRAG, SLOTS, [&](int p) { lds_read1(f1, cur, 1, p); }); });
     group(f1, [&](int n) {
       spread(n, FRAG, SLOTS, [&](int p) { lds_read1(f0, cur, 2, p); });
@@ -336,7 +345,7 @@ __global__ __launch_bounds__(WM * WN * TL_WAVE) void gemm_bf16_kernel(const bf16
 template <int BM, int BN, int WM, int WN, typename TO, bool SWIGLU, bool FULL>
 static int launch_gemm_bf16_full(const bf16_t* a, const bf16_t* w, TO* out, const float* residual,
                                  const float* row_scale, int M, int N, int K, int64_t lda, int64_t ldo,
-                                 hipStream_t stream) {
+                                 int k_per_split, hipStream_t stream) {
   using S = GemmShape<BM, BN, WM, WN>;
   static bool configured = false;
   if (!configured) {
@@ -345,22 +354,23 @@ static int launch_gemm_bf16_full(const bf16_t* a, const bf16_t* w, TO* out, cons
       return TL_ERR_LAUNCH;
     configured = true;
   }
-  const int64_t total = (int64_t)((N + BN - 1) / BN) * ((M + BM - 1) / BM);
+  const int64_t splits = k_per_split > 0 ? (K + k_per_split - 1) / k_per_split : 1;
+  const int64_t total = (int64_t)((N + BN - 1) / BN) * ((M + BM - 1) / BM) * splits;
   const int64_t grid = (total + B_XCDS - 1) / B_XCDS * B_XCDS;
   if (grid > 0x7fffffff) return TL_ERR_ARG;
   hipLaunchKernelGGL((gemm_bf16_kernel<BM, BN, WM, WN, TO, SWIGLU, FULL>), dim3((unsigned)grid), dim3(S::THREADS),
-                     S::SMEM, stream, a, w, out, residual, row_scale, M, N, K, lda, ldo);
+                     S::SMEM, stream, a, w, out, residual, row_scale, M, N, K, lda, ldo, k_per_split);
   return TL_OK;
 }
 
 template <int BM, int BN, int WM, int WN, typename TO, bool SWIGLU>
 static int launch_gemm_bf16(const bf16_t* a, const bf16_t* w, TO* out, const float* residual, const float* row_scale,
-                            int M, int N, int K, int64_t lda, int64_t ldo, hipStream_t stream) {
+                            int M, int N, int K, int64_t lda, int64_t ldo, int k_per_split, hipStream_t stream) {
   if (M % BM == 0 && N % BN == 0 && K % B_BK == 0)
     return launch_gemm_bf16_full<BM, BN, WM, WN, TO, SWIGLU, true>(a, w, out, residual, row_scale, M, N, K, lda, ldo,
-                                                                   stream);
+                                                                   k_per_split, stream);
   return launch_gemm_bf16_full<BM, BN, WM, WN, TO, SWIGLU, false>(a, w, out, residual, row_scale, M, N, K, lda, ldo,
-                                                                  stream);
+                                                                  k_per_split, stream);
 }
 
 // Which tile: the one with the smallest estimated time.  A compute unit works through
@@ -369,7 +379,7 @@ static int launch_gemm_bf16(const bf16_t* a, const bf16_t* w, TO* out, const flo
 template <typename TO, bool SWIGLU>
 static int launch_gemm_bf16_any(const bf16_t* a, const bf16_t* w, TO* out, const float* residual,
                                 const float* row_scale, int M, int N, int K, int64_t lda, int64_t ldo,
-                                int tile, hipStream_t stream) {
+                                int tile, int k_per_split, hipStream_t stream) {
   struct Choice {
     int bm, bn;
     double rate;
@@ -388,14 +398,117 @@ static int launch_gemm_bf16_any(const bf16_t* a, const bf16_t* w, TO* out, const
   if (tile >= 1 && tile <= 4) best = tile - 1;     // the caller's choice (tests, tuning)
   switch (best) {
     case 0:
-      return launch_gemm_bf16<256, 256, 2, 4, TO, SWIGLU>(a, w, out, residual, row_scale, M, N, K, lda, ldo, stream);
+      return launch_gemm_bf16<256, 256, 2, 4, TO, SWIGLU>(a, w, out, residual, row_scale, M, N, K, lda, ldo, k_per_split,
+                                                          stream);
     case 1:
-      return launch_gemm_bf16<256, 128, 4, 2, TO, SWIGLU>(a, w, out, residual, row_scale, M, N, K, lda, ldo, stream);
+      return launch_gemm_bf16<256, 128, 4, 2, TO, SWIGLU>(a, w, out, residual, row_scale, M, N, K, lda, ldo, k_per_split,
+                                                          stream);
     case 2:
-      return launch_gemm_bf16<128, 128, 2, 2, TO, SWIGLU>(a, w, out, residual, row_scale, M, N, K, lda, ldo, stream);
+      return launch_gemm_bf16<128, 128, 2, 2, TO, SWIGLU>(a, w, out, residual, row_scale, M, N, K, lda, ldo, k_per_split,
+                                                          stream);
     default:
-      return launch_gemm_bf16<64, 128, 2, 2, TO, SWIGLU>(a, w, out, residual, row_scale, M, N, K, lda, ldo, stream);
+      return launch_gemm_bf16<64, 128, 2, 2, TO, SWIGLU>(a, w, out, residual, row_scale, M, N, K, lda, ldo, k_per_split,
+                                                          stream);
   }
+}
+
+// ------------------------------------------------------------ split k: the second kernel
+// Adds up the partial products [splits, M, N] of a product whose inner size was split over
+// workgroups and applies what the product's own epilogue would have: row factor (given, or from
+// sums of squares handed over by the producer of the input), residual, SiLU-gate, output type; it
+// can also prepare the next norm (operand and sums of squares per chunk of 1024 columns).  One
+// workgroup per (row, chunk of 1024 columns), four consecutive columns per thread.
+constexpr int R_THREADS = 256, R_CHUNK = R_THREADS * 4;
+
+struct ReduceArgs {
+  const float* partial;
+  int splits, M, N;
+  void* out;
+  int64_t ldo;
+  const float* residual;
+  const float* row_scale;
+  const float* in_sumsq;
+  int in_parts, in_width;
+  float in_eps;
+  const void* emit_w;
+  int emit_w_is_f32;
+  bf16_t* emit_operand;
+  float* emit_sumsq;
+};
+
+template <typename TO, bool SWIGLU>
+__global__ __launch_bounds__(R_THREADS) void splitk_reduce_kernel(const ReduceArgs p) {
+  __shared__ float red[R_THREADS / TL_WAVE];
+  const int m = blockIdx.x, tid = threadIdx.x;
+  const int n = blockIdx.y * R_CHUNK + tid * 4;
+  const int N = p.N;
+  float scale = p.row_scale ? p.row_scale[m] : 1.f;
+  if (p.in_sumsq) {
+    float t = 0.f;
+    for (int q = tid; q < p.in_parts; q += R_THREADS) t += p.in_sumsq[(int64_t)m * p.in_parts + q];
+    t = block_sum<R_THREADS / TL_WAVE>(t, red);
+    scale = 1.f / sqrtf(t / (float)p.in_width + p.in_eps);
+  }
+  const bool vec = (N % 4 == 0);
+  float v[4] = {0.f, 0.f, 0.f, 0.f};
+  if (n < N) {
+    for (int sp = 0; sp < p.splits; ++sp) {
+      const float* src = p.partial + ((int64_t)sp * p.M + m) * N + n;
+      if (vec) {
+        const f32x4 x = *(const f32x4*)src;
+        v[0] += x[0]; v[1] += x[1]; v[2] += x[2]; v[3] += x[3];
+      } else {
+        for (int e = 0; e < 4 && n + e < N; ++e) v[e] += src[e];
+      }
+    }
+  }
+  TO* out = (TO*)p.out;
+  float sq = 0.f;
+  if (n < N) {
+    if constexpr (SWIGLU) {   // (gate, up, gate, up) -> two outputs; N is even and n a multiple of 4
+      out[(int64_t)m * p.ldo + n / 2] = from_f32<TO>(swiglu_pair(v[0] * scale, v[1] * scale));
+      if (n + 2 < N) out[(int64_t)m * p.ldo + n / 2 + 1] = from_f32<TO>(swiglu_pair(v[2] * scale, v[3] * scale));
+    } else {
+      for (int e = 0; e < 4 && n + e < N; ++e) {
+        float x = v[e] * scale;
+        const int64_t o = (int64_t)m * p.ldo + n + e;
+        if (p.residual) x += p.residual[o];
+        out[o] = from_f32<TO>(x);
+        if (p.emit_operand) {
+          const float wn = p.emit_w_is_f32 ? ((const float*)p.emit_w)[n + e] : (float)((const bf16_t*)p.emit_w)[n + e];
+          p.emit_operand[(int64_t)m * N + n + e] = (bf16_t)(wn * x);
+          sq += x * x;
+        }
+      }
+    }
+  }
+  if (p.emit_operand) {       // uniform
+    sq = block_sum<R_THREADS / TL_WAVE>(sq, red);
+    if (tid == 0) p.emit_sumsq[(int64_t)m * gridDim.y + blockIdx.y] = sq;
+  }
+}
+
+// How a bfloat16 product of these sizes is best split: returns the number of splits (1: not at
+// all) and sets the tile (as tl_linear_tile's) and the inner size per split.  Splitting pays when
+// the output has too few tiles to fill 256 compute units and the rows are too many for the
+// few-row kernel to stream the weights at full rate.
+static int splitk_plan(int M, int N, int K, int* tile, int* k_per_split) {
+  *tile = 0;
+  *k_per_split = 0;
+  if (M <= 16 || K < 8 * B_BK) return 1;
+  const int bm = M <= 64 ? 64 : 128, bn = 128;
+  const int64_t wgs = (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+  if (wgs >= 160) return 1;
+  if (M <= 64 && (int64_t)N * K < (int64_t)8 << 20) return 1;      // small weights: the few-row kernel is faster
+  const int nk = (K + B_BK - 1) / B_BK;
+  const int want = (int)((256 + wgs - 1) / wgs);
+  int per = (nk + want - 1) / want;
+  if (per < 4) per = 4;
+  const int splits = (nk + per - 1) / per;
+  if (splits < 2) return 1;
+  *tile = M <= 64 ? 4 : 3;
+  *k_per_split = per * B_BK;
+  return splits;
 }
 
 // ============================================================ bfloat16, few rows
@@ -799,13 +912,13 @@ int tl_linear_tile(const void* a, const void* w, void* out, const float* residua
       int rc;
       if (swiglu)
         rc = launch_gemm_bf16_any<bf16_t, true>((const bf16_t*)a, (const bf16_t*)w, (bf16_t*)out, residual, row_scale,
-                                                M, N, K, lda, ldo, tile, stream);
+                                                M, N, K, lda, ldo, tile, 0, stream);
       else if (out_dtype == 0)
         rc = launch_gemm_bf16_any<float, false>((const bf16_t*)a, (const bf16_t*)w, (float*)out, residual, row_scale,
-                                                M, N, K, lda, ldo, tile, stream);
+                                                M, N, K, lda, ldo, tile, 0, stream);
       else
         rc = launch_gemm_bf16_any<bf16_t, false>((const bf16_t*)a, (const bf16_t*)w, (bf16_t*)out, residual,
-                                                 row_scale, M, N, K, lda, ldo, tile, stream);
+                                                 row_scale, M, N, K, lda, ldo, tile, 0, stream);
       if (rc != TL_OK) return rc;
     }
   } else {
@@ -854,6 +967,49 @@ int tl_linear_handoff(const void* a, const void* w, void* out, const float* resi
   }
   const int rc = launch_skinny_out<PRO_NONE>(p, out_dtype, swiglu, stream);
   if (rc != TL_OK) return rc;
+  return tl_launch_status();
+}
+
+// See splitk_plan.  A caller that gets more than one split allocates a float32 workspace of
+// splits * M * N elements and calls tl_linear_splitk with the same sizes.
+int tl_splitk_plan(int M, int N, int K) {
+  int tile, kps;
+  return splitk_plan(M, N, K, &tile, &kps);
+}
+
+// The bfloat16 product with its inner size split over workgroups: partial products into
+// `workspace` (float32 [splits, M, N], splits as tl_splitk_plan says), then one kernel that adds
+// them up and applies the epilogue.  Arguments as tl_linear and tl_linear_handoff (no row gather);
+// emit_sumsq is float [M, ceil(N / 1024)].
+int tl_linear_splitk(const void* a, const void* w, void* out, const float* residual, const float* row_scale,
+                     const float* in_sumsq, int in_parts, float in_eps, int in_width, const void* emit_w,
+                     int emit_w_dtype, void* emit_operand, float* emit_sumsq, int M, int N, int K, int64_t lda,
+                     int64_t ldo, int out_dtype, int epilogue, float* workspace, hipStream_t stream) {
+  const bool swiglu = epilogue == 1;
+  if (M <= 0 || N <= 0 || K <= 0 || K % 8 || lda % 8 || lda < K || ldo < (swiglu ? N / 2 : N) || epilogue < 0 ||
+      epilogue > 1 || (out_dtype != 0 && out_dtype != 1) || !workspace)
+    return TL_ERR_ARG;
+  if (swiglu && ((N & 1) || residual || out_dtype != 1)) return TL_ERR_ARG;
+  if (in_sumsq && (in_parts <= 0 || in_width <= 0)) return TL_ERR_ARG;
+  const bool emit = emit_operand != nullptr;
+  if (emit && (!emit_w || !emit_sumsq || swiglu || out_dtype != 0 || (emit_w_dtype != 0 && emit_w_dtype != 1)))
+    return TL_ERR_ARG;
+  int tile, kps;
+  const int splits = splitk_plan(M, N, K, &tile, &kps);
+  if (splits < 2) return TL_ERR_ARG;
+  int rc = launch_gemm_bf16_any<float, false>((const bf16_t*)a, (const bf16_t*)w, workspace, nullptr, nullptr, M, N, K,
+                                              lda, N, tile, kps, stream);
+  if (rc != TL_OK) return rc;
+  ReduceArgs p{workspace, splits, M, N, out, ldo, residual, row_scale, in_sumsq, in_parts, in_width, in_eps, emit_w,
+               emit_w_dtype == 0 ? 1 : 0, (bf16_t*)emit_operand, emit_sumsq};
+  if (M > 65535) return TL_ERR_ARG;
+  dim3 g(M, (N + R_CHUNK - 1) / R_CHUNK), b(R_THREADS);
+  if (swiglu)
+    hipLaunchKernelGGL((splitk_reduce_kernel<bf16_t, true>), g, b, 0, stream, p);
+  else if (out_dtype == 0)
+    hipLaunchKernelGGL((splitk_reduce_kernel<float, false>), g, b, 0, stream, p);
+  else
+    hipLaunchKernelGGL((splitk_reduce_kernel<bf16_t, false>), g, b, 0, stream, p);
   return tl_launch_status();
 }
 

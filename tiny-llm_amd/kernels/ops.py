@@ -140,6 +140,10 @@ def linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, residual: Option
         _need(dt == 1 and row_scale.dtype == torch.float32 and row_scale.is_contiguous()
               and row_scale.numel() == M, "row scales go with the bfloat16 product: float32, one per row")
     _need(0 <= tile <= 4, "tile is 0 (by size) or 1 to 4")
+    if dt == 1 and tile == 0 and M > 16:
+        splits = split_k(M, N, K)
+        if splits > 1:
+            return _linear_split(a, w, out, residual, swiglu, row_scale, None, 0, 0.0, 0, None, splits)
     _check(_lib().tl_linear_tile(_ptr(a, al), _ptr(w, al), _ptr(out, ao), _ptr(residual, ao), _ptr(row_scale),
                                  c_int(M), c_int(N), c_int(K), c_int64(a.stride(0)), c_int64(out.stride(0)), c_int(dt),
                                  c_int(odt), c_int(swiglu), c_int(tile), _stream()), "linear")
@@ -200,24 +204,60 @@ def linear_norm(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: torch
                                  _stream()), "linear_norm")
     return out
 
-HANDOFF_MAX_ROWS = 64   # most rows for which a product can hand a norm to the next one
+FEW_ROWS = 64   # most rows the few-row product takes
 
 
-def can_hand_off(rows: int, width: int, dtype: torch.dtype) -> bool:
-    """Whether `linear_handoff` can prepare a norm over `width` columns for `rows` rows."""
-    return dtype == torch.bfloat16 and 0 < rows <= HANDOFF_MAX_ROWS and width % 8 == 0
+def split_k(rows: int, cols: int, inner: int) -> int:
+    """Into how many parts the bfloat16 product [rows, inner] x [cols, inner]^T has its inner size
+    split over workgroups (1: not at all): products with few output tiles and more rows than the
+    few-row kernel likes."""
+    if inner % 8:
+        return 1
+    return int(_lib().tl_splitk_plan(c_int(rows), c_int(cols), c_int(inner)))
+
+
+def can_hand_off(rows: int, width: int, inner: int, dtype: torch.dtype) -> bool:
+    """Whether `linear_handoff` can prepare a norm over `width` columns for `rows` rows, as the
+    epilogue of the product with inner size `inner`."""
+    if dtype != torch.bfloat16 or rows <= 0 or width % 8 or inner % 8:
+        return False
+    return rows <= FEW_ROWS or split_k(rows, width, inner) > 1
+
+
+def handoff_parts(rows: int, width: int, inner: int) -> int:
+    """How many partial sums of squares per row the product [rows, inner] x [width, inner]^T writes
+    when it prepares a norm: per 16 columns in the few-row kernel, per 1024 after a split inner size."""
+    if split_k(rows, width, inner) > 1:
+        return (width + 1023) // 1024
+    _need(rows <= FEW_ROWS, f"without a split inner size a norm is prepared for at most {FEW_ROWS} rows")
+    return (width + 15) // 16
+
+
+def _linear_split(a, w, out, residual, swiglu, row_scale, sumsq_in, parts, eps, width, emit, splits) -> torch.Tensor:
+    """Partial products into a workspace, then one kernel that adds them and applies the epilogue."""
+    M, K = a.shape
+    N = w.shape[0]
+    work = torch.empty(splits * M * N, dtype=torch.float32, device=a.device)
+    emit_w, emit_op, emit_sq = emit if emit is not None else (None, None, None)
+    _check(_lib().tl_linear_splitk(
+        _ptr(a, 16), _ptr(w, 16), _ptr(out), _ptr(residual), _ptr(row_scale), _ptr(sumsq_in), c_int(parts),
+        c_float(eps), c_int(width), _ptr(emit_w), c_int(_dt(emit_w) if emit_w is not None else 0), _ptr(emit_op),
+        _ptr(emit_sq), c_int(M), c_int(N), c_int(K), c_int64(a.stride(0)), c_int64(out.stride(0)), c_int(_dt(out)),
+        c_int(swiglu), _ptr(work, 16), _stream()), "linear_splitk")
+    return out
 
 
 def linear_handoff(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, residual: Optional[torch.Tensor] = None,
                    epilogue: Optional[str] = None, rows: Optional[torch.Tensor] = None, prepared=None,
                    emit=None) -> torch.Tensor:
-    """The few-row bfloat16 product with a norm handed over between products, in one launch each.
+    """The bfloat16 product with a norm handed over between products.
 
-    emit = (norm_weight [N], operand [M, N] bfloat16, sumsq [M, ceil(N / 16)] float32): besides
-    out = a @ w.T + residual (float32) the kernel writes operand = bf16(norm_weight * out) and the
-    sums of out^2 over groups of 16 columns.  prepared = (sumsq [R, P], eps, width): `a` is such an
-    operand ([R, K]; `rows` picks rows of both) and the product is multiplied by
-    1 / sqrt(sum(sumsq[row]) / width + eps): together the two are rmsnorm(out) @ w.T."""
+    emit = (norm_weight [N], operand [M, N] bfloat16, sumsq [M, handoff_parts(M, N, K)] float32):
+    besides out = a @ w.T + residual (float32) the kernel writes operand = bf16(norm_weight * out)
+    and the sums of out^2 over groups of columns.  prepared = (sumsq [R, P], eps, width): `a` is
+    such an operand ([R, K]; `rows` picks rows of both) and the product is multiplied by
+    1 / sqrt(sum(sumsq[row]) / width + eps): together the two are rmsnorm(out) @ w.T.
+    For at most 64 rows (one launch), or a product whose inner size is split (`split_k`)."""
     _dev(a, w, out, residual, rows)
     _rows_2d(a, "linear input")
     _rows_2d(out, "linear output")
@@ -225,7 +265,9 @@ def linear_handoff(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, residual
     M = a.shape[0] if rows is None else rows.numel()
     N = w.shape[0]
     swiglu = _epilogue(epilogue)
-    _need(0 < M <= HANDOFF_MAX_ROWS, f"a norm is handed over for at most {HANDOFF_MAX_ROWS} rows")
+    splits = split_k(M, N, K) if rows is None and M > 16 else 1
+    _need(0 < M <= FEW_ROWS or splits > 1,
+          f"a norm is handed over for at most {FEW_ROWS} rows or with a split inner size")
     _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_contiguous()
           and w.shape[1] == K, f"input and weight must be bfloat16, weight contiguous [N, {K}]")
     _need(K % 8 == 0 and a.stride(0) % 8 == 0, "inner size must be a multiple of 8")
@@ -258,7 +300,10 @@ def linear_handoff(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, residual
         _need(emit_op.dtype == torch.bfloat16 and emit_op.is_contiguous() and tuple(emit_op.shape) == (M, N),
               f"operand must be contiguous bfloat16 [{M}, {N}]")
         _need(emit_sq.dtype == torch.float32 and emit_sq.is_contiguous()
-              and tuple(emit_sq.shape) == (M, (N + 15) // 16), f"sums of squares must be float32 [{M}, {(N + 15) // 16}]")
+              and tuple(emit_sq.shape) == (M, handoff_parts(M, N, K)),
+              f"sums of squares must be float32 [{M}, {handoff_parts(M, N, K)}]")
+    if splits > 1:
+        return _linear_split(a, w, out, residual, swiglu, None, sumsq_in, parts, eps, width, emit, splits)
     _check(_lib().tl_linear_handoff(
         _ptr(a, 16), _ptr(w, 16), _ptr(out), _ptr(residual), _ptr(rows), _ptr(sumsq_in), c_int(parts), c_float(eps),
         c_int(width), _ptr(emit_w), c_int(_dt(emit_w) if emit_w is not None else 0), _ptr(emit_op), _ptr(emit_sq),

@@ -146,7 +146,7 @@ def project_into_residual(z: torch.Tensor, w: torch.Tensor, residual: torch.Tens
     from ..kernels import ops
     bufs = None
     if next_norm is not None and hasattr(next_norm, "hand_off_buffers") and residual.is_contiguous():
-        bufs = next_norm.hand_off_buffers(residual.shape[0], residual.device)
+        bufs = next_norm.hand_off_buffers(residual.shape[0], z.shape[1], residual.device)
     if bufs is not None and z.dtype == torch.bfloat16 and bufs[1].shape == residual.shape:
         ops.linear_handoff(z, w, residual, residual, emit=bufs)
         return residual, (bufs[1], bufs[2])

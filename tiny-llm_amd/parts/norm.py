@@ -29,7 +29,8 @@ class LazyNorm:
 
     def linear(self, w: torch.Tensor, out: torch.Tensor, epilogue: Optional[str] = None) -> torch.Tensor:
         """out = norm(x)[rows] @ w.T (then the epilogue), by the cheapest route there is."""
-        if self.prepared is not None and self.num_rows <= ops.HANDOFF_MAX_ROWS:
+        if self.prepared is not None and (self.num_rows <= ops.FEW_ROWS or (
+                self.rows is None and ops.split_k(self.num_rows, w.shape[0], w.shape[1]) > 1)):
             operand, sumsq = self.prepared
             return ops.linear_handoff(operand, w, out, epilogue=epilogue, rows=self.rows,
                                       prepared=(sumsq, self.eps, self.x.shape[1]))
@@ -65,13 +66,14 @@ class RMSNorm(Norm):
             return LazyNorm(self, x, rows, prepared)
         return self.forward(x, rows)
 
-    def hand_off_buffers(self, n_rows: int, device):
-        """(weight, operand, sumsq) for a product that writes this norm's input and can prepare the
-        norm on the way (`ops.linear_handoff`), or None where that does not apply."""
-        if not ops.can_hand_off(n_rows, self.hidden_size, self.dtype):
+    def hand_off_buffers(self, n_rows: int, inner: int, device):
+        """(weight, operand, sumsq) for a product (inner size `inner`) that writes this norm's input
+        and can prepare the norm on the way (`ops.linear_handoff`), or None where that does not apply."""
+        if not ops.can_hand_off(n_rows, self.hidden_size, inner, self.dtype):
             return None
         operand = torch.empty((n_rows, self.hidden_size), dtype=torch.bfloat16, device=device)
-        sumsq = torch.empty((n_rows, (self.hidden_size + 15) // 16), dtype=torch.float32, device=device)
+        sumsq = torch.empty((n_rows, ops.handoff_parts(n_rows, self.hidden_size, inner)), dtype=torch.float32,
+                            device=device)
         return self.weight, operand, sumsq
 
     def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
