@@ -139,6 +139,18 @@ class CacheManager:
         first_pos = max(0, context_len - g.spec.window + 1)
         return first_pos // self.block_size
 
+    def has_room(self, req_id, new_len: int) -> bool:
+        """True if the request is live and holds blocks for positions < new_len in every group
+        (the common case of a decoded token that does not start a new block)."""
+        rc = self.requests.get(req_id)
+        if rc is None:
+            return False
+        want = -(-new_len // self.block_size)
+        for b in rc.blocks:
+            if len(b) < want:
+                return False
+        return True
+
     def blocks_needed(self, req_id, new_len: int) -> List[int]:
         """New blocks per group to hold positions up to new_len - 1."""
         rc = self.requests.get(req_id)
@@ -172,19 +184,23 @@ class CacheManager:
         new = [rid for rid, _ in entries if rid not in self.requests]
         if len(new) > len(self._free_slots):
             raise NoFreeSlot(f"{len(new)} new requests, {len(self._free_slots)} request slots are free")
-        before, needs = [], []
+        before, needs, growing = [], [], []
         for rid, n in entries:
-            c = self.requests[rid].num_tokens if rid in self.requests else 0
+            rc = self.requests.get(rid)
+            c = rc.num_tokens if rc is not None else 0
             before.append(c)
+            if rc is not None and self.has_room(rid, c + n):
+                continue                      # nothing to take for this one
             needs.append(self.blocks_needed(rid, c + n))
+            growing.append((rid, c + n))
         if not self.can_grow(needs):
             raise OutOfBlocks("the step needs more cache blocks than are free: needs "
                               f"{[sum(n[g] for n in needs) for g in range(len(self.groups))]}, "
                               f"free {self.free_blocks()}")
         for rid in new:
             self.add_request(rid)
-        for (rid, n), c in zip(entries, before):
-            self.grow(rid, c + n)
+        for rid, new_len in growing:
+            self.grow(rid, new_len)
         return before
 
     def commit(self, req_id, new_len: int) -> None:

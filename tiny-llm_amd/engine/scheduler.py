@@ -40,7 +40,7 @@ from ..sampling.params import SamplingParams
 WAITING, RUNNING, FINISHED = "waiting", "running", "finished"
 
 
-@dataclass
+@dataclass(eq=False)          # a request is itself: membership tests compare identities, not token lists
 class Request:
     req_id: Hashable
     prompt: List[int]
@@ -175,9 +175,15 @@ class Scheduler:
         order = [r for r in self.running if r.pending == 1] + [r for r in self.running if r.pending > 1]
         scheduled_ids = set()
         for req in order:
-            if req not in self.running or budget <= 0:   # preempted meanwhile / no budget left
+            if req.status != RUNNING or budget <= 0:      # preempted meanwhile / no budget left
                 continue
             want = min(req.pending, budget)
+            if want == 1 and self.cache.has_room(req.req_id, req.num_computed + 1):
+                # the usual decoded token: its block is there already, nothing to weigh
+                entries.append(Scheduled(req, req.num_computed, 1, req.num_computed + 1 == req.num_tokens))
+                scheduled_ids.add(req.req_id)
+                budget -= 1
+                continue
             while True:
                 count = self._largest_fit(req, want, taken)
                 if count >= 1 and (count == want or req.pending > 1):

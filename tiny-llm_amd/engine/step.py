@@ -280,6 +280,7 @@ class DecodeGraph:
         self.out_host = torch.zeros(R, dtype=torch.int32, pin_memory=True)
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.runs = 0
+        self._tables = [[None] * R for _ in range(G)]     # (table, its length) last written per row
         # the attention kernel's query tiles of a decode step never change: one token per request
         ar = torch.arange(R, dtype=torch.int32, device=dev)
         one = torch.ones(R, dtype=torch.int32, device=dev)
@@ -303,11 +304,18 @@ class DecodeGraph:
         for g in range(G):
             bt = h[offs[7 + G + g]:offs[7 + G + g] + R * MB].reshape(R, MB)
             sm = h[offs[7 + g]:offs[7 + g] + R]
+            seen = self._tables[g]
             for r, (rid, c) in enumerate(zip(req_ids, ctx_lens)):
                 table = cm.block_table(rid, g)
-                tb = np.maximum(np.asarray(table, dtype=np.int32), 0)
-                bt[r, :len(table)] = tb
-                sm[r] = tb[c // bs] * bs + c % bs
+                # a row is rewritten only when it belongs to another admission than last time (the
+                # table object is made when a request is admitted) or has changed length (released
+                # blocks turn into -1 without a change of length, but a decode step never reads
+                # them: they lie before the window)
+                last = seen[r]
+                if last is None or last[0] is not table or last[1] != len(table):
+                    bt[r, :len(table)] = np.maximum(np.asarray(table, dtype=np.int32), 0)
+                    seen[r] = (table, len(table))
+                sm[r] = max(table[c // bs], 0) * bs + c % bs
         s0 = self.s0
         fview = self.host.view(torch.float32).numpy()
         fview[offs[s0]:offs[s0] + R] = [p.temperature if p.do_sample else 0.0 for p in params]
