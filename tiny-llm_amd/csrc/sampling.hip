@@ -192,6 +192,37 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
   r.inv_t = greedy ? 1.f : 1.f / temp;
   r.xmax = 0.f;
 
+  if (greedy) {
+    // One pass: the largest (key, lowest index) pair.  The index is stored inverted in the low
+    // half, so the maximum of the pairs is the first maximum of the row.
+    unsigned long long best = 0;
+    const bool vec = (vocab % 4 == 0) && (((uintptr_t)r.logits & 15) == 0);
+    if (vec) {
+      for (int i = threadIdx.x * 4; i < vocab; i += S_THREADS * 4) {
+        const f32x4 x = *(const f32x4*)(r.logits + i);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          best = max(best, ((unsigned long long)order_key(x[e]) << 32) | (uint32_t)(0xffffffffu - (uint32_t)(i + e)));
+      }
+    } else {
+      for (int i = threadIdx.x; i < vocab; i += S_THREADS)
+        best = max(best, ((unsigned long long)order_key(r.logits[i]) << 32) | (uint32_t)(0xffffffffu - (uint32_t)i));
+    }
+#pragma unroll
+    for (int off = TL_WAVE / 2; off > 0; off >>= 1) {
+      const uint32_t hi = (uint32_t)__shfl_xor((int)(best >> 32), off, TL_WAVE);
+      const uint32_t lo = (uint32_t)__shfl_xor((int)(best & 0xffffffffu), off, TL_WAVE);
+      best = max(best, ((unsigned long long)hi << 32) | lo);
+    }
+    if (threadIdx.x % TL_WAVE == 0) sh.red64[threadIdx.x / TL_WAVE] = best;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      for (int wv = 0; wv < S_WAVES; ++wv) best = max(best, sh.red64[wv]);
+      out[row] = (int32_t)(0xffffffffu - (uint32_t)(best & 0xffffffffu));
+    }
+    return;
+  }
+
   // maximum key of the row
   uint32_t kmax = 0;
   for (int i = threadIdx.x; i < vocab; i += S_THREADS) kmax = max(kmax, order_key(scaled(r, i)));
@@ -203,11 +234,6 @@ __global__ __launch_bounds__(S_THREADS) void sample_kernel(
   for (int wv = 0; wv < S_WAVES; ++wv) kmax = max(kmax, sh.red32[wv]);
   __syncthreads();
 
-  if (greedy) {
-    const int tok = nth_with_key(r, sh, kmax, 1);
-    if (threadIdx.x == 0) out[row] = tok;
-    return;
-  }
   r.xmax = key_value(kmax);
 
   // top-k: mass of the k largest
