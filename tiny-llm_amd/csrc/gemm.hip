@@ -648,16 +648,34 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
   }
 
   // Row factors of a norm whose sums of squares arrive in parts: one wave per row, fixed order.
-  // Called after the first stage's loads have been issued, so that its own loads queue behind
-  // them instead of holding them up.
+  // The first 128 parts of a row are requested here, ahead of everything else, and added up after
+  // the main loop: the request then costs no wait of its own.
   float* scale_s = ss_part + S_WAVES * MT * 16;                      // [MT * 16]
+  constexpr int RPW = MT * 16 / S_WAVES;                             // rows per wave
+  float pre[RPW][2];
+  if (p.in_sumsq) {
+#pragma unroll
+    for (int rr = 0; rr < RPW; ++rr) {
+      const int m = min(wave + rr * S_WAVES, M - 1);
+      const int64_t src = p.rows ? p.rows[m] : m;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int q = lane + h * TL_WAVE;
+        pre[rr][h] = q < p.in_parts ? p.in_sumsq[src * p.in_parts + q] : 0.f;
+      }
+    }
+  }
   auto row_factors = [&]() {
     if (!p.in_sumsq) return;
-    for (int r = wave; r < MT * 16; r += S_WAVES) {
-      const int m = min(r, M - 1);
-      const int64_t src = p.rows ? p.rows[m] : m;
-      float t = 0.f;
-      for (int q = lane; q < p.in_parts; q += TL_WAVE) t += p.in_sumsq[src * p.in_parts + q];
+#pragma unroll
+    for (int rr = 0; rr < RPW; ++rr) {
+      const int r = wave + rr * S_WAVES;
+      float t = pre[rr][0] + pre[rr][1];
+      if (p.in_parts > 2 * TL_WAVE) {
+        const int m = min(r, M - 1);
+        const int64_t src = p.rows ? p.rows[m] : m;
+        for (int q = lane + 2 * TL_WAVE; q < p.in_parts; q += TL_WAVE) t += p.in_sumsq[src * p.in_parts + q];
+      }
       t = wave_sum(t);
       if (lane == 0) scale_s[r] = 1.f / sqrtf(t / (float)p.in_width + p.in_eps);
     }
@@ -732,13 +750,11 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
     }
   };
   constexpr int STEP = S_WAVES * UN;
-  if (wave >= nblk) row_factors();        // a wave without a k block
   if constexpr (TWO_STAGES) {
     Stage s0, s1;
     int blk = wave;
     if (blk < nblk) {
       load(s0, blk);
-      row_factors();
       while (true) {
         const int b1 = blk + STEP;
         if (b1 < nblk) load(s1, b1);
@@ -755,10 +771,10 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
     Stage s0;
     for (int blk = wave; blk < nblk; blk += STEP) {
       load(s0, blk);
-      if (blk == wave) row_factors();
       multiply(s0, blk);
     }
   }
+  row_factors();
   // tile layout: lane holds rows (weight rows) g*4 + r, column (activation row) r16
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
