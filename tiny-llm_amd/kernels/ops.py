@@ -30,7 +30,16 @@ def _lib():
     return library.load()
 
 
+try:                                        # the raw handle without building a Stream object
+    from torch._C import _cuda_getCurrentRawStream as _raw_stream
+except ImportError:                          # pragma: no cover
+    _raw_stream = None
+
+
 def _stream():
+    """The current stream of the current device (also while a graph is being captured)."""
+    if _raw_stream is not None:
+        return c_void_p(_raw_stream(torch.cuda.current_device()))
     return c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
@@ -41,6 +50,10 @@ def _dt(t: torch.Tensor) -> int:
         raise KernelError(f"element type {t.dtype} is not float32 or bfloat16") from None
 
 
+def _fail(msg: str) -> None:
+    raise KernelError(msg)
+
+
 def _need(cond: bool, msg: str) -> None:
     if not cond:
         raise KernelError(msg)
@@ -49,14 +62,16 @@ def _need(cond: bool, msg: str) -> None:
 def _dev(*tensors) -> None:
     for t in tensors:
         if t is not None:
-            _need(t.is_cuda, "kernel operands must live on the GPU (there is no CPU path)")
+            if not (t.is_cuda):
+                _fail("kernel operands must live on the GPU (there is no CPU path)")
 
 
 def _ptr(t: Optional[torch.Tensor], align: int = 1) -> c_void_p:
     if t is None:
         return c_void_p(0)
     p = t.data_ptr()
-    _need(p % align == 0, f"operand is not {align}-byte aligned")
+    if not (p % align == 0):
+        _fail(f"operand is not {align}-byte aligned")
     return c_void_p(p)
 
 
@@ -68,7 +83,8 @@ def _check(code: int, what: str) -> None:
 
 
 def _rows_2d(t: torch.Tensor, name: str) -> None:
-    _need(t.dim() == 2 and t.stride(1) == 1, f"{name} must be 2-D with unit inner stride")
+    if not (t.dim() == 2 and t.stride(1) == 1):
+        _fail(f"{name} must be 2-D with unit inner stride")
 
 
 # --------------------------------------------------------------------------- ops
@@ -77,10 +93,12 @@ def embedding(tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> t
     _dev(tokens, table, out)
     T = tokens.numel()
     V, H = table.shape
-    _need(tokens.dtype == torch.int32 and tokens.is_contiguous(), "tokens must be contiguous int32")
-    _need(table.is_contiguous(), "embedding table must be contiguous")
-    _need(out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (T, H),
-          f"embedding output must be float32 [{T}, {H}]")
+    if not (tokens.dtype == torch.int32 and tokens.is_contiguous()):
+        _fail("tokens must be contiguous int32")
+    if not (table.is_contiguous()):
+        _fail("embedding table must be contiguous")
+    if not (out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (T, H)):
+        _fail(f"embedding output must be float32 [{T}, {H}]")
     _check(_lib().tl_embedding(_ptr(tokens), _ptr(table), _ptr(out), c_int(T), c_int(H), c_int(V),
                                c_int(_dt(table)), _stream()), "embedding")
     return out
@@ -90,16 +108,20 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor
             rows: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[i] = weight * x[rows[i] or i] / sqrt(mean(x^2) + eps); x is float32."""
     _dev(x, weight, out, rows)
-    _need(x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous(), "norm input must be contiguous float32 [T, H]")
+    if not (x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous()):
+        _fail("norm input must be contiguous float32 [T, H]")
     H = x.shape[1]
     n = out.shape[0]
-    _need(weight.is_contiguous() and weight.numel() == H, f"norm weight must have {H} elements")
-    _need(out.dim() == 2 and out.is_contiguous() and out.shape[1] == H, "norm output must be contiguous [n, H]")
+    if not (weight.is_contiguous() and weight.numel() == H):
+        _fail(f"norm weight must have {H} elements")
+    if not (out.dim() == 2 and out.is_contiguous() and out.shape[1] == H):
+        _fail("norm output must be contiguous [n, H]")
     if rows is None:
-        _need(n == x.shape[0], "norm output rows must match input rows")
+        if not (n == x.shape[0]):
+            _fail("norm output rows must match input rows")
     else:
-        _need(rows.dtype == torch.int32 and rows.is_contiguous() and rows.numel() == n,
-              "row index must be contiguous int32, one per output row")
+        if not (rows.dtype == torch.int32 and rows.is_contiguous() and rows.numel() == n):
+            _fail("row index must be contiguous int32, one per output row")
     _check(_lib().tl_rmsnorm(_ptr(x), _ptr(weight), _ptr(rows), _ptr(out), c_int(n), c_int(H),
                              c_float(eps), c_int(_dt(weight)), c_int(_dt(out)), _stream()), "rmsnorm")
     return out
@@ -119,27 +141,34 @@ def linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, residual: Option
     M, K = a.shape
     N = w.shape[0]
     swiglu = _epilogue(epilogue)
-    _need(w.dim() == 2 and w.is_contiguous() and w.shape[1] == K, f"weight must be contiguous [N, {K}]")
-    _need(a.dtype == w.dtype, "input and weight must share an element type")
+    if not (w.dim() == 2 and w.is_contiguous() and w.shape[1] == K):
+        _fail(f"weight must be contiguous [N, {K}]")
+    if not (a.dtype == w.dtype):
+        _fail("input and weight must share an element type")
     dt, odt = _dt(a), _dt(out)
     if swiglu:
-        _need(N % 2 == 0 and tuple(out.shape) == (M, N // 2) and odt == dt and residual is None,
-              f"the SiLU-gate epilogue writes [{M}, {N // 2}] of the input's type and takes no residual")
+        if not (N % 2 == 0 and tuple(out.shape) == (M, N // 2) and odt == dt and residual is None):
+            _fail(f"the SiLU-gate epilogue writes [{M}, {N // 2}] of the input's type and takes no residual")
     else:
-        _need(tuple(out.shape) == (M, N), f"linear output must be [{M}, {N}]")
-        _need(odt == dt or odt == 0, "linear output must have the input's type or float32")
+        if not (tuple(out.shape) == (M, N)):
+            _fail(f"linear output must be [{M}, {N}]")
+        if not (odt == dt or odt == 0):
+            _fail("linear output must have the input's type or float32")
     if residual is not None:
-        _need(residual.dtype == torch.float32 and residual.shape == out.shape
-              and residual.stride() == out.stride(), "residual must be float32 with the output's layout")
+        if not (residual.dtype == torch.float32 and residual.shape == out.shape
+                and residual.stride() == out.stride()):
+            _fail("residual must be float32 with the output's layout")
     if dt == 1:
-        _need(K % 8 == 0 and a.stride(0) % 8 == 0,
-              f"bfloat16 linear needs an inner size that is a multiple of 8, got K={K}")
+        if not (K % 8 == 0 and a.stride(0) % 8 == 0):
+            _fail(f"bfloat16 linear needs an inner size that is a multiple of 8, got K={K}")
     al = 16 if dt == 1 else 4      # the bfloat16 kernel moves 16-byte vectors
     ao = 16 if (dt == 1 and not swiglu and M > 64) else 4
     if row_scale is not None:
-        _need(dt == 1 and row_scale.dtype == torch.float32 and row_scale.is_contiguous()
-              and row_scale.numel() == M, "row scales go with the bfloat16 product: float32, one per row")
-    _need(0 <= tile <= 4, "tile is 0 (by size) or 1 to 4")
+        if not (dt == 1 and row_scale.dtype == torch.float32 and row_scale.is_contiguous()
+                and row_scale.numel() == M):
+            _fail("row scales go with the bfloat16 product: float32, one per row")
+    if not (0 <= tile <= 4):
+        _fail("tile is 0 (by size) or 1 to 4")
     if dt == 1 and tile == 0 and M > 16:
         splits = split_k(M, N, K)
         if splits > 1:
@@ -153,7 +182,8 @@ def linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, residual: Option
 def _epilogue(name: Optional[str]) -> int:
     if name is None:
         return 0
-    _need(name == "swiglu", f"unknown epilogue {name!r}")
+    if not (name == "swiglu"):
+        _fail(f"unknown epilogue {name!r}")
     return 1
 
 FUSED_MAX_ROWS = 16    # most rows for which the few-row product kernel normalises its input itself
@@ -170,20 +200,26 @@ def linear_norm(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: torch
     while one round of workgroups covers the columns); otherwise a pre-scale kernel writes the
     operand and the row factors once and the plain product applies them."""
     _dev(x, norm_weight, w, out, residual, rows)
-    _need(x.dtype == torch.float32 and x.dim() == 2 and x.stride(1) == 1, "norm input must be float32 [T, K]")
+    if not (x.dtype == torch.float32 and x.dim() == 2 and x.stride(1) == 1):
+        _fail("norm input must be float32 [T, K]")
     K = x.shape[1]
     M = x.shape[0] if rows is None else rows.numel()
     N = w.shape[0]
     swiglu = _epilogue(epilogue)
-    _need(M > 0, "the product needs at least one row")
-    _need(w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_contiguous() and w.shape[1] == K,
-          f"weight must be contiguous bfloat16 [N, {K}]")
-    _need(norm_weight.is_contiguous() and norm_weight.numel() == K, f"norm weight must have {K} elements")
-    _need(K % 8 == 0 and x.stride(0) % 8 == 0, "inner size must be a multiple of 8")
+    if not (M > 0):
+        _fail("the product needs at least one row")
+    if not (w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_contiguous() and w.shape[1] == K):
+        _fail(f"weight must be contiguous bfloat16 [N, {K}]")
+    if not (norm_weight.is_contiguous() and norm_weight.numel() == K):
+        _fail(f"norm weight must have {K} elements")
+    if not (K % 8 == 0 and x.stride(0) % 8 == 0):
+        _fail("inner size must be a multiple of 8")
     if rows is not None:
-        _need(rows.dtype == torch.int32 and rows.is_contiguous(), "row index must be contiguous int32")
+        if not (rows.dtype == torch.int32 and rows.is_contiguous()):
+            _fail("row index must be contiguous int32")
     if M > FUSED_MAX_ROWS or N > FUSED_MAX_COLS:
-        _need(x.is_contiguous(), "norm input must be contiguous")
+        if not (x.is_contiguous()):
+            _fail("norm input must be contiguous")
         h = torch.empty((M, K), dtype=torch.bfloat16, device=x.device)
         inv_rms = torch.empty(M, dtype=torch.float32, device=x.device)
         _check(_lib().tl_norm_prescale(_ptr(x), _ptr(norm_weight), _ptr(rows), _ptr(h), _ptr(inv_rms), c_int(M),
@@ -191,13 +227,15 @@ def linear_norm(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: torch
         return linear(h, w, out, residual, epilogue, row_scale=inv_rms)
     _rows_2d(out, "linear output")
     if swiglu:
-        _need(N % 2 == 0 and tuple(out.shape) == (M, N // 2) and out.dtype == torch.bfloat16 and residual is None,
-              f"the SiLU-gate epilogue writes bfloat16 [{M}, {N // 2}] and takes no residual")
+        if not (N % 2 == 0 and tuple(out.shape) == (M, N // 2) and out.dtype == torch.bfloat16 and residual is None):
+            _fail(f"the SiLU-gate epilogue writes bfloat16 [{M}, {N // 2}] and takes no residual")
     else:
-        _need(tuple(out.shape) == (M, N), f"linear output must be [{M}, {N}]")
+        if not (tuple(out.shape) == (M, N)):
+            _fail(f"linear output must be [{M}, {N}]")
     if residual is not None:
-        _need(residual.dtype == torch.float32 and residual.shape == out.shape
-              and residual.stride() == out.stride(), "residual must be float32 with the output's layout")
+        if not (residual.dtype == torch.float32 and residual.shape == out.shape
+                and residual.stride() == out.stride()):
+            _fail("residual must be float32 with the output's layout")
     _check(_lib().tl_linear_norm(_ptr(x, 16), _ptr(w, 16), _ptr(out), _ptr(residual), _ptr(norm_weight, 16),
                                  _ptr(rows), c_float(eps), c_int(_dt(norm_weight)), c_int(M), c_int(N), c_int(K),
                                  c_int64(x.stride(0)), c_int64(out.stride(0)), c_int(_dt(out)), c_int(swiglu),
@@ -213,7 +251,14 @@ def split_k(rows: int, cols: int, inner: int) -> int:
     few-row kernel likes."""
     if inner % 8:
         return 1
-    return int(_lib().tl_splitk_plan(c_int(rows), c_int(cols), c_int(inner)))
+    key = (rows, cols, inner)
+    n = _SPLITS.get(key)
+    if n is None:
+        n = _SPLITS[key] = int(_lib().tl_splitk_plan(c_int(rows), c_int(cols), c_int(inner)))
+    return n
+
+
+_SPLITS: dict = {}      # the plan is a pure function of the sizes
 
 
 def can_hand_off(rows: int, width: int, inner: int, dtype: torch.dtype) -> bool:
@@ -229,7 +274,8 @@ def handoff_parts(rows: int, width: int, inner: int) -> int:
     when it prepares a norm: per 16 columns in the few-row kernel, per 1024 after a split inner size."""
     if split_k(rows, width, inner) > 1:
         return (width + 1023) // 1024
-    _need(rows <= FEW_ROWS, f"without a split inner size a norm is prepared for at most {FEW_ROWS} rows")
+    if not (rows <= FEW_ROWS):
+        _fail(f"without a split inner size a norm is prepared for at most {FEW_ROWS} rows")
     return (width + 15) // 16
 
 
@@ -266,42 +312,47 @@ def linear_handoff(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, residual
     N = w.shape[0]
     swiglu = _epilogue(epilogue)
     splits = split_k(M, N, K) if rows is None and M > 16 else 1
-    _need(0 < M <= FEW_ROWS or splits > 1,
-          f"a norm is handed over for at most {FEW_ROWS} rows or with a split inner size")
-    _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_contiguous()
-          and w.shape[1] == K, f"input and weight must be bfloat16, weight contiguous [N, {K}]")
-    _need(K % 8 == 0 and a.stride(0) % 8 == 0, "inner size must be a multiple of 8")
+    if not (0 < M <= FEW_ROWS or splits > 1):
+        _fail(f"a norm is handed over for at most {FEW_ROWS} rows or with a split inner size")
+    if not (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_contiguous()
+            and w.shape[1] == K):
+        _fail(f"input and weight must be bfloat16, weight contiguous [N, {K}]")
+    if not (K % 8 == 0 and a.stride(0) % 8 == 0):
+        _fail("inner size must be a multiple of 8")
     if rows is not None:
-        _need(rows.dtype == torch.int32 and rows.is_contiguous(), "row index must be contiguous int32")
+        if not (rows.dtype == torch.int32 and rows.is_contiguous()):
+            _fail("row index must be contiguous int32")
     if swiglu:
-        _need(N % 2 == 0 and tuple(out.shape) == (M, N // 2) and out.dtype == torch.bfloat16 and residual is None,
-              f"the SiLU-gate epilogue writes bfloat16 [{M}, {N // 2}] and takes no residual")
+        if not (N % 2 == 0 and tuple(out.shape) == (M, N // 2) and out.dtype == torch.bfloat16 and residual is None):
+            _fail(f"the SiLU-gate epilogue writes bfloat16 [{M}, {N // 2}] and takes no residual")
     else:
-        _need(tuple(out.shape) == (M, N) and out.dtype in (torch.float32, torch.bfloat16),
-              f"linear output must be [{M}, {N}], float32 or bfloat16")
+        if not (tuple(out.shape) == (M, N) and out.dtype in (torch.float32, torch.bfloat16)):
+            _fail(f"linear output must be [{M}, {N}], float32 or bfloat16")
     if residual is not None:
-        _need(residual.dtype == torch.float32 and residual.shape == out.shape
-              and residual.stride() == out.stride(), "residual must be float32 with the output's layout")
+        if not (residual.dtype == torch.float32 and residual.shape == out.shape
+                and residual.stride() == out.stride()):
+            _fail("residual must be float32 with the output's layout")
     sumsq_in, parts, eps, width = None, 0, 0.0, 0
     if prepared is not None:
         sumsq_in, eps, width = prepared
         _dev(sumsq_in)
-        _need(sumsq_in.dtype == torch.float32 and sumsq_in.dim() == 2 and sumsq_in.is_contiguous()
-              and sumsq_in.shape[0] == a.shape[0] and width > 0,
-              "sums of squares must be contiguous float32 [rows of the input, parts]")
+        if not (sumsq_in.dtype == torch.float32 and sumsq_in.dim() == 2 and sumsq_in.is_contiguous()
+                and sumsq_in.shape[0] == a.shape[0] and width > 0):
+            _fail("sums of squares must be contiguous float32 [rows of the input, parts]")
         parts = sumsq_in.shape[1]
     emit_w = emit_op = emit_sq = None
     if emit is not None:
         emit_w, emit_op, emit_sq = emit
         _dev(emit_w, emit_op, emit_sq)
-        _need(not swiglu and out.dtype == torch.float32, "only a float32 product without SiLU-gate prepares a norm")
-        _need(emit_w.is_contiguous() and emit_w.numel() == N and emit_w.dtype in (torch.float32, torch.bfloat16),
-              f"norm weight must have {N} elements, float32 or bfloat16")
-        _need(emit_op.dtype == torch.bfloat16 and emit_op.is_contiguous() and tuple(emit_op.shape) == (M, N),
-              f"operand must be contiguous bfloat16 [{M}, {N}]")
-        _need(emit_sq.dtype == torch.float32 and emit_sq.is_contiguous()
-              and tuple(emit_sq.shape) == (M, handoff_parts(M, N, K)),
-              f"sums of squares must be float32 [{M}, {handoff_parts(M, N, K)}]")
+        if not (not swiglu and out.dtype == torch.float32):
+            _fail("only a float32 product without SiLU-gate prepares a norm")
+        if not (emit_w.is_contiguous() and emit_w.numel() == N and emit_w.dtype in (torch.float32, torch.bfloat16)):
+            _fail(f"norm weight must have {N} elements, float32 or bfloat16")
+        if not (emit_op.dtype == torch.bfloat16 and emit_op.is_contiguous() and tuple(emit_op.shape) == (M, N)):
+            _fail(f"operand must be contiguous bfloat16 [{M}, {N}]")
+        if not (emit_sq.dtype == torch.float32 and emit_sq.is_contiguous()
+                and tuple(emit_sq.shape) == (M, handoff_parts(M, N, K))):
+            _fail(f"sums of squares must be float32 [{M}, {handoff_parts(M, N, K)}]")
     if splits > 1:
         return _linear_split(a, w, out, residual, swiglu, None, sumsq_in, parts, eps, width, emit, splits)
     _check(_lib().tl_linear_handoff(
@@ -316,9 +367,10 @@ def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     """out[t, j] = silu(gate_up[t, j]) * gate_up[t, I + j]."""
     _dev(gate_up, out)
     T, I2 = gate_up.shape
-    _need(I2 % 2 == 0 and gate_up.is_contiguous(), "gate_up must be contiguous [T, 2I]")
-    _need(out.dtype == gate_up.dtype and out.is_contiguous() and tuple(out.shape) == (T, I2 // 2),
-          "silu_mul output must be contiguous [T, I] of the input's type")
+    if not (I2 % 2 == 0 and gate_up.is_contiguous()):
+        _fail("gate_up must be contiguous [T, 2I]")
+    if not (out.dtype == gate_up.dtype and out.is_contiguous() and tuple(out.shape) == (T, I2 // 2)):
+        _fail("silu_mul output must be contiguous [T, I] of the input's type")
     _check(_lib().tl_silu_mul(_ptr(gate_up), _ptr(out), c_int(T), c_int(I2 // 2), c_int(_dt(gate_up)),
                               _stream()), "silu_mul")
     return out
@@ -327,8 +379,8 @@ def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
 def add_residual(x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
     """x += y with x float32."""
     _dev(x, y)
-    _need(x.dtype == torch.float32 and x.is_contiguous() and y.is_contiguous() and x.shape == y.shape,
-          "residual add needs contiguous operands of one shape, the sum in float32")
+    if not (x.dtype == torch.float32 and x.is_contiguous() and y.is_contiguous() and x.shape == y.shape):
+        _fail("residual add needs contiguous operands of one shape, the sum in float32")
     _check(_lib().tl_add_residual(_ptr(x), _ptr(y), c_int64(x.numel()), c_int(_dt(y)), _stream()), "add_residual")
     return x
 
@@ -343,22 +395,25 @@ def rope_store(qkv: torch.Tensor, positions: torch.Tensor, cos: Optional[torch.T
     _rows_2d(qkv, "qkv")
     T = qkv.shape[0]
     width = (num_heads + 2 * num_kv_heads) * head_dim
-    _need(qkv.shape[1] == width, f"qkv rows must be {width} wide")
-    _need(positions.dtype == torch.int32 and positions.is_contiguous() and positions.numel() == T,
-          "positions must be contiguous int32, one per row")
+    if not (qkv.shape[1] == width):
+        _fail(f"qkv rows must be {width} wide")
+    if not (positions.dtype == torch.int32 and positions.is_contiguous() and positions.numel() == T):
+        _fail("positions must be contiguous int32, one per row")
     block_size = 1
     if rotary_dim:
-        _need(cos is not None and sin is not None and cos.dtype == torch.float32 and sin.dtype == torch.float32
-              and cos.is_contiguous() and sin.is_contiguous() and cos.shape == sin.shape
-              and cos.shape[1] == rotary_dim // 2, "angle tables must be float32 [positions, rotary_dim/2]")
+        if not (cos is not None and sin is not None and cos.dtype == torch.float32
+                and sin.dtype == torch.float32 and cos.is_contiguous() and sin.is_contiguous()
+                and cos.shape == sin.shape and cos.shape[1] == rotary_dim // 2):
+            _fail("angle tables must be float32 [positions, rotary_dim/2]")
     if slot_mapping is not None:
-        _need(slot_mapping.dtype == torch.int32 and slot_mapping.is_contiguous() and slot_mapping.numel() == T,
-              "slot mapping must be contiguous int32, one per row")
+        if not (slot_mapping.dtype == torch.int32 and slot_mapping.is_contiguous() and slot_mapping.numel() == T):
+            _fail("slot mapping must be contiguous int32, one per row")
         for c in (k_cache, v_cache):
-            _need(c is not None and c.dtype == qkv.dtype and c.is_contiguous() and c.dim() == 4
-                  and c.shape[1] == num_kv_heads and c.shape[3] == head_dim,
-                  "cache must be contiguous [blocks, kv_heads, block, head_dim] of the activations' type")
-        _need(k_cache.shape == v_cache.shape, "key and value caches must have one shape")
+            if not (c is not None and c.dtype == qkv.dtype and c.is_contiguous() and c.dim() == 4
+                    and c.shape[1] == num_kv_heads and c.shape[3] == head_dim):
+                _fail("cache must be contiguous [blocks, kv_heads, block, head_dim] of the activations' type")
+        if not (k_cache.shape == v_cache.shape):
+            _fail("key and value caches must have one shape")
         block_size = k_cache.shape[2]
     _check(_lib().tl_rope_store(_ptr(qkv), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(slot_mapping),
                                 _ptr(k_cache), _ptr(v_cache), c_int(T), c_int(num_heads), c_int(num_kv_heads),
@@ -376,19 +431,23 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     _rows_2d(q, "q")
     _rows_2d(out, "attention output")
     T = q.shape[0]
-    _need(q.shape[1] == num_heads * head_dim and tuple(out.shape) == (T, num_heads * head_dim),
-          "q and the attention output must be [T, heads * head_dim]")
-    _need(q.dtype == k_cache.dtype == v_cache.dtype == out.dtype, "q, caches and output must share an element type")
-    _need(k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dim() == 4
-          and k_cache.shape == v_cache.shape and k_cache.shape[1] == num_kv_heads
-          and k_cache.shape[3] == head_dim, "cache must be contiguous [blocks, kv_heads, block, head_dim]")
-    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(),
-          "block tables must be contiguous int32 [requests, max_blocks]")
+    if not (q.shape[1] == num_heads * head_dim and tuple(out.shape) == (T, num_heads * head_dim)):
+        _fail("q and the attention output must be [T, heads * head_dim]")
+    if not (q.dtype == k_cache.dtype == v_cache.dtype == out.dtype):
+        _fail("q, caches and output must share an element type")
+    if not (k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dim() == 4
+            and k_cache.shape == v_cache.shape and k_cache.shape[1] == num_kv_heads
+            and k_cache.shape[3] == head_dim):
+        _fail("cache must be contiguous [blocks, kv_heads, block, head_dim]")
+    if not (block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()):
+        _fail("block tables must be contiguous int32 [requests, max_blocks]")
     for t in (req_of_token, positions):
-        _need(t.dtype == torch.int32 and t.is_contiguous() and t.numel() == T,
-              "per-token request ids and positions must be contiguous int32")
-    _need(num_kv_heads > 0 and num_heads % num_kv_heads == 0, "heads must be a multiple of kv heads")
-    _need(head_dim <= 256, f"head_dim {head_dim} exceeds the attention kernel's limit of 256")
+        if not (t.dtype == torch.int32 and t.is_contiguous() and t.numel() == T):
+            _fail("per-token request ids and positions must be contiguous int32")
+    if not (num_kv_heads > 0 and num_heads % num_kv_heads == 0):
+        _fail("heads must be a multiple of kv heads")
+    if not (head_dim <= 256):
+        _fail(f"head_dim {head_dim} exceeds the attention kernel's limit of 256")
     _check(_lib().tl_paged_attention(
         _ptr(q), c_int64(q.stride(0)), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
         c_int(block_tables.shape[1]), _ptr(req_of_token), _ptr(positions), _ptr(out), c_int64(out.stride(0)),
@@ -420,39 +479,47 @@ def flash_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     _rows_2d(q, "q")
     _rows_2d(out, "attention output")
     T = q.shape[0]
-    _need(flash_attention_supported(q.dtype, num_heads, num_kv_heads, head_dim),
-          "the MFMA attention kernel takes bfloat16, head sizes in steps of 16 up to 128, up to 16 heads per kv head")
-    _need(q.shape[1] == num_heads * head_dim and tuple(out.shape) == (T, num_heads * head_dim),
-          "q and the attention output must be [T, heads * head_dim]")
-    _need(q.dtype == k_cache.dtype == v_cache.dtype == out.dtype, "q, caches and output must share an element type")
-    _need(k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dim() == 4
-          and k_cache.shape == v_cache.shape and k_cache.shape[1] == num_kv_heads
-          and k_cache.shape[3] == head_dim, "cache must be contiguous [blocks, kv_heads, block, head_dim]")
-    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(),
-          "block tables must be contiguous int32 [requests, max_blocks]")
-    _need(positions.dtype == torch.int32 and positions.is_contiguous() and positions.numel() == T,
-          "positions must be contiguous int32, one per row")
+    if not (flash_attention_supported(q.dtype, num_heads, num_kv_heads, head_dim)):
+        _fail("the MFMA attention kernel takes bfloat16, head sizes in steps of 16 up to 128, up to 16 "
+              "heads per kv head")
+    if not (q.shape[1] == num_heads * head_dim and tuple(out.shape) == (T, num_heads * head_dim)):
+        _fail("q and the attention output must be [T, heads * head_dim]")
+    if not (q.dtype == k_cache.dtype == v_cache.dtype == out.dtype):
+        _fail("q, caches and output must share an element type")
+    if not (k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dim() == 4
+            and k_cache.shape == v_cache.shape and k_cache.shape[1] == num_kv_heads
+            and k_cache.shape[3] == head_dim):
+        _fail("cache must be contiguous [blocks, kv_heads, block, head_dim]")
+    if not (block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()):
+        _fail("block tables must be contiguous int32 [requests, max_blocks]")
+    if not (positions.dtype == torch.int32 and positions.is_contiguous() and positions.numel() == T):
+        _fail("positions must be contiguous int32, one per row")
     n_tiles = tile_req.numel()
     for t in (tile_req, tile_tok0, tile_ntok):
-        _need(t.dtype == torch.int32 and t.is_contiguous() and t.numel() == n_tiles, "tile arrays must be int32 [tiles]")
-    _need(q.stride(0) % 8 == 0, "q rows must be 16-byte aligned")
+        if not (t.dtype == torch.int32 and t.is_contiguous() and t.numel() == n_tiles):
+            _fail("tile arrays must be int32 [tiles]")
+    if not (q.stride(0) % 8 == 0):
+        _fail("q rows must be 16-byte aligned")
     part_o = part_ml = None
     if n_splits > 1:
         need = n_splits * T * num_heads * (head_dim + 2)
-        _need(scratch is not None and scratch.dtype == torch.float32 and scratch.is_contiguous()
-              and scratch.numel() >= need, f"split attention needs {need} float32 of scratch")
+        if not (scratch is not None and scratch.dtype == torch.float32 and scratch.is_contiguous()
+                and scratch.numel() >= need):
+            _fail(f"split attention needs {need} float32 of scratch")
         part_o = scratch[:n_splits * T * num_heads * head_dim]
         part_ml = scratch[n_splits * T * num_heads * head_dim:]
     cos = sin = None
     if fused_rope is not None:
         cos, sin = fused_rope
         _dev(cos, sin)
-        _need(n_tiles == T, "the fused rotation and cache write take one token per tile")
-        _need(cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.is_contiguous() and sin.is_contiguous()
-              and cos.shape == sin.shape and cos.shape[1] == head_dim // 2,
-              "angle tables must be float32 [positions, head_dim / 2]")
+        if not (n_tiles == T):
+            _fail("the fused rotation and cache write take one token per tile")
+        if not (cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.is_contiguous()
+                and sin.is_contiguous() and cos.shape == sin.shape and cos.shape[1] == head_dim // 2):
+            _fail("angle tables must be float32 [positions, head_dim / 2]")
         # q must be the head of a [q | k | v] row
-        _need(q.stride(0) >= (num_heads + 2 * num_kv_heads) * head_dim, "fused mode needs q inside its qkv rows")
+        if not (q.stride(0) >= (num_heads + 2 * num_kv_heads) * head_dim):
+            _fail("fused mode needs q inside its qkv rows")
     _check(_lib().tl_flash_attention(
         _ptr(q, 16), c_int64(q.stride(0)), _ptr(k_cache, 16), _ptr(v_cache, 16), _ptr(block_tables),
         c_int(block_tables.shape[1]), _ptr(tile_req), _ptr(tile_tok0), _ptr(tile_ntok), _ptr(positions),
@@ -477,22 +544,27 @@ def flash_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
     _rows_2d(q, "q")
     _rows_2d(out, "attention output")
     T = q.shape[0]
-    _need(flash_attention_supported(q.dtype, num_heads, num_kv_heads, head_dim),
-          "the MFMA attention kernel takes bfloat16, head sizes in steps of 16 up to 128, up to 16 heads per kv head")
-    _need(q.shape[1] == num_heads * head_dim and tuple(out.shape) == (T, num_heads * head_dim),
-          "q and the attention output must be [T, heads * head_dim]")
-    _need(q.dtype == k_cache.dtype == v_cache.dtype == out.dtype, "q, caches and output must share an element type")
-    _need(k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dim() == 4
-          and k_cache.shape == v_cache.shape and k_cache.shape[1] == num_kv_heads
-          and k_cache.shape[3] == head_dim, "cache must be contiguous [blocks, kv_heads, block, head_dim]")
-    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(),
-          "block tables must be contiguous int32 [requests, max_blocks]")
-    _need(positions.dtype == torch.int32 and positions.is_contiguous() and positions.numel() == T,
-          "positions must be contiguous int32, one per row")
+    if not (flash_attention_supported(q.dtype, num_heads, num_kv_heads, head_dim)):
+        _fail("the MFMA attention kernel takes bfloat16, head sizes in steps of 16 up to 128, up to 16 "
+              "heads per kv head")
+    if not (q.shape[1] == num_heads * head_dim and tuple(out.shape) == (T, num_heads * head_dim)):
+        _fail("q and the attention output must be [T, heads * head_dim]")
+    if not (q.dtype == k_cache.dtype == v_cache.dtype == out.dtype):
+        _fail("q, caches and output must share an element type")
+    if not (k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dim() == 4
+            and k_cache.shape == v_cache.shape and k_cache.shape[1] == num_kv_heads
+            and k_cache.shape[3] == head_dim):
+        _fail("cache must be contiguous [blocks, kv_heads, block, head_dim]")
+    if not (block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()):
+        _fail("block tables must be contiguous int32 [requests, max_blocks]")
+    if not (positions.dtype == torch.int32 and positions.is_contiguous() and positions.numel() == T):
+        _fail("positions must be contiguous int32, one per row")
     n_tiles = tile_req.numel()
     for t in (tile_req, tile_tok0, tile_ntok):
-        _need(t.dtype == torch.int32 and t.is_contiguous() and t.numel() == n_tiles, "tile arrays must be int32 [tiles]")
-    _need(q.stride(0) % 8 == 0 and out.stride(0) % 4 == 0, "q and output rows must be vector aligned")
+        if not (t.dtype == torch.int32 and t.is_contiguous() and t.numel() == n_tiles):
+            _fail("tile arrays must be int32 [tiles]")
+    if not (q.stride(0) % 8 == 0 and out.stride(0) % 4 == 0):
+        _fail("q and output rows must be vector aligned")
     _check(_lib().tl_flash_prefill(
         _ptr(q, 16), c_int64(q.stride(0)), _ptr(k_cache, 16), _ptr(v_cache, 16), _ptr(block_tables),
         c_int(block_tables.shape[1]), _ptr(tile_req), _ptr(tile_tok0), _ptr(tile_ntok), _ptr(positions),
@@ -510,13 +582,16 @@ def sample(logits: torch.Tensor, out: torch.Tensor, temperature: Optional[torch.
     _dev(logits, out, temperature, top_k, top_p, seeds, counters)
     _rows_2d(logits, "logits")
     n, V = logits.shape
-    _need(logits.dtype == torch.float32, "logits must be float32")
-    _need(out.dtype == torch.int32 and out.is_contiguous() and out.numel() == n, "token output must be int32 [rows]")
+    if not (logits.dtype == torch.float32):
+        _fail("logits must be float32")
+    if not (out.dtype == torch.int32 and out.is_contiguous() and out.numel() == n):
+        _fail("token output must be int32 [rows]")
     for t, dt, name in ((temperature, torch.float32, "temperature"), (top_k, torch.int32, "top_k"),
                         (top_p, torch.float32, "top_p"), (seeds, torch.int64, "seeds"),
                         (counters, torch.int32, "counters")):
         if t is not None:
-            _need(t.dtype == dt and t.is_contiguous() and t.numel() == n, f"{name} must be contiguous {dt} [rows]")
+            if not (t.dtype == dt and t.is_contiguous() and t.numel() == n):
+                _fail(f"{name} must be contiguous {dt} [rows]")
     _check(_lib().tl_sample(_ptr(logits), c_int64(logits.stride(0)), c_int(n), c_int(V), _ptr(temperature),
                             _ptr(top_k), _ptr(top_p), _ptr(seeds), _ptr(counters), _ptr(out), _stream()), "sample")
     return out
