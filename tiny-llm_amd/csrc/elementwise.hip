@@ -61,10 +61,28 @@ __global__ void norm_prescale_kernel(const float* __restrict__ x, const TW* __re
   const float* src = x + in_row * hidden;
   bf16_t* dst = out + (int64_t)blockIdx.x * hidden;
   float ss = 0.f;
-  for (int j = threadIdx.x; j < hidden; j += kThreads) {
-    const float v = src[j];
-    ss += v * v;
-    dst[j] = (bf16_t)(to_f32(w[j]) * v);
+  const bool aligned = (((uintptr_t)x | (uintptr_t)out) & 15) == 0 && ((uintptr_t)w & (4 * sizeof(TW) - 1)) == 0;
+  if (hidden % 4 == 0 && aligned) {       // four elements per access
+    for (int j = threadIdx.x * 4; j < hidden; j += kThreads * 4) {
+      const f32x4 v = *(const f32x4*)(src + j);
+      float wv[4];
+      if constexpr (sizeof(TW) == 4) {
+        const f32x4 w4 = *(const f32x4*)(w + j);
+        wv[0] = w4[0]; wv[1] = w4[1]; wv[2] = w4[2]; wv[3] = w4[3];
+      } else {
+        const bf16x4 w4 = *(const bf16x4*)(w + j);
+        wv[0] = (float)w4[0]; wv[1] = (float)w4[1]; wv[2] = (float)w4[2]; wv[3] = (float)w4[3];
+      }
+      ss += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+      bf16x4 o = {(bf16_t)(wv[0] * v[0]), (bf16_t)(wv[1] * v[1]), (bf16_t)(wv[2] * v[2]), (bf16_t)(wv[3] * v[3])};
+      *(bf16x4*)(dst + j) = o;
+    }
+  } else {
+    for (int j = threadIdx.x; j < hidden; j += kThreads) {
+      const float v = src[j];
+      ss += v * v;
+      dst[j] = (bf16_t)(to_f32(w[j]) * v);
+    }
   }
   ss = block_sum<kWaves>(ss, red);
   if (threadIdx.x == 0) inv_rms[blockIdx.x] = 1.f / sqrtf(ss / (float)hidden + eps);
@@ -112,6 +130,45 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const int32_t* __restrict
   const int64_t blk = slot >= 0 ? slot / block_size : 0;
   const int in_blk = slot >= 0 ? slot % block_size : 0;
 
+  if constexpr (sizeof(T) == 2) {
+    // bfloat16, whole heads rotated, halves that are multiples of 8 and 16-byte aligned rows:
+    // eight pairs per thread and 16-byte accesses throughout
+    const bool aligned = (((uintptr_t)qkv | (uintptr_t)k_cache | (uintptr_t)v_cache | (uintptr_t)cos_t |
+                           (uintptr_t)sin_t) & 15) == 0;
+    if (rot == hd && half % 8 == 0 && row_stride % 8 == 0 && aligned) {
+      const int chunks = half / 8;
+      for (int i = threadIdx.x; i < (nq + nkv) * chunks; i += kThreads) {
+        const int head = i / chunks, j = (i - head * chunks) * 8;
+        bf16_t* h = (bf16_t*)row + (int64_t)head * hd;
+        const bf16x8 a8 = *(const bf16x8*)(h + j), b8 = *(const bf16x8*)(h + j + half);
+        const f32x4 c0 = *(const f32x4*)(cs + j), c1 = *(const f32x4*)(cs + j + 4);
+        const f32x4 s0 = *(const f32x4*)(sn + j), s1 = *(const f32x4*)(sn + j + 4);
+        bf16x8 ra, rb;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float c = e < 4 ? c0[e] : c1[e - 4], sv = e < 4 ? s0[e] : s1[e - 4];
+          const float a = (float)a8[e], b = (float)b8[e];
+          ra[e] = (bf16_t)(c * a - sv * b);
+          rb[e] = (bf16_t)(sv * a + c * b);
+        }
+        if (head < nq) {
+          *(bf16x8*)(h + j) = ra;
+          *(bf16x8*)(h + j + half) = rb;
+        } else if (slot >= 0) {
+          bf16_t* dst = (bf16_t*)k_cache + ((blk * nkv + (head - nq)) * block_size + in_blk) * hd;
+          *(bf16x8*)(dst + j) = ra;
+          *(bf16x8*)(dst + j + half) = rb;
+        }
+      }
+      if (slot < 0) return;
+      for (int i = threadIdx.x; i < nkv * hd / 8; i += kThreads) {
+        const int head = (i * 8) / hd, j = i * 8 - head * hd;
+        *(bf16x8*)((bf16_t*)v_cache + ((blk * nkv + head) * block_size + in_blk) * hd + j) =
+            *(const bf16x8*)((const bf16_t*)row + (int64_t)(nq + nkv + head) * hd + j);
+      }
+      return;
+    }
+  }
   // rotated pairs of q and k heads
   const int pairs = (nq + nkv) * half;
   for (int i = threadIdx.x; i < pairs; i += kThreads) {
