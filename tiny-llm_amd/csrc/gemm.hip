@@ -419,7 +419,7 @@ static int launch_gemm_bf16_tile(int c, const bf16_t* a, const bf16_t* w, TO* ou
       return launch_gemm_bf16<256, 128, 4, 2, TO, SWIGLU>(a, w, out, residual, row_scale, M, N, K, lda, ldo, k_per_split,
                                                           stream);
     case 2:
-      return launch_gemm_bf16<128, 128, 2, 2, TO, SWIGLU>(a, w, out, residual, row_scale, M, N, K, lda, ldo, k_per_split,
+      return launch_gemm_bf16<128, 128, 4, 2, TO, SWIGLU>(a, w, out, residual, row_scale, M, N, K, lda, ldo, k_per_split,
                                                           stream);
     default:
       return launch_gemm_bf16<64, 128, 2, 2, TO, SWIGLU>(a, w, out, residual, row_scale, M, N, K, lda, ldo, k_per_split,
