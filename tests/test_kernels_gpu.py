@@ -229,6 +229,33 @@ def test_linear_handoff(M, K, N, N2):
                              rows=torch.arange(65, dtype=torch.int32, device=DEV))
 
 
+@pytest.mark.parametrize("M,K,N", [(2048, 64, 8576), (1000, 136, 16390)])
+def test_linear_two_part_launch(M, K, N):
+    """Wide products are launched in two parts (whole rounds of the largest tile, then the rest with
+    another tile): every epilogue must land in the right columns of both parts."""
+    g = torch.Generator().manual_seed(N)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    res = torch.randn(M, N, generator=g)
+    scale = torch.rand(M, generator=g) + 0.5
+    ref = a.double() @ w.double().T
+    out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops().linear(a.to(DEV), w.to(DEV), out)
+    assert rel(out, ref) < 6e-3
+    x = res.clone().to(DEV)
+    ops().linear(a.to(DEV), w.to(DEV), x, x, row_scale=scale.to(DEV))
+    assert rel(x, ref * scale.double()[:, None] + res.double()) < 1e-5
+    z = torch.full((M, N // 2), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops().linear(a.to(DEV), w.to(DEV), z, epilogue="swiglu")
+    assert rel(z, plain.silu(ref[:, 0::2]) * ref[:, 1::2]) < 6e-3
+    # the same values as one launch with one tile shape
+    one = torch.empty(M, N, dtype=torch.float32, device=DEV)
+    two = torch.empty(M, N, dtype=torch.float32, device=DEV)
+    ops().linear(a.to(DEV), w.to(DEV), one, tile=3)
+    ops().linear(a.to(DEV), w.to(DEV), two)
+    assert rel(two, one.double()) < 1e-6
+
+
 @pytest.mark.parametrize("M", [17, 64, 65, 200, 512])
 @pytest.mark.parametrize("K,N", [(5632, 2048), (2048, 4100), (1096, 518)])
 def test_linear_split_k(M, K, N):
