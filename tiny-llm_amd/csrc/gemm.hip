@@ -662,7 +662,9 @@ __device__ __forceinline__ bf16x8 skinny_operand(const SkinnyChunk<PRO_NORM>& c,
   return r;
 }
 
-template <int MT, int CT, typename TO, int PRO, bool SWIGLU>
+// DEEP: two register stages also with one tile, for long inner sizes, where a wave works through
+// several stages and the chain of their memory round trips sets the kernel's duration.
+template <int MT, int CT, bool DEEP, typename TO, int PRO, bool SWIGLU>
 __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const SkinnyArgs p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char skinny_smem[];
   typedef float Tile[16][17];
@@ -737,7 +739,7 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
   // load would become a branch and the stages could not overlap.  Rows beyond M or N only feed
   // outputs that are never written; a chunk beyond K is zeroed on the weight side when it is used.
   constexpr int UN = TILES == 1 ? 2 : 1;
-  constexpr bool TWO_STAGES = TILES > 1 && MT + CT <= 5;
+  constexpr bool TWO_STAGES = DEEP || (TILES > 1 && MT + CT <= 5);
   struct Stage {
     bf16x8 fw[UN][CT][4];
     SkinnyChunk<PRO> fa[UN][MT][4];
@@ -891,19 +893,27 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
 
 // Column tiles per workgroup: every workgroup reads all M activation rows, so with more rows it
 // should own more columns, or the activations are read more often than the weights.
-template <int MT, int CT, typename TO, int PRO, bool SWIGLU>
-static int launch_skinny_tile(const SkinnyArgs& p, hipStream_t stream) {
+template <int MT, int CT, bool DEEP, typename TO, int PRO, bool SWIGLU>
+static int launch_skinny_deep(const SkinnyArgs& p, hipStream_t stream) {
   constexpr size_t smem = (size_t)S_WAVES * MT * CT * 16 * 17 * sizeof(float) + (size_t)(S_WAVES + 1) * MT * 16 * sizeof(float);
   static bool configured = false;
   if (!configured) {
-    if (hipFuncSetAttribute((const void*)gemm_skinny_bf16_kernel<MT, CT, TO, PRO, SWIGLU>,
+    if (hipFuncSetAttribute((const void*)gemm_skinny_bf16_kernel<MT, CT, DEEP, TO, PRO, SWIGLU>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
       return TL_ERR_LAUNCH;
     configured = true;
   }
   dim3 g((p.N + S_COLS * CT - 1) / (S_COLS * CT)), b(S_THREADS);
-  hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, CT, TO, PRO, SWIGLU>), g, b, smem, stream, p);
+  hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, CT, DEEP, TO, PRO, SWIGLU>), g, b, smem, stream, p);
   return TL_OK;
+}
+
+template <int MT, int CT, typename TO, int PRO, bool SWIGLU>
+static int launch_skinny_tile(const SkinnyArgs& p, hipStream_t stream) {
+  if constexpr (MT * CT == 1 && PRO == PRO_NONE) {
+    if (p.K > 4096) return launch_skinny_deep<MT, CT, true, TO, PRO, SWIGLU>(p, stream);
+  }
+  return launch_skinny_deep<MT, CT, false, TO, PRO, SWIGLU>(p, stream);
 }
 
 // More column tiles only while at least 256 workgroups remain: fewer cannot pull the weights
