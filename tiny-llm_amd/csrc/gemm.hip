@@ -884,7 +884,8 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
           float sq = valid ? v * v : 0.f;
 #pragma unroll
           for (int off = 1; off < 16; off <<= 1) sq += __shfl_xor(sq, off, TL_WAVE);
-          if (nn == 0 && m < M) p.emit_sumsq[(int64_t)m * ((N + 15) / 16) + (n0 / 16 + tile % CT)] = sq;
+          // a column group that begins beyond N has no part of its own
+          if (nn == 0 && m < M && n < N) p.emit_sumsq[(int64_t)m * ((N + 15) / 16) + (n0 / 16 + tile % CT)] = sq;
         }
       }
     }
