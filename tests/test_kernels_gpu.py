@@ -99,7 +99,7 @@ def test_lm_head_last_rows_reference_vector():
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,K,N", [(127, 255, 353), (1, 64, 251), (7, 176, 64), (130, 96, 517), (64, 2048, 256),
-                                   (300, 5632, 136)])
+                                   (300, 5632, 136), (9, 5640, 520), (16, 4104, 40)])
 def test_linear_sizes(dtype, M, K, N):
     if dtype == torch.bfloat16 and K % 8:
         K = K + 8 - K % 8
