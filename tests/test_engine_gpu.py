@@ -2,6 +2,7 @@
 seeded sampling, preemption, and a toy architecture with a stateful mixer that is
 registered here, in the test, without touching the framework's files."""
 import math
+import json
 import os
 import subprocess
 import sys
@@ -248,6 +249,31 @@ def test_command_line_generates_from_prompt_ids(folders):
     bad = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "tiny_llm"), "--model_path", "/nonexistent"],
                          capture_output=True, text=True, timeout=120)
     assert bad.returncode == 1 and "[Fatal]" in bad.stderr
+
+
+def test_command_line_random_weights_and_prompt_file(tmp_path):
+    """--random_weights takes only config.json from the folder and fills the weights on the device
+    from --weights_seed, as the Python entry point does for a configuration; --prompt_ids_file
+    holds one prompt a line."""
+    from tiny_llm_amd import Engine, SamplingParams
+    cfg = CONFIGS["A"][0]
+    only_config = tmp_path / "only_config"
+    only_config.mkdir()
+    with open(only_config / "config.json", "w") as f:
+        json.dump(cfg, f)
+    prompts = [random_tokens(9, cfg["vocab_size"], 21), random_tokens(14, cfg["vocab_size"], 22)]
+    ids_file = tmp_path / "prompts.txt"
+    ids_file.write_text("\n".join(" ".join(map(str, p)) for p in prompts) + "\n")
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "tiny_llm"), "--model_path", str(only_config),
+                           "--random_weights", "--weights_seed=11", "--init_std=0.05", "--nodo_sample",
+                           "--max_new_tokens=4", "--dtype", "float32", "--ignore_eos",
+                           "--prompt_ids_file", str(ids_file)], capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    got = [[int(t) for t in line.split()] for line in proc.stdout.strip().splitlines()[-2:]]
+    engine = Engine(config=cfg, dtype="float32", weights_seed=11, init_std=0.05)
+    assert got == engine.generate(prompts, SamplingParams.greedy(4, ignore_eos=True))
+    other = Engine(config=cfg, dtype="float32", weights_seed=12, init_std=0.05)
+    assert got != other.generate(prompts, SamplingParams.greedy(4, ignore_eos=True))
 
 
 # ------------------------------------------------------ a toy architecture

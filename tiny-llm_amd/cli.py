@@ -27,6 +27,10 @@ FLAGS: Dict[str, Tuple[type, Any, str]] = {
     "dtype": (str, "bfloat16", "bfloat16 (serving) or float32 (true 32-bit path)"),
     "seed": (int, 0, "Seed of the sampling random numbers"),
     "prompt_ids": (str, "", "Token ids of one prompt (\"1,2,3\"): generate once and exit"),
+    "prompt_ids_file": (str, "", "File with one prompt of token ids per line: generate for all of them and exit"),
+    "random_weights": (bool, False, "Take only config.json from --model_path and fill the weights from --weights_seed"),
+    "weights_seed": (int, 0, "Seed of the random weights"),
+    "init_std": (float, 0.0, "Standard deviation of the random matrices (0: the configuration's initializer_range)"),
     "ignore_eos": (bool, False, "Keep generating after the end-of-sequence token"),
     "kv_block_size": (int, 16, "Tokens per cache page"),
     "num_kv_blocks": (int, 0, "Cache pages (0: enough for max_num_seqs full-length requests)"),
@@ -137,14 +141,26 @@ def main(argv: List[str] = None) -> int:
                            num_kv_blocks=flags["num_kv_blocks"] or None, max_num_seqs=flags["max_num_seqs"],
                            max_num_batched_tokens=flags["max_num_batched_tokens"], device=flags["device"],
                            seed=flags["seed"])
-        engine = Engine(flags["model_path"], engine_config=cfg)
+        if flags["random_weights"]:
+            import json
+            import os
+            with open(os.path.join(flags["model_path"], "config.json")) as f:
+                raw = json.load(f)
+            engine = Engine(config=raw, engine_config=cfg, weights_seed=flags["weights_seed"],
+                            init_std=flags["init_std"] or None)
+        else:
+            engine = Engine(flags["model_path"], engine_config=cfg)
         text = _Text(flags["model_path"])
         params = SamplingParams(max_new_tokens=flags["max_new_tokens"], do_sample=flags["do_sample"],
                                 temperature=flags["temperature"], top_k=flags["top_k"], top_p=flags["top_p"],
                                 ignore_eos=flags["ignore_eos"])
-        if flags["prompt_ids"]:
-            out = engine.generate([parse_ids(flags["prompt_ids"])], params)[0]
-            print(text.decode(out))
+        if flags["prompt_ids"] or flags["prompt_ids_file"]:
+            prompts = [parse_ids(flags["prompt_ids"])] if flags["prompt_ids"] else []
+            if flags["prompt_ids_file"]:
+                with open(flags["prompt_ids_file"]) as f:
+                    prompts += [parse_ids(line) for line in f if line.strip()]
+            for out in engine.generate(prompts, params):
+                print(text.decode(out))
             return 0
         print("\n>>> [Page Mode] Interactive Mode (Multi-line enabled) <<<")
         print(">>> Enter your prompt. Enter a blank line to end the current input. "
