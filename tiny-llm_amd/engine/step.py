@@ -15,7 +15,7 @@ kernels need no search over sequence separators (tiny_llm/ops/details.hpp:19-36)
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Dict, Hashable, List, Optional, Sequence
+from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
@@ -96,7 +96,7 @@ class ModelRunner:
             decoder.states[i] = cache.states[i]
         self._pinned: Optional[torch.Tensor] = None
         self._uploaded: Optional[torch.cuda.Event] = None
-        self._graphs: Dict[int, "DecodeGraph"] = {}
+        self._graphs: Dict[Tuple[int, int], "DecodeGraph"] = {}
 
     # ----------------------------------------------------------------- metadata
     def _host_buffer(self, n: int) -> torch.Tensor:
@@ -216,9 +216,15 @@ class ModelRunner:
             if (cm.num_tokens(rid) if cm.has(rid) else 0) + 1 > self.max_model_len:
                 raise StepError(f"request {rid!r} would exceed {self.max_model_len} tokens")
         ctx_lens = cm.reserve_step([(rid, 1) for rid in req_ids])
-        dg = self._graphs.get(R)
+        # One graph per batch size and context bound: the bound (a power of two, at least 512) decides
+        # into how many workgroups the attention kernel splits a request's keys, which is fixed at capture.
+        bound = 512
+        while bound < max(ctx_lens) + 1:
+            bound *= 2
+        bound = min(bound, self.max_model_len)
+        dg = self._graphs.get((R, bound))
         if dg is None:
-            dg = self._graphs[R] = DecodeGraph(self, R)
+            dg = self._graphs[(R, bound)] = DecodeGraph(self, R, bound)
         toks = dg.run(req_ids, tokens, ctx_lens, params, seeds, counters,
                       capture=use_graph and self.decoder.graph_safe)
         for rid, c in zip(req_ids, ctx_lens):
@@ -232,15 +238,16 @@ class ModelRunner:
 
 
 class DecodeGraph:
-    """Static buffers and the captured HIP graph of a decode-only step of `R` requests.
+    """Static buffers and the captured HIP graph of a decode-only step of `R` requests whose
+    contexts stay within `max_seq_len` tokens.
 
-    Everything whose size depends on the step (block-table width, key splits of the attention
-    kernel) is fixed at its maximum, so one capture serves every step of that batch size.  The
+    The block-table width is fixed at its maximum and the key splits of the attention kernel follow
+    `max_seq_len`, so one capture serves every step of that batch size and context bound.  The
     first run of a size executes eagerly (kernels configure themselves, the allocator warms up);
     the second is captured; later ones are replayed.  No memset node is recorded: buffers are
     written by kernels and by the upload only."""
 
-    def __init__(self, runner: ModelRunner, R: int):
+    def __init__(self, runner: ModelRunner, R: int, max_seq_len: int):
         self.runner, self.R = runner, R
         cm = runner.cache
         dev = runner.device
@@ -268,7 +275,7 @@ class DecodeGraph:
             block_tables=[sec(7 + G + g, R * MB).view(R, MB) for g in range(G)],
             slot_mappings=[sec(7 + g, R) for g in range(G)],
             q_lens=[1] * R, context_lens=[0] * R, slots_host=[0] * R, max_q_len=1,
-            max_seq_len=runner.max_model_len, block_size=bs)
+            max_seq_len=max_seq_len, block_size=bs)
         s0 = 7 + 2 * G
         self.temperature = sec(s0, R).view(torch.float32)
         self.top_p = sec(s0 + 1, R).view(torch.float32)
