@@ -11,8 +11,6 @@ from __future__ import annotations
 import itertools
 from typing import Dict, Hashable, List, Mapping, Optional, Sequence, Union
 
-import torch
-
 from ..config import EngineConfig
 from ..sampling import Sampler, SamplingParams
 from .loading import build_runner, load_model, random_model

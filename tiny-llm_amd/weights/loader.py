@@ -22,7 +22,7 @@ from typing import Callable, Dict, Iterable, List, Mapping, Optional, Sequence, 
 import torch
 
 from ..parts.base import WeightSpec
-from .safetensors_io import SafetensorsError, SafetensorsFile, open_model_files, save_file
+from .safetensors_io import SafetensorsFile, open_model_files, save_file
 
 # tensors that checkpoints of this family carry and no part needs
 IGNORABLE = ("*.rotary_emb.inv_freq",)
