@@ -374,3 +374,113 @@ def test_toy_stateful_mixer_registers_builds_and_steps(tmp_path):
     finally:
         MIXERS.unregister("toy_decay")
         unregister_architecture("ToyForCausalLM")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_routed_feed_forward_and_other_position_encoding(dtype):
+    """A feed-forward with routing (two experts, the larger router logit takes the token) and a
+    position encoding of its own (a rotation of the first half of each head with doubled angles),
+    both defined here, in a toy architecture: registered, built, and stepped in different cuttings."""
+    from tiny_llm_amd.config import (EngineConfig, LayerSpec, ModelSpec, PartSpec, PlanEntry, register_architecture,
+                                     unregister_architecture)
+    from tiny_llm_amd.engine.loading import build_runner, random_model
+    from tiny_llm_amd.engine.step import StepEntry
+    from tiny_llm_amd.kernels import ops
+    from tiny_llm_amd.parts import (FEED_FORWARDS, POSITION_ENCODINGS, FeedForward, PositionEncoding, WeightSpec,
+                                    add_to_residual, register_feed_forward, register_position_encoding)
+
+    class DoubledHalfRotary(PositionEncoding):
+        def __init__(self, prefix, dtype, device, *, head_dim, max_position):
+            super().__init__(prefix, dtype, device)
+            self.rot = head_dim // 2
+            inv = torch.pow(torch.tensor(50.0, dtype=torch.float64), -torch.arange(self.rot // 2, dtype=torch.float64)
+                            / (self.rot // 2))
+            ang = 2.0 * torch.arange(max_position, dtype=torch.float64)[:, None] * inv[None, :]
+            self.cos, self.sin = torch.cos(ang).float().to(device), torch.sin(ang).float().to(device)
+
+        def rotary_tables(self):
+            return self.cos, self.sin, self.rot
+
+    used = set()
+
+    class TwoExperts(FeedForward):
+        def __init__(self, prefix, dtype, device, *, hidden_size, intermediate_size):
+            super().__init__(prefix, dtype, device)
+            self.H, self.I = hidden_size, intermediate_size
+
+        def weights(self):
+            w = [WeightSpec(f"{self.prefix}.router.weight", (2, self.H))]
+            for e in range(2):
+                w += [WeightSpec(f"{self.prefix}.experts.{e}.up.weight", (self.I, self.H)),
+                      WeightSpec(f"{self.prefix}.experts.{e}.down.weight", (self.H, self.I))]
+            return w
+
+        def bind(self, tensors):
+            self.router = tensors[f"{self.prefix}.router.weight"].float()
+            self.up = [tensors[f"{self.prefix}.experts.{e}.up.weight"].contiguous() for e in range(2)]
+            self.down = [tensors[f"{self.prefix}.experts.{e}.down.weight"].contiguous() for e in range(2)]
+
+        def forward(self, h, ctx, residual):
+            choice = (h.float() @ self.router.T).argmax(dim=-1)          # router logits in float32
+            y = torch.zeros_like(residual)
+            for e in range(2):
+                rows = (choice == e).nonzero().flatten()
+                if rows.numel() == 0:
+                    continue
+                used.add(e)
+                mid = torch.empty((rows.numel(), self.I), dtype=h.dtype, device=h.device)
+                ops.linear(h[rows].contiguous(), self.up[e], mid)
+                out = torch.empty((rows.numel(), self.H), dtype=torch.float32, device=h.device)
+                ops.linear(torch.relu(mid), self.down[e], out)
+                y[rows] = out
+            return add_to_residual(residual, y)
+
+    def build(cfg):
+        H = cfg["hidden_size"]
+        norm = PartSpec("rmsnorm", {"hidden_size": H, "eps": 1e-5})
+        attn = PartSpec("attention", {"hidden_size": H, "num_heads": 4, "num_kv_heads": 1, "head_dim": 16,
+                                      "position": {"kind": "doubled_half_rotary", "head_dim": 16, "max_position": 256}})
+        dense = PartSpec("swiglu", {"hidden_size": H, "intermediate_size": 96})
+        routed = PartSpec("two_experts", {"hidden_size": H, "intermediate_size": 40})
+        layers = (LayerSpec("model.layers.0", "pre_norm", norm, attn, norm, routed),
+                  LayerSpec("model.layers.1", "pre_norm", norm, attn, norm, dense))
+        return ModelSpec("Toy2ForCausalLM", cfg["vocab_size"], H, 256,
+                         PartSpec("token_embedding", {"vocab_size": cfg["vocab_size"], "hidden_size": H}), layers,
+                         (PlanEntry(0), PlanEntry(1)), norm,
+                         PartSpec("lm_head", {"vocab_size": cfg["vocab_size"], "hidden_size": H, "tied": True}))
+
+    register_position_encoding("doubled_half_rotary", DoubledHalfRotary)
+    register_feed_forward("two_experts", TwoExperts)
+    register_architecture("Toy2ForCausalLM", dict, build)
+    try:
+        raw = {"architectures": ["Toy2ForCausalLM"], "hidden_size": 64, "vocab_size": 101}
+        engine = EngineConfig(dtype=dtype, kv_block_size=8, max_cache_tokens=256, max_num_seqs=3,
+                              max_num_batched_tokens=256, use_graphs=False)
+        _, dec = random_model(raw, engine, seed=3, std=0.3)
+        runner = build_runner(dec, engine)
+        a, b = random_tokens(41, 101, 5), random_tokens(18, 101, 6)
+        whole = runner.step([StepEntry("a", a, list(range(41))), StepEntry("b", b, list(range(18)))]).cpu()
+        assert used == {0, 1}                       # both experts got tokens
+        runner.finish("a")
+        runner.finish("b")
+        got_a, got_b, at_a, at_b = [], [], 0, 0
+        for na, nb in [(9, 3), (2, 0), (14, 6), (1, 1), (15, 8)]:
+            ents = [StepEntry("a", a[at_a:at_a + na], list(range(na)))] if na else []
+            if nb:
+                ents.append(StepEntry("b", b[at_b:at_b + nb], list(range(nb))))
+            l = runner.step(ents).cpu()
+            got_a.append(l[:na])
+            got_b.append(l[na:])
+            at_a, at_b = at_a + na, at_b + nb
+        tol = 1e-5 if dtype == "float32" else 2e-2
+        assert rel_err(torch.cat(got_a), whole[:41]) < tol and rel_err(torch.cat(got_b), whole[41:]) < tol
+        # the position encoding matters: a shift of the positions' angles changes the logits
+        for layer in dec.layers:
+            layer.mixer.position.cos, layer.mixer.position.sin = layer.mixer.position.sin, layer.mixer.position.cos
+        runner.finish("a")
+        runner.finish("b")
+        assert rel_err(runner.step([StepEntry("c", a, list(range(41)))]).cpu(), whole[:41]) > 1e-3
+    finally:
+        FEED_FORWARDS.unregister("two_experts")
+        POSITION_ENCODINGS.unregister("doubled_half_rotary")
+        unregister_architecture("Toy2ForCausalLM")
