@@ -410,6 +410,20 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
   }
 }
 
+// Two probabilities as two bfloat16 terms each, p = hi + lo, packed pairwise.  hi is p with the low
+// 16 bits cut off (exact, one mask), lo = p - hi is exact in float32 and rounded to bfloat16: the
+// pair carries 16 bits of p, as rounding hi would, for three vector instructions a value
+// instead of four.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void split_pair(float pa, float pc, uint32_t& hi, uint32_t& lo) {
+  const uint32_t ba = __float_as_uint(pa), bc = __float_as_uint(pc);
+  hi = __builtin_amdgcn_perm(bc, ba, 0x07060302u);          // upper halves of both, a in the low word
+  const f32x2 rest = {pa - __uint_as_float(ba & 0xffff0000u), pc - __uint_as_float(bc & 0xffff0000u)};
+  lo = __builtin_bit_cast(uint32_t, __builtin_convertvector(rest, bf16x2));
+}
+
 // flash_prefill_bf16_kernel: the same mathematics arranged for prompt portions.  A workgroup
 // owns up to 8 query tiles (one per wave, 128 rows: for 8 heads per kv head that is 16 tokens) of
 // consecutive tokens of one request, and all eight waves work on the SAME 64-key tile, staged and
@@ -642,15 +656,20 @@ __global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
             for (int r = 0; r < 4; ++r) o[rt][dt][r] *= alpha;
         }
 #pragma unroll
-        for (int st = 0; st < 2; ++st)
+        for (int st = 0; st < 2; ++st) {
+          u32x4 hi_w, lo_w;
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const float p0 = sc[rt][2 * st][r], p1 = sc[rt][2 * st + 1][r];
-            pb[rt][st][r] = (bf16_t)p0;
-            pb[rt][st][4 + r] = (bf16_t)p1;
-            pl[rt][st][r] = (bf16_t)(p0 - (float)pb[rt][st][r]);
-            pl[rt][st][4 + r] = (bf16_t)(p1 - (float)pb[rt][st][4 + r]);
+          for (int w = 0; w < 4; ++w) {
+            // probabilities 2w and 2w + 1 of this step (two of key block 2 st, then two of 2 st + 1)
+            const float pa = sc[rt][2 * st + w / 2][(w % 2) * 2], pc = sc[rt][2 * st + w / 2][(w % 2) * 2 + 1];
+            uint32_t hi, lo;
+            split_pair(pa, pc, hi, lo);
+            hi_w[w] = hi;
+            lo_w[w] = lo;
           }
+          pb[rt][st] = __builtin_bit_cast(bf16x8, hi_w);
+          pl[rt][st] = __builtin_bit_cast(bf16x8, lo_w);
+        }
       }
       bf16x8 vfr[2][HDT];
 #pragma unroll
