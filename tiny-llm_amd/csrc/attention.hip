@@ -499,12 +499,17 @@ __global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
 
   // The running maximum starts at a large negative FINITE number, so exp2(m - m') is never
   // exp2(-inf + inf); a masked score is -inf and its probability exp2(-inf) = 0.
-  float m_run[FP_RT], l_run[FP_RT];
+  // The softmax denominator is accumulated by the matrix cores: a row of ones beside V^T adds up
+  // the very probabilities (both bfloat16 terms) that enter the output, in an accumulator of its
+  // own, which is rescaled with the output.  That saves the adds and two cross-lane exchanges per
+  // key tile, and numerator and denominator see the same rounding.
+  float m_run[FP_RT];
+  f32x4 l_acc[FP_RT];
   f32x4 o[FP_RT][HDT];
 #pragma unroll
   for (int rt = 0; rt < FP_RT; ++rt) {
     m_run[rt] = kNegBig;
-    l_run[rt] = 0.f;
+    l_acc[rt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int dt = 0; dt < HDT; ++dt) o[rt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
@@ -636,24 +641,18 @@ __global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
         // the maximum is taken over raw scores (the scale is positive) and scaled once
         const float m_new = fmaxf(m_run[rt], m_tile * c_log2);
         const float alpha = __builtin_amdgcn_exp2f(m_run[rt] - m_new);
-        float psum = 0.f;
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const float p = __builtin_amdgcn_exp2f(fmaf(sc[rt][kt][r], c_log2, -m_new));
-            sc[rt][kt][r] = p;
-            psum += p;
-          }
-        psum += __shfl_xor(psum, 16, TL_WAVE);
-        psum += __shfl_xor(psum, 32, TL_WAVE);
-        l_run[rt] = l_run[rt] * alpha + psum;
+          for (int r = 0; r < 4; ++r) sc[rt][kt][r] = __builtin_amdgcn_exp2f(fmaf(sc[rt][kt][r], c_log2, -m_new));
         m_run[rt] = m_new;
         if (__any(alpha != 1.f)) {
 #pragma unroll
           for (int dt = 0; dt < HDT; ++dt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) o[rt][dt][r] *= alpha;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) l_acc[rt][r] *= alpha;
         }
 #pragma unroll
         for (int st = 0; st < 2; ++st) {
@@ -687,24 +686,32 @@ __global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
           }
           vfr[st][dt] = vf;
         }
-      // the four products into one accumulator are kept four MFMAs apart
+      // the four products into one accumulator are kept at least four MFMAs apart
+      bf16x8 ones;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ones[e] = (bf16_t)1.f;
 #pragma unroll
       for (int st = 0; st < 2; ++st)
 #pragma unroll
-        for (int lo = 0; lo < 2; ++lo)
+        for (int lo = 0; lo < 2; ++lo) {
 #pragma unroll
           for (int dt = 0; dt < HDT; ++dt)
 #pragma unroll
             for (int rt = 0; rt < FP_RT; ++rt)
               o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vfr[st][dt], lo ? pl[rt][st] : pb[rt][st], o[rt][dt],
                                                                   0, 0, 0);
+#pragma unroll
+          for (int rt = 0; rt < FP_RT; ++rt)
+            l_acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, lo ? pl[rt][st] : pb[rt][st], l_acc[rt], 0, 0, 0);
+        }
     }
     __syncthreads();
   }
 #pragma unroll
   for (int rt = 0; rt < FP_RT; ++rt) {
     if (!row_valid[rt]) continue;
-    const float inv = l_run[rt] > 0.f ? 1.f / l_run[rt] : 0.f;
+    const float l = l_acc[rt][0];         // every element of the lane's column holds the row's sum
+    const float inv = l > 0.f ? 1.f / l : 0.f;
     bf16_t* orow = out + (int64_t)tok[rt] * out_stride + (int64_t)head * HD + g * 4;
 #pragma unroll
     for (int dt = 0; dt < HDT; ++dt) {
