@@ -92,22 +92,50 @@ __global__ __launch_bounds__(TL_WAVE) void paged_attention_kernel(
 // flash_attn_bf16_kernel: the same function on the matrix cores, for head sizes
 // that are multiples of 16 up to 128 and up to 16 query heads per kv head.
 //
-// A workgroup (eight wave64, four for wide heads) owns a tile of 16 query rows that share one
-// request and one kv head: `tile_ntok` consecutive tokens times the G query heads of the group,
-// row = token * G + head.  The waves split the 64-key tiles of the request's
+// A workgroup (eight wave64) owns a tile of 16 query rows that
+// share one request and one kv head: `tile_ntok` consecutive tokens times the G query heads of the
+// group, row = token * G + head.  The waves split the 64-key tiles of the request's
 // cache between them (and `n_splits` workgroups split them further for decoding
-// with few requests), each with a private LDS staging area, and merge their running
-// (max, sum, output) at the end.  Scores are computed transposed, S^T = K Q^T, with
+// with few requests) and merge their running (max, sum, output) at the end.  A wave reads its
+// tile by itself: keys straight from memory into MFMA operands, values through a private LDS
+// area.  (Sixteen waves a workgroup were measured slower at every context length: what a compute
+// unit can have in flight is the limit, so keys are better spread over more workgroups.)
+// Scores are computed transposed, S^T = K Q^T, with
 // v_mfma_f32_16x16x32_bf16: a lane then holds 16 scores of ONE query row, so the
 // online softmax is lane-local up to two shuffles, the probabilities are already in
 // the B-operand layout of the second product O^T = V^T P^T, and the output
 // accumulator of a lane belongs to that same row.  The probabilities enter the second
 // product as a sum of two bfloat16 terms, so no accuracy is lost against a float32
 // softmax times bfloat16 values.  V is transposed on its way into
-// LDS.  Rows of a tile outside [kv_begin, kv_end) are zero-filled instead of read:
+// LDS.  Rows of a tile outside [kv_begin, kv_end) are zeroed:
 // stale pages may hold anything, and 0 * NaN is NaN.
-constexpr int FA_THREADS = 256, FA_WAVES = 4, FA_KT = 64, FA_VP = 68;
+constexpr int FA_KT = 64, FA_VP = 68;
+constexpr int FA_VPAD = 8;      // padding of a row of the row-major V tile of the decode kernel (elements)
 constexpr float kNegBig = -1.0e30f;   // "no key yet": finite, so exp2(m - m') never sees inf - inf
+
+// Two probabilities as two bfloat16 terms each, p = hi + lo, packed pairwise.  hi is p with the low
+// 16 bits cut off (exact, one mask), lo = p - hi is exact in float32 and rounded to bfloat16: the
+// pair carries 16 bits of p, as rounding hi would, for three vector instructions a value
+// instead of four.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void split_pair(float pa, float pc, uint32_t& hi, uint32_t& lo) {
+  const uint32_t ba = __float_as_uint(pa), bc = __float_as_uint(pc);
+  hi = __builtin_amdgcn_perm(bc, ba, 0x07060302u);          // upper halves of both, a in the low word
+  const f32x2 rest = {pa - __uint_as_float(ba & 0xffff0000u), pc - __uint_as_float(bc & 0xffff0000u)};
+  lo = __builtin_bit_cast(uint32_t, __builtin_convertvector(rest, bf16x2));
+}
+
+// The LDS transpose load of gfx950 (ds_read_b64_tr_b16).  The 16 lanes of a group each name four
+// consecutive 16-bit elements; lane i of the group receives element i % 4 of the four chunks named
+// by lanes i / 4, 4 + i / 4, 8 + i / 4 and 12 + i / 4.  With lane s naming V[key0 + s / 4][d0 + 4 * (s % 4) ..]
+// of a row-major tile, lane i gets V[key0 .. key0 + 3][d0 + i]: four consecutive keys of one dim,
+// half an MFMA operand of V^T, without the tile ever being stored transposed.
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ bf16x4 lds_read_transposed(const bf16_t* p) {
+  return __builtin_bit_cast(bf16x4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)p));
+}
 
 // Optional fusion for decode steps (every tile is ONE new token): the query and the new key are
 // rotated here and the new key and value are written to the cache here, instead of by a kernel of
@@ -149,9 +177,8 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
     int block_size, float scale, int window, int n_splits, int n_tokens, const FusedRope fused) {
   constexpr int HD = HDT * 16;
   constexpr int KS = (HD + 31) / 32;       // k-steps of the score product
-  constexpr int KP = KS * 32 + 8;          // LDS row stride of the K tile (elements)
-  constexpr int K_ELEMS = FA_KT * KP, V_ELEMS = HD * FA_VP;
-  constexpr int WAVE_ELEMS = K_ELEMS + V_ELEMS;
+  constexpr int VS = HD + FA_VPAD;         // row stride of a wave's V tile in LDS
+  constexpr int WAVE_ELEMS = FA_KT * VS;   // a wave's LDS area: its V tile, [key][dim]
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   bf16_t* smem = (bf16_t*)smem_raw;
 
@@ -161,13 +188,18 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
   const int G = nq / nkv;
   const int req = tile_req[tile], tok0 = tile_tok0[tile], ntok = tile_ntok[tile];
   const int32_t* bt = block_tables + (int64_t)req * max_blocks;
-  bf16_t* Kl = smem + wave * WAVE_ELEMS;
-  bf16_t* Vl = Kl + K_ELEMS;
+  bf16_t* Vl = smem + wave * WAVE_ELEMS;
   const bool do_rope = fused.cos_t != nullptr;
   // Key tiles are dealt out in turn (see below), so without a window this wave's first tile is
-  // known here: the page of this lane's row in it is requested together with the position.  The
-  // index is clamped into the table; an entry that belongs to no key of the request is not used.
-  const int spec_blk = max(bt[min(((split * WAVES + wave) * FA_KT + lane) / block_size, max_blocks - 1)], 0);
+  // known here: the pages of this lane's rows in it (one value row, four key rows) are requested
+  // together with the position.  The index is clamped into the table; an entry that belongs to no
+  // key of the request is not used.
+  const int spec_j = (split * WAVES + wave) * FA_KT;
+  const int spec_v = max(bt[min((spec_j + lane) / block_size, max_blocks - 1)], 0);
+  int spec_k[4];
+#pragma unroll
+  for (int kt = 0; kt < 4; ++kt)
+    spec_k[kt] = max(bt[min((spec_j + kt * 16 + (lane % 16)) / block_size, max_blocks - 1)], 0);
 
   // this lane's query row
   const int tok_local = r16 / G, hh = r16 % G;
@@ -219,81 +251,120 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
   for (int dt = 0; dt < HDT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   const float c_log2 = scale * 1.44269504088896341f;     // scores are kept in units of log2 e
 
-  // A wave stages its tile in an LDS area of its own (lane = key row), so nothing in this loop
-  // waits for another wave.  The rows of the next tile are requested before the current tile is
-  // worked on.
-  constexpr int KCH = KS * 4, VCH = HD / 8;
-  bf16x8 k_stage[KCH], v_stage[VCH];
-  int64_t stage_off = 0;        // element offset of this lane's row in the caches
-  bool stage_in = false;        // the row is a key of this tile's range
-  auto fetch = [&](int it, int spec_blk) {
-    const int j = ((it0 + it) * stride + mine) * FA_KT + lane;
-    stage_in = j >= kv_begin && j < kv_end;
-    stage_off = 0;
-    if (stage_in) {
-      const int jb = j / block_size;
-      const int64_t blk = spec_blk >= 0 ? spec_blk : bt[jb];
-      stage_off = ((blk * nkv + kvh) * block_size + (j - jb * block_size)) * HD;
-    }
-    const bf16_t* kp = k_cache + stage_off;
-    const bf16_t* vp = v_cache + stage_off;
-    bf16x8 z = {};
-#pragma unroll
-    for (int c = 0; c < KCH; ++c) k_stage[c] = (stage_in && c * 8 < HD) ? *(const bf16x8*)(kp + c * 8) : z;
-#pragma unroll
-    for (int c = 0; c < VCH; ++c) v_stage[c] = stage_in ? *(const bf16x8*)(vp + c * 8) : z;
+  // A wave reads its 64-key tile by itself, so nothing in this loop waits for another wave.  Keys
+  // go straight from memory into MFMA operands (lane (r16, g) holds dims ks*32 + g*8.. of key rows
+  // kt*16 + r16: the layout the score product wants); values pass through an LDS area of the wave's
+  // own (lane = key row), where they are transposed.
+  constexpr int VCH = HD / 8;
+  bf16x8 k_op[4][KS], v_stage[VCH];
+  auto row_offset = [&](int j, int blk) {
+    const int jb = j / block_size;
+    return (((int64_t)blk * nkv + kvh) * block_size + (j - jb * block_size)) * HD;
   };
-  if (iters > 0) fetch(0, it0 == 0 ? spec_blk : -1);
+  // Fused mode: the new token's key is rotated here, by the lanes that will hold its chunks as
+  // operands (in the wave whose tile it falls into), and written to the cache; its value is read
+  // from the qkv row where the loop would read the cache.
+  const int new_tile = new_pos / FA_KT;
+  const bf16_t* new_v = nullptr;
+  int64_t new_off = 0;
+  bf16x8 new_k[KS];
+  if (do_rope) {
+    new_v = q + (int64_t)tok0 * q_stride + fused.v_off + (int64_t)kvh * HD;
+    if (new_tile % stride == mine) {
+      new_off = row_offset(new_pos, bt[new_pos / block_size]);     // the same for every lane
+      if (r16 == new_pos % 16) {
+        const bf16_t* krow = q + (int64_t)tok0 * q_stride + fused.k_off + (int64_t)kvh * HD;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const int d = ks * 32 + g * 8;
+          if (d < HD) {
+            new_k[ks] = rotate_chunk<HD>(*(const bf16x8*)(krow + d), *(const bf16x8*)(krow + (d + HD / 2) % HD), d,
+                                         cs, sn);
+            *(bf16x8*)(fused.k_cache_w + new_off + d) = new_k[ks];
+          }
+        }
+      }
+    }
+  }
+  // Loads are unconditional, with the address clamped into the caches (a row outside the tile's
+  // key range reads row 0 of page 0 and is zeroed afterwards: stale pages may hold anything, and
+  // 0 * NaN is NaN): a predicated load would become a branch, and the loads could not all be in
+  // flight together.
+  auto page_of = [&](int j) { return max(bt[min(j / block_size, max_blocks - 1)], 0); };
+  auto fetch = [&](int it, bool spec) {
+    const int base = ((it0 + it) * stride + mine) * FA_KT;
+    bf16x8 z = {};
+    bool k_in[4];
+    const bf16_t* kp[4];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) {
+      const int j = base + kt * 16 + r16;
+      k_in[kt] = j >= kv_begin && j < kv_end;
+      const int64_t off = row_offset(j, spec ? spec_k[kt] : page_of(j));
+      kp[kt] = k_cache + (k_in[kt] ? off : 0);
+    }
+    const int jv = base + lane;
+    const bool v_in = jv >= kv_begin && jv < kv_end;
+    const int64_t v_off = row_offset(jv, spec ? spec_v : page_of(jv));
+    const bf16_t* vp = v_cache + (v_in ? v_off : 0);
+    if (do_rope && jv == new_pos) vp = new_v;      // not in the cache yet
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) k_op[kt][ks] = *(const bf16x8*)(kp[kt] + min(ks * 32 + g * 8, HD - 8));
+#pragma unroll
+    for (int c = 0; c < VCH; ++c) v_stage[c] = *(const bf16x8*)(vp + c * 8);
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        if (!k_in[kt] || ks * 32 + g * 8 >= HD) k_op[kt][ks] = z;
+#pragma unroll
+    for (int c = 0; c < VCH; ++c)
+      if (!v_in) v_stage[c] = z;
+  };
+  // The next tile is requested as soon as the registers of this one are free.
+  if (iters > 0) {
+    if (it0 == 0) fetch(0, true);
+    else fetch(0, false);
+  }
 
   for (int it = 0; it < iters; ++it) {
     const int kt_idx = (it0 + it) * stride + mine;
-    {
-      const int j = kt_idx * FA_KT + lane;
-      if (do_rope && j == new_pos) {
-        // the new token's own key and value: made here from its qkv row, and written to the cache
-        const bf16_t* krow = q + (int64_t)tok0 * q_stride + fused.k_off + (int64_t)kvh * HD;
-        const bf16_t* vrow = q + (int64_t)tok0 * q_stride + fused.v_off + (int64_t)kvh * HD;
+    if (do_rope && kt_idx == new_tile) {
+      // the new token's own key (rotated above) takes the place of what its cache row held, and its
+      // value, fetched from the qkv row instead of the cache, is written to the cache
+      if (r16 == new_pos % 16) {
 #pragma unroll
-        for (int c = 0; c < KCH; ++c) {
-          if (c * 8 < HD) {
-            k_stage[c] = rotate_chunk<HD>(*(const bf16x8*)(krow + c * 8),
-                                          *(const bf16x8*)(krow + (c * 8 + HD / 2) % HD), c * 8, cs, sn);
-            *(bf16x8*)(fused.k_cache_w + stage_off + c * 8) = k_stage[c];
-          }
-        }
+        for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
-        for (int c = 0; c < VCH; ++c) {
-          v_stage[c] = *(const bf16x8*)(vrow + c * 8);
-          *(bf16x8*)(fused.v_cache_w + stage_off + c * 8) = v_stage[c];
-        }
+          for (int ks = 0; ks < KS; ++ks)
+            if (kt == (new_pos % FA_KT) / 16) k_op[kt][ks] = new_k[ks];
       }
-      // registers -> this wave's LDS area; V is transposed on the way
+      if (lane == new_pos % FA_KT) {
 #pragma unroll
-      for (int c = 0; c < KCH; ++c) *(bf16x8*)(Kl + lane * KP + c * 8) = k_stage[c];
-#pragma unroll
-      for (int c = 0; c < VCH; ++c) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) Vl[(c * 8 + e) * FA_VP + lane] = v_stage[c][e];
+        for (int c = 0; c < VCH; ++c) *(bf16x8*)(fused.v_cache_w + new_off + c * 8) = v_stage[c];
       }
     }
-    if (it + 1 < iters) fetch(it + 1, -1);
+    // values: registers -> this wave's LDS area, as they are (the reads transpose)
+#pragma unroll
+    for (int c = 0; c < VCH; ++c) *(bf16x8*)(Vl + lane * VS + c * 8) = v_stage[c];
+    // scores, transposed: sc[kt][r] = S^T[key kt*16 + g*4 + r][row r16]
+    f32x4 sc[4];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) {
+      sc[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        sc[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_op[kt][ks], qf[ks], sc[kt], 0, 0, 0);
+    }
+    if (it + 1 < iters) fetch(it + 1, false);
     // the LDS operations of one wave are carried out in order; the fences keep the compiler from
     // moving the reads of other lanes' rows above the writes
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     {
-      // scores, transposed: acc[kt][r] = S^T[key kt*16 + g*4 + r][row r16]
-      f32x4 sc[4];
-#pragma unroll
-      for (int kt = 0; kt < 4; ++kt) {
-        sc[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const bf16x8 kf = *(const bf16x8*)(Kl + (kt * 16 + r16) * KP + ks * 32 + g * 8);
-          sc[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], sc[kt], 0, 0, 0);
-        }
-      }
       float m_tile = kNegBig;
 #pragma unroll
       for (int kt = 0; kt < 4; ++kt)
@@ -330,20 +401,24 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
 #pragma unroll
       for (int st = 0; st < 2; ++st) {
         // probabilities as two bfloat16 terms, p = hi + lo: the product then carries 16 bits of p
-        bf16x8 pb, pl;
+        u32x4 hi, lo;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float p0 = sc[2 * st][r], p1 = sc[2 * st + 1][r];
-          pb[r] = (bf16_t)p0;
-          pb[4 + r] = (bf16_t)p1;
-          pl[r] = (bf16_t)(p0 - (float)pb[r]);
-          pl[4 + r] = (bf16_t)(p1 - (float)pb[4 + r]);
+        for (int r = 0; r < 2; ++r) {
+          uint32_t h0, l0, h1, l1;
+          split_pair(sc[2 * st][2 * r], sc[2 * st][2 * r + 1], h0, l0);
+          split_pair(sc[2 * st + 1][2 * r], sc[2 * st + 1][2 * r + 1], h1, l1);
+          hi[r] = h0;
+          lo[r] = l0;
+          hi[2 + r] = h1;
+          lo[2 + r] = l1;
         }
+        const bf16x8 pb = __builtin_bit_cast(bf16x8, hi), pl = __builtin_bit_cast(bf16x8, lo);
+        // lane s of a group names keys g*4 + s/4 of a 16-key block, dims dt*16 + 4*(s%4) ..
+        const bf16_t* vsrc = Vl + ((2 * st) * 16 + g * 4 + r16 / 4) * VS + 4 * (r16 % 4);
 #pragma unroll
         for (int dt = 0; dt < HDT; ++dt) {
-          const bf16_t* vrow = Vl + (dt * 16 + r16) * FA_VP + g * 4;
-          const bf16x4 lo4 = *(const bf16x4*)(vrow + (2 * st) * 16);
-          const bf16x4 hi4 = *(const bf16x4*)(vrow + (2 * st + 1) * 16);
+          const bf16x4 lo4 = lds_read_transposed(vsrc + dt * 16);
+          const bf16x4 hi4 = lds_read_transposed(vsrc + 16 * VS + dt * 16);
           bf16x8 vf;
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
@@ -374,8 +449,8 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
     Mw[r16 * MROW + HD + 1] = l_run;
   }
   __syncthreads();
-  for (int e = tid; e < 16 * 16; e += WAVES * TL_WAVE) {
-    const int row = e / 16, dl = e % 16;
+  for (int e = tid; e < 16 * HD; e += WAVES * TL_WAVE) {      // one output element a thread
+    const int row = e / HD, d = e % HD;
     const int t_local = row / G, h_local = row % G;
     if (t_local >= ntok) continue;
     const int t = tok0 + t_local, h = kvh * G + h_local;
@@ -385,43 +460,25 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
       mw[wv] = ((const float*)(smem + wv * WAVE_ELEMS))[row * MROW + HD];
       M = fmaxf(M, mw[wv]);
     }
-    float L = 0.f, wgt[WAVES];
+    float L = 0.f, acc = 0.f;
 #pragma unroll
     for (int wv = 0; wv < WAVES; ++wv) {
-      wgt[wv] = __builtin_amdgcn_exp2f(mw[wv] - M);      // a wave without keys has l = 0 and O = 0
-      L += wgt[wv] * ((const float*)(smem + wv * WAVE_ELEMS))[row * MROW + HD + 1];
+      const float* area = (const float*)(smem + wv * WAVE_ELEMS) + row * MROW;
+      const float wgt = __builtin_amdgcn_exp2f(mw[wv] - M);      // a wave without keys has l = 0 and O = 0
+      L += wgt * area[HD + 1];
+      acc += wgt * area[d];
     }
-    for (int d = dl; d < HD; d += 16) {
-      float acc = 0.f;
-#pragma unroll
-      for (int wv = 0; wv < WAVES; ++wv)
-        acc += wgt[wv] * ((const float*)(smem + wv * WAVE_ELEMS))[row * MROW + d];
-      if (n_splits == 1) {
-        out[(int64_t)t * out_stride + (int64_t)h * HD + d] = (bf16_t)(L > 0.f ? acc / L : 0.f);
-      } else {
-        part_o[(((int64_t)split * n_tokens + t) * nq + h) * HD + d] = acc;
+    if (n_splits == 1) {
+      out[(int64_t)t * out_stride + (int64_t)h * HD + d] = (bf16_t)(L > 0.f ? acc / L : 0.f);
+    } else {
+      part_o[(((int64_t)split * n_tokens + t) * nq + h) * HD + d] = acc;
+      if (d == 0) {
+        float* ml = part_ml + (((int64_t)split * n_tokens + t) * nq + h) * 2;
+        ml[0] = M;       // in units of log2 e
+        ml[1] = L;
       }
     }
-    if (n_splits > 1 && dl == 0) {
-      float* ml = part_ml + (((int64_t)split * n_tokens + t) * nq + h) * 2;
-      ml[0] = M;       // in units of log2 e
-      ml[1] = L;
-    }
   }
-}
-
-// Two probabilities as two bfloat16 terms each, p = hi + lo, packed pairwise.  hi is p with the low
-// 16 bits cut off (exact, one mask), lo = p - hi is exact in float32 and rounded to bfloat16: the
-// pair carries 16 bits of p, as rounding hi would, for three vector instructions a value
-// instead of four.
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ void split_pair(float pa, float pc, uint32_t& hi, uint32_t& lo) {
-  const uint32_t ba = __float_as_uint(pa), bc = __float_as_uint(pc);
-  hi = __builtin_amdgcn_perm(bc, ba, 0x07060302u);          // upper halves of both, a in the low word
-  const f32x2 rest = {pa - __uint_as_float(ba & 0xffff0000u), pc - __uint_as_float(bc & 0xffff0000u)};
-  lo = __builtin_bit_cast(uint32_t, __builtin_convertvector(rest, bf16x2));
 }
 
 // flash_prefill_bf16_kernel: the same mathematics arranged for prompt portions.  A workgroup
@@ -752,9 +809,9 @@ static int launch_flash_w(const bf16_t* q, int64_t q_stride, const bf16_t* k_cac
                           int64_t out_stride, float* part_o, float* part_ml, int n_tiles, int n_tokens, int nq,
                           int nkv, int block_size, float scale, int window, int n_splits, const FusedRope& fused,
                           hipStream_t stream) {
-  constexpr int HD = HDT * 16, KS = (HD + 31) / 32, KP = KS * 32 + 8;
-  constexpr size_t stage = (size_t)WAVES * (FA_KT * KP + HD * FA_VP) * sizeof(bf16_t);
-  static_assert((size_t)(FA_KT * KP + HD * FA_VP) * sizeof(bf16_t) >= 16 * (HD + 2) * sizeof(float),
+  constexpr int HD = HDT * 16;
+  constexpr size_t stage = (size_t)WAVES * FA_KT * (HD + FA_VPAD) * sizeof(bf16_t);
+  static_assert((size_t)FA_KT * (HD + FA_VPAD) * sizeof(bf16_t) >= 16 * (HD + 2) * sizeof(float),
                 "a wave's merge area must fit its staging area");
   static bool configured = false;
   if (!configured) {
@@ -770,7 +827,8 @@ static int launch_flash_w(const bf16_t* q, int64_t q_stride, const bf16_t* k_cac
   return TL_OK;
 }
 
-// Eight waves share a query tile where their staging areas fit the 160 KB of LDS, else four.
+constexpr int flash_waves(int) { return 8; }
+
 template <int HDT>
 static int launch_flash(const bf16_t* q, int64_t q_stride, const bf16_t* k_cache, const bf16_t* v_cache,
                         const int32_t* block_tables, int max_blocks, const int32_t* tile_req,
@@ -778,16 +836,10 @@ static int launch_flash(const bf16_t* q, int64_t q_stride, const bf16_t* k_cache
                         int64_t out_stride, float* part_o, float* part_ml, int n_tiles, int n_tokens, int nq, int nkv,
                         int block_size, float scale, int window, int n_splits, const FusedRope& fused,
                         hipStream_t stream) {
-  constexpr int HD = HDT * 16, KS = (HD + 31) / 32, KP = KS * 32 + 8;
-  constexpr size_t per_wave = (size_t)(FA_KT * KP + HD * FA_VP) * sizeof(bf16_t);
-  if constexpr (8 * per_wave <= 150 * 1024)
-    return launch_flash_w<HDT, 8>(q, q_stride, k_cache, v_cache, block_tables, max_blocks, tile_req, tile_tok0,
-                                  tile_ntok, positions, out, out_stride, part_o, part_ml, n_tiles, n_tokens, nq, nkv,
-                                  block_size, scale, window, n_splits, fused, stream);
-  else
-    return launch_flash_w<HDT, 4>(q, q_stride, k_cache, v_cache, block_tables, max_blocks, tile_req, tile_tok0,
-                                  tile_ntok, positions, out, out_stride, part_o, part_ml, n_tiles, n_tokens, nq, nkv,
-                                  block_size, scale, window, n_splits, fused, stream);
+  return launch_flash_w<HDT, flash_waves(HDT * 16)>(q, q_stride, k_cache, v_cache, block_tables, max_blocks, tile_req,
+                                                    tile_tok0, tile_ntok, positions, out, out_stride, part_o, part_ml,
+                                                    n_tiles, n_tokens, nq, nkv, block_size, scale, window, n_splits,
+                                                    fused, stream);
 }
 
 }  // namespace
@@ -848,6 +900,10 @@ int tl_flash_prefill(const void* q, int64_t q_stride, const void* k_cache, const
 #undef TL_PREFILL_CASE
   return tl_launch_status();
 }
+
+// How many waves of a workgroup of tl_flash_attention share a query tile's keys, a 64-key tile each at
+// a time (the caller sizes n_splits by it).
+int tl_flash_waves(int hd) { return flash_waves(hd); }
 
 // bfloat16 only.  Tiles: tile_req / tile_tok0 / tile_ntok [n_tiles] describe groups of at most
 // 16 / (nq / nkv) consecutive tokens of one request.  With n_splits > 1, part_o

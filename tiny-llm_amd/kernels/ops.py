@@ -530,6 +530,17 @@ def flash_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     return out
 
 
+def flash_waves(head_dim: int) -> int:
+    """Waves of a `flash_attention` workgroup: each takes one 64-key tile per round trip to memory."""
+    n = _WAVES.get(head_dim)
+    if n is None:
+        n = _WAVES[head_dim] = int(_lib().tl_flash_waves(c_int(head_dim)))
+    return n
+
+
+_WAVES: dict = {}
+
+
 PREFILL_TILES = 8     # query tiles (of 16 rows) one workgroup of the prefill attention kernel owns
 
 

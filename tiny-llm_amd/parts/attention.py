@@ -106,14 +106,14 @@ class Attention(Mixer):
         return out if next_norm is None else (out, prepared)
 
     def _splits(self, ctx, T: int, device):
-        """How many workgroups share one query tile's keys.  Eight waves of a workgroup take a
+        """How many workgroups share one query tile's keys.  The waves of a workgroup take a
         64-key tile each per round trip to memory, and every further round costs about as much as
         the whole rest of the kernel; so long contexts are split until a wave has one tile, as far
         as that keeps the launch within about 256 workgroups (beyond that the splits only queue up,
         and their partial results have to be merged by a second kernel)."""
         key_tiles = -(-ctx.max_seq_len // 64)
         room = max(1, 256 // max(1, T * self.num_kv_heads))
-        n_splits = max(1, min(-(-key_tiles // 8), room, 16))
+        n_splits = max(1, min(-(-key_tiles // ops.flash_waves(self.head_dim)), room, 16))
         if n_splits == 1:
             return 1, None
         return n_splits, torch.empty(n_splits * T * self.num_heads * (self.head_dim + 2), dtype=torch.float32,
