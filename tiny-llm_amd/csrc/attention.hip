@@ -109,8 +109,8 @@ __global__ __launch_bounds__(TL_WAVE) void paged_attention_kernel(
 // softmax times bfloat16 values.  V is transposed on its way into
 // LDS.  Rows of a tile outside [kv_begin, kv_end) are zeroed:
 // stale pages may hold anything, and 0 * NaN is NaN.
-constexpr int FA_KT = 64, FA_VP = 68;
-constexpr int FA_VPAD = 8;      // padding of a row of the row-major V tile of the decode kernel (elements)
+constexpr int FA_KT = 64;
+constexpr int FA_VPAD = 8;      // padding of a row of the row-major V tile in LDS (elements)
 constexpr float kNegBig = -1.0e30f;   // "no key yet": finite, so exp2(m - m') never sees inf - inf
 
 // Two probabilities as two bfloat16 terms each, p = hi + lo, packed pairwise.  hi is p with the low
@@ -505,7 +505,8 @@ __global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
   // two staging buffers: the next key tile is written while the current one is worked on, so a
   // key tile costs one barrier
   __shared__ __attribute__((aligned(16))) bf16_t Kbuf[2][FA_KT * KP];
-  __shared__ __attribute__((aligned(16))) bf16_t Vbuf[2][HD * FA_VP];
+  constexpr int VS = HD + FA_VPAD;         // row stride of the row-major V tile
+  __shared__ __attribute__((aligned(16))) bf16_t Vbuf[2][FA_KT * VS];
 
   const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
   const int r16 = lane % 16, g = lane / 16;
@@ -618,7 +619,7 @@ __global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
       v_stage[ci] = (in_range && c < HD / 8) ? *(const bf16x8*)(vp + c * 8) : z;
     }
   };
-  // registers -> LDS; V is transposed on the way
+  // registers -> LDS, both tiles as they are (the reads of V transpose)
   auto store_tile = [&](int buf) {
     bf16_t* Kl = Kbuf[buf];
     bf16_t* Vl = Vbuf[buf];
@@ -630,10 +631,7 @@ __global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
 #pragma unroll
     for (int ci = 0; ci < VC; ++ci) {
       const int c = ci * FP_WAVES + wave;
-      if (c < HD / 8) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) Vl[(c * 8 + e) * FA_VP + lane] = v_stage[ci][e];
-      }
+      if (c < HD / 8) *(bf16x8*)(Vl + lane * VS + c * 8) = v_stage[ci];
     }
   };
   if (first_tile < last_tile) {
@@ -732,9 +730,10 @@ __global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
       for (int st = 0; st < 2; ++st)
 #pragma unroll
         for (int dt = 0; dt < HDT; ++dt) {
-          const bf16_t* vrow = Vl + (dt * 16 + r16) * FA_VP + g * 4;
-          const bf16x4 lo4 = *(const bf16x4*)(vrow + (2 * st) * 16);
-          const bf16x4 hi4 = *(const bf16x4*)(vrow + (2 * st + 1) * 16);
+          // lane s of a group names keys g*4 + s/4 of a 16-key block, dims dt*16 + 4*(s%4) ..
+          const bf16_t* vsrc = Vl + ((2 * st) * 16 + g * 4 + r16 / 4) * VS + dt * 16 + 4 * (r16 % 4);
+          const bf16x4 lo4 = lds_read_transposed(vsrc);
+          const bf16x4 hi4 = lds_read_transposed(vsrc + 16 * VS);
           bf16x8 vf;
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
