@@ -593,9 +593,10 @@ struct SkinnyArgs {
   int M, N, K;
   int64_t lda, ldo;
   // A norm handed from producer to consumer.  The producer (float32 output, no SiLU-gate) also
-  // writes emit_operand[m, n] = bf16(emit_w[n] * out[m, n]) and, per group of 16 columns, the sum
-  // of out^2 into emit_sumsq[m, group] (ceil(N / 16) groups).  The consumer takes such an operand
-  // as `a` and turns in_sumsq [rows, in_parts] into its row factor 1 / sqrt(sum / in_width + in_eps).
+  // writes emit_operand[m, n] = bf16(emit_w[n] * out[m, n]) and, per group of columns (one group
+  // a workgroup: 16 columns, or 8), the sum of out^2 into emit_sumsq[m, group].  The consumer takes
+  // such an operand as `a` and turns in_sumsq [rows, in_parts] into its row factor
+  // 1 / sqrt(sum / in_width + in_eps).
   const void* emit_w = nullptr;
   int emit_w_is_f32 = 0;
   bf16_t* emit_operand = nullptr;
@@ -664,19 +665,33 @@ __device__ __forceinline__ bf16x8 skinny_operand(const SkinnyChunk<PRO_NORM>& c,
 
 // DEEP: two register stages also with one tile, for long inner sizes, where a wave works through
 // several stages and the chain of their memory round trips sets the kernel's duration.
-template <int MT, int CT, bool DEEP, typename TO, int PRO, bool SWIGLU>
+//
+// HALF (at most 8 activation rows, one tile, no prologue): a workgroup owns 8 columns only, so that
+// a matrix with few rows still gives every compute unit a workgroup; what a workgroup can have in
+// flight, not the memory system, bounds these kernels.  The 16 x 16 MFMA tile is then used as two
+// 8 x 8 tiles that split k: weight row i of the operand is column i % 8 at k offset (i / 8) * 32,
+// activation column j is row j % 8 at k offset (j / 8) * 32, and the wanted products are the two
+// diagonal blocks of the result, added in the epilogue.  One MFMA so covers 64 k, and a load
+// instruction reads whole 128-byte lines of 8 weight rows.
+template <int MT, int CT, bool DEEP, typename TO, int PRO, bool SWIGLU, bool HALF>
 __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const SkinnyArgs p) {
+  static_assert(!HALF || (MT == 1 && CT == 1 && PRO == PRO_NONE && !SWIGLU), "HALF: one plain tile");
+  constexpr int COLS = HALF ? 8 : S_COLS;          // columns of a tile that are outputs
+  constexpr int KW = HALF ? 64 : 32;               // k covered by one MFMA
+  constexpr int KBLK = 4 * KW;                     // k covered by a block of four MFMAs
   extern __shared__ __attribute__((aligned(16))) unsigned char skinny_smem[];
   typedef float Tile[16][17];
   Tile* part = (Tile*)skinny_smem;                                  // [S_WAVES][MT * CT]
   float* ss_part = (float*)(part + S_WAVES * MT * CT);              // [S_WAVES][MT * 16]
   const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
   const int M = p.M, N = p.N, K = p.K;
-  const int n0 = blockIdx.x * (S_COLS * CT);
+  const int n0 = blockIdx.x * (COLS * CT);
   const int r16 = lane % 16, g = lane / 16;
+  const int rr = HALF ? r16 % 8 : r16;             // the weight row / activation row this lane feeds
+  const int kh = HALF ? (r16 / 8) * 32 : 0;        // and its k offset inside an MFMA's range
   const bf16_t* wrow[CT];
 #pragma unroll
-  for (int ct = 0; ct < CT; ++ct) wrow[ct] = p.w + (int64_t)min(n0 + ct * 16 + r16, N - 1) * K;
+  for (int ct = 0; ct < CT; ++ct) wrow[ct] = p.w + (int64_t)min(n0 + ct * 16 + rr, N - 1) * K;
 
   // epilogue operands first: their latency hides behind the main loop
   constexpr int TILES = MT * CT;
@@ -685,47 +700,50 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
 #pragma unroll
   for (int j = 0; j < EPT; ++j) {
     const int e = tid + j * S_THREADS;
-    const int tile = e / 256, m = (tile / CT) * 16 + (e % 256) / 16, n = n0 + (tile % CT) * 16 + e % 16;
-    res_v[j] = (p.residual && e < TILES * 256 && m < M && n < N) ? p.residual[(int64_t)m * p.ldo + n] : 0.f;
+    const int tile = e / 256;
+    const int m = HALF ? e / 8 : (tile / CT) * 16 + (e % 256) / 16;
+    const int n = HALF ? n0 + e % 8 : n0 + (tile % CT) * 16 + e % 16;
+    res_v[j] = (p.residual && e < (HALF ? 64 : TILES * 256) && m < M && n < N) ? p.residual[(int64_t)m * p.ldo + n] : 0.f;
   }
 
   // input row of each activation row this lane feeds
   int64_t row_off[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    const int m = mt * 16 + r16;
+    const int m = mt * 16 + rr;
     const int src = p.rows ? p.rows[min(m, M - 1)] : min(m, M - 1);
     row_off[mt] = (int64_t)src * p.lda;
   }
 
   // Row factors of a norm whose sums of squares arrive in parts: one wave per row, fixed order.
-  // The first 128 parts of a row are requested here, ahead of everything else, and added up after
+  // The first 256 parts of a row are requested here, ahead of everything else, and added up after
   // the main loop: the request then costs no wait of its own.
   float* scale_s = ss_part + S_WAVES * MT * 16;                      // [MT * 16]
   constexpr int RPW = MT * 16 / S_WAVES;                             // rows per wave
-  float pre[RPW][2];
+  constexpr int PRE = 4;                                             // parts requested ahead, in wavefuls
+  float pre[RPW][PRE];
   if (p.in_sumsq) {
 #pragma unroll
-    for (int rr = 0; rr < RPW; ++rr) {
-      const int m = min(wave + rr * S_WAVES, M - 1);
+    for (int ri = 0; ri < RPW; ++ri) {
+      const int m = min(wave + ri * S_WAVES, M - 1);
       const int64_t src = p.rows ? p.rows[m] : m;
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
+      for (int h = 0; h < PRE; ++h) {
         const int q = lane + h * TL_WAVE;
-        pre[rr][h] = q < p.in_parts ? p.in_sumsq[src * p.in_parts + q] : 0.f;
+        pre[ri][h] = q < p.in_parts ? p.in_sumsq[src * p.in_parts + q] : 0.f;
       }
     }
   }
   auto row_factors = [&]() {
     if (!p.in_sumsq) return;
 #pragma unroll
-    for (int rr = 0; rr < RPW; ++rr) {
-      const int r = wave + rr * S_WAVES;
-      float t = pre[rr][0] + pre[rr][1];
-      if (p.in_parts > 2 * TL_WAVE) {
+    for (int ri = 0; ri < RPW; ++ri) {
+      const int r = wave + ri * S_WAVES;
+      float t = (pre[ri][0] + pre[ri][1]) + (pre[ri][2] + pre[ri][3]);
+      if (p.in_parts > PRE * TL_WAVE) {
         const int m = min(r, M - 1);
         const int64_t src = p.rows ? p.rows[m] : m;
-        for (int q = lane + 2 * TL_WAVE; q < p.in_parts; q += TL_WAVE) t += p.in_sumsq[src * p.in_parts + q];
+        for (int q = lane + PRE * TL_WAVE; q < p.in_parts; q += TL_WAVE) t += p.in_sumsq[src * p.in_parts + q];
       }
       t = wave_sum(t);
       if (lane == 0) scale_s[r] = 1.f / sqrtf(t / (float)p.in_width + p.in_eps);
@@ -745,24 +763,24 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
     SkinnyChunk<PRO> fa[UN][MT][4];
     NormChunk nw[PRO == PRO_NORM ? UN : 1][PRO == PRO_NORM ? 4 : 1];
   };
-  const int nblk = (K + S_KBLK - 1) / S_KBLK;
+  const int nblk = (K + KBLK - 1) / KBLK;
   auto load = [&](Stage& st, int blk) {
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
       // MFMA i of the block covers k = i*32 .. i*32+31, lane group g its 8 k from g*8: one load
       // instruction then reads 64 contiguous bytes of each of the 16 weight rows
-      const int kb = (blk + u * S_WAVES) * S_KBLK + g * 8;
+      const int kb = (blk + u * S_WAVES) * KBLK + kh + g * 8;
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) st.fw[u][ct][i] = *(const bf16x8*)(wrow[ct] + min(kb + i * 32, K - 8));
+        for (int i = 0; i < 4; ++i) st.fw[u][ct][i] = *(const bf16x8*)(wrow[ct] + min(kb + i * KW, K - 8));
     }
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
-      const int kb = (blk + u * S_WAVES) * S_KBLK + g * 8;
+      const int kb = (blk + u * S_WAVES) * KBLK + kh + g * 8;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int k = min(kb + i * 32, K - 8);
+        const int k = min(kb + i * KW, K - 8);
         if constexpr (PRO == PRO_NORM) st.nw[u][i].load(p, k);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) st.fa[u][mt][i].load(p, row_off[mt] + k);
@@ -780,10 +798,10 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
   auto multiply = [&](const Stage& st, int blk) {
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
-      const int kb = (blk + u * S_WAVES) * S_KBLK + g * 8;
+      const int kb = (blk + u * S_WAVES) * KBLK + kh + g * 8;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const bool k_ok = kb + i * 32 < K;
+        const bool k_ok = kb + i * KW < K;
         bf16x8 z = {};
         bf16x8 fa[MT];
 #pragma unroll
@@ -847,8 +865,8 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
 #pragma unroll
   for (int j = 0; j < EPT; ++j) {
     const int e = tid + j * S_THREADS;
-    if (e >= TILES * 256) continue;       // whole waves: 256 elements are four waves
-    const int tile = e / 256, m_local = (e % 256) / 16, nn = e % 16;
+    if (e >= (HALF ? 64 : TILES * 256)) continue;       // whole waves: 256 elements are four waves
+    const int tile = e / 256, m_local = HALF ? e / 8 : (e % 256) / 16, nn = HALF ? e % 8 : e % 16;
     const int m = (tile / CT) * 16 + m_local, n = n0 + (tile % CT) * 16 + nn;
     const bool valid = m < M && n < N;
     float scale = 1.f;                    // the row factor left out of the operands
@@ -872,20 +890,23 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
     } else {
       float v = 0.f;
 #pragma unroll
-      for (int wv = 0; wv < S_WAVES; ++wv) v += part[wv * TILES + tile][nn][m_local];
+      for (int wv = 0; wv < S_WAVES; ++wv) {
+        v += part[wv * TILES + tile][nn][m_local];
+        if constexpr (HALF) v += part[wv * TILES + tile][nn + 8][m_local + 8];
+      }
       v = v * scale + res_v[j];
       if (valid) out[(int64_t)m * p.ldo + n] = from_f32<TO>(v);
       if constexpr (sizeof(TO) == 4) {
-        if (p.emit_operand) {             // uniform: the 16 lanes of a row group stay together
+        if (p.emit_operand) {             // uniform: the lanes of a row group stay together
           if (valid) {
             const float wn = p.emit_w_is_f32 ? ((const float*)p.emit_w)[n] : (float)((const bf16_t*)p.emit_w)[n];
             p.emit_operand[(int64_t)m * N + n] = (bf16_t)(wn * v);
           }
           float sq = valid ? v * v : 0.f;
 #pragma unroll
-          for (int off = 1; off < 16; off <<= 1) sq += __shfl_xor(sq, off, TL_WAVE);
+          for (int off = 1; off < COLS; off <<= 1) sq += __shfl_xor(sq, off, TL_WAVE);
           // a column group that begins beyond N has no part of its own
-          if (nn == 0 && m < M && n < N) p.emit_sumsq[(int64_t)m * ((N + 15) / 16) + (n0 / 16 + tile % CT)] = sq;
+          if (nn == 0 && m < M && n < N) p.emit_sumsq[(int64_t)m * ((N + COLS - 1) / COLS) + (n0 / COLS + tile % CT)] = sq;
         }
       }
     }
@@ -894,23 +915,35 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
 
 // Column tiles per workgroup: every workgroup reads all M activation rows, so with more rows it
 // should own more columns, or the activations are read more often than the weights.
-template <int MT, int CT, bool DEEP, typename TO, int PRO, bool SWIGLU>
+template <int MT, int CT, bool DEEP, typename TO, int PRO, bool SWIGLU, bool HALF = false>
 static int launch_skinny_deep(const SkinnyArgs& p, hipStream_t stream) {
   constexpr size_t smem = (size_t)S_WAVES * MT * CT * 16 * 17 * sizeof(float) + (size_t)(S_WAVES + 1) * MT * 16 * sizeof(float);
   static bool configured = false;
   if (!configured) {
-    if (hipFuncSetAttribute((const void*)gemm_skinny_bf16_kernel<MT, CT, DEEP, TO, PRO, SWIGLU>,
+    if (hipFuncSetAttribute((const void*)gemm_skinny_bf16_kernel<MT, CT, DEEP, TO, PRO, SWIGLU, HALF>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
       return TL_ERR_LAUNCH;
     configured = true;
   }
-  dim3 g((p.N + S_COLS * CT - 1) / (S_COLS * CT)), b(S_THREADS);
-  hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, CT, DEEP, TO, PRO, SWIGLU>), g, b, smem, stream, p);
+  constexpr int cols = HALF ? 8 : S_COLS * CT;
+  dim3 g((p.N + cols - 1) / cols), b(S_THREADS);
+  hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, CT, DEEP, TO, PRO, SWIGLU, HALF>), g, b, smem, stream, p);
   return TL_OK;
 }
 
+// 8 columns a workgroup: for at most 8 rows, where a wave would otherwise work through its share
+// of a long inner size in several dependent round trips to memory, and where that still gives
+// no more workgroups than there are compute units (measured: otherwise it is slower).
+static bool skinny_half(int M, int N, int K) { return M <= 8 && K > 2048 && (N + 7) / 8 <= 256; }
+
 template <int MT, int CT, typename TO, int PRO, bool SWIGLU>
 static int launch_skinny_tile(const SkinnyArgs& p, hipStream_t stream) {
+  if constexpr (MT * CT == 1 && PRO == PRO_NONE && !SWIGLU) {
+    if (skinny_half(p.M, p.N, p.K)) {
+      if (p.K > 4096) return launch_skinny_deep<MT, CT, true, TO, PRO, SWIGLU, true>(p, stream);
+      return launch_skinny_deep<MT, CT, false, TO, PRO, SWIGLU, true>(p, stream);
+    }
+  }
   if constexpr (MT * CT == 1 && PRO == PRO_NONE) {
     if (p.K > 4096) return launch_skinny_deep<MT, CT, true, TO, PRO, SWIGLU>(p, stream);
   }
@@ -1012,7 +1045,7 @@ int tl_linear(const void* a, const void* w, void* out, const float* residual, co
 // Few-row (M <= 64) bfloat16 product that takes part in handing a norm from one product to the
 // next (see SkinnyArgs).  Consumer side: in_sumsq [rows of a, in_parts] (a is then the operand a
 // producer wrote; `rows` gathers rows of both).  Producer side (out_dtype 0, epilogue 0): emit_w
-// [N] (element type emit_w_dtype), emit_operand bf16 [M, N], emit_sumsq float [M, ceil(N / 16)].
+// [N] (element type emit_w_dtype), emit_operand bf16 [M, N], emit_sumsq float [M, tl_handoff_parts(M, N, K)].
 // Either side may be absent.
 int tl_linear_handoff(const void* a, const void* w, void* out, const float* residual, const int32_t* rows,
                       const float* in_sumsq, int in_parts, float in_eps, int in_width, const void* emit_w,
@@ -1045,6 +1078,10 @@ int tl_linear_handoff(const void* a, const void* w, void* out, const float* resi
   if (rc != TL_OK) return rc;
   return tl_launch_status();
 }
+
+// How many partial sums of squares per row tl_linear_handoff writes as a producer for these sizes
+// (one per workgroup: per 16 columns, or per 8 where workgroups own 8).
+int tl_handoff_parts(int M, int N, int K) { return skinny_half(M, N, K) ? (N + 7) / 8 : (N + 15) / 16; }
 
 // See splitk_plan.  A caller that gets more than one split allocates a float32 workspace of
 // splits * M * N elements and calls tl_linear_splitk with the same sizes.

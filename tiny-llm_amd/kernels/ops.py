@@ -271,12 +271,20 @@ def can_hand_off(rows: int, width: int, inner: int, dtype: torch.dtype) -> bool:
 
 def handoff_parts(rows: int, width: int, inner: int) -> int:
     """How many partial sums of squares per row the product [rows, inner] x [width, inner]^T writes
-    when it prepares a norm: per 16 columns in the few-row kernel, per 1024 after a split inner size."""
+    when it prepares a norm: one per workgroup in the few-row kernel (16 or 8 columns), per 1024
+    after a split inner size."""
     if split_k(rows, width, inner) > 1:
         return (width + 1023) // 1024
     if not (rows <= FEW_ROWS):
         _fail(f"without a split inner size a norm is prepared for at most {FEW_ROWS} rows")
-    return (width + 15) // 16
+    key = (rows, width, inner)
+    n = _PARTS.get(key)
+    if n is None:
+        n = _PARTS[key] = int(_lib().tl_handoff_parts(c_int(rows), c_int(width), c_int(inner)))
+    return n
+
+
+_PARTS: dict = {}
 
 
 def _linear_split(a, w, out, residual, swiglu, row_scale, sumsq_in, parts, eps, width, emit, splits) -> torch.Tensor:
