@@ -490,25 +490,47 @@ __global__ __launch_bounds__(R_THREADS) void splitk_reduce_kernel(const ReduceAr
   const int m = blockIdx.x, tid = threadIdx.x;
   const int n = blockIdx.y * R_CHUNK + tid * 4;
   const int N = p.N;
-  float scale = p.row_scale ? p.row_scale[m] : 1.f;
-  if (p.in_sumsq) {
-    float t = 0.f;
+  // Everything that has to come from memory is requested before anything is used: the kernel is
+  // a few dependent round trips long, and every one it saves counts.
+  float t = 0.f;
+  if (p.in_sumsq)
     for (int q = tid; q < p.in_parts; q += R_THREADS) t += p.in_sumsq[(int64_t)m * p.in_parts + q];
-    t = block_sum<R_THREADS / TL_WAVE>(t, red);
-    scale = 1.f / sqrtf(t / (float)p.in_width + p.in_eps);
+  float scale = p.row_scale ? p.row_scale[m] : 1.f;
+  float res[4] = {0.f, 0.f, 0.f, 0.f}, wn[4] = {0.f, 0.f, 0.f, 0.f};
+  if constexpr (!SWIGLU) {
+    for (int e = 0; e < 4 && n + e < N; ++e) {
+      if (p.residual) res[e] = p.residual[(int64_t)m * p.ldo + n + e];
+      if (p.emit_operand)
+        wn[e] = p.emit_w_is_f32 ? ((const float*)p.emit_w)[n + e] : (float)((const bf16_t*)p.emit_w)[n + e];
+    }
   }
   const bool vec = (N % 4 == 0);
   float v[4] = {0.f, 0.f, 0.f, 0.f};
   if (n < N) {
-    for (int sp = 0; sp < p.splits; ++sp) {
-      const float* src = p.partial + ((int64_t)sp * p.M + m) * N + n;
-      if (vec) {
-        const f32x4 x = *(const f32x4*)src;
-        v[0] += x[0]; v[1] += x[1]; v[2] += x[2]; v[3] += x[3];
-      } else {
+    if (vec) {
+      // eight splits at a time, their loads in flight together; added in the order of the splits
+      for (int sp0 = 0; sp0 < p.splits; sp0 += 8) {
+        f32x4 x[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          x[u] = *(const f32x4*)(p.partial + ((int64_t)min(sp0 + u, p.splits - 1) * p.M + m) * N + n);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          if (sp0 + u < p.splits) {
+            v[0] += x[u][0]; v[1] += x[u][1]; v[2] += x[u][2]; v[3] += x[u][3];
+          }
+        }
+      }
+    } else {
+      for (int sp = 0; sp < p.splits; ++sp) {
+        const float* src = p.partial + ((int64_t)sp * p.M + m) * N + n;
         for (int e = 0; e < 4 && n + e < N; ++e) v[e] += src[e];
       }
     }
+  }
+  if (p.in_sumsq) {      // uniform
+    t = block_sum<R_THREADS / TL_WAVE>(t, red);
+    scale = 1.f / sqrtf(t / (float)p.in_width + p.in_eps);
   }
   TO* out = (TO*)p.out;
   float sq = 0.f;
@@ -519,13 +541,10 @@ __global__ __launch_bounds__(R_THREADS) void splitk_reduce_kernel(const ReduceAr
         out[(int64_t)m * p.ldo + n / 2 + 1] = from_f32<TO>(swiglu_pair_fast(v[2] * scale, v[3] * scale));
     } else {
       for (int e = 0; e < 4 && n + e < N; ++e) {
-        float x = v[e] * scale;
-        const int64_t o = (int64_t)m * p.ldo + n + e;
-        if (p.residual) x += p.residual[o];
-        out[o] = from_f32<TO>(x);
+        const float x = v[e] * scale + res[e];
+        out[(int64_t)m * p.ldo + n + e] = from_f32<TO>(x);
         if (p.emit_operand) {
-          const float wn = p.emit_w_is_f32 ? ((const float*)p.emit_w)[n + e] : (float)((const bf16_t*)p.emit_w)[n + e];
-          p.emit_operand[(int64_t)m * N + n + e] = (bf16_t)(wn * x);
+          p.emit_operand[(int64_t)m * N + n + e] = (bf16_t)(wn[e] * x);
           sq += x * x;
         }
       }
