@@ -587,13 +587,16 @@ def test_flash_attention_decode_batch():
 
 @pytest.mark.parametrize("nq,nkv,hd,bs", [(32, 4, 64, 16), (3, 1, 32, 8), (8, 8, 16, 16), (16, 2, 128, 32), (6, 2, 80, 16)])
 @pytest.mark.parametrize("n_splits", [1, 3])
-def test_flash_attention_fused_rotation_and_cache_write(nq, nkv, hd, bs, n_splits):
-    """Decode step with rotation and cache write inside the attention kernel == rope_store + attention."""
+@pytest.mark.parametrize("window", [0, 150])
+def test_flash_attention_fused_rotation_and_cache_write(nq, nkv, hd, bs, n_splits, window):
+    """Decode step with rotation and cache write inside the attention kernel == rope_store + attention.
+    The long requests give a wave several key tiles in turn (the new token's in the last), the
+    window lets a wave's first tile be another than the one whose pages it looked up ahead."""
     from tiny_llm_amd.parts.rotary import RotaryEmbedding
     g = torch.Generator().manual_seed(nq + hd)
-    lens = [1, 2, 63, 64, 65, 129, 300, 17]
+    lens = [1, 2, 63, 64, 65, 129, 300, 17, 600, 1100]
     R = len(lens)
-    rot = RotaryEmbedding("r", torch.bfloat16, DEV, head_dim=hd, theta=10000.0, max_position=512)
+    rot = RotaryEmbedding("r", torch.bfloat16, DEV, head_dim=hd, theta=10000.0, max_position=1200)
     cos, sin, rd = rot.rotary_tables()
     nblocks = sum(-(-l // bs) for l in lens) + 2
     perm = torch.randperm(nblocks, generator=g).tolist()
@@ -615,12 +618,12 @@ def test_flash_attention_fused_rotation_and_cache_write(nq, nkv, hd, bs, n_split
     kc1, vc1, qkv1 = kc.clone().to(DEV), vc.clone().to(DEV), qkv.clone().to(DEV)
     ops().rope_store(qkv1, pos, cos, sin, i32(slots), kc1, vc1, nq, nkv, hd, rd)
     out1 = torch.empty(R, nq * hd, dtype=torch.bfloat16, device=DEV)
-    ops().flash_attention(qkv1[:, :nq * hd], kc1, vc1, bt.to(DEV), tiles, pos, out1, nq, nkv, hd, hd ** -0.5, 0,
+    ops().flash_attention(qkv1[:, :nq * hd], kc1, vc1, bt.to(DEV), tiles, pos, out1, nq, nkv, hd, hd ** -0.5, window,
                           n_splits, scratch)
     # fused
     kc2, vc2, qkv2 = kc.clone().to(DEV), vc.clone().to(DEV), qkv.clone().to(DEV)
     out2 = torch.empty(R, nq * hd, dtype=torch.bfloat16, device=DEV)
-    ops().flash_attention(qkv2[:, :nq * hd], kc2, vc2, bt.to(DEV), tiles, pos, out2, nq, nkv, hd, hd ** -0.5, 0,
+    ops().flash_attention(qkv2[:, :nq * hd], kc2, vc2, bt.to(DEV), tiles, pos, out2, nq, nkv, hd, hd ** -0.5, window,
                           n_splits, scratch, fused_rope=(cos, sin))
     assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2)      # the same rows, the same bits
     assert torch.equal(qkv2.cpu(), qkv)                          # the input rows are left as they were
