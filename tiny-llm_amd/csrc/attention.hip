@@ -254,7 +254,7 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
   // A wave reads its 64-key tile by itself, so nothing in this loop waits for another wave.  Keys
   // go straight from memory into MFMA operands (lane (r16, g) holds dims ks*32 + g*8.. of key rows
   // kt*16 + r16: the layout the score product wants); values pass through an LDS area of the wave's
-  // own (lane = key row), where they are transposed.
+  // own (lane = key row), stored as they are; the reads for the second product transpose them.
   constexpr int VCH = HD / 8;
   bf16x8 k_op[4][KS], v_stage[VCH];
   auto row_offset = [&](int j, int blk) {
