@@ -236,6 +236,31 @@ def test_graph_replays_equal_eager_steps(dtype, folders):
         assert same >= 0.8 * sum(min(len(x), 8) for x in outs[True])
 
 
+def test_collector_rests_while_a_decode_graph_is_captured(folders, monkeypatch):
+    """Python's garbage collector must not run while a decode step is captured: finalising the
+    pinned buffers or graphs of an engine that is no longer referenced is not allowed during a
+    capture and would end the process.  (torch.cuda.graph no longer collects before a capture.)"""
+    import gc
+    from tiny_llm_amd import Engine, SamplingParams
+    from tiny_llm_amd.engine import step as step_module
+    cfg = CONFIGS["A"][0]
+    seen = []
+    body = step_module.DecodeGraph._body
+
+    def watched(self):
+        seen.append((torch.cuda.is_current_stream_capturing(), gc.isenabled()))
+        return body(self)
+
+    monkeypatch.setattr(step_module.DecodeGraph, "_body", watched)
+    assert gc.isenabled()
+    prompts = [random_tokens(12, cfg["vocab_size"], 77)]
+    for _ in range(2):      # the second engine is built while the first one is garbage
+        Engine(folders["A"], dtype="bfloat16", use_graphs=True).generate(prompts, SamplingParams.greedy(6, ignore_eos=True))
+    assert any(capturing for capturing, _ in seen)
+    assert all(not collecting for capturing, collecting in seen if capturing)
+    assert gc.isenabled()
+
+
 def test_command_line_generates_from_prompt_ids(folders):
     cfg = CONFIGS["A"][0]
     prompt = random_tokens(12, cfg["vocab_size"], 5)

@@ -322,15 +322,33 @@ def test_linear_swiglu_epilogue(dtype, M, K, N):
         ops().linear(a.to(DEV), w.to(DEV), torch.empty(M, N, dtype=dtype, device=DEV), epilogue="swiglu")
 
 
-def test_linear_row_alone_equals_row_in_batch_fp32():
-    g = torch.Generator().manual_seed(5)
-    a = torch.randn(70, 200, generator=g).to(DEV)
-    w = torch.randn(90, 200, generator=g).to(DEV)
-    full = torch.empty(70, 90, device=DEV)
-    ops().linear(a, w, full)
-    one = torch.empty(1, 90, device=DEV)
-    ops().linear(a[37:38], w, one)
-    assert torch.equal(full[37:38], one)
+@pytest.mark.parametrize("K,N", [(200, 90), (1000, 72), (5632, 130), (256, 8), (258, 34)])
+def test_linear_row_alone_equals_row_in_batch_fp32(K, N):
+    """In float32 a row gives the same bits alone, among a few rows and among many: the tiled kernel
+    (more than 16 rows, or an inner size that is no multiple of 4) and the few-row kernel add in one
+    order.  With residual and with the SiLU-gate epilogue too."""
+    g = torch.Generator().manual_seed(5 + K)
+    a = torch.randn(70, K, generator=g).to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(DEV)
+    res = torch.randn(70, N, generator=g).to(DEV)
+    for kwargs in ({}, {"residual": True}, {"epilogue": "swiglu"}):
+        width = N // 2 if "epilogue" in kwargs else N
+        def run(rows):
+            x = a[rows].contiguous()
+            out = torch.empty(x.shape[0], width, device=DEV)
+            r = res[rows].contiguous() if kwargs.get("residual") else None
+            ops().linear(x, w, out, r, epilogue=kwargs.get("epilogue"))
+            return out
+        full = run(slice(0, 70))
+        assert torch.equal(full[37:38], run(slice(37, 38)))
+        assert torch.equal(full[30:43], run(slice(30, 43)))
+        assert torch.equal(full[3:67], run(slice(3, 67)))
+        ref = a.double() @ w.double().T
+        if kwargs.get("residual"):
+            ref = ref + res.double()
+        if "epilogue" in kwargs:
+            ref = plain.silu(ref[:, 0::2]) * ref[:, 1::2]
+        assert rel(full, ref) < 1e-5
 
 
 def test_linear_refuses_bad_inner_size_in_bf16():

@@ -4,9 +4,10 @@
 // residual add that the reference runs as a separate kernel
 // (tiny_llm/ops/cuda/arithmetic.cu:13) is folded into the epilogue.
 //
-//  * gemm_f32_kernel: true float32, FMA on the vector units, no reduced-precision
-//    matrix mode.  The k order of the accumulation does not depend on M, so a row
-//    gives the same bits whether it is computed alone or in a batch.
+//  * gemm_f32_kernel, and gemm_f32_rows_kernel for at most 16 rows: true float32, FMA on the
+//    vector units, no reduced-precision matrix mode.  Both add in ONE order: k ascending inside
+//    blocks of 256, each block from zero, the block sums added in ascending order.  So a row
+//    gives the same bits whether it is computed alone or in a batch, by either kernel.
 //  * gemm_bf16_kernel: bf16 inputs on the MFMA matrix cores
 //    (v_mfma_f32_32x32x16_bf16), float32 accumulation, 256x256, 128x128 or 64x128 tiles with
 //    k steps of 64 staged through double-buffered LDS.
@@ -18,6 +19,7 @@ namespace {
 
 // ===================================================================== float32
 constexpr int F_BM = 64, F_BN = 64, F_BK = 16, F_THREADS = 256;
+constexpr int F_KBLOCK = 256;     // the k block of the order of addition (a multiple of F_BK)
 
 // silu(g) * u of an interleaved gate|up pair of output columns, as the reference computes it
 // (tiny_llm/ops/cuda/silu.cu:10, arithmetic.cu:13), from the float32 accumulators.
@@ -40,7 +42,7 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f32_kernel(const float* __rest
   const int tid = threadIdx.x;
   const int m0 = blockIdx.y * F_BM, n0 = blockIdx.x * F_BN;
   const int ty = tid / 16, tx = tid % 16;
-  float acc[4][4] = {};
+  float acc[4][4] = {}, tot[4][4] = {};
   // each thread stages 4 consecutive k of one row of each operand
   const int lr = tid / 4, lk = (tid % 4) * 4;
   for (int k0 = 0; k0 < K; k0 += F_BK) {
@@ -71,7 +73,20 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f32_kernel(const float* __rest
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(ar[i], wr[j], acc[i][j]);
     }
+    if ((k0 + F_BK) % F_KBLOCK == 0 || k0 + F_BK >= K) {     // a block of the order of addition ends
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          tot[i][j] += acc[i][j];
+          acc[i][j] = 0.f;
+        }
+    }
   }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = tot[i][j];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int m = m0 + ty * 4 + i;
@@ -93,6 +108,71 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f32_kernel(const float* __rest
         out[(int64_t)m * ldo + n] = from_f32<TO>(v);
       }
     }
+  }
+}
+
+// The same product for few rows (decode steps), where the tiled kernel leaves most of the chip
+// idle.  A workgroup owns 8 output columns; a thread owns one k block of 256 of one column (and the
+// blocks 32, 64, ... further on) and works through it in ascending k for 8 rows at a time; the
+// block sums meet in LDS and are added in ascending order: the order of gemm_f32_kernel, to the bit.
+constexpr int FR_COLS = 8, FR_LANES = 32, FR_THREADS = FR_COLS * FR_LANES, FR_ROWS = 8;
+
+template <bool SWIGLU>
+__global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* __restrict__ a,
+                                                                   const float* __restrict__ w,
+                                                                   float* __restrict__ out,
+                                                                   const float* __restrict__ residual, int M,
+                                                                   int N, int K, int64_t lda, int64_t ldo) {
+  extern __shared__ float rows_smem[];
+  const int nkb = (K + F_KBLOCK - 1) / F_KBLOCK;
+  float* part = rows_smem;                                   // [FR_COLS][nkb][FR_ROWS]
+  float* sums = rows_smem + FR_COLS * nkb * FR_ROWS;         // [FR_COLS][FR_ROWS]
+  const int tid = threadIdx.x, c = tid / FR_LANES, bl = tid % FR_LANES;
+  const int n0 = blockIdx.x * FR_COLS;
+  const float* wrow = w + (int64_t)min(n0 + c, N - 1) * K;
+  for (int m0 = 0; m0 < M; m0 += FR_ROWS) {
+    const float* arow[FR_ROWS];
+#pragma unroll
+    for (int r = 0; r < FR_ROWS; ++r) arow[r] = a + (int64_t)min(m0 + r, M - 1) * lda;
+    for (int b = bl; b < nkb; b += FR_LANES) {
+      float acc[FR_ROWS];
+#pragma unroll
+      for (int r = 0; r < FR_ROWS; ++r) acc[r] = 0.f;
+      const int k_end = min((b + 1) * F_KBLOCK, K);          // K is a multiple of 4
+#pragma unroll 4
+      for (int k = b * F_KBLOCK; k < k_end; k += 4) {
+        const f32x4 wv = *(const f32x4*)(wrow + k);
+#pragma unroll
+        for (int r = 0; r < FR_ROWS; ++r) {
+          const f32x4 av = *(const f32x4*)(arow[r] + k);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[r] = fmaf(av[e], wv[e], acc[r]);
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < FR_ROWS; ++r) part[(c * nkb + b) * FR_ROWS + r] = acc[r];
+    }
+    __syncthreads();
+    if (tid < FR_COLS * FR_ROWS) {
+      const int cc = tid / FR_ROWS, r = tid % FR_ROWS;
+      float t = 0.f;
+      for (int b = 0; b < nkb; ++b) t += part[(cc * nkb + b) * FR_ROWS + r];
+      sums[tid] = t;
+    }
+    __syncthreads();
+    if (tid < FR_COLS * FR_ROWS) {
+      const int cc = tid / FR_ROWS, r = tid % FR_ROWS;
+      const int m = m0 + r, n = n0 + cc;
+      if (m < M && n < N) {
+        if constexpr (SWIGLU) {   // columns (2j, 2j+1) = (gate_j, up_j); N and n0 are even
+          if ((cc & 1) == 0) out[(int64_t)m * ldo + n / 2] = swiglu_pair(sums[tid], sums[tid + FR_ROWS]);
+        } else {
+          const float v = sums[tid];
+          out[(int64_t)m * ldo + n] = residual ? v + residual[(int64_t)m * ldo + n] : v;
+        }
+      }
+    }
+    // the next pass writes `part` only after the barrier above and `sums` only after its own first barrier
   }
 }
 
@@ -1022,6 +1102,18 @@ int tl_linear_tile(const void* a, const void* w, void* out, const float* residua
   if (swiglu && ((N & 1) || residual || out_dtype != dtype)) return TL_ERR_ARG;
   if (dtype == 0) {
     if (out_dtype != 0) return TL_ERR_ARG;
+    if (M <= 16 && K % 4 == 0 && K <= 32768 && lda % 4 == 0 && ((uintptr_t)a | (uintptr_t)w) % 16 == 0) {
+      const int nkb = (K + F_KBLOCK - 1) / F_KBLOCK;
+      const size_t smem = (size_t)(FR_COLS * nkb * FR_ROWS + FR_COLS * FR_ROWS) * sizeof(float);   // at most 33 KB
+      dim3 gr((N + FR_COLS - 1) / FR_COLS);
+      if (swiglu)
+        hipLaunchKernelGGL((gemm_f32_rows_kernel<true>), gr, dim3(FR_THREADS), smem, stream, (const float*)a,
+                           (const float*)w, (float*)out, residual, M, N, K, lda, ldo);
+      else
+        hipLaunchKernelGGL((gemm_f32_rows_kernel<false>), gr, dim3(FR_THREADS), smem, stream, (const float*)a,
+                           (const float*)w, (float*)out, residual, M, N, K, lda, ldo);
+      return tl_launch_status();
+    }
     dim3 g((N + F_BN - 1) / F_BN, (M + F_BM - 1) / F_BM);
     if (swiglu)
       hipLaunchKernelGGL((gemm_f32_kernel<float, true>), g, dim3(F_THREADS), 0, stream, (const float*)a,

@@ -14,6 +14,7 @@ kernels need no search over sequence separators (tiny_llm/ops/details.hpp:19-36)
 """
 from __future__ import annotations
 
+import gc
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
@@ -338,9 +339,20 @@ class DecodeGraph:
             self._body()
         elif self.graph is None:
             torch.cuda.synchronize()
-            self.graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(self.graph):
-                self._body()
+            # Nothing may be finalised while the stream is capturing: the release of pinned buffers,
+            # graphs or events of an engine that is no longer referenced is not allowed then and
+            # ends the process.  So dead objects are collected now, and the collector rests until
+            # the capture is over (torch.cuda.graph does not collect by itself any more).
+            gc.collect()
+            collecting = gc.isenabled()
+            gc.disable()
+            try:
+                self.graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(self.graph):
+                    self._body()
+            finally:
+                if collecting:
+                    gc.enable()
             self.graph.replay()
         else:
             self.graph.replay()
