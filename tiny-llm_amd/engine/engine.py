@@ -14,7 +14,7 @@ from typing import Dict, Hashable, List, Mapping, Optional, Sequence, Union
 from ..config import EngineConfig
 from ..sampling import Sampler, SamplingParams
 from .loading import build_runner, load_model, random_model
-from .scheduler import Request, Scheduler, StepPlan
+from .scheduler import Request, Scheduler
 from .step import StepEntry
 
 

@@ -21,7 +21,7 @@ from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 import numpy as np
 import torch
 
-from ..cache import CacheManager, OutOfBlocks
+from ..cache import CacheManager
 
 
 @dataclass

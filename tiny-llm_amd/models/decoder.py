@@ -11,7 +11,7 @@ from typing import List, Optional
 
 import torch
 
-from ..config.spec import ModelSpec, PartSpec
+from ..config.spec import ModelSpec
 from ..parts import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, CacheSpec, LayerCache, StateSpec, WeightSpec)
 from ..parts.embedding import LMHead, TokenEmbedding
 

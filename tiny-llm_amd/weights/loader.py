@@ -17,12 +17,12 @@ import fnmatch
 import hashlib
 import json
 import os
-from typing import Callable, Dict, Iterable, List, Mapping, Optional, Sequence, Tuple
+from typing import Callable, Dict, Iterable, Mapping, Optional, Sequence, Tuple
 
 import torch
 
 from ..parts.base import WeightSpec
-from .safetensors_io import SafetensorsFile, open_model_files, save_file
+from .safetensors_io import open_model_files, save_file
 
 # tensors that checkpoints of this family carry and no part needs
 IGNORABLE = ("*.rotary_emb.inv_freq",)
