@@ -212,6 +212,27 @@ def test_preemption_recomputes_and_gives_the_same_tokens(folders):
     assert tight.runner.cache.free_blocks() == [9]
 
 
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_float32_generation_does_not_depend_on_the_schedule(name, folders):
+    """In float32 a row gives the same bits alone and in any batch, so greedy generation must give
+    the same tokens whatever the token budget, the page size, the number of live requests, the
+    number of pages (with preemption) and graphs or eager steps."""
+    from tiny_llm_amd import Engine, SamplingParams
+    cfg, eng_kw, _ = CONFIGS[name]
+    kw = {k: v for k, v in eng_kw.items() if k != "kv_block_size"}
+    prompts = [random_tokens(n, cfg["vocab_size"], 900 + n) for n in (70, 3, 33, 64, 17, 129, 5)]
+    sps = [SamplingParams.greedy(n, ignore_eos=True) for n in (40, 60, 25, 33, 50, 20, 64)]
+    outs = []
+    for budget, bs, seqs, graphs, blocks in [(256, 16, 8, True, None), (7, 8, 2, False, None), (32, 32, 4, True, 12),
+                                             (256, 8, 8, False, 40), (7, 16, 4, True, 16), (32, 16, 2, False, None)]:
+        extra = {} if blocks is None else {"num_kv_blocks": blocks}
+        eng = Engine(folders[name], dtype="float32", max_num_seqs=seqs, max_num_batched_tokens=budget, kv_block_size=bs,
+                     use_graphs=graphs, **extra, **kw)
+        outs.append(eng.generate(prompts, sps))
+        eng.runner.cache.audit()
+    assert all(o == outs[0] for o in outs[1:])
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_graph_replays_equal_eager_steps(dtype, folders):
     """Decode steps captured in a HIP graph: every replay, with eager work (prefill of new requests,
