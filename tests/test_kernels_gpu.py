@@ -646,6 +646,12 @@ def test_flash_attention_fused_rotation_and_cache_write(nq, nkv, hd, bs, n_split
     assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2)      # the same rows, the same bits
     assert torch.equal(qkv2.cpu(), qkv)                          # the input rows are left as they were
     assert rel(out2, out1.double()) < 1e-6
+    # without tile arrays: row i is the one new token of request i
+    kc3, vc3 = kc.clone().to(DEV), vc.clone().to(DEV)
+    out3 = torch.empty(R, nq * hd, dtype=torch.bfloat16, device=DEV)
+    ops().flash_attention(qkv2[:, :nq * hd], kc3, vc3, bt.to(DEV), None, pos, out3, nq, nkv, hd, hd ** -0.5, window,
+                          n_splits, scratch, fused_rope=(cos, sin))
+    assert torch.equal(out3, out2) and torch.equal(kc3, kc2) and torch.equal(vc3, vc2)
 
 
 def test_paged_attention_reduces_to_library_routine():

@@ -186,7 +186,9 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
   const int r16 = lane % 16, g = lane / 16;
   const int tile = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
   const int G = nq / nkv;
-  const int req = tile_req[tile], tok0 = tile_tok0[tile], ntok = tile_ntok[tile];
+  // no tile lists: tile i is token i of request i (a decode step), known without a round trip
+  const int req = tile_req ? tile_req[tile] : tile, tok0 = tile_req ? tile_tok0[tile] : tile;
+  const int ntok = tile_req ? tile_ntok[tile] : 1;
   const int32_t* bt = block_tables + (int64_t)req * max_blocks;
   bf16_t* Vl = smem + wave * WAVE_ELEMS;
   const bool do_rope = fused.cos_t != nullptr;
@@ -779,23 +781,44 @@ __global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
   }
 }
 
-// Merges the partial results of `n_splits` workgroups per (token, head).
-__global__ void flash_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                     bf16_t* __restrict__ out, int64_t out_stride, int n_tokens, int nq, int hd,
-                                     int n_splits) {
-  const int t = blockIdx.x, h = blockIdx.y;
+// Merges the partial results of `n_splits` workgroups per (token, head).  One wave per (token,
+// head); everything is requested before anything is used (up to 16 splits at a time), because a
+// dependent round trip to memory costs as much as the rest of this kernel.  FC_BATCH is the
+// smallest of 2, 4, 8, 16 that covers n_splits (16 beyond), so that few splits ask for little.
+template <int FC_BATCH>
+__global__ __launch_bounds__(TL_WAVE) void flash_combine_kernel(const float* __restrict__ part_o,
+                                                                const float* __restrict__ part_ml,
+                                                                bf16_t* __restrict__ out, int64_t out_stride,
+                                                                int n_tokens, int nq, int hd, int n_splits) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int64_t row = (int64_t)t * nq + h, step = (int64_t)n_tokens * nq;      // split s: row + s * step
+  // lane s holds (maximum, sum) of split s, s + 64, ...: one request each
   float M = kNegBig;       // maxima are in units of log2 e; a split without keys has l = 0 and O = 0
-  for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part_ml[(((int64_t)s * n_tokens + t) * nq + h) * 2]);
-  float L = 0.f;
-  for (int s = 0; s < n_splits; ++s) {
-    const float* ml = part_ml + (((int64_t)s * n_tokens + t) * nq + h) * 2;
-    L += __builtin_amdgcn_exp2f(ml[0] - M) * ml[1];
+  for (int s0 = 0; s0 < n_splits; s0 += TL_WAVE) {
+    const int s = s0 + lane;
+    M = fmaxf(M, s < n_splits ? part_ml[(row + s * step) * 2] : kNegBig);
   }
-  for (int d = threadIdx.x; d < hd; d += blockDim.x) {
-    float acc = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-      const int64_t base = ((int64_t)s * n_tokens + t) * nq + h;
-      acc += __builtin_amdgcn_exp2f(part_ml[base * 2] - M) * part_o[base * hd + d];
+#pragma unroll
+  for (int off = 1; off < TL_WAVE; off <<= 1) M = fmaxf(M, __shfl_xor(M, off, TL_WAVE));
+  for (int d = lane; d < hd; d += TL_WAVE) {
+    float acc = 0.f, L = 0.f;
+    for (int s0 = 0; s0 < n_splits; s0 += FC_BATCH) {
+      float m[FC_BATCH], l[FC_BATCH], o[FC_BATCH];
+#pragma unroll
+      for (int u = 0; u < FC_BATCH; ++u) {
+        const int64_t base = row + (int64_t)min(s0 + u, n_splits - 1) * step;
+        m[u] = part_ml[base * 2];
+        l[u] = part_ml[base * 2 + 1];
+        o[u] = part_o[base * hd + d];
+      }
+#pragma unroll
+      for (int u = 0; u < FC_BATCH; ++u) {
+        if (s0 + u < n_splits) {
+          const float wgt = __builtin_amdgcn_exp2f(m[u] - M);
+          L += wgt * l[u];
+          acc += wgt * o[u];
+        }
+      }
     }
     out[(int64_t)t * out_stride + (int64_t)h * hd + d] = (bf16_t)(L > 0.f ? acc / L : 0.f);
   }
@@ -905,7 +928,7 @@ int tl_flash_prefill(const void* q, int64_t q_stride, const void* k_cache, const
 int tl_flash_waves(int hd) { return flash_waves(hd); }
 
 // bfloat16 only.  Tiles: tile_req / tile_tok0 / tile_ntok [n_tiles] describe groups of at most
-// 16 / (nq / nkv) consecutive tokens of one request.  With n_splits > 1, part_o
+// 16 / (nq / nkv) consecutive tokens of one request; all three null: tile i is token i of request i.  With n_splits > 1, part_o
 // [n_splits, n_tokens, nq, hd] and part_ml [n_splits, n_tokens, nq, 2] (float32) are scratch.
 int tl_flash_attention(const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
                        const int32_t* block_tables, int max_blocks, const int32_t* tile_req,
@@ -918,6 +941,8 @@ int tl_flash_attention(const void* q, int64_t q_stride, const void* k_cache, con
       max_blocks <= 0 || window < 0 || n_splits < 1 || nkv > 65535 || n_splits > 65535 || q_stride % 8)
     return TL_ERR_ARG;
   if (n_splits > 1 && (!part_o || !part_ml)) return TL_ERR_ARG;
+  if (!tile_req && (tile_tok0 || tile_ntok || n_tiles != n_tokens)) return TL_ERR_ARG;
+  if (tile_req && (!tile_tok0 || !tile_ntok)) return TL_ERR_ARG;
   // fused rotation and cache write: q is the first slice of rows [q heads | k heads | v heads], every
   // tile is one token, the whole head is rotated
   if (fuse_store && (!rope_cos || !rope_sin || n_tiles != n_tokens)) return TL_ERR_ARG;
@@ -937,9 +962,14 @@ int tl_flash_attention(const void* q, int64_t q_stride, const void* k_cache, con
   }
 #undef TL_FLASH_CASE
   if (rc != TL_OK) return rc;
-  if (n_splits > 1)
-    hipLaunchKernelGGL(flash_combine_kernel, dim3(n_tokens, nq), dim3(64), 0, stream, part_o, part_ml, (bf16_t*)out,
-                       out_stride, n_tokens, nq, hd, n_splits);
+#define TL_COMBINE(B)                                                                                          \
+  hipLaunchKernelGGL(flash_combine_kernel<B>, dim3(n_tokens, nq), dim3(TL_WAVE), 0, stream, part_o, part_ml, \
+                     (bf16_t*)out, out_stride, n_tokens, nq, hd, n_splits)
+  if (n_splits > 8) TL_COMBINE(16);
+  else if (n_splits > 4) TL_COMBINE(8);
+  else if (n_splits > 2) TL_COMBINE(4);
+  else if (n_splits > 1) TL_COMBINE(2);
+#undef TL_COMBINE
   return tl_launch_status();
 }
 

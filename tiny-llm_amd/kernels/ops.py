@@ -476,13 +476,14 @@ def flash_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                     scratch: Optional[torch.Tensor] = None, fused_rope=None) -> torch.Tensor:
     """The same function as `paged_attention` on the matrix cores (bfloat16).  `tiles` =
     (tile_req, tile_tok0, tile_ntok): groups of at most 16 // (heads / kv_heads) consecutive
-    tokens of one request.  n_splits > 1 needs float32 `scratch` of at least
+    tokens of one request; None for a decode step, where row i is the one new token of request i
+    (the kernel then starts without waiting for the tile arrays).  n_splits > 1 needs float32 `scratch` of at least
     n_splits * T * heads * (head_dim + 2) elements.
 
     fused_rope=(cos, sin), for steps of ONE new token per request: `q` is the first slice of the
     unrotated rows [q heads | k heads | v heads]; the kernel rotates q and the new key over the
     whole head and writes the new key and value into the caches itself (no `rope_store` before)."""
-    tile_req, tile_tok0, tile_ntok = tiles
+    tile_req, tile_tok0, tile_ntok = tiles if tiles is not None else (None, None, None)
     _dev(q, k_cache, v_cache, block_tables, tile_req, tile_tok0, tile_ntok, positions, out, scratch)
     _rows_2d(q, "q")
     _rows_2d(out, "attention output")
@@ -502,10 +503,15 @@ def flash_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         _fail("block tables must be contiguous int32 [requests, max_blocks]")
     if not (positions.dtype == torch.int32 and positions.is_contiguous() and positions.numel() == T):
         _fail("positions must be contiguous int32, one per row")
-    n_tiles = tile_req.numel()
-    for t in (tile_req, tile_tok0, tile_ntok):
-        if not (t.dtype == torch.int32 and t.is_contiguous() and t.numel() == n_tiles):
-            _fail("tile arrays must be int32 [tiles]")
+    if tiles is None:        # a decode step: row i is the one new token of request i
+        n_tiles = T
+        if not (block_tables.shape[0] >= T):
+            _fail("without tile arrays every row is a request of its own and needs a block table row")
+    else:
+        n_tiles = tile_req.numel()
+        for t in (tile_req, tile_tok0, tile_ntok):
+            if not (t.dtype == torch.int32 and t.is_contiguous() and t.numel() == n_tiles):
+                _fail("tile arrays must be int32 [tiles]")
     if not (q.stride(0) % 8 == 0):
         _fail("q rows must be 16-byte aligned")
     part_o = part_ml = None

@@ -93,7 +93,8 @@ class Attention(Mixer):
         elif flash:
             # decoding: one token per request, its keys split over the waves of a workgroup (and over
             # workgroups when the context is long)
-            tiles = ctx.attention_tiles(16 // group)
+            # (no tile arrays when every request brings exactly one token: row i is request i)
+            tiles = None if T == ctx.num_requests else ctx.attention_tiles(16 // group)
             n_splits, scratch = self._splits(ctx, T, residual.device)
             ops.flash_attention(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, attn,
                                 self.num_heads, self.num_kv_heads, self.head_dim, self.scale, self.window,
