@@ -1061,7 +1061,19 @@ static int launch_skinny_rows(const SkinnyArgs& p, hipStream_t stream) {
 template <typename TO, int PRO, bool SWIGLU>
 static int launch_skinny(const SkinnyArgs& p, hipStream_t stream) {
   const int mt = (p.M + 15) / 16;
-  if (mt == 1) return launch_skinny_tile<1, 1, TO, PRO, SWIGLU>(p, stream);
+  if (mt == 1) {
+    if constexpr (PRO == PRO_NONE) {
+      // A workgroup fetches at a rate of its own, and every workgroup fetches all activation rows:
+      // the product is fastest with ONE round of workgroups over the 256 compute units, each owning
+      // as many column tiles as that takes (up to four; wider products stay at one).  Below 8 rows
+      // the activations are too few to matter and more workgroups are faster.
+      const int ct = p.M >= 8 ? (p.N + 256 * S_COLS - 1) / (256 * S_COLS) : 1;
+      if (ct == 2) return launch_skinny_tile<1, 2, TO, PRO, SWIGLU>(p, stream);
+      if (ct == 3) return launch_skinny_tile<1, 3, TO, PRO, SWIGLU>(p, stream);
+      if (ct == 4) return launch_skinny_tile<1, 4, TO, PRO, SWIGLU>(p, stream);
+    }
+    return launch_skinny_tile<1, 1, TO, PRO, SWIGLU>(p, stream);
+  }
   if constexpr (PRO == PRO_NONE) {       // the norm prologue exists for one row tile only
     if (mt == 2) return launch_skinny_rows<2, TO, SWIGLU>(p, stream);
     if (mt == 3) return launch_skinny_rows<3, TO, SWIGLU>(p, stream);
