@@ -868,6 +868,7 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
     for (int u = 0; u < UN; ++u) {
       // MFMA i of the block covers k = i*32 .. i*32+31, lane group g its 8 k from g*8: one load
       // instruction then reads 64 contiguous bytes of each of the 16 weight rows
+      if (HALF && u > 0 && blk + u * S_WAVES >= nblk) continue;      // the same for the whole wave: no such block
       const int kb = (blk + u * S_WAVES) * KBLK + kh + g * 8;
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct)
@@ -876,6 +877,7 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
     }
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
+      if (HALF && u > 0 && blk + u * S_WAVES >= nblk) continue;
       const int kb = (blk + u * S_WAVES) * KBLK + kh + g * 8;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -897,6 +899,7 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
   auto multiply = [&](const Stage& st, int blk) {
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
+      if (HALF && u > 0 && blk + u * S_WAVES >= nblk) continue;      // nothing was loaded for it
       const int kb = (blk + u * S_WAVES) * KBLK + kh + g * 8;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -1030,10 +1033,10 @@ static int launch_skinny_deep(const SkinnyArgs& p, hipStream_t stream) {
   return TL_OK;
 }
 
-// 8 columns a workgroup: for at most 8 rows, where a wave would otherwise work through its share
-// of a long inner size in several dependent round trips to memory, and where that still gives
-// no more workgroups than there are compute units (measured: otherwise it is slower).
-static bool skinny_half(int M, int N, int K) { return M <= 8 && K > 2048 && (N + 7) / 8 <= 256; }
+// 8 columns a workgroup: for at most 8 rows and an inner size that gives every wave at least
+// one block of four MFMAs, where that still gives no more workgroups than there are compute
+// units (measured: otherwise it is slower).
+static bool skinny_half(int M, int N, int K) { return M <= 8 && K >= 2048 && (N + 7) / 8 <= 256; }
 
 template <int MT, int CT, typename TO, int PRO, bool SWIGLU>
 static int launch_skinny_tile(const SkinnyArgs& p, hipStream_t stream) {
