@@ -100,7 +100,8 @@ def test_lm_head_last_rows_reference_vector():
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,K,N", [(127, 255, 353), (1, 64, 251), (7, 176, 64), (130, 96, 517), (64, 2048, 256),
                                    (300, 5632, 136), (9, 5640, 520), (16, 4104, 40), (8, 5640, 524), (3, 2056, 2044),
-                                   (5, 9000, 72), (8, 64, 4100), (12, 96, 8200), (16, 72, 12300), (7, 64, 8200)])
+                                   (5, 9000, 72), (8, 64, 4100), (12, 96, 8200), (16, 72, 12300), (7, 64, 8200),
+                                   (5, 64, 2500), (16, 96, 3302)])
 def test_linear_sizes(dtype, M, K, N):
     if dtype == torch.bfloat16 and K % 8:
         K = K + 8 - K % 8
@@ -188,7 +189,7 @@ def test_linear_norm(M, K, N):
 
 
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 40, 64])
-@pytest.mark.parametrize("K,N,N2", [(64, 248, 96), (5632, 2048, 516), (176, 64, 40), (96, 520, 1030), (2120, 1000, 72), (64, 4200, 40), (64, 64, 8300)])
+@pytest.mark.parametrize("K,N,N2", [(64, 248, 96), (5632, 2048, 516), (176, 64, 40), (96, 520, 1030), (2120, 1000, 72), (64, 4200, 40), (64, 64, 8300), (64, 2600, 3000)])
 def test_linear_handoff(M, K, N, N2):
     """A norm handed from the product that writes the residual stream to the product that reads
     it: the first also writes bf16(w * x) and partial sums of x^2, the second applies 1 / rms."""

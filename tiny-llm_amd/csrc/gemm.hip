@@ -703,6 +703,9 @@ struct SkinnyArgs {
   const float* in_sumsq = nullptr;
   int in_parts = 0, in_width = 0;
   float in_eps = 0.f;
+  // One row tile, one column tile: the columns a workgroup owns, at most 16 and even (0: all 16).
+  // Fewer make one balanced round of workgroups out of a product with 129 to 255 column tiles.
+  int cols_wg = 0;
 };
 
 // One 8-wide k chunk of an activation row, as loaded (Raw) and as an MFMA operand.  With the norm
@@ -784,13 +787,14 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
   float* ss_part = (float*)(part + S_WAVES * MT * CT);              // [S_WAVES][MT * 16]
   const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
   const int M = p.M, N = p.N, K = p.K;
-  const int n0 = blockIdx.x * (COLS * CT);
+  const int cw = (MT * CT == 1 && !HALF && p.cols_wg > 0) ? p.cols_wg : COLS * CT;      // columns of this workgroup
+  const int n0 = blockIdx.x * cw;
   const int r16 = lane % 16, g = lane / 16;
   const int rr = HALF ? r16 % 8 : r16;             // the weight row / activation row this lane feeds
   const int kh = HALF ? (r16 / 8) * 32 : 0;        // and its k offset inside an MFMA's range
   const bf16_t* wrow[CT];
 #pragma unroll
-  for (int ct = 0; ct < CT; ++ct) wrow[ct] = p.w + (int64_t)min(n0 + ct * 16 + rr, N - 1) * K;
+  for (int ct = 0; ct < CT; ++ct) wrow[ct] = p.w + (int64_t)min(n0 + min(ct * 16 + rr, cw - 1), N - 1) * K;
 
   // epilogue operands first: their latency hides behind the main loop
   constexpr int TILES = MT * CT;
@@ -802,7 +806,7 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
     const int tile = e / 256;
     const int m = HALF ? e / 8 : (tile / CT) * 16 + (e % 256) / 16;
     const int n = HALF ? n0 + e % 8 : n0 + (tile % CT) * 16 + e % 16;
-    res_v[j] = (p.residual && e < (HALF ? 64 : TILES * 256) && m < M && n < N) ? p.residual[(int64_t)m * p.ldo + n] : 0.f;
+    res_v[j] = (p.residual && e < (HALF ? 64 : TILES * 256) && m < M && n < N && n - n0 < cw) ? p.residual[(int64_t)m * p.ldo + n] : 0.f;
   }
 
   // input row of each activation row this lane feeds
@@ -970,7 +974,7 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
     if (e >= (HALF ? 64 : TILES * 256)) continue;       // whole waves: 256 elements are four waves
     const int tile = e / 256, m_local = HALF ? e / 8 : (e % 256) / 16, nn = HALF ? e % 8 : e % 16;
     const int m = (tile / CT) * 16 + m_local, n = n0 + (tile % CT) * 16 + nn;
-    const bool valid = m < M && n < N;
+    const bool valid = m < M && n < N && n - n0 < cw;
     float scale = 1.f;                    // the row factor left out of the operands
     if (p.row_scale) scale = p.row_scale[min(m, M - 1)];
     if (p.in_sumsq) scale = scale_s[(tile / CT) * 16 + m_local];
@@ -1008,7 +1012,10 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
 #pragma unroll
           for (int off = 1; off < COLS; off <<= 1) sq += __shfl_xor(sq, off, TL_WAVE);
           // a column group that begins beyond N has no part of its own
-          if (nn == 0 && m < M && n < N) p.emit_sumsq[(int64_t)m * ((N + COLS - 1) / COLS) + (n0 / COLS + tile % CT)] = sq;
+          if (nn == 0 && m < M && n < N) {
+            if (cw == COLS * CT) p.emit_sumsq[(int64_t)m * ((N + COLS - 1) / COLS) + (n0 / COLS + tile % CT)] = sq;
+            else p.emit_sumsq[(int64_t)m * ((N + cw - 1) / cw) + blockIdx.x] = sq;
+          }
         }
       }
     }
@@ -1028,9 +1035,19 @@ static int launch_skinny_deep(const SkinnyArgs& p, hipStream_t stream) {
     configured = true;
   }
   constexpr int cols = HALF ? 8 : S_COLS * CT;
-  dim3 g((p.N + cols - 1) / cols), b(S_THREADS);
+  const int cw = (MT * CT == 1 && !HALF && p.cols_wg > 0) ? p.cols_wg : cols;
+  dim3 g((p.N + cw - 1) / cw), b(S_THREADS);
   hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, CT, DEEP, TO, PRO, SWIGLU, HALF>), g, b, smem, stream, p);
   return TL_OK;
+}
+
+// Columns a workgroup owns in the plain one-tile kernel: 16, or fewer (even) where that turns 129
+// to 255 workgroups, which leave compute units idle, into one round of at most 256.
+static int skinny_cols_wg(int N) {
+  const int tiles = (N + S_COLS - 1) / S_COLS;
+  if (tiles <= 128 || tiles >= 256) return S_COLS;
+  const int cw = (N + 255) / 256;
+  return cw + (cw & 1);
 }
 
 // 8 columns a workgroup: for at most 8 rows and an inner size that gives every wave at least
@@ -1046,8 +1063,13 @@ static int launch_skinny_tile(const SkinnyArgs& p, hipStream_t stream) {
       return launch_skinny_deep<MT, CT, false, TO, PRO, SWIGLU, true>(p, stream);
     }
   }
-  if constexpr (MT * CT == 1 && PRO == PRO_NONE) {
-    if (p.K > 4096) return launch_skinny_deep<MT, CT, true, TO, PRO, SWIGLU>(p, stream);
+  if constexpr (MT * CT == 1) {
+    SkinnyArgs q = p;
+    q.cols_wg = skinny_cols_wg(p.N);
+    if constexpr (PRO == PRO_NONE) {
+      if (p.K > 4096) return launch_skinny_deep<MT, CT, true, TO, PRO, SWIGLU>(q, stream);
+    }
+    return launch_skinny_deep<MT, CT, false, TO, PRO, SWIGLU>(q, stream);
   }
   return launch_skinny_deep<MT, CT, false, TO, PRO, SWIGLU>(p, stream);
 }
@@ -1207,7 +1229,12 @@ int tl_linear_handoff(const void* a, const void* w, void* out, const float* resi
 
 // How many partial sums of squares per row tl_linear_handoff writes as a producer for these sizes
 // (one per workgroup: per 16 columns, or per 8 where workgroups own 8).
-int tl_handoff_parts(int M, int N, int K) { return skinny_half(M, N, K) ? (N + 7) / 8 : (N + 15) / 16; }
+int tl_handoff_parts(int M, int N, int K) {
+  if (skinny_half(M, N, K)) return (N + 7) / 8;
+  const bool one_tile = M <= 16 && !(M >= 8 && N > 256 * S_COLS && N <= 4 * 256 * S_COLS);
+  const int cw = one_tile ? skinny_cols_wg(N) : S_COLS;
+  return (N + cw - 1) / cw;
+}
 
 // See splitk_plan.  A caller that gets more than one split allocates a float32 workspace of
 // splits * M * N elements and calls tl_linear_splitk with the same sizes.
