@@ -212,12 +212,7 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
   const int row_lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
 
   // key range of the tile: union over its rows
-  int hi = pos, lo = row_valid ? row_lo : 0x7fffffff;
-#pragma unroll
-  for (int off = 8; off > 0; off >>= 1) {
-    hi = max(hi, __shfl_xor(hi, off, TL_WAVE));
-    lo = min(lo, __shfl_xor(lo, off, TL_WAVE));
-  }
+  const int hi = row_max_i32(pos), lo = row_min_i32(row_valid ? row_lo : 0x7fffffff);
   const int kv_end = hi + 1, kv_begin = lo;
   const int first_tile = kv_begin / FA_KT, last_tile = (kv_end + FA_KT - 1) / FA_KT;
   // Key tiles are dealt out in turn: tile (it0 + it) * stride + split * WAVES + wave belongs to
@@ -378,8 +373,7 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
           sc[kt][r] = sv;
           m_tile = fmaxf(m_tile, sv);
         }
-      m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, TL_WAVE));
-      m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, TL_WAVE));
+      m_tile = max_over_rows(m_tile);
       const float m_new = fmaxf(m_run, m_tile * c_log2);   // the scale is positive: the maximum commutes
       const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
       float psum = 0.f;
@@ -391,8 +385,7 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
           sc[kt][r] = p;
           psum += p;
         }
-      psum += __shfl_xor(psum, 16, TL_WAVE);
-      psum += __shfl_xor(psum, 32, TL_WAVE);
+      psum = sum_over_rows(psum);
       l_run = l_run * alpha + psum;
       m_run = m_new;
 #pragma unroll
@@ -693,8 +686,7 @@ __global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
               m_tile = fmaxf(m_tile, sv);
             }
         }
-        m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, TL_WAVE));
-        m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, TL_WAVE));
+        m_tile = max_over_rows(m_tile);
         // the maximum is taken over raw scores (the scale is positive) and scaled once
         const float m_new = fmaxf(m_run[rt], m_tile * c_log2);
         const float alpha = __builtin_amdgcn_exp2f(m_run[rt] - m_new);
@@ -798,8 +790,7 @@ __global__ __launch_bounds__(TL_WAVE) void flash_combine_kernel(const float* __r
     const int s = s0 + lane;
     M = fmaxf(M, s < n_splits ? part_ml[(row + s * step) * 2] : kNegBig);
   }
-#pragma unroll
-  for (int off = 1; off < TL_WAVE; off <<= 1) M = fmaxf(M, __shfl_xor(M, off, TL_WAVE));
+  M = wave_max(M);
   for (int d = lane; d < hd; d += TL_WAVE) {
     float acc = 0.f, L = 0.f;
     for (int s0 = 0; s0 < n_splits; s0 += FC_BATCH) {

@@ -819,8 +819,8 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
   }
 
   // Row factors of a norm whose sums of squares arrive in parts: one wave per row, fixed order.
-  // The first 256 parts of a row are requested here, ahead of everything else, and added up after
-  // the main loop: the request then costs no wait of its own.
+  // The first 256 parts of a row are requested here, ahead of everything else, and added up once
+  // the first weights have been requested (see the main loop).
   float* scale_s = ss_part + S_WAVES * MT * 16;                      // [MT * 16]
   constexpr int RPW = MT * 16 / S_WAVES;                             // rows per wave
   constexpr int PRE = 4;                                             // parts requested ahead, in wavefuls
@@ -830,10 +830,11 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
     for (int ri = 0; ri < RPW; ++ri) {
       const int m = min(wave + ri * S_WAVES, M - 1);
       const int64_t src = p.rows ? p.rows[m] : m;
+      const bool row_there = wave + ri * S_WAVES < M;        // the same for the whole wave
 #pragma unroll
       for (int h = 0; h < PRE; ++h) {
         const int q = lane + h * TL_WAVE;
-        pre[ri][h] = q < p.in_parts ? p.in_sumsq[src * p.in_parts + q] : 0.f;
+        pre[ri][h] = (row_there && q < p.in_parts) ? p.in_sumsq[src * p.in_parts + q] : 0.f;
       }
     }
   }
@@ -925,14 +926,17 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
     }
   };
   constexpr int STEP = S_WAVES * UN;
+  // The row factors are worked out while the first weights are on their way: their operands were
+  // requested before and arrive first, and the wave has nothing else to do until the weights come.
   if constexpr (TWO_STAGES) {
     Stage s0, s1;
     int blk = wave;
+    if (blk < nblk) load(s0, blk);
+    if (blk + STEP < nblk) load(s1, blk + STEP);
+    row_factors();
     if (blk < nblk) {
-      load(s0, blk);
       while (true) {
         const int b1 = blk + STEP;
-        if (b1 < nblk) load(s1, b1);
         multiply(s0, blk);
         if (b1 >= nblk) break;
         const int b2 = b1 + STEP;
@@ -940,16 +944,20 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
         multiply(s1, b1);
         if (b2 >= nblk) break;
         blk = b2;
+        if (blk + STEP < nblk) load(s1, blk + STEP);
       }
     }
   } else {
     Stage s0;
-    for (int blk = wave; blk < nblk; blk += STEP) {
-      load(s0, blk);
+    int blk = wave;
+    if (blk < nblk) load(s0, blk);
+    row_factors();
+    while (blk < nblk) {
       multiply(s0, blk);
+      blk += STEP;
+      if (blk < nblk) load(s0, blk);
     }
   }
-  row_factors();
   // tile layout: lane holds rows (weight rows) g*4 + r, column (activation row) r16
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
@@ -961,8 +969,7 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       float t = ss[mt];
-      t += __shfl_xor(t, 16, TL_WAVE);
-      t += __shfl_xor(t, 32, TL_WAVE);
+      t = sum_over_rows(t);
       if (g == 0) ss_part[wave * (MT * 16) + mt * 16 + r16] = t;
     }
   }
@@ -1009,8 +1016,7 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
             p.emit_operand[(int64_t)m * N + n] = (bf16_t)(wn * v);
           }
           float sq = valid ? v * v : 0.f;
-#pragma unroll
-          for (int off = 1; off < COLS; off <<= 1) sq += __shfl_xor(sq, off, TL_WAVE);
+          sq = group_sum<COLS>(sq);
           // a column group that begins beyond N has no part of its own
           if (nn == 0 && m < M && n < N) {
             if (cw == COLS * CT) p.emit_sumsq[(int64_t)m * ((N + COLS - 1) / COLS) + (n0 / COLS + tile % CT)] = sq;
