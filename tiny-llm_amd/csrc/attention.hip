@@ -410,19 +410,22 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
         const bf16x8 pb = __builtin_bit_cast(bf16x8, hi), pl = __builtin_bit_cast(bf16x8, lo);
         // lane s of a group names keys g*4 + s/4 of a 16-key block, dims dt*16 + 4*(s%4) ..
         const bf16_t* vsrc = Vl + ((2 * st) * 16 + g * 4 + r16 / 4) * VS + 4 * (r16 % 4);
+        bf16x8 vf[HDT];
 #pragma unroll
         for (int dt = 0; dt < HDT; ++dt) {
           const bf16x4 lo4 = lds_read_transposed(vsrc + dt * 16);
           const bf16x4 hi4 = lds_read_transposed(vsrc + 16 * VS + dt * 16);
-          bf16x8 vf;
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            vf[r] = lo4[r];
-            vf[4 + r] = hi4[r];
+            vf[dt][r] = lo4[r];
+            vf[dt][4 + r] = hi4[r];
           }
-          o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb, o[dt], 0, 0, 0);
-          o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pl, o[dt], 0, 0, 0);
         }
+        // the two products into one accumulator are kept HDT MFMAs apart
+#pragma unroll
+        for (int dt = 0; dt < HDT; ++dt) o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pb, o[dt], 0, 0, 0);
+#pragma unroll
+        for (int dt = 0; dt < HDT; ++dt) o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pl, o[dt], 0, 0, 0);
       }
     }
     // this wave's reads of its area are done before the next tile is written over it
