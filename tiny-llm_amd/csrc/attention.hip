@@ -787,8 +787,37 @@ __global__ __launch_bounds__(TL_WAVE) void flash_combine_kernel(const float* __r
                                                                 int n_tokens, int nq, int hd, int n_splits) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int64_t row = (int64_t)t * nq + h, step = (int64_t)n_tokens * nq;      // split s: row + s * step
-  // lane s holds (maximum, sum) of split s, s + 64, ...: one request each
-  float M = kNegBig;       // maxima are in units of log2 e; a split without keys has l = 0 and O = 0
+  // maxima are in units of log2 e; a split without keys has l = 0 and O = 0
+  if (n_splits <= FC_BATCH) {      // the usual case: ONE round trip, the maximum comes from the same loads
+    float m[FC_BATCH], l[FC_BATCH];
+#pragma unroll
+    for (int u = 0; u < FC_BATCH; ++u) {
+      const int64_t base = row + (int64_t)min(u, n_splits - 1) * step;
+      m[u] = part_ml[base * 2];
+      l[u] = part_ml[base * 2 + 1];
+    }
+    for (int d = lane; d < hd; d += TL_WAVE) {
+      float o[FC_BATCH];
+#pragma unroll
+      for (int u = 0; u < FC_BATCH; ++u) o[u] = part_o[(row + (int64_t)min(u, n_splits - 1) * step) * hd + d];
+      float M = kNegBig;
+#pragma unroll
+      for (int u = 0; u < FC_BATCH; ++u) M = fmaxf(M, m[u]);      // a repeated split changes nothing
+      float acc = 0.f, L = 0.f;
+#pragma unroll
+      for (int u = 0; u < FC_BATCH; ++u) {
+        if (u < n_splits) {
+          const float wgt = __builtin_amdgcn_exp2f(m[u] - M);
+          L += wgt * l[u];
+          acc += wgt * o[u];
+        }
+      }
+      out[(int64_t)t * out_stride + (int64_t)h * hd + d] = (bf16_t)(L > 0.f ? acc / L : 0.f);
+    }
+    return;
+  }
+  // lane s holds the maximum of split s, s + 64, ...
+  float M = kNegBig;
   for (int s0 = 0; s0 < n_splits; s0 += TL_WAVE) {
     const int s = s0 + lane;
     M = fmaxf(M, s < n_splits ? part_ml[(row + s * step) * 2] : kNegBig);
