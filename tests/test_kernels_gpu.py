@@ -543,7 +543,7 @@ def test_paged_attention_window_edge(dtype, window):
 
 
 FLASH_SHAPES = [(4, 2, 48, 32), (32, 4, 64, 16), (3, 1, 32, 8), (8, 8, 16, 16), (6, 2, 80, 16), (16, 1, 128, 64),
-                (5, 5, 112, 8), (12, 4, 96, 16)]
+                (5, 5, 112, 8), (12, 4, 96, 16), (8, 2, 64, 24), (4, 4, 32, 1), (2, 1, 64, 100)]
 
 
 @pytest.mark.parametrize("n_splits", [1, 3])
