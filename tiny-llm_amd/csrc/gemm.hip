@@ -834,7 +834,9 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
 #pragma unroll
       for (int h = 0; h < PRE; ++h) {
         const int q = lane + h * TL_WAVE;
-        pre[ri][h] = (row_there && q < p.in_parts) ? p.in_sumsq[src * p.in_parts + q] : 0.f;
+        pre[ri][h] = 0.f;
+        if (!row_there || h * TL_WAVE >= p.in_parts) continue;      // the same for the whole wave: nothing to ask for
+        if (q < p.in_parts) pre[ri][h] = p.in_sumsq[src * p.in_parts + q];
       }
     }
   }
