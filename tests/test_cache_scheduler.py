@@ -30,12 +30,12 @@ def test_pool_reference_vectors():
 
 
 def full(n=1):
-    return [CacheSpec(2, 16)] * n
+    return [CacheSpec.keys_and_values(2, 16)] * n
 
 
 def test_groups_by_need():
-    specs = [CacheSpec(2, 16), CacheSpec(2, 16, "window", 8), None, CacheSpec(2, 16), CacheSpec(2, 16, "window", 8),
-             CacheSpec(4, 16)]
+    kv = CacheSpec.keys_and_values
+    specs = [kv(2, 16), kv(2, 16, "window", 8), None, kv(2, 16), kv(2, 16, "window", 8), kv(4, 16)]
     cm = CacheManager(specs, [None] * 6, block_size=4, num_blocks=10, max_seqs=2)
     assert [g.entries for g in cm.groups] == [[0, 3], [1, 4], [5]]
     assert cm.group_of_entry == {0: 0, 3: 0, 1: 1, 4: 1, 5: 2}
@@ -81,7 +81,7 @@ def test_slots_run_out_and_come_back():
 
 
 def test_window_gives_blocks_back_as_it_passes():
-    spec = [CacheSpec(1, 8), CacheSpec(1, 8, "window", 6)]
+    spec = [CacheSpec.keys_and_values(1, 8), CacheSpec.keys_and_values(1, 8, "window", 6)]
     cm = CacheManager(spec, [None, None], block_size=4, num_blocks=8, max_seqs=2)
     cm.reserve_step([("a", 10)])
     cm.commit("a", 10)        # next query at >= 10 reads keys >= 5: block 0 (0..3) of the window group is done
@@ -102,7 +102,7 @@ def test_window_gives_blocks_back_as_it_passes():
 @pytest.mark.parametrize("seed", range(6))
 def test_no_page_lost_held_twice_or_freed_twice_under_random_orders(seed):
     rng = random.Random(seed)
-    spec = [CacheSpec(2, 16), CacheSpec(2, 16, "window", 11), CacheSpec(2, 16)]
+    spec = [CacheSpec.keys_and_values(2, 16), CacheSpec.keys_and_values(2, 16, "window", 11), CacheSpec.keys_and_values(2, 16)]
     cm = CacheManager(spec, [None, StateSpec((2,)), None], block_size=4, num_blocks=40, max_seqs=5)
     live = {}
     n_new = 0
@@ -225,11 +225,14 @@ def test_admission_waits_for_slots_and_blocks():
     assert [e.request.req_id for e in p.entries] == ["a", "b"]      # two slots
     run_plan(cm, s, p)
     assert [r.req_id for r in s.waiting] == ["c"]
-    while s.running:
-        run_plan(cm, s, s.schedule())
-    assert [r.req_id for r in s.running + list(s.waiting)] == [] or s.has_work()
+    admitted_c_with_finished = None
     while s.has_work():
-        run_plan(cm, s, s.schedule())
+        p = s.schedule()
+        if admitted_c_with_finished is None and any(e.request.req_id == "c" for e in p.entries):
+            admitted_c_with_finished = sorted(r.req_id for r in s.finished)
+        assert len(s.running) <= 2
+        run_plan(cm, s, p)
+    assert admitted_c_with_finished == ["a", "b"]                   # c got a slot only when one was given back
     assert sorted(r.req_id for r in s.finished) == ["a", "b", "c"]
     assert all(len(r.output) == 3 for r in s.finished)
 

@@ -5,7 +5,7 @@ import os
 import pytest
 import torch
 
-from util import TINY_A, TINY_B
+from util import REFERENCE_DATA, TINY_A, TINY_B
 
 from tiny_llm_amd.config import (ConfigError, EngineConfig, LlamaConfig, UnknownArchitecture, known_architectures,
                                  resolve)
@@ -18,14 +18,22 @@ from tiny_llm_amd.parts.base import WeightSpec
 
 def test_reference_config_file_parses_to_tinyllama_sizes():
     # the reference's own fixture (tests/datas/llama_config.json), as tests/parser/test_llama_parser.cpp:12-20 reads it
-    path = "/root/reference/tests/datas/llama_config.json"
+    path = os.path.join(REFERENCE_DATA, "llama_config.json")
     if not os.path.exists(path):
         pytest.skip("reference checkout not mounted")
     cfg = LlamaConfig.from_json(path)
     assert (cfg.num_hidden_layers, cfg.hidden_size, cfg.num_attention_heads, cfg.num_key_value_heads) == (22, 2048, 32, 4)
     assert (cfg.head_dim, cfg.intermediate_size, cfg.vocab_size, cfg.max_position_embeddings) == (64, 5632, 32000, 2048)
     assert cfg.rope_theta == 10000.0 and cfg.rms_norm_eps == 1e-5 and not cfg.tie_word_embeddings
-    assert cfg.eos_token_id == 2
+    assert cfg.eos_token_id == 2 and cfg.eos_token_ids == (2,)
+
+
+def test_every_end_of_sequence_id_is_kept():
+    d = dict(TINY_A, eos_token_id=[7, 9, 11])
+    cfg, spec = resolve(d)
+    assert cfg.eos_token_ids == (7, 9, 11) and spec.eos_token_ids == (7, 9, 11)
+    assert cfg.to_dict()["eos_token_id"] == [7, 9, 11]
+    assert resolve(dict(TINY_A, eos_token_id=None))[1].eos_token_ids == ()
 
 
 def test_defaults_and_head_dim_key():
@@ -56,9 +64,11 @@ def test_registry_chooses_by_architecture_name():
     assert "LlamaForCausalLM" in known_architectures()
     cfg, spec = resolve(TINY_B)
     assert spec.architecture == "LlamaForCausalLM" and len(spec.layers) == 3 and len(spec.plan) == 3
-    assert spec.layers[1].mixer.kind == "attention" and spec.layers[1].ffn.kind == "swiglu"
-    assert spec.layers[0].mixer.params["position"]["theta"] == 500000.0
-    assert spec.lm_head.params["tied"] is True
+    assert spec.layers[1].parts["mixer"].kind == "attention" and spec.layers[1].parts["ffn"].kind == "swiglu"
+    assert spec.layers[1].parts["mixer"].name == "self_attn" and spec.layers[1].block == "pre_norm"
+    assert spec.layers[0].parts["mixer"].params["position"]["theta"] == 500000.0
+    assert spec.lm_head.params["tied_to"] == "model.embed_tokens" and spec.embedding.name == "model.embed_tokens"
+    assert "tied_to" not in resolve(TINY_A)[1].lm_head.params
     with pytest.raises(UnknownArchitecture) as e:
         resolve(dict(TINY_A, architectures=["MambaForCausalLM"]))
     assert "LlamaForCausalLM" in str(e.value)
@@ -77,6 +87,38 @@ def test_no_size_stands_in_code():
     assert shapes["model.layers.0.mlp.down_proj.weight"] == (80, 72)
     assert shapes["lm_head.weight"] == (99, 80)
     assert len(shapes) == 3 + 4 * 9
+
+
+def test_sizes_a_kernel_refuses_are_refused_when_the_model_is_built():
+    """bfloat16 products move 16-byte vectors: a width that is no multiple of 8 fails at build time,
+    with the part and the size named; float32 takes it."""
+    from tiny_llm_amd.kernels.ops import KernelError
+    odd = dict(TINY_A, hidden_size=68, num_attention_heads=2, num_key_value_heads=1, head_dim=34)
+    _, spec = resolve(odd)
+    Decoder(spec, "float32", "cpu")
+    with pytest.raises(KernelError) as e:
+        Decoder(spec, "bfloat16", "cpu")
+    assert "68" in str(e.value) and "multiple of 8" in str(e.value)
+    _, spec = resolve(dict(TINY_A, intermediate_size=177))
+    with pytest.raises(KernelError) as e:
+        Decoder(spec, "bfloat16", "cpu")
+    assert "intermediate_size = 177" in str(e.value)
+    _, spec = resolve(dict(TINY_A, hidden_size=1056, num_attention_heads=4, num_key_value_heads=4, head_dim=264))
+    with pytest.raises(KernelError) as e:
+        Decoder(spec, "float32", "cpu")
+    assert "head_dim 264" in str(e.value)
+
+
+def test_cache_pool_is_sized_by_configuration_or_by_free_memory():
+    from tiny_llm_amd.engine.loading import plan_cache_blocks
+    e = EngineConfig(kv_block_size=16, max_num_seqs=4)
+    assert plan_cache_blocks(EngineConfig(num_kv_blocks=7), 100, 1000, 10 ** 9) == 7
+    assert plan_cache_blocks(EngineConfig(kv_block_size=16, max_cache_tokens=100), 100, 1000, 10 ** 9) == 7
+    assert plan_cache_blocks(e, 100, 1000, None) == 4 * 7                      # worst case: can never run out
+    assert plan_cache_blocks(e, 100, 1000, 10 ** 9) == 28                      # memory is plenty
+    assert plan_cache_blocks(e, 100, 1000, 20000) == 18                        # 0.9 of 20000 bytes / 1000
+    with pytest.raises(MemoryError):
+        plan_cache_blocks(e, 100, 1000, 500)
 
 
 def test_engine_config_checks():
@@ -121,6 +163,70 @@ def test_safetensors_rejects_damaged_files(tmp_path):
         SafetensorsFile(str(tmp_path / "absent.safetensors"))
 
 
+def test_tensors_set_by_hand_shadow_the_file(tmp_path):
+    # (ref) tests/weight_managers/test_safetensors.cpp:31-56: a missing name throws; set, read back,
+    # set again with another shape, read back; tensors of the file stay readable
+    from tiny_llm_amd.weights import Checkpoint
+    save_file({"embedding": torch.arange(6, dtype=torch.float32).reshape(2, 3),
+               "attention": torch.arange(10, 14, dtype=torch.float32).reshape(2, 2)},
+              str(tmp_path / "model.safetensors"))
+    ck = Checkpoint(str(tmp_path))
+    with pytest.raises(SafetensorsError):
+        ck.get("random")
+    mine = torch.tensor([100.0, 200.0])
+    ck.set_tensor("random", mine)
+    mine[0] = -1.0                                   # the checkpoint holds a copy
+    assert ck.info("random") == (torch.float32, (2,)) and ck.get("random").tolist() == [100.0, 200.0]
+    ck.set_tensor("random", torch.tensor([[50.0, 100.0]]))
+    assert ck.info("random") == (torch.float32, (1, 2)) and ck.get("random").tolist() == [[50.0, 100.0]]
+    ck.set_tensor("attention", torch.zeros(3))       # shadows the file's tensor
+    assert ck.get("attention").tolist() == [0, 0, 0] and ck.get("embedding").tolist() == [[0, 1, 2], [3, 4, 5]]
+    assert sorted(ck.names()) == ["attention", "embedding", "random"]
+    with pytest.raises(ValueError):
+        ck.set_tensor("empty", torch.zeros(0))
+
+
+def test_loading_through_a_checkpoint_with_tensors_set_by_hand(tmp_path):
+    from tiny_llm_amd.weights import Checkpoint
+    folder = write_random_model(str(tmp_path), TINY_A, seed=5)
+    ck = Checkpoint(folder)
+    ck.set_tensor("model.norm.weight", torch.full((64,), 3.0))
+    dec = _specs(TINY_A)
+    load_weights(dec, ck)
+    assert dec.final_norm.weight.tolist() == [3.0] * 64
+    ck.set_tensor("model.norm.weight", torch.full((63,), 3.0))
+    with pytest.raises(WeightLoadError) as e:
+        load_weights(_specs(TINY_A), ck)
+    assert e.value.wrong_shape == [("model.norm.weight", (64,), (63,))]
+
+
+def test_sharded_folder_loads_like_a_single_file(tmp_path):
+    """model.safetensors.index.json and its shards (how larger checkpoints are published)."""
+    single = write_random_model(str(tmp_path / "single"), TINY_B, seed=4, norm_std=0.1)
+    f = SafetensorsFile(os.path.join(single, "model.safetensors"))
+    names = f.names()
+    shard_dir = tmp_path / "sharded"
+    shard_dir.mkdir()
+    weight_map = {}
+    for i in range(3):
+        part = {n: f.get(n).clone() for n in names[i::3]}
+        fname = f"model-{i + 1:05d}-of-00003.safetensors"
+        save_file(part, str(shard_dir / fname))
+        weight_map.update({n: fname for n in part})
+    json.dump({"metadata": {}, "weight_map": weight_map}, open(shard_dir / "model.safetensors.index.json", "w"))
+    json.dump(json.load(open(os.path.join(single, "config.json"))), open(shard_dir / "config.json", "w"))
+    a, b = _specs(TINY_B), _specs(TINY_B)
+    load_weights(a, single)
+    load_weights(b, str(shard_dir))
+    for pa, pb in zip(a.parts(), b.parts()):
+        for k, v in vars(pa).items():
+            if isinstance(v, torch.Tensor):
+                assert torch.equal(v, getattr(pb, k)), (pa.prefix, k)
+    os.remove(shard_dir / "model-00002-of-00003.safetensors")
+    with pytest.raises(SafetensorsError):
+        load_weights(_specs(TINY_B), str(shard_dir))
+
+
 # ---------------------------------------------------------------------- loading
 def _specs(cfg):
     _, spec = resolve(cfg)
@@ -133,7 +239,7 @@ def test_random_model_folder_round_trip(tmp_path):
     dec = _specs(TINY_A)
     load_weights(dec, folder)       # device "cpu": binding needs no kernel
     assert dec.layers[0].mixer.w_qkv.shape == ((4 + 2 * 2) * 16, 64)
-    assert dec.layers[1].ffn.w_gate_up.shape == (2 * 176, 64)
+    assert dec.layers[1].by_role["ffn"].w_gate_up.shape == (2 * 176, 64)
     assert dec.lm_head.weight.shape == (251, 64)
     # the same (seed, name) gives the same tensor whatever else is generated, another seed another one
     again = write_random_model(str(tmp_path / "again"), TINY_A, seed=5)
@@ -145,6 +251,23 @@ def test_random_model_folder_round_trip(tmp_path):
     assert abs(float(a.std()) - 0.02) < 0.002
     spec = WeightSpec("model.layers.1.mlp.up_proj.weight", (176, 64))
     assert torch.equal(random_tensor(spec, 5, 0.02, 0.0), a)
+
+
+def test_seeded_numbers_are_normal_and_a_pure_function_of_seed_name_and_index():
+    from tiny_llm_amd.weights.loader import _standard_normal_host, tensor_key
+    z = torch.from_numpy(_standard_normal_host(tensor_key(1, "x"), 1 << 20)).double()
+    assert abs(float(z.mean())) < 5e-3 and abs(float(z.std()) - 1) < 5e-3
+    assert abs(float((z ** 4).mean()) - 3) < 0.05 and abs(float((z ** 3).mean())) < 0.02
+    assert abs(float((z.abs() < 1).double().mean()) - 0.6827) < 3e-3
+    # element i does not depend on how many elements are made, nor on the chunking
+    a = _standard_normal_host(tensor_key(1, "x"), 1000, chunk=64)
+    assert torch.equal(torch.from_numpy(a), z[:1000].float())
+    # a norm weight: 1 + norm_std * z, each operation rounded to float32
+    n = random_tensor(WeightSpec("n.weight", (50,), role="vector", init="ones"), 9, 0.02, 0.1)
+    zz = torch.from_numpy(_standard_normal_host(tensor_key(9, "n.weight"), 50))
+    assert torch.equal(n, zz * torch.tensor(0.1, dtype=torch.float32) + 1.0)
+    assert torch.equal(random_tensor(WeightSpec("n.weight", (50,), role="vector", init="ones"), 9, 0.02, 0.0),
+                       torch.ones(50))
 
 
 def test_tied_head_is_not_stored_and_shares_the_table(tmp_path):
@@ -168,7 +291,7 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     del tensors["model.norm.weight"]
     tensors["model.layers.1.self_attn.o_proj.weight"] = torch.zeros(64, 32)
     tensors["model.layers.7.mlp.up_proj.weight"] = torch.zeros(2, 2)
-    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)      # known and ignorable
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)      # the architecture says: ignorable
     save_file(tensors, path)
     with pytest.raises(WeightLoadError) as e:
         load_weights(_specs(TINY_A), folder)
@@ -180,6 +303,24 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     text = str(err)
     for word in ("missing", "unexpected", "wrong shapes", "model.norm.weight", "[64, 32]"):
         assert word in text
+
+
+def test_what_may_be_ignored_is_the_architectures_to_say(tmp_path):
+    import dataclasses
+    folder = write_random_model(str(tmp_path), TINY_A, seed=5)
+    path = os.path.join(folder, "model.safetensors")
+    f = SafetensorsFile(path)
+    tensors = {n: f.get(n).clone() for n in f.names()}
+    del f
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)
+    save_file(tensors, path)
+    _, spec = resolve(TINY_A)
+    assert spec.ignorable_tensors == ("*.rotary_emb.inv_freq",)
+    load_weights(Decoder(spec, "float32", "cpu"), folder)
+    strict = dataclasses.replace(spec, ignorable_tensors=())
+    with pytest.raises(WeightLoadError) as e:
+        load_weights(Decoder(strict, "float32", "cpu"), folder)
+    assert e.value.unexpected == ["model.layers.0.self_attn.rotary_emb.inv_freq"]
 
 
 def test_untied_model_needs_its_head(tmp_path):

@@ -57,8 +57,8 @@ def fake_ctx(lens, q_lens, block_size, n_groups=1, shuffle_seed=0):
 # ----------------------------------------------------------------- parts alone
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_norm_ffn_embedding_head_parts(dtype):
-    from tiny_llm_amd.parts import FEED_FORWARDS, NORMS
-    from tiny_llm_amd.parts.embedding import LMHead, TokenEmbedding
+    from tiny_llm_amd.parts import EMBEDDINGS, FEED_FORWARDS, HEADS, NORMS
+    TokenEmbedding, LMHead = EMBEDDINGS.get("token_embedding"), HEADS.get("lm_head")
     g = torch.Generator().manual_seed(3)
     H, I, V, T = 80, 136, 123, 19
     tol = 1e-5 if dtype == torch.float32 else 1e-2
@@ -122,7 +122,7 @@ def test_attention_part_alone(dtype, nq, nkv, hd, bs, window):
     ctx2, nblocks = fake_ctx(lens, [l - c for l, c in zip(lens, cut)], bs)
     kc = torch.full((nblocks, nkv, bs, hd), float("nan"), dtype=dtype, device=DEV)
     vc = torch.full((nblocks, nkv, bs, hd), float("nan"), dtype=dtype, device=DEV)
-    cache = LayerCache(kc, vc, 0, True)
+    cache = LayerCache({"k": kc, "v": vc}, 0, True)
     live = [r for r, c in enumerate(cut) if c > 0]
     ctx1, _ = fake_ctx([cut[r] for r in live], [cut[r] for r in live], bs)
     ctx1.block_tables = [ctx2.block_tables[0][live][:, :ctx1.block_tables[0].shape[1]].contiguous()]
@@ -327,8 +327,8 @@ def test_toy_stateful_mixer_registers_builds_and_steps(tmp_path):
     """A mixer with per-request state of fixed size (an exponential running mean), defined here.
     The toy model mixes it with attention layers, runs one layer twice and lets one run read
     another run's cache.  Cutting its input differently must not change its logits."""
-    from tiny_llm_amd.config import (EngineConfig, LayerSpec, ModelSpec, PartSpec, PlanEntry, register_architecture,
-                                     unregister_architecture)
+    from tiny_llm_amd.config import (EngineConfig, ModelSpec, PartSpec, PlanEntry, pre_norm_layer,
+                                     register_architecture, unregister_architecture)
     from tiny_llm_amd.engine.loading import build_runner, random_model
     from tiny_llm_amd.engine.step import StepEntry
     from tiny_llm_amd.parts import MIXERS, Mixer, StateSpec, WeightSpec, add_to_residual, register_mixer
@@ -371,13 +371,14 @@ def test_toy_stateful_mixer_registers_builds_and_steps(tmp_path):
         win = PartSpec("attention", {"hidden_size": H, "num_heads": 4, "num_kv_heads": 2, "head_dim": 16, "window": 5,
                                      "position": {"kind": "none"}})
         toy = PartSpec("toy_decay", {"hidden_size": H, "decay": 0.5})
-        layers = tuple(LayerSpec(f"model.layers.{i}", "pre_norm", norm, m, norm, ffn) for i, m in enumerate([attn, toy, win]))
+        layers = tuple(pre_norm_layer(f"model.layers.{i}", norm, m, norm, ffn) for i, m in enumerate([attn, toy, win]))
         # layer 0, layer 1 (state), layer 2 (window), layer 0 again with a cache of its own,
         # then layer 0 once more reading the first run's cache
         plan = (PlanEntry(0), PlanEntry(1), PlanEntry(2), PlanEntry(0), PlanEntry(0, cache_of=0))
-        return ModelSpec("ToyForCausalLM", cfg["vocab_size"], H, 256, PartSpec("token_embedding", {
-            "vocab_size": cfg["vocab_size"], "hidden_size": H}), layers, plan, norm,
-            PartSpec("lm_head", {"vocab_size": cfg["vocab_size"], "hidden_size": H, "tied": True}))
+        sizes = {"vocab_size": cfg["vocab_size"], "hidden_size": H}
+        return ModelSpec("ToyForCausalLM", cfg["vocab_size"], H, 256, PartSpec("token_embedding", sizes, "model.embed_tokens"),
+                         layers, plan, norm.named("model.norm"),
+                         PartSpec("lm_head", dict(sizes, tied_to="model.embed_tokens"), "lm_head"))
 
     register_mixer("toy_decay", DecayMixer)
     register_architecture("ToyForCausalLM", read, build)
@@ -387,8 +388,8 @@ def test_toy_stateful_mixer_registers_builds_and_steps(tmp_path):
                               max_num_batched_tokens=256, use_graphs=False)
         _, dec = random_model(raw, engine, seed=1, std=0.3)
         runner = build_runner(dec, engine)
-        assert [g.entries for g in runner.cache.groups] == [[0, 3], [2]]       # full and windowed groups
-        assert runner.decoder.states[1].shape == (3, 64) and runner.decoder.states[0] is None
+        assert [g.entries for g in runner.cache.groups] == [[(0, "mixer"), (3, "mixer")], [(2, "mixer")]]   # full, windowed
+        assert runner.decoder.states[1]["mixer"].shape == (3, 64) and runner.decoder.states[0] == {}
         a, b = random_tokens(45, 101, 1), random_tokens(23, 101, 2)
         whole = runner.step([StepEntry("a", a, list(range(45))), StepEntry("b", b, list(range(23)))]).cpu()
         runner.finish("a")
@@ -427,13 +428,14 @@ def test_toy_routed_feed_forward_and_other_position_encoding(dtype):
     """A feed-forward with routing (two experts, the larger router logit takes the token) and a
     position encoding of its own (a rotation of the first half of each head with doubled angles),
     both defined here, in a toy architecture: registered, built, and stepped in different cuttings."""
-    from tiny_llm_amd.config import (EngineConfig, LayerSpec, ModelSpec, PartSpec, PlanEntry, register_architecture,
-                                     unregister_architecture)
+    from tiny_llm_amd.config import (EngineConfig, ModelSpec, PartSpec, PlanEntry, pre_norm_layer,
+                                     register_architecture, unregister_architecture)
     from tiny_llm_amd.engine.loading import build_runner, random_model
     from tiny_llm_amd.engine.step import StepEntry
     from tiny_llm_amd.kernels import ops
-    from tiny_llm_amd.parts import (FEED_FORWARDS, POSITION_ENCODINGS, FeedForward, PositionEncoding, WeightSpec,
-                                    add_to_residual, register_feed_forward, register_position_encoding)
+    from tiny_llm_amd.parts import (EMBEDDINGS, FEED_FORWARDS, HEADS, POSITION_ENCODINGS, Embedding, FeedForward, Head,
+                                    PositionEncoding, WeightSpec, add_to_residual, register_embedding,
+                                    register_feed_forward, register_head, register_position_encoding)
 
     class DoubledHalfRotary(PositionEncoding):
         def __init__(self, prefix, dtype, device, *, head_dim, max_position):
@@ -481,6 +483,37 @@ def test_toy_routed_feed_forward_and_other_position_encoding(dtype):
                 y[rows] = out
             return add_to_residual(residual, y)
 
+    class ScaledEmbedding(Embedding):
+        """An embedding with a scale and a table under another name, looked up with torch."""
+        def __init__(self, prefix, dtype, device, *, vocab_size, hidden_size, scale):
+            super().__init__(prefix, dtype, device)
+            self.V, self.H, self.scale = vocab_size, hidden_size, scale
+
+        def weights(self):
+            return [WeightSpec(f"{self.prefix}.table", (self.V, self.H))]
+
+        def bind(self, tensors):
+            self.table = tensors[f"{self.prefix}.table"]
+
+        def forward(self, tokens, ctx=None):
+            return (self.table[tokens.long()].float() * self.scale).contiguous()
+
+    class CappedHead(Head):
+        """A head of its own name whose logits are soft-capped: cap * tanh(logits / cap)."""
+        def __init__(self, prefix, dtype, device, *, vocab_size, hidden_size, cap):
+            super().__init__(prefix, dtype, device)
+            self.V, self.H, self.cap = vocab_size, hidden_size, cap
+
+        def weights(self):
+            return [WeightSpec(f"{self.prefix}.proj", (self.V, self.H))]
+
+        def bind(self, tensors):
+            self.w = tensors[f"{self.prefix}.proj"].contiguous()
+
+        def forward(self, h):
+            out = torch.empty((h.shape[0], self.V), dtype=torch.float32, device=h.device)
+            return self.cap * torch.tanh(ops.linear(h, self.w, out) / self.cap)
+
     def build(cfg):
         H = cfg["hidden_size"]
         norm = PartSpec("rmsnorm", {"hidden_size": H, "eps": 1e-5})
@@ -488,25 +521,36 @@ def test_toy_routed_feed_forward_and_other_position_encoding(dtype):
                                       "position": {"kind": "doubled_half_rotary", "head_dim": 16, "max_position": 256}})
         dense = PartSpec("swiglu", {"hidden_size": H, "intermediate_size": 96})
         routed = PartSpec("two_experts", {"hidden_size": H, "intermediate_size": 40})
-        layers = (LayerSpec("model.layers.0", "pre_norm", norm, attn, norm, routed),
-                  LayerSpec("model.layers.1", "pre_norm", norm, attn, norm, dense))
+        names = {"mixer_norm": "ln1", "mixer": "attn", "ffn_norm": "ln2", "ffn": "moe"}
+        layers = (pre_norm_layer("decoder.h.0", norm, attn, norm, routed, names),
+                  pre_norm_layer("decoder.h.1", norm, attn, norm, dense, names))
         return ModelSpec("Toy2ForCausalLM", cfg["vocab_size"], H, 256,
-                         PartSpec("token_embedding", {"vocab_size": cfg["vocab_size"], "hidden_size": H}), layers,
-                         (PlanEntry(0), PlanEntry(1)), norm,
-                         PartSpec("lm_head", {"vocab_size": cfg["vocab_size"], "hidden_size": H, "tied": True}))
+                         PartSpec("scaled_embedding", {"vocab_size": cfg["vocab_size"], "hidden_size": H, "scale": 2.0},
+                                  "decoder.wte"), layers,
+                         (PlanEntry(0), PlanEntry(1)), norm.named("decoder.ln_f"),
+                         PartSpec("capped_head", {"vocab_size": cfg["vocab_size"], "hidden_size": H, "cap": 3.0},
+                                  "output"))
 
     register_position_encoding("doubled_half_rotary", DoubledHalfRotary)
     register_feed_forward("two_experts", TwoExperts)
+    register_embedding("scaled_embedding", ScaledEmbedding)
+    register_head("capped_head", CappedHead)
     register_architecture("Toy2ForCausalLM", dict, build)
     try:
         raw = {"architectures": ["Toy2ForCausalLM"], "hidden_size": 64, "vocab_size": 101}
         engine = EngineConfig(dtype=dtype, kv_block_size=8, max_cache_tokens=256, max_num_seqs=3,
                               max_num_batched_tokens=256, use_graphs=False)
         _, dec = random_model(raw, engine, seed=3, std=0.3)
+        # embedding, head and layers carry the names this architecture gave them
+        names = {s.name for s in dec.weight_specs()}
+        assert {"decoder.wte.table", "output.proj", "decoder.ln_f.weight", "decoder.h.0.attn.q_proj.weight",
+                "decoder.h.0.moe.router.weight", "decoder.h.1.ln2.weight"} <= names
+        assert not any(n.startswith(("model.", "lm_head")) for n in names)
         runner = build_runner(dec, engine)
         a, b = random_tokens(41, 101, 5), random_tokens(18, 101, 6)
         whole = runner.step([StepEntry("a", a, list(range(41))), StepEntry("b", b, list(range(18)))]).cpu()
         assert used == {0, 1}                       # both experts got tokens
+        assert float(whole.abs().max()) <= 3.0 and float(whole.abs().max()) > 1.0      # the head's cap is at work
         runner.finish("a")
         runner.finish("b")
         got_a, got_b, at_a, at_b = [], [], 0, 0
@@ -529,4 +573,6 @@ def test_toy_routed_feed_forward_and_other_position_encoding(dtype):
     finally:
         FEED_FORWARDS.unregister("two_experts")
         POSITION_ENCODINGS.unregister("doubled_half_rotary")
+        EMBEDDINGS.unregister("scaled_embedding")
+        HEADS.unregister("capped_head")
         unregister_architecture("Toy2ForCausalLM")

@@ -11,8 +11,8 @@ import pytest
 import torch
 
 import plain_llama as plain
+from util import REFERENCE_DATA as DATA
 
-DATA = "/root/reference/tests/datas"
 needs_reference = pytest.mark.skipif(not os.path.isdir(DATA), reason="reference checkout not mounted")
 
 
@@ -184,14 +184,98 @@ def test_window_and_shift_of_all_positions():
     assert torch.allclose(plain.attention(q, k, v, range(100, 112), window=3), w3)
 
 
-def test_model_invariants():
-    from util import TINY_B, random_tokens
+def _tiny_weights(cfg, seed=3, std=0.05, norm_std=0.1):
     from tiny_llm_amd.weights.loader import random_tensor
     from tiny_llm_amd.config import resolve
     from tiny_llm_amd.models.decoder import Decoder
-    _, spec = resolve(TINY_B)
+    _, spec = resolve(cfg)
     dec = Decoder(spec, "float32", "cpu")
-    w = {s.name: random_tensor(s, 3, 0.05, 0.1).double() for s in dec.weight_specs() if not s.alias_of}
+    return {s.name: random_tensor(s, seed, std, norm_std).double() for s in dec.weight_specs() if not s.alias_of}
+
+
+def _library_model(w, cfg, tokens, causal):
+    """The whole model from torch's own routines only, for the cases in which the rotation is the
+    identity (every token at position 0): embedding, rms_norm, linear, scaled_dot_product_attention
+    with keys and values repeated per group, silu.  Layer order as tiny_llm/parser/llama_parser.cpp:194-271."""
+    F = torch.nn.functional
+    H, nq = cfg["hidden_size"], cfg["num_attention_heads"]
+    nkv = cfg.get("num_key_value_heads", nq)
+    hd = cfg.get("head_dim") or H // nq
+    eps = cfg["rms_norm_eps"]
+    T = len(tokens)
+    x = F.embedding(torch.tensor(tokens), w["model.embed_tokens.weight"])
+    for i in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{i}"
+        h = F.rms_norm(x, (H,), w[f"{p}.input_layernorm.weight"], eps)
+        q = F.linear(h, w[f"{p}.self_attn.q_proj.weight"]).view(T, nq, hd).transpose(0, 1)
+        k = F.linear(h, w[f"{p}.self_attn.k_proj.weight"]).view(T, nkv, hd).transpose(0, 1)
+        v = F.linear(h, w[f"{p}.self_attn.v_proj.weight"]).view(T, nkv, hd).transpose(0, 1)
+        k, v = k.repeat_interleave(nq // nkv, 0), v.repeat_interleave(nq // nkv, 0)
+        o = F.scaled_dot_product_attention(q, k, v, is_causal=causal).transpose(0, 1).reshape(T, nq * hd)
+        x = x + F.linear(o, w[f"{p}.self_attn.o_proj.weight"])
+        h = F.rms_norm(x, (H,), w[f"{p}.post_attention_layernorm.weight"], eps)
+        x = x + F.linear(F.silu(F.linear(h, w[f"{p}.mlp.gate_proj.weight"])) * F.linear(h, w[f"{p}.mlp.up_proj.weight"]),
+                         w[f"{p}.mlp.down_proj.weight"])
+    head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings") else w["lm_head.weight"]
+    return F.linear(F.rms_norm(x, (H,), w["model.norm.weight"], eps), head)
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_whole_model_reduces_to_library_routines_where_the_rotation_is_the_identity(name):
+    """With every token at position 0 nothing is rotated and (the mask comparing positions) every
+    token sees every other: the model is embedding, rms_norm, linear, unmasked attention and silu
+    of the library, in the reference's layer order.  A norm in another place, gate and up swapped,
+    the residual taken before instead of after, a missing final norm or another head-to-group
+    mapping all fail this.  One token alone is the causal case of it."""
+    from util import CONFIGS, random_tokens
+    cfg, _, init = CONFIGS[name]
+    w = _tiny_weights(cfg, 3, init["std"] * 3, max(init["norm_std"], 0.1))
+    toks = random_tokens(13, cfg["vocab_size"], 4)
+    got = plain.llama_forward(w, cfg, toks, positions=[0] * 13)
+    want = _library_model(w, cfg, toks, causal=False)
+    assert (got - want).abs().max() < 1e-9 * max(1.0, float(want.abs().max()))
+    one = plain.llama_forward(w, cfg, toks[:1])
+    assert (one - _library_model(w, cfg, toks[:1], causal=True)).abs().max() < 1e-9
+    # and the causal model agrees with the library on its FIRST row whatever follows (position 0)
+    assert (plain.llama_forward(w, cfg, toks)[0] - one[0]).abs().max() < 1e-9
+
+
+def test_whole_model_invariants_that_plausible_mistakes_break():
+    from util import TINY_A, random_tokens
+    cfg = TINY_A
+    w = _tiny_weights(cfg, 5, 0.08, 0.1)
+    toks = random_tokens(17, cfg["vocab_size"], 6)
+    base = plain.llama_forward(w, cfg, toks)
+    scaled = lambda key, c: {**w, **{k: v * c for k, v in w.items() if key in k}}
+    # the feed-forward is linear in `up` and in `down` but not in `gate` (SiLU sits on gate only)
+    up2, down2, gate2 = (plain.llama_forward(scaled(k, 2.0), cfg, toks) for k in ("up_proj", "down_proj", "gate_proj"))
+    assert (up2 - down2).abs().max() < 1e-9 and (up2 - base).abs().max() > 1e-3
+    assert (gate2 - up2).abs().max() > 1e-3
+    # attention is linear in `v` and in `o` alike, and only distances between positions count
+    v2, o2 = (plain.llama_forward(scaled(k, 2.0), cfg, toks) for k in ("v_proj", "o_proj"))
+    assert (v2 - o2).abs().max() < 1e-9 and (v2 - base).abs().max() > 1e-3
+    shifted = plain.llama_forward(w, cfg, toks, positions=range(300, 317))
+    assert (shifted - base).abs().max() < 1e-6       # the angle table is rounded to float32, as the reference's
+    # pre-norm: a norm's weight times c is its consumers' weights times c (the residual stream itself
+    # is not normed: scaling the embedding changes the logits, scaling after the final norm does not exist)
+    n2 = plain.llama_forward(scaled("input_layernorm", 3.0), cfg, toks)
+    qkv3 = plain.llama_forward({**w, **{k: v * 3.0 for k, v in w.items() if any(
+        p in k for p in ("q_proj", "k_proj", "v_proj"))}}, cfg, toks)
+    assert (n2 - qkv3).abs().max() < 1e-8 and (n2 - base).abs().max() > 1e-3
+    f2 = plain.llama_forward(scaled("model.norm", 3.0), cfg, toks)
+    assert (f2 - 3.0 * base).abs().max() < 1e-8                              # the final norm feeds the head alone
+    # zeroed o and down projections: the layers add nothing and the logits are head(norm(embedding))
+    z = scaled("down_proj", 0.0)
+    z = {k: (v * 0.0 if "o_proj" in k else v) for k, v in z.items()}
+    F = torch.nn.functional
+    x = F.embedding(torch.tensor(toks), w["model.embed_tokens.weight"])
+    want = F.linear(F.rms_norm(x, (cfg["hidden_size"],), w["model.norm.weight"], cfg["rms_norm_eps"]), w["lm_head.weight"])
+    assert (plain.llama_forward(z, cfg, toks) - want).abs().max() < 1e-9
+
+
+def test_model_invariants():
+    from util import TINY_B, random_tokens
+    w = _tiny_weights(TINY_B)
     toks = random_tokens(24, TINY_B["vocab_size"], 9)
     logits = plain.llama_forward(w, TINY_B, toks)
     assert logits.shape == (24, TINY_B["vocab_size"])

@@ -55,8 +55,8 @@ def make_runner(folder, dtype, block_size, max_tokens, poison=True):
     runner = build_runner(dec, engine)
     if poison:                      # stale or unwritten cache contents must never reach a result
         for g in runner.cache.groups:
-            g.k.fill_(float("nan"))
-            g.v.fill_(float("nan"))
+            for t in g.tensors.values():
+                t.fill_(float("nan"))
     return runner
 
 

@@ -4,6 +4,10 @@ import os
 
 import torch
 
+# Where the reference's checkout lies (its tests' fixtures are read from there, never run).
+REFERENCE = os.environ.get("TINY_LLM_REFERENCE", "/root/reference")
+REFERENCE_DATA = os.path.join(REFERENCE, "tests", "datas")
+
 # Two tiny configurations of the architecture that differ in every size and option.
 TINY_A = {
     "architectures": ["LlamaForCausalLM"], "model_type": "llama",

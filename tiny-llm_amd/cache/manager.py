@@ -7,8 +7,8 @@ never run out and frees everything when the whole batch is done
 
 * Layers whose mixers declare the same CacheSpec form a group.  A group has ONE
   block-id space and one block table per request that serves all its layers; each
-  layer has its own key and value tensor [blocks, kv_heads, block_size, head_dim]
-  indexed by those ids.
+  layer has its own tensors, the ones its CacheSpec describes (keys and values
+  [blocks, kv_heads, block_size, head_dim] for attention), indexed by those ids.
 * A "window" group gives a request's blocks back as soon as every position in them
   is more than `window` behind the next query; a "full" group when the request ends.
 * Blocks that are given back are used again by later growth, most recently freed first.
@@ -19,8 +19,9 @@ Everything here is host bookkeeping; device tensors are only allocated (by
 """
 from __future__ import annotations
 
+import math
 from dataclasses import dataclass, field
-from typing import Dict, Hashable, List, Optional, Sequence, Tuple
+from typing import Dict, Hashable, List, Mapping, Optional, Sequence, Tuple
 
 import torch
 
@@ -37,14 +38,15 @@ class NoFreeSlot(CacheError):
 @dataclass
 class CacheGroup:
     spec: CacheSpec
-    entries: List[int]                 # plan entries that own a cache in this group
+    entries: List[Hashable]            # owners (runs of layers) that keep a cache in this group
     pool: BlockPool
-    k: Optional[torch.Tensor] = None   # [len(entries), blocks, kv_heads, block_size, head_dim]
-    v: Optional[torch.Tensor] = None
+    # by tensor name: [len(entries), blocks, *page_shape]
+    tensors: Dict[str, torch.Tensor] = field(default_factory=dict)
 
-    @property
-    def bytes_per_block_per_layer(self) -> int:
-        return 0 if self.k is None else 2 * self.k[0, 0].numel() * self.k.element_size()
+    def elements_per_block(self, block_size: int) -> int:
+        """Elements one block takes over all owners and tensors of the group."""
+        per_token = sum(math.prod(t.shape) for t in self.spec.tensors)
+        return len(self.entries) * per_token * block_size
 
 
 @dataclass
@@ -55,21 +57,23 @@ class RequestCache:
 
 
 class CacheManager:
-    def __init__(self, cache_specs: Sequence[Optional[CacheSpec]], state_specs: Sequence[Optional[StateSpec]],
-                 block_size: int, num_blocks: int, max_seqs: int):
-        """cache_specs / state_specs: per plan entry, None where the entry has none."""
+    def __init__(self, cache_specs, state_specs, block_size: int, num_blocks: int, max_seqs: int):
+        """cache_specs / state_specs: {owner: spec} for the runs of layers that keep a cache or a
+        state (any hashable owner), or a sequence indexed by owner with None where there is none."""
+        if not isinstance(cache_specs, Mapping):
+            cache_specs = {i: c for i, c in enumerate(cache_specs) if c is not None}
+        if not isinstance(state_specs, Mapping):
+            state_specs = {i: c for i, c in enumerate(state_specs) if c is not None}
         if block_size <= 0:
             raise ValueError("block_size must be positive")
         self.block_size = int(block_size)
         self.num_blocks = int(num_blocks)
         self.max_seqs = int(max_seqs)
         self.groups: List[CacheGroup] = []
-        self.group_of_entry: Dict[int, int] = {}
-        self.index_in_group: Dict[int, int] = {}
+        self.group_of_entry: Dict[Hashable, int] = {}
+        self.index_in_group: Dict[Hashable, int] = {}
         by_key: Dict[Tuple, int] = {}
-        for i, cs in enumerate(cache_specs):
-            if cs is None:
-                continue
+        for i, cs in cache_specs.items():
             key = cs.group_key()
             if key not in by_key:
                 by_key[key] = len(self.groups)
@@ -78,30 +82,33 @@ class CacheManager:
             self.group_of_entry[i] = g
             self.index_in_group[i] = len(self.groups[g].entries)
             self.groups[g].entries.append(i)
-        self.state_specs = list(state_specs)
-        self.states: List[Optional[torch.Tensor]] = [None] * len(self.state_specs)
+        self.state_specs: Dict[Hashable, StateSpec] = dict(state_specs)
+        self.states: Dict[Hashable, torch.Tensor] = {}
         self._free_slots: List[int] = list(range(self.max_seqs - 1, -1, -1))
         self.requests: Dict[Hashable, RequestCache] = {}
 
     # ------------------------------------------------------------------- tensors
+    def elements_per_block(self) -> int:
+        """Cache elements one more block costs, over all groups (every group has `num_blocks`)."""
+        return sum(g.elements_per_block(self.block_size) for g in self.groups)
+
     def allocate_tensors(self, dtype: torch.dtype, device) -> None:
         for g in self.groups:
-            shape = (len(g.entries), self.num_blocks, g.spec.num_kv_heads, self.block_size, g.spec.head_dim)
-            g.k = torch.zeros(shape, dtype=dtype, device=device)
-            g.v = torch.zeros(shape, dtype=dtype, device=device)
-        for i, ss in enumerate(self.state_specs):
-            if ss is not None:
-                self.states[i] = torch.zeros((self.max_seqs, *ss.shape), dtype=ss.dtype, device=device)
+            for t in g.spec.tensors:
+                shape = (len(g.entries), self.num_blocks, *t.page_shape(self.block_size))
+                g.tensors[t.name] = torch.zeros(shape, dtype=dtype, device=device)
+        for owner, ss in self.state_specs.items():
+            self.states[owner] = torch.zeros((self.max_seqs, *ss.shape), dtype=ss.dtype, device=device)
 
-    def layer_cache(self, entry: int, cache_of: Optional[int] = None) -> Optional[LayerCache]:
-        """The view a plan entry's mixer gets: its own cache, or (read-only) the cache of `cache_of`."""
-        owner = entry if cache_of is None else cache_of
+    def layer_cache(self, owner: Hashable, cache_of: Optional[Hashable] = None) -> Optional[LayerCache]:
+        """The view a run's part gets: its own cache, or (read-only) the cache that `cache_of` owns."""
+        owner = owner if cache_of is None else cache_of
         if owner not in self.group_of_entry:
             return None
         g = self.group_of_entry[owner]
         grp = self.groups[g]
         j = self.index_in_group[owner]
-        return LayerCache(k=grp.k[j], v=grp.v[j], group=g, write=cache_of is None)
+        return LayerCache({name: t[j] for name, t in grp.tensors.items()}, group=g, write=cache_of is None)
 
     # ------------------------------------------------------------------ requests
     def has(self, req_id) -> bool:
@@ -118,9 +125,8 @@ class CacheManager:
             raise NoFreeSlot(f"all {self.max_seqs} request slots are taken")
         slot = self._free_slots.pop()
         self.requests[req_id] = RequestCache(slot, 0, [[] for _ in self.groups])
-        for st in self.states:
-            if st is not None:
-                st[slot].zero_()
+        for st in self.states.values():
+            st[slot].zero_()
         return slot
 
     def num_tokens(self, req_id) -> int:

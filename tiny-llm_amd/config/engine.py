@@ -19,7 +19,8 @@ class EngineConfig:
     dtype: str = "bfloat16"            # "bfloat16" (serving) or "float32" (true 32-bit)
     kv_block_size: int = 16            # tokens per cache page
     num_kv_blocks: Optional[int] = None  # pages per cache group; None = from max_cache_tokens
-    max_cache_tokens: Optional[int] = None
+    max_cache_tokens: Optional[int] = None  # None too: worst case, capped by free device memory
+    cache_memory_fraction: float = 0.9   # share of the free device memory the cache may take then
     max_num_seqs: int = 64             # live requests (state slots)
     max_num_batched_tokens: int = 2048  # token budget of one step
     max_model_len: Optional[int] = None  # None = the model's max_position_embeddings
@@ -33,5 +34,7 @@ class EngineConfig:
         self.dtype = DTYPES[self.dtype]
         if self.kv_block_size <= 0:
             raise ValueError("kv_block_size must be positive")
+        if not (0.0 < self.cache_memory_fraction <= 1.0):
+            raise ValueError("cache_memory_fraction must be in (0, 1]")
         if self.max_num_seqs <= 0 or self.max_num_batched_tokens <= 0:
             raise ValueError("max_num_seqs and max_num_batched_tokens must be positive")

@@ -10,7 +10,7 @@ from __future__ import annotations
 import json
 import os
 from dataclasses import dataclass, asdict
-from typing import Any, Mapping, Optional
+from typing import Any, Mapping, Optional, Tuple
 
 
 class ConfigError(ValueError):
@@ -42,7 +42,7 @@ class LlamaConfig:
     hidden_act: str
     attention_bias: bool
     mlp_bias: bool
-    eos_token_id: Optional[int]
+    eos_token_ids: Tuple[int, ...]       # every id that ends a request (config.json may list several)
     bos_token_id: Optional[int]
     torch_dtype: str
     initializer_range: float
@@ -70,8 +70,10 @@ class LlamaConfig:
                     "and config.json gives no head_dim")
             head_dim = hidden // nq
         eos = d.get("eos_token_id")
-        if isinstance(eos, (list, tuple)):
-            eos = eos[0] if eos else None
+        if eos is None:
+            eos = ()
+        elif not isinstance(eos, (list, tuple)):
+            eos = (eos,)
         arch = d.get("architectures") or ["LlamaForCausalLM"]
         cfg = cls(
             vocab_size=int(d["vocab_size"]),
@@ -88,7 +90,7 @@ class LlamaConfig:
             hidden_act=str(d.get("hidden_act", "silu")),
             attention_bias=bool(d.get("attention_bias", False)),
             mlp_bias=bool(d.get("mlp_bias", False)),
-            eos_token_id=None if eos is None else int(eos),
+            eos_token_ids=tuple(int(e) for e in eos),
             bos_token_id=None if d.get("bos_token_id") is None else int(d["bos_token_id"]),
             torch_dtype=str(d.get("torch_dtype", "float32")),
             initializer_range=float(d.get("initializer_range", 0.02)),
@@ -129,9 +131,16 @@ class LlamaConfig:
         if not (self.rope_theta > 0):
             raise ConfigError("rope_theta must be positive")
 
+    @property
+    def eos_token_id(self) -> Optional[int]:
+        """The first end-of-sequence id (None if the checkpoint names none)."""
+        return self.eos_token_ids[0] if self.eos_token_ids else None
+
     # ---------------------------------------------------------------- writing
     def to_dict(self) -> dict:
         d = asdict(self)
+        eos = d.pop("eos_token_ids")
+        d["eos_token_id"] = None if not eos else (eos[0] if len(eos) == 1 else list(eos))
         d["architectures"] = list(self.architectures)
         d["model_type"] = "llama"
         d["rope_scaling"] = None

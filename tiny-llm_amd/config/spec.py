@@ -12,24 +12,40 @@ from typing import Any, Mapping, Optional, Tuple
 
 @dataclass(frozen=True)
 class PartSpec:
-    """One part by registry name, with every size and constant it needs."""
+    """One part by registry name, with every size and constant it needs.
+
+    `name` is where its weights live: for the parts of a layer the component below the layer's
+    prefix ("self_attn" -> "model.layers.3.self_attn.*"), for the model's own parts (embedding,
+    final norm, output head) the whole prefix ("model.embed_tokens")."""
     kind: str
     params: Mapping[str, Any] = field(default_factory=dict)
+    name: str = ""
+
+    def named(self, name: str) -> "PartSpec":
+        return PartSpec(self.kind, self.params, name)
 
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """One layer: a mixer and a feed-forward, each behind its norm, in a block."""
+    """One layer: parts by role, and the block arrangement that runs them.
+
+    The roles are the arrangement's own ("pre_norm" has mixer_norm, mixer, ffn_norm and ffn; an
+    arrangement registered elsewhere may have others); the arrangement says which registry each
+    role is looked up in."""
     prefix: str                 # weight-name prefix, e.g. "model.layers.3"
-    block: str                  # arrangement of the four parts, e.g. "pre_norm"
-    mixer_norm: PartSpec
-    mixer: PartSpec
-    ffn_norm: PartSpec
-    ffn: PartSpec
-    # weight-name component of each part below `prefix`
-    part_names: Mapping[str, str] = field(default_factory=lambda: {
-        "mixer_norm": "input_layernorm", "mixer": "self_attn",
-        "ffn_norm": "post_attention_layernorm", "ffn": "mlp"})
+    block: str                  # arrangement, e.g. "pre_norm"
+    parts: Mapping[str, PartSpec]
+
+
+def pre_norm_layer(prefix: str, mixer_norm: PartSpec, mixer: PartSpec, ffn_norm: PartSpec, ffn: PartSpec,
+                   names: Optional[Mapping[str, str]] = None) -> LayerSpec:
+    """The usual layer: x + mixer(norm(x)), then x + ffn(norm(x)).  `names` gives the weight-name
+    component of each role; a part that already has a name keeps it, the others get the role."""
+    names = dict(names or {})
+    parts = {}
+    for role, ps in (("mixer_norm", mixer_norm), ("mixer", mixer), ("ffn_norm", ffn_norm), ("ffn", ffn)):
+        parts[role] = ps if ps.name else ps.named(names.get(role, role))
+    return LayerSpec(prefix, "pre_norm", parts)
 
 
 @dataclass(frozen=True)
@@ -46,17 +62,22 @@ class ModelSpec:
     vocab_size: int
     hidden_size: int
     max_position: int
-    embedding: PartSpec
+    embedding: PartSpec          # its `name` is the whole weight prefix
     layers: Tuple[LayerSpec, ...]
     plan: Tuple[PlanEntry, ...]
     final_norm: PartSpec
     lm_head: PartSpec
-    eos_token_id: Optional[int] = None
+    eos_token_ids: Tuple[int, ...] = ()
+    # glob patterns of tensors that checkpoints of this architecture carry and no part needs
+    ignorable_tensors: Tuple[str, ...] = ()
 
     def validate(self) -> None:
         n = len(self.layers)
         if not self.plan:
             raise ValueError("a model needs at least one plan entry")
+        for what in ("embedding", "final_norm", "lm_head"):
+            if not getattr(self, what).name:
+                raise ValueError(f"the model's {what} needs a weight prefix (PartSpec.name)")
         for i, e in enumerate(self.plan):
             if not (0 <= e.layer < n):
                 raise ValueError(f"plan entry {i} names layer {e.layer}, model has {n}")

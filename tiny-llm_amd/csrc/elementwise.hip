@@ -200,6 +200,25 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const int32_t* __restrict
   }
 }
 
+// ------------------------------------------------------- seeded normal numbers
+// out[i] = shift + scale * table[splitmix64(key + (i + 1) * golden) >> (64 - table_bits)]: a pure
+// function of (key, i).  The product and the sum are rounded to float32 one after the other (no
+// fused multiply-add), so a host that does the same two operations gets the same bits.
+template <typename T>
+__global__ void random_normal_kernel(T* __restrict__ out, int64_t n, uint64_t key, const float* __restrict__ table,
+                                     int table_bits, float scale, float shift) {
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (int64_t)gridDim.x * kThreads) {
+    uint64_t x = key + ((uint64_t)i + 1ull) * 0x9E3779B97F4A7C15ull;
+    x ^= x >> 30;
+    x *= 0xBF58476D1CE4E5B9ull;
+    x ^= x >> 27;
+    x *= 0x94D049BB133111EBull;
+    x ^= x >> 31;
+    const float z = table[x >> (64 - table_bits)];
+    out[i] = from_f32<T>(__fadd_rn(__fmul_rn(scale, z), shift));
+  }
+}
+
 }  // namespace
 
 #define TL_DISPATCH_T(dtype, ...)                 \
@@ -280,6 +299,21 @@ int tl_rope_store(void* qkv, const int32_t* positions, const float* cos_t, const
   TL_DISPATCH_T(dtype, hipLaunchKernelGGL(rope_store_kernel<T>, dim3(n_tokens), dim3(kThreads), 0, stream,
                                           (T*)qkv, positions, cos_t, sin_t, slot_mapping, (T*)k_cache,
                                           (T*)v_cache, nq, nkv, hd, rot, block_size, row_stride);)
+  return tl_launch_status();
+}
+
+// Seeded normal numbers (random-weights mode).  table: 2^table_bits float32 quantiles of N(0, 1).
+int tl_random_normal(void* out, int64_t n, uint64_t key, const float* table, int table_bits, float scale,
+                     float shift, int dtype, hipStream_t stream) {
+  if (n <= 0) return TL_OK;
+  if (table_bits < 1 || table_bits > 30 || (dtype != 0 && dtype != 1)) return TL_ERR_ARG;
+  const int blocks = (int)(ceil_div64(n, kThreads) < 65536 ? ceil_div64(n, kThreads) : 65536);
+  if (dtype == 0)
+    hipLaunchKernelGGL(random_normal_kernel<float>, dim3(blocks), dim3(kThreads), 0, stream, (float*)out, n, key,
+                       table, table_bits, scale, shift);
+  else
+    hipLaunchKernelGGL(random_normal_kernel<bf16_t>, dim3(blocks), dim3(kThreads), 0, stream, (bf16_t*)out, n, key,
+                       table, table_bits, scale, shift);
   return tl_launch_status();
 }
 

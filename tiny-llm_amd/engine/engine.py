@@ -32,10 +32,10 @@ class Engine:
         else:
             self.model_config, self.decoder = random_model(config, self.engine_config, weights_seed, init_std, norm_std)
         self.runner = build_runner(self.decoder, self.engine_config)
-        self.eos_token_id = self.decoder.spec.eos_token_id
+        self.eos_token_ids = tuple(self.decoder.spec.eos_token_ids)
         self.scheduler = Scheduler(self.runner.cache, self.engine_config.max_num_seqs,
                                    self.engine_config.max_num_batched_tokens, self.runner.max_model_len,
-                                   self.eos_token_id)
+                                   self.eos_token_ids)
         self.sampler = Sampler(self.decoder.device)
         self._ids = itertools.count()
         self.requests: Dict[Hashable, Request] = {}

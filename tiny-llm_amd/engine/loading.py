@@ -48,16 +48,37 @@ def random_model(config: Mapping, engine: EngineConfig, seed: int = 0, std: Opti
     return cfg, dec
 
 
+def plan_cache_blocks(engine: EngineConfig, max_len: int, bytes_per_block: int, free_bytes: Optional[int]) -> int:
+    """How many cache blocks every group gets.  A number in the configuration is taken as it is
+    (`num_kv_blocks`, or `max_cache_tokens` in blocks).  Otherwise: the worst case of
+    `max_num_seqs` requests of `max_len` tokens, which can never run out (the reference's rule,
+    tiny_llm/runtime/cuda/cuda_runtime.cpp:510-515), capped by `cache_memory_fraction` of the
+    device memory that is free once the weights are resident; a smaller pool is what the
+    scheduler's preemption is for."""
+    bs = engine.kv_block_size
+    if engine.num_kv_blocks is not None:
+        return max(1, int(engine.num_kv_blocks))
+    if engine.max_cache_tokens is not None:
+        return max(1, -(-engine.max_cache_tokens // bs))
+    blocks = engine.max_num_seqs * (-(-max_len // bs))
+    if free_bytes is not None and bytes_per_block > 0:
+        fit = int(free_bytes * engine.cache_memory_fraction) // bytes_per_block
+        if fit < 1:
+            raise MemoryError(f"no device memory for the cache: one block of {bs} tokens takes "
+                              f"{bytes_per_block} bytes, {free_bytes} bytes are free")
+        blocks = min(blocks, fit)
+    return max(1, blocks)
+
+
 def build_runner(dec: Decoder, engine: EngineConfig) -> ModelRunner:
     max_len = engine.max_model_len or dec.spec.max_position
     max_len = min(max_len, dec.spec.max_position)
     bs = engine.kv_block_size
-    if engine.num_kv_blocks is not None:
-        blocks = engine.num_kv_blocks
-    elif engine.max_cache_tokens is not None:
-        blocks = -(-engine.max_cache_tokens // bs)
-    else:
-        blocks = engine.max_num_seqs * (-(-max_len // bs))
-    cache = CacheManager(dec.cache_specs(), dec.state_specs(), bs, max(1, blocks), engine.max_num_seqs)
+    cache_specs, state_specs = dec.cache_specs(), dec.state_specs()
+    elt = torch.empty((), dtype=dec.dtype).element_size()
+    per_block = CacheManager(cache_specs, state_specs, bs, 1, 1).elements_per_block() * elt
+    free = torch.cuda.mem_get_info(dec.device)[0] if dec.device.type == "cuda" else None
+    blocks = plan_cache_blocks(engine, max_len, per_block, free)
+    cache = CacheManager(cache_specs, state_specs, bs, blocks, engine.max_num_seqs)
     cache.allocate_tensors(dec.dtype, dec.device)
     return ModelRunner(dec, cache, engine.max_num_batched_tokens, max_len)

@@ -95,7 +95,8 @@ class StepPlan:
 
 class Scheduler:
     def __init__(self, cache: CacheManager, max_num_seqs: int, max_num_batched_tokens: int, max_model_len: int,
-                 eos_token_id: Optional[int] = None):
+                 eos_token_id=None):
+        """eos_token_id: one id, several, or None (nothing ends a request but its length)."""
         self.cache = cache
         self.max_num_seqs = int(max_num_seqs)
         self.budget = int(max_num_batched_tokens)
@@ -104,6 +105,20 @@ class Scheduler:
         self.waiting: Deque[Request] = deque()
         self.running: List[Request] = []       # in order of admission
         self.finished: List[Request] = []
+
+    @property
+    def eos_token_id(self):
+        return self._eos
+
+    @eos_token_id.setter
+    def eos_token_id(self, value) -> None:
+        self._eos = value
+        if value is None:
+            self.eos_token_ids = frozenset()
+        elif isinstance(value, (list, tuple, set, frozenset)):
+            self.eos_token_ids = frozenset(int(v) for v in value)
+        else:
+            self.eos_token_ids = frozenset([int(value)])
 
     # ---------------------------------------------------------------- requests
     def add(self, req: Request) -> None:
@@ -249,7 +264,7 @@ class Scheduler:
             tok = int(sampled[req.req_id])
             req.output.append(tok)
             reason = None
-            if self.eos_token_id is not None and tok == self.eos_token_id and not req.params.ignore_eos:
+            if tok in self.eos_token_ids and not req.params.ignore_eos:
                 reason = "stop"
             elif len(req.output) >= req.params.max_new_tokens:
                 reason = "length"

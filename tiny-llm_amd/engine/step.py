@@ -92,9 +92,11 @@ class ModelRunner:
         self.max_tokens = int(max_num_batched_tokens)
         self.max_model_len = int(max_model_len)
         self.vocab_size = decoder.spec.vocab_size
-        for i, e in enumerate(decoder.spec.plan):
-            decoder.caches[i] = cache.layer_cache(i, e.cache_of)
-            decoder.states[i] = cache.states[i]
+        readers = decoder.cache_readers()
+        for (i, role) in list(decoder.cache_specs()) + list(readers):
+            decoder.caches[i][role] = cache.layer_cache((i, role), readers.get((i, role)))
+        for (i, role) in decoder.state_specs():
+            decoder.states[i][role] = cache.states[(i, role)]
         self._pinned: Optional[torch.Tensor] = None
         self._uploaded: Optional[torch.cuda.Event] = None
         self._graphs: Dict[Tuple[int, int], "DecodeGraph"] = {}

@@ -87,6 +87,27 @@ def _rows_2d(t: torch.Tensor, name: str) -> None:
         _fail(f"{name} must be 2-D with unit inner stride")
 
 
+# ------------------------------------------------- sizes, checked when parts are built
+MAX_HEAD_DIM = 256      # the general attention kernel keeps a head's row in one wave's registers
+
+
+def check_linear_sizes(dtype: torch.dtype, inner: int, what: str = "inner size") -> None:
+    """Raises KernelError if no product kernel takes rows of `inner` elements in `dtype`
+    (the bfloat16 kernels move 16-byte vectors: multiples of 8)."""
+    if dtype == torch.bfloat16 and inner % 8:
+        _fail(f"{what} = {inner}: the bfloat16 products need a multiple of 8 (float32 takes any size)")
+    if inner <= 0:
+        _fail(f"{what} = {inner} must be positive")
+
+
+def check_attention_sizes(dtype: torch.dtype, num_heads: int, num_kv_heads: int, head_dim: int) -> None:
+    """Raises KernelError for head shapes no attention kernel takes."""
+    if head_dim > MAX_HEAD_DIM or head_dim <= 0:
+        _fail(f"head_dim {head_dim} is outside the attention kernels' range of 1 to {MAX_HEAD_DIM}")
+    if num_heads <= 0 or num_kv_heads <= 0 or num_heads % num_kv_heads or num_heads > 65535:
+        _fail(f"{num_heads} heads over {num_kv_heads} kv heads: heads must be a multiple of kv heads, at most 65535")
+
+
 # --------------------------------------------------------------------------- ops
 def embedding(tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     """out[t, :] = table[tokens[t], :] as float32."""
@@ -454,8 +475,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             _fail("per-token request ids and positions must be contiguous int32")
     if not (num_kv_heads > 0 and num_heads % num_kv_heads == 0):
         _fail("heads must be a multiple of kv heads")
-    if not (head_dim <= 256):
-        _fail(f"head_dim {head_dim} exceeds the attention kernel's limit of 256")
+    if not (head_dim <= MAX_HEAD_DIM):
+        _fail(f"head_dim {head_dim} exceeds the attention kernel's limit of {MAX_HEAD_DIM}")
     _check(_lib().tl_paged_attention(
         _ptr(q), c_int64(q.stride(0)), _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
         c_int(block_tables.shape[1]), _ptr(req_of_token), _ptr(positions), _ptr(out), c_int64(out.stride(0)),
@@ -619,4 +640,19 @@ def sample(logits: torch.Tensor, out: torch.Tensor, temperature: Optional[torch.
                 _fail(f"{name} must be contiguous {dt} [rows]")
     _check(_lib().tl_sample(_ptr(logits), c_int64(logits.stride(0)), c_int(n), c_int(V), _ptr(temperature),
                             _ptr(top_k), _ptr(top_p), _ptr(seeds), _ptr(counters), _ptr(out), _stream()), "sample")
+    return out
+
+
+def random_normal(out: torch.Tensor, table: torch.Tensor, key: int, scale: float, shift: float) -> torch.Tensor:
+    """out.flat[i] = shift + scale * table[hash(key, i)], a pure function of (key, i): the numbers of
+    random-weights mode (weights/loader.py gives the formula).  table: float32, a power of two long."""
+    _dev(out, table)
+    n = table.numel()
+    if not (table.dtype == torch.float32 and table.is_contiguous() and n >= 2 and n & (n - 1) == 0):
+        _fail("the quantile table must be contiguous float32 with a power-of-two length")
+    if not out.is_contiguous():
+        _fail("the output must be contiguous")
+    _check(_lib().tl_random_normal(_ptr(out), c_int64(out.numel()), ctypes.c_uint64(key & ((1 << 64) - 1)), _ptr(table),
+                                   c_int(n.bit_length() - 1), c_float(scale), c_float(shift), c_int(_dt(out)),
+                                   _stream()), "random_normal")
     return out

@@ -1,36 +1,55 @@
 """The generic decoder: a ModelSpec made into parts, and the forward pass of one step.
 
-It does not know Llama.  It instantiates the parts each LayerSpec names, collects
-what they declare (weights, cache needs, per-request state), and runs the plan:
-a list of layer runs, in which a layer may appear twice or read the cache of an
-earlier run.
+It knows no architecture.  Every part (embedding, the parts of each layer, final norm,
+output head) is looked up by kind in the part registries and built from its PartSpec;
+weight prefixes come from the spec.  The decoder collects what the parts declare
+(weights, cache needs, per-request state) and runs the plan: a list of layer runs, in
+which a layer may appear twice or read the cache of an earlier run.
 """
 from __future__ import annotations
 
-from typing import List, Optional
+from typing import Dict, List, Optional, Tuple
 
 import torch
 
-from ..config.spec import ModelSpec
-from ..parts import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, CacheSpec, LayerCache, StateSpec, WeightSpec)
-from ..parts.embedding import LMHead, TokenEmbedding
+from ..config.spec import LayerSpec, ModelSpec, PartSpec
+from ..parts import BLOCKS, REGISTRIES, CacheSpec, LayerCache, Part, StateSpec, WeightSpec
 
 TORCH_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 
+# (plan entry, role of the part within its layer): who owns a cache or a state
+Owner = Tuple[int, str]
+
+
+def build_part(category: str, spec: PartSpec, prefix: str, dtype, device) -> Part:
+    return REGISTRIES[category].get(spec.kind)(prefix, dtype, device, **dict(spec.params))
+
 
 class Layer:
-    def __init__(self, spec, dtype, device):
-        p = spec.prefix
-        part_names = spec.part_names
-        mk = lambda reg, ps, sub: reg.get(ps.kind)(f"{p}.{part_names[sub]}", dtype, device, **dict(ps.params))
-        self.mixer_norm = mk(NORMS, spec.mixer_norm, "mixer_norm")
-        self.mixer = mk(MIXERS, spec.mixer, "mixer")
-        self.ffn_norm = mk(NORMS, spec.ffn_norm, "ffn_norm")
-        self.ffn = mk(FEED_FORWARDS, spec.ffn, "ffn")
-        self.block = BLOCKS.get(spec.block)(self.mixer_norm, self.mixer, self.ffn_norm, self.ffn)
+    def __init__(self, spec: LayerSpec, dtype, device):
+        arrangement = BLOCKS.get(spec.block)
+        roles = getattr(arrangement, "roles", None)
+        if not roles:
+            raise ValueError(f"block arrangement {spec.block!r} does not say which parts it takes (`roles`)")
+        unknown = [r for r in spec.parts if r not in roles]
+        if unknown:
+            raise ValueError(f"layer {spec.prefix}: arrangement {spec.block!r} has no role {unknown}; "
+                             f"it takes {sorted(roles)}")
+        self.by_role: Dict[str, Part] = {}
+        for role, category in roles.items():
+            if role not in spec.parts:
+                raise ValueError(f"layer {spec.prefix}: arrangement {spec.block!r} needs a part for role {role!r}")
+            ps = spec.parts[role]
+            self.by_role[role] = build_part(category, ps, f"{spec.prefix}.{ps.name or role}", dtype, device)
+        self.block = arrangement(self.by_role)
 
-    def parts(self):
-        return [self.mixer_norm, self.mixer, self.ffn_norm, self.ffn]
+    def parts(self) -> List[Part]:
+        return list(self.by_role.values())
+
+    @property
+    def mixer(self):
+        """The layer's part of role "mixer" (None in an arrangement without that role)."""
+        return self.by_role.get("mixer")
 
 
 class Decoder:
@@ -39,20 +58,16 @@ class Decoder:
         self.spec = spec
         self.dtype = TORCH_DTYPES[dtype] if isinstance(dtype, str) else dtype
         self.device = torch.device(device)
-        e = dict(spec.embedding.params)
-        self.embedding = TokenEmbedding("model.embed_tokens", self.dtype, self.device, **e)
+        self.embedding = build_part("embedding", spec.embedding, spec.embedding.name, self.dtype, self.device)
         self.layers: List[Layer] = [Layer(ls, self.dtype, self.device) for ls in spec.layers]
-        self.final_norm = NORMS.get(spec.final_norm.kind)("model.norm", self.dtype, self.device,
-                                                          **dict(spec.final_norm.params))
-        h = dict(spec.lm_head.params)
-        tied = h.pop("tied", False)
-        self.lm_head = LMHead("lm_head", self.dtype, self.device, tied_to="model.embed_tokens" if tied else None, **h)
-        # cache and state views are attached by the runner once the pools exist
-        self.caches: List[Optional[LayerCache]] = [None] * len(spec.plan)
-        self.states: List[Optional[torch.Tensor]] = [None] * len(spec.plan)
+        self.final_norm = build_part("norm", spec.final_norm, spec.final_norm.name, self.dtype, self.device)
+        self.lm_head = build_part("head", spec.lm_head, spec.lm_head.name, self.dtype, self.device)
+        # cache and state views by role, per plan entry; attached by the runner once the pools exist
+        self.caches: List[Dict[str, LayerCache]] = [{} for _ in spec.plan]
+        self.states: List[Dict[str, torch.Tensor]] = [{} for _ in spec.plan]
 
     # ---------------------------------------------------------------- declarations
-    def parts(self):
+    def parts(self) -> List[Part]:
         out = [self.embedding]
         for l in self.layers:
             out.extend(l.parts())
@@ -61,8 +76,9 @@ class Decoder:
 
     @property
     def graph_safe(self) -> bool:
-        """True if every part (and every mixer's position encoding) may be captured in a HIP graph."""
-        parts = self.parts() + [getattr(l.mixer, "position", None) for l in self.layers]
+        """True if every part (and every part's position encoding) may be captured in a HIP graph."""
+        parts = self.parts()
+        parts += [getattr(p, "position", None) for p in parts]
         return all(p.graph_safe for p in parts if p is not None)
 
     def weight_specs(self) -> List[WeightSpec]:
@@ -71,21 +87,45 @@ class Decoder:
             specs.extend(p.weights())
         return specs
 
-    def cache_specs(self) -> List[Optional[CacheSpec]]:
-        """Per plan entry: the cache it owns (None if it has none or reads another's)."""
-        out = []
-        for e in self.spec.plan:
-            out.append(None if e.cache_of is not None else self.layers[e.layer].mixer.cache_spec())
+    def cache_specs(self) -> Dict[Owner, CacheSpec]:
+        """The caches the plan's runs own (a run that reads another run's cache owns none)."""
+        out: Dict[Owner, CacheSpec] = {}
+        for i, e in enumerate(self.spec.plan):
+            if e.cache_of is not None:
+                continue
+            for role, part in self.layers[e.layer].by_role.items():
+                cs = part.cache_spec()
+                if cs is not None:
+                    out[(i, role)] = cs
         return out
 
-    def state_specs(self) -> List[Optional[StateSpec]]:
-        return [self.layers[e.layer].mixer.state_spec() for e in self.spec.plan]
+    def cache_readers(self) -> Dict[Owner, Owner]:
+        """Runs that read the cache of an earlier run: reader -> owner."""
+        out: Dict[Owner, Owner] = {}
+        for i, e in enumerate(self.spec.plan):
+            if e.cache_of is None:
+                continue
+            for role, part in self.layers[e.layer].by_role.items():
+                if part.cache_spec() is not None:
+                    out[(i, role)] = (e.cache_of, role)
+        return out
+
+    def state_specs(self) -> Dict[Owner, StateSpec]:
+        out: Dict[Owner, StateSpec] = {}
+        for i, e in enumerate(self.spec.plan):
+            for role, part in self.layers[e.layer].by_role.items():
+                ss = part.state_spec()
+                if ss is not None:
+                    out[(i, role)] = ss
+        return out
 
     # --------------------------------------------------------------------- compute
     def forward(self, ctx) -> torch.Tensor:
         """Runs the tokens of `ctx` through the plan; float32 logits at ctx.logit_rows."""
-        x = self.embedding.forward(ctx.tokens)
+        x = self.embedding.forward(ctx.tokens, ctx)
         wants_logits = ctx.logit_rows is not None and ctx.logit_rows.numel() > 0
+        # a head that says so may receive the final norm unevaluated and fuse it into its product
+        lazy_head = hasattr(self.final_norm, "lazy") and getattr(self.lm_head, "accepts_lazy_norm", False)
         plan = self.spec.plan
         # A block may prepare the norm that reads its result (the next block's first norm, or the
         # final norm) in its last product; `prepared` carries that from one block to the next.
@@ -99,12 +139,12 @@ class Decoder:
                 nxt = self.layers[plan[i + 1].layer].block
                 next_norm = getattr(nxt, "first_norm", None) if hasattr(nxt, "forward_chained") else None
             else:
-                next_norm = self.final_norm if wants_logits and hasattr(self.final_norm, "lazy") else None
+                next_norm = self.final_norm if wants_logits and lazy_head else None
             x, prepared = block.forward_chained(x, ctx, self.caches[i], self.states[i], prepared, next_norm)
         if not wants_logits:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=x.device)
         norm = self.final_norm
-        if hasattr(norm, "lazy"):
+        if lazy_head:
             h = norm.lazy(x, ctx.logit_rows, prepared=prepared) if prepared is not None else norm.lazy(x, ctx.logit_rows)
         else:
             h = norm.forward(x, ctx.logit_rows)

@@ -36,8 +36,12 @@ class Attention(Mixer):
         self.num_heads = int(num_heads)
         self.num_kv_heads = int(num_kv_heads)
         self.head_dim = int(head_dim)
-        if self.num_heads % self.num_kv_heads:
+        if self.num_kv_heads <= 0 or self.num_heads % self.num_kv_heads:
             raise ValueError("num_heads must be a multiple of num_kv_heads")
+        # sizes a kernel refuses are refused here, when the model is built, not at its first step
+        ops.check_attention_sizes(dtype, self.num_heads, self.num_kv_heads, self.head_dim)
+        ops.check_linear_sizes(dtype, self.hidden_size, f"{prefix}: hidden_size")
+        ops.check_linear_sizes(dtype, self.num_heads * self.head_dim, f"{prefix}: num_heads * head_dim")
         self.window = int(window or 0)
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
         pos = dict(position or {"kind": "none"})
@@ -63,7 +67,8 @@ class Attention(Mixer):
         self.w_o = tensors[f"{p}.o_proj.weight"].contiguous()
 
     def cache_spec(self) -> CacheSpec:
-        return CacheSpec(self.num_kv_heads, self.head_dim, "window" if self.window else "full", self.window)
+        return CacheSpec.keys_and_values(self.num_kv_heads, self.head_dim, "window" if self.window else "full",
+                                         self.window)
 
     # --------------------------------------------------------------------- compute
     def forward(self, h, ctx, cache: LayerCache, state, residual, next_norm=None):

@@ -48,16 +48,38 @@ class WeightSpec:
 
 
 @dataclass(frozen=True)
+class CacheTensor:
+    """One paged tensor of a cache: per token it keeps `shape` elements, and a page is
+    [block_size tokens] put at axis `token_axis` of that shape (keys of 4 heads of 64 are
+    shape (4, 64) with token_axis 1: pages [4, block_size, 64]; one latent vector of 96 per token is
+    shape (96,) with token_axis 0: pages [block_size, 96])."""
+    name: str
+    shape: Tuple[int, ...]
+    token_axis: int = 0
+
+    def page_shape(self, block_size: int) -> Tuple[int, ...]:
+        s = list(self.shape)
+        s.insert(self.token_axis, block_size)
+        return tuple(s)
+
+
+@dataclass(frozen=True)
 class CacheSpec:
-    """What a mixer keeps per token: keys and values of `num_kv_heads` heads.
-    kind "full" keeps every position, "window" the last `window` positions."""
-    num_kv_heads: int
-    head_dim: int
+    """What a mixer keeps per token, as a list of paged tensors.
+    kind "full" keeps every position, "window" the last `window` positions.
+    Layers whose specs are equal share one block-id space and one block table per request."""
+    tensors: Tuple[CacheTensor, ...]
     kind: str = "full"
     window: int = 0
 
+    @classmethod
+    def keys_and_values(cls, num_kv_heads: int, head_dim: int, kind: str = "full", window: int = 0) -> "CacheSpec":
+        """The usual attention cache: tensors "k" and "v", pages [kv_heads, block_size, head_dim]."""
+        t = (int(num_kv_heads), int(head_dim))
+        return cls((CacheTensor("k", t, 1), CacheTensor("v", t, 1)), kind, int(window))
+
     def group_key(self):
-        return (self.kind, self.window, self.num_kv_heads, self.head_dim)
+        return (self.kind, self.window, self.tensors)
 
 
 @dataclass(frozen=True)
@@ -69,11 +91,19 @@ class StateSpec:
 
 @dataclass
 class LayerCache:
-    """A mixer's view of the paged cache for one plan entry."""
-    k: torch.Tensor            # [blocks, kv_heads, block_size, head_dim]
-    v: torch.Tensor
+    """A mixer's view of the paged cache for one run of its layer: the tensors its CacheSpec
+    names, each [blocks, *page_shape]."""
+    tensors: Dict[str, torch.Tensor]
     group: int                 # which block table / slot mapping of the context applies
-    write: bool = True         # False: the entry reads a cache that another entry fills
+    write: bool = True         # False: the run reads a cache that another run fills
+
+    @property
+    def k(self) -> torch.Tensor:
+        return self.tensors["k"]
+
+    @property
+    def v(self) -> torch.Tensor:
+        return self.tensors["v"]
 
 
 class Part:
@@ -95,6 +125,28 @@ class Part:
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         """Receives the device tensors named by `weights()` (full names)."""
 
+    def cache_spec(self) -> Optional[CacheSpec]:
+        """Paged per-token memory this part needs (None: none)."""
+        return None
+
+    def state_spec(self) -> Optional[StateSpec]:
+        """Per-request memory of fixed size this part needs (None: none)."""
+        return None
+
+
+class Embedding(Part):
+    """Token ids [T] (int32) -> the residual stream, float32 [T, hidden]."""
+
+    def forward(self, tokens: torch.Tensor, ctx=None) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Head(Part):
+    """Normed activations at the wanted rows -> float32 logits [rows, vocab]."""
+
+    def forward(self, h) -> torch.Tensor:
+        raise NotImplementedError
+
 
 class Norm(Part):
     def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -110,12 +162,6 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
-    def cache_spec(self) -> Optional[CacheSpec]:
-        return None
-
-    def state_spec(self) -> Optional[StateSpec]:
-        return None
-
     def forward(self, h: torch.Tensor, ctx, cache: Optional[LayerCache], state: Optional[torch.Tensor],
                 residual: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
@@ -127,15 +173,27 @@ class FeedForward(Part):
 
 
 class Block:
-    """Arrangement of (mixer_norm, mixer, ffn_norm, ffn) around the residual stream."""
+    """An arrangement of a layer's parts around the residual stream.
 
-    def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Norm, ffn: FeedForward):
-        self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
+    `roles` names the parts the arrangement wants and the registry each is looked up in
+    ("norm", "mixer", "feed_forward", ...: the keys of REGISTRIES).  The decoder builds them and
+    hands them over as a dict; `caches` and `states` in `forward` are dicts by role that hold an
+    entry for every part that declared a cache or a state."""
 
-    def parts(self):
-        return [self.mixer_norm, self.mixer, self.ffn_norm, self.ffn]
+    roles: Dict[str, str] = {}
 
-    def forward(self, x, ctx, cache, state):
+    def __init__(self, parts: Dict[str, Part]):
+        missing = [r for r in self.roles if r not in parts]
+        extra = [r for r in parts if r not in self.roles]
+        if missing or extra:
+            raise ValueError(f"{type(self).__name__} takes the parts {sorted(self.roles)}; "
+                             f"missing {missing}, not taken {extra}")
+        self._parts = dict(parts)
+
+    def parts(self) -> List[Part]:
+        return list(self._parts.values())
+
+    def forward(self, x, ctx, caches, states):
         raise NotImplementedError
 
 
@@ -182,6 +240,8 @@ class Registry:
         return sorted(self._items)
 
 
+EMBEDDINGS = Registry("embedding")
+HEADS = Registry("output head")
 NORMS = Registry("norm")
 MIXERS = Registry("mixer")
 FEED_FORWARDS = Registry("feed-forward")
@@ -189,6 +249,13 @@ POSITION_ENCODINGS = Registry("position encoding")
 BLOCKS = Registry("block arrangement")
 
 
+# a block's roles and the model's own parts name their registry by these keys
+REGISTRIES = {"embedding": EMBEDDINGS, "head": HEADS, "norm": NORMS, "mixer": MIXERS,
+              "feed_forward": FEED_FORWARDS, "position_encoding": POSITION_ENCODINGS}
+
+
+def register_embedding(name, factory, **kw): EMBEDDINGS.register(name, factory, **kw)
+def register_head(name, factory, **kw): HEADS.register(name, factory, **kw)
 def register_norm(name, factory, **kw): NORMS.register(name, factory, **kw)
 def register_mixer(name, factory, **kw): MIXERS.register(name, factory, **kw)
 def register_feed_forward(name, factory, **kw): FEED_FORWARDS.register(name, factory, **kw)

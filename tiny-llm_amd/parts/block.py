@@ -6,21 +6,28 @@ from .base import Block, register_block
 
 
 class PreNormBlock(Block):
-    def forward(self, x, ctx, cache, state):
-        return self.forward_chained(x, ctx, cache, state)[0]
+    roles = {"mixer_norm": "norm", "mixer": "mixer", "ffn_norm": "norm", "ffn": "feed_forward"}
+
+    def __init__(self, parts):
+        super().__init__(parts)
+        self.mixer_norm, self.mixer = parts["mixer_norm"], parts["mixer"]
+        self.ffn_norm, self.ffn = parts["ffn_norm"], parts["ffn"]
+
+    def forward(self, x, ctx, caches, states):
+        return self.forward_chained(x, ctx, caches, states)[0]
 
     @property
     def first_norm(self):
         """The norm that reads this block's input, for whoever writes that input."""
         return self.mixer_norm if getattr(self.mixer, "accepts_lazy_norm", False) else None
 
-    def forward_chained(self, x, ctx, cache, state, prepared=None, next_norm=None):
+    def forward_chained(self, x, ctx, caches, states, prepared=None, next_norm=None):
         """As `forward`, between neighbours: `prepared` is this block's first norm as prepared by the
         product that wrote x (or None); `next_norm` is the norm that will read this block's result
         (or None).  Returns (x, that norm prepared or None)."""
         h = self._normed(self.mixer_norm, self.mixer, x, prepared)
         ffn_norm = self.ffn_norm if getattr(self.ffn, "accepts_lazy_norm", False) else None
-        x, prep = self._run(self.mixer, (h, ctx, cache, state, x), ffn_norm)
+        x, prep = self._run(self.mixer, (h, ctx, caches.get("mixer"), states.get("mixer"), x), ffn_norm)
         h = self._normed(self.ffn_norm, self.ffn, x, prep)
         return self._run(self.ffn, (h, ctx, x), next_norm)
 

@@ -9,11 +9,11 @@ from typing import Dict, List, Optional
 import torch
 
 from ..kernels import ops
-from .base import Part, WeightSpec
+from .base import Embedding, Head, WeightSpec, register_embedding, register_head
 from .norm import LazyNorm
 
 
-class TokenEmbedding(Part):
+class TokenEmbedding(Embedding):
     graph_safe = True
 
     def __init__(self, prefix, dtype, device, *, vocab_size: int, hidden_size: int):
@@ -27,18 +27,20 @@ class TokenEmbedding(Part):
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.weight = tensors[f"{self.prefix}.weight"].contiguous()
 
-    def forward(self, tokens: torch.Tensor) -> torch.Tensor:
+    def forward(self, tokens: torch.Tensor, ctx=None) -> torch.Tensor:
         out = torch.empty((tokens.numel(), self.hidden_size), dtype=torch.float32, device=tokens.device)
         return ops.embedding(tokens, self.weight, out)
 
 
-class LMHead(Part):
+class LMHead(Head):
     graph_safe = True
+    accepts_lazy_norm = True
 
     def __init__(self, prefix, dtype, device, *, vocab_size: int, hidden_size: int, tied_to: str = None):
         super().__init__(prefix, dtype, device)
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
-        self.tied_to = tied_to
+        self.tied_to = tied_to          # weight prefix of the embedding whose table this head shares
+        ops.check_linear_sizes(dtype, self.hidden_size, f"{prefix}: hidden_size")
         self.weight: Optional[torch.Tensor] = None
 
     def weights(self) -> List[WeightSpec]:
@@ -55,3 +57,7 @@ class LMHead(Part):
             return h.linear(self.weight, out)
         out = torch.empty((h.shape[0], self.vocab_size), dtype=torch.float32, device=h.device)
         return ops.linear(h, self.weight, out)
+
+
+register_embedding("token_embedding", TokenEmbedding)
+register_head("lm_head", LMHead)

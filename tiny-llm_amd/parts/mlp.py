@@ -26,6 +26,8 @@ class SwiGLU(FeedForward):
         super().__init__(prefix, dtype, device)
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
+        ops.check_linear_sizes(dtype, self.hidden_size, f"{prefix}: hidden_size")
+        ops.check_linear_sizes(dtype, self.intermediate_size, f"{prefix}: intermediate_size")
         self.w_gate_up: Optional[torch.Tensor] = None
         self.w_down: Optional[torch.Tensor] = None
 

@@ -1,3 +1,3 @@
 from .safetensors_io import SafetensorsFile, SafetensorsError, save_file, open_model_files
-from .loader import (WeightLoadError, load_weights, init_random_weights, write_random_model, random_tensor,
+from .loader import (Checkpoint, WeightLoadError, load_weights, init_random_weights, write_random_model, random_tensor,
                      check_against, target_dtype)
