@@ -304,3 +304,99 @@ def test_scheduler_invariants_under_random_load(seed):
         assert r.finish_reason in ("stop", "length", "capacity")
         if r.finish_reason == "stop":
             assert r.output[-1] == 3
+
+
+# ------------------------------------------------------------- step metadata
+def _rows(specs, bs):
+    """specs: (context_len, new tokens, wanted places) per request, with made-up block tables."""
+    from tiny_llm_amd.engine.step import _Row
+    rows, nxt = [], 3
+    for i, (c, toks, want) in enumerate(specs):
+        nb = -(-(c + len(toks)) // bs)
+        rows.append(_Row(f"r{i}", toks, want, c, slot=10 + i, tables=[list(range(nxt, nxt + nb))]))
+        nxt += nb + 1
+    return rows
+
+
+def test_step_metadata_layout_and_padding():
+    """One routine lays out eager steps (exact sizes) and captured steps (capacities): the padded
+    layout holds the exact one in its first entries, and what is padding can do no harm."""
+    import numpy as np
+    from tiny_llm_amd.engine.step import Layout, SampleSpec, fill_metadata, tile_lists
+    bs = 4
+    rows = _rows([(5, [7, 8, 9], [2]), (0, [1, 2, 3, 4, 5, 6], []), (9, [4], [0])], bs)
+    exact = Layout(10, 3, 2, 1, 3, {2: 6, 16: 3}, True)
+    a = np.full(exact.total, -7, dtype=np.int32)
+    samples = [SampleSpec(0.8, 5, 0.9, 123456789012345, 8), SampleSpec()]
+    fill_metadata(a, exact, rows, bs, samples)
+    assert exact.sec(a, "tokens").tolist() == [7, 8, 9, 1, 2, 3, 4, 5, 6, 4]
+    assert exact.sec(a, "positions").tolist() == [5, 6, 7, 0, 1, 2, 3, 4, 5, 9]
+    assert exact.sec(a, "req_of_token").tolist() == [0, 0, 0, 1, 1, 1, 1, 1, 1, 2]
+    assert exact.sec(a, "cu_seqlens").tolist() == [0, 3, 9, 10] and exact.sec(a, "seq_lens").tolist() == [8, 6, 10]
+    assert exact.sec(a, "state_slots").tolist() == [10, 11, 12] and exact.sec(a, "logit_rows").tolist() == [2, 9]
+    # slots: request 0 holds blocks 3, 4 (positions 5..7 -> block 4), request 1 blocks 6, 7, request 2 blocks 9, 10, 11
+    assert exact.sec(a, "slots0").tolist() == [17, 18, 19, 24, 25, 26, 27, 28, 29, 11 * 4 + 1]
+    assert exact.sec(a, "tables0").reshape(3, 3).tolist() == [[3, 4, -7], [6, 7, -7], [9, 10, 11]]
+    t2 = exact.sec(a, "tiles2").reshape(3, 6)
+    assert t2.tolist() == [[0, 0, 1, 1, 1, 2], [0, 2, 3, 5, 7, 9], [2, 1, 2, 2, 2, 1]]
+    assert exact.sec(a, "tiles16").reshape(3, 3).tolist() == [[0, 1, 2], [0, 3, 9], [3, 6, 1]]
+    assert exact.sec(a, "temperature").view(np.float32).tolist() == [np.float32(0.8), 0.0]
+    assert exact.sec(a, "top_k").tolist() == [5, 0] and exact.sec(a, "counters").tolist() == [8, 0]
+    assert exact.sec(a, "seeds").view(np.int64).tolist() == [123456789012345, 0]
+
+    padded = Layout(16, 4, 4, 1, 5, {2: 12, 16: 5}, True)
+    b = np.full(padded.total, -7, dtype=np.int32)
+    fill_metadata(b, padded, rows, bs, samples)
+    for name in ("tokens", "positions", "req_of_token", "slots0"):
+        n = exact.off[name][1]
+        assert padded.sec(b, name)[:n].tolist() == exact.sec(a, name).tolist()
+    assert padded.sec(b, "tokens")[10:].tolist() == [0] * 6 and padded.sec(b, "positions")[10:].tolist() == [0] * 6
+    assert padded.sec(b, "slots0")[10:].tolist() == [-1] * 6            # a padding token stores nothing
+    assert padded.sec(b, "cu_seqlens").tolist() == [0, 3, 9, 10, 10]    # the padding request has no tokens
+    assert padded.sec(b, "logit_rows").tolist() == [2, 9, 0, 0]
+    assert padded.sec(b, "tables0").reshape(4, 5)[:3, :3].tolist() == [[3, 4, -7], [6, 7, -7], [9, 10, 11]]
+    p2 = padded.sec(b, "tiles2").reshape(3, 12)
+    assert p2[:, :6].tolist() == t2.tolist() and p2[2, 6:].tolist() == [0] * 6     # padding tiles hold no token
+    assert padded.sec(b, "top_p").view(np.float32).tolist() == [np.float32(0.9), 1.0, 1.0, 1.0]
+    # too many tiles for the layout is an error, not an overrun
+    small = Layout(10, 3, 2, 1, 3, {2: 5}, False)
+    with pytest.raises(ValueError):
+        fill_metadata(np.zeros(small.total, dtype=np.int32), small, rows, bs)
+    assert tile_lists([3, 0, 5], 2) == ([0, 0, 2, 2, 2], [0, 2, 3, 5, 7], [2, 1, 2, 2, 1])
+
+
+def test_static_block_table_rows_are_rewritten_when_they_change():
+    import numpy as np
+    from tiny_llm_amd.engine.step import Layout, fill_metadata
+    bs = 4
+    lay = Layout(2, 2, 2, 1, 4, {}, False)
+    buf = np.zeros(lay.total, dtype=np.int32)
+    seen = [[None, None]]
+    rows = _rows([(5, [1], [0]), (2, [1], [0])], bs)
+    fill_metadata(buf, lay, rows, bs, None, seen)
+    assert lay.sec(buf, "tables0").reshape(2, 4).tolist() == [[3, 4, 0, 0], [6, 0, 0, 0]]
+    assert lay.sec(buf, "slots0").tolist() == [4 * 4 + 1, 6 * 4 + 2]
+    rows[0].tables[0].append(20)                      # the same request grew by a block
+    rows[0].context_len = 8
+    rows[1] = _rows([(0, [5], [0])], bs)[0]           # another request took row 1
+    fill_metadata(buf, lay, rows, bs, None, seen)
+    assert lay.sec(buf, "tables0").reshape(2, 4).tolist() == [[3, 4, 20, 0], [3, 0, 0, 0]]
+    assert lay.sec(buf, "slots0").tolist() == [20 * 4, 3 * 4]
+
+
+def test_reservation_of_a_step_that_did_not_run_is_undone():
+    cm = CacheManager(full(1), [None], block_size=4, num_blocks=8, max_seqs=2)
+    cm.reserve_step([("a", 6)])
+    cm.commit("a", 6)
+    cm.forget_reservation()
+    before = (cm.free_blocks(), cm.free_slots, list(cm.block_table("a", 0)))
+    cm.reserve_step([("a", 5), ("b", 9)])              # a: one more block; b: admitted with three
+    assert cm.free_blocks() == [2] and cm.has("b")
+    cm.undo_reservation()
+    assert (cm.free_blocks(), cm.free_slots, list(cm.block_table("a", 0))) == before and not cm.has("b")
+    cm.audit()
+    assert cm.reserve_step([("a", 5), ("b", 9)]) == [6, 0]
+    assert cm.block_table("a", 0) == [0, 1, 2] and cm.block_table("b", 0) == [3, 4, 5]    # the same pages again
+    cm.undo_reservation()
+    cm.undo_reservation()                               # nothing open: nothing happens
+    cm.audit()

@@ -233,32 +233,118 @@ def test_float32_generation_does_not_depend_on_the_schedule(name, folders):
     assert all(o == outs[0] for o in outs[1:])
 
 
+def spy_on_steps(eng):
+    """Records, for every step the engine runs, (request, position) and the logits of each row a
+    token was chosen from."""
+    log = []
+    run = eng.runner.run
+    cache = eng.runner.cache
+
+    def spy(entries, samples, use_graph=True):
+        rows = [(e.req_id, (cache.num_tokens(e.req_id) if cache.has(e.req_id) else 0) + len(e.tokens) - 1)
+                for e in entries if e.want]
+        toks = run(entries, samples, use_graph)
+        if rows:
+            log.append((rows, eng.runner.last_logits.float().cpu().clone()))
+        return toks
+
+    eng.runner.run = spy
+    return log
+
+
+def check_logged_logits(log, tokens_of, w, c, act, tol):
+    """Every logged row against the plain model run over the request's final token list."""
+    refs = {rid: plain.llama_forward(w, c, toks, act_dtype=act) for rid, toks in tokens_of.items()}
+    worst, n = 0.0, 0
+    for rows, logits in log:
+        assert logits.shape[0] == len(rows)
+        for i, (rid, pos) in enumerate(rows):
+            assert torch.isfinite(logits[i]).all(), (rid, pos)
+            e = rel_err(logits[i], refs[rid][pos])
+            worst, n = max(worst, e), n + 1
+            assert e < tol, f"request {rid} position {pos}: rel err {e:.3e}"
+    return worst, n
+
+
+def poison(eng):
+    for g in eng.runner.cache.groups:
+        for t in g.tensors.values():
+            t.fill_(float("nan"))
+
+
+@pytest.mark.parametrize("graphs", [True, False])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_graph_replays_equal_eager_steps(dtype, folders):
-    """Decode steps captured in a HIP graph: every replay, with eager work (prefill of new requests,
-    other batch sizes) between replays, gives the tokens of the eager path."""
+def test_graph_replays_against_the_plain_model(dtype, graphs, folders):
+    """Steps captured in HIP graphs, decode steps and steps with prompt portions alike: every
+    replay, with other shapes of step between replays as requests come and go, gives the plain
+    model's logits at every row a token is chosen from."""
     from tiny_llm_amd import Engine, SamplingParams
     cfg, eng_kw, _ = CONFIGS["A"]
-    prompts = [random_tokens(n, cfg["vocab_size"], 300 + n) for n in (40, 3, 17, 64, 9)]
-    sp = [SamplingParams.greedy(n, ignore_eos=True) for n in (50, 20, 35, 8, 44)]     # batch sizes change as they end
+    act = torch.bfloat16 if dtype == "bfloat16" else None
+    w, c = read_weights(folders["A"], round_to=act)
+    prompts = [random_tokens(n, cfg["vocab_size"], 300 + n) for n in (40, 3, 17, 64, 9, 77, 30)]
+    sp = [SamplingParams.greedy(n, ignore_eos=True) for n in (50, 20, 35, 8, 44, 12, 25)]     # batch sizes change as they end
     sp[2] = SamplingParams(max_new_tokens=35, temperature=0.9, top_k=20, top_p=0.9, seed=5, ignore_eos=True)
-    outs = {}
-    for graphs in (False, True):
-        eng = Engine(folders["A"], dtype=dtype, max_num_seqs=3, max_num_batched_tokens=32, use_graphs=graphs, **eng_kw)
-        outs[graphs] = eng.generate(prompts, sp)
-        if graphs:
-            assert any(g.graph is not None for g in eng.runner._graphs.values())
-            assert sum(g.runs for g in eng.runner._graphs.values()) > 60
-    if dtype == "float32":
-        assert outs[True] == outs[False]
+    eng = Engine(folders["A"], dtype=dtype, max_num_seqs=3, max_num_batched_tokens=32, use_graphs=graphs, **eng_kw)
+    poison(eng)
+    log = spy_on_steps(eng)
+    out = eng.generate(prompts, sp)
+    tokens_of = {i: p + o for i, (p, o) in enumerate(zip(prompts, out))}
+    worst, n = check_logged_logits(log, tokens_of, w, c, act, 1e-4 if dtype == "float32" else 2e-2)
+    print(f"{dtype} graphs={graphs}: {n} rows, worst rel err {worst:.2e}, graph steps {eng.runner.graph_steps}, "
+          f"eager {eng.runner.eager_steps}")
+    assert n == sum(len(o) for o in out)
+    if graphs:
+        kinds = {k[0] for k, g in eng.runner._graphs.items() if g.graph is not None}
+        assert kinds == {"decode", "mixed"}                 # both kinds of step were captured and replayed
+        assert eng.runner.graph_steps > 60
+        assert not any(g.capture_failed for g in eng.runner._graphs.values())
     else:
-        # bfloat16: key splits differ between the two paths, so sums round differently now and then
-        same = sum(a == b for x, y in zip(outs[True], outs[False]) for a, b in zip(x[:8], y[:8]))
-        assert same >= 0.8 * sum(min(len(x), 8) for x in outs[True])
+        assert eng.runner.graph_steps == 0
+    eng.runner.cache.audit()
 
 
-def test_collector_rests_while_a_decode_graph_is_captured(folders, monkeypatch):
-    """Python's garbage collector must not run while a decode step is captured: finalising the
+@pytest.mark.parametrize("graphs", [True, False])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decoding_past_the_first_context_bucket(dtype, graphs, tmp_path_factory):
+    """Contexts that grow from below 512 to beyond: the decode graph of the next context bound
+    takes over a live batch, the attention kernel splits the keys of a request over workgroups
+    and merges them, inside a graph and outside.  Logits of every step against the plain model."""
+    from tiny_llm_amd import Engine, SamplingParams
+    cfg, eng_kw, init = CONFIGS["B"]
+    key = ("past512",)
+    if key not in _folders:
+        _folders[key] = make_folder(tmp_path_factory.mktemp("past512"), cfg, seed=21, **init)
+    folder = _folders[key]
+    act = torch.bfloat16 if dtype == "bfloat16" else None
+    w, c = read_weights(folder, round_to=act)
+    prompts = [random_tokens(n, cfg["vocab_size"], 700 + n) for n in (497, 490, 505)]
+    eng = Engine(folder, dtype=dtype, max_num_seqs=4, max_num_batched_tokens=512, use_graphs=graphs,
+                 max_cache_tokens=3 * 576, **eng_kw)
+    poison(eng)
+    log = spy_on_steps(eng)
+    out = eng.generate(prompts, SamplingParams.greedy(44, ignore_eos=True))
+    tokens_of = {i: p + o for i, (p, o) in enumerate(zip(prompts, out))}
+    worst, n = check_logged_logits(log, tokens_of, w, c, act, 1e-4 if dtype == "float32" else 2e-2)
+    print(f"{dtype} graphs={graphs}: {n} rows across the 512 boundary, worst rel err {worst:.2e}")
+    assert n == 3 * 44
+    if graphs:
+        bounds = sorted({k[2] for k, g in eng.runner._graphs.items() if k[0] == "decode" and g.graph is not None})
+        assert bounds == [512, 1024]
+    if dtype == "bfloat16":
+        # the split path was really taken beyond 512 keys
+        attn = eng.decoder.layers[0].mixer
+
+        class Ctx:
+            max_seq_len = 1024
+        assert attn._splits(Ctx, 3, eng.decoder.device)[0] >= 2
+
+
+_folders = {}
+
+
+def test_collector_rests_while_a_step_is_captured(folders, monkeypatch):
+    """Python's garbage collector must not run while a step is captured: finalising the
     pinned buffers or graphs of an engine that is no longer referenced is not allowed during a
     capture and would end the process.  (torch.cuda.graph no longer collects before a capture.)"""
     import gc
@@ -266,13 +352,13 @@ def test_collector_rests_while_a_decode_graph_is_captured(folders, monkeypatch):
     from tiny_llm_amd.engine import step as step_module
     cfg = CONFIGS["A"][0]
     seen = []
-    body = step_module.DecodeGraph._body
+    body = step_module.StepGraph._body
 
     def watched(self):
         seen.append((torch.cuda.is_current_stream_capturing(), gc.isenabled()))
         return body(self)
 
-    monkeypatch.setattr(step_module.DecodeGraph, "_body", watched)
+    monkeypatch.setattr(step_module.StepGraph, "_body", watched)
     assert gc.isenabled()
     prompts = [random_tokens(12, cfg["vocab_size"], 77)]
     for _ in range(2):      # the second engine is built while the first one is garbage
@@ -280,6 +366,133 @@ def test_collector_rests_while_a_decode_graph_is_captured(folders, monkeypatch):
     assert any(capturing for capturing, _ in seen)
     assert all(not collecting for capturing, collecting in seen if capturing)
     assert gc.isenabled()
+
+
+def test_abort_gives_everything_back_mid_generation(folders):
+    from tiny_llm_amd import Engine, SamplingParams
+    cfg, eng_kw, _ = CONFIGS["A"]
+    w, c = read_weights(folders["A"])
+    prompts = [random_tokens(n, cfg["vocab_size"], 400 + n) for n in (20, 45, 33)]
+    eng = Engine(folders["A"], dtype="float32", max_num_seqs=4, max_num_batched_tokens=16, **eng_kw)
+    ids = [eng.add_request(p, SamplingParams.greedy(30, ignore_eos=True)) for p in prompts]
+    for _ in range(4):
+        eng.step()                      # request 1 is still in its prompt, the others decode
+    assert eng.requests[ids[1]].num_computed < 45 and len(eng.requests[ids[0]].output) > 0
+    held = eng.runner.cache.free_blocks()[0]
+    eng.abort(ids[0])                   # a decoding request
+    eng.abort(ids[1])                   # a request in the middle of its prompt
+    eng.runner.cache.audit()
+    assert eng.runner.cache.free_blocks()[0] > held and eng.runner.cache.free_slots == 4
+    assert eng.requests[ids[0]].finish_reason == "abort" and eng.requests[ids[1]].status == "finished"
+    late = eng.add_request(prompts[1], SamplingParams.greedy(5, ignore_eos=True))     # takes the pages over
+    while eng.has_unfinished():
+        eng.step()
+    assert eng.requests[ids[2]].output == plain.greedy_generate(w, c, prompts[2], 30)
+    assert eng.requests[late].output == plain.greedy_generate(w, c, prompts[1], 5)
+    assert eng.runner.cache.free_blocks() == [g.pool.num_blocks for g in eng.runner.cache.groups]
+    eng.abort(ids[2])                   # finished already: nothing happens
+    eng.runner.cache.audit()
+
+
+def test_a_request_that_cannot_go_on_even_alone_ends_with_capacity(folders):
+    from tiny_llm_amd import Engine, SamplingParams
+    cfg, eng_kw, _ = CONFIGS["A"]
+    w, c = read_weights(folders["A"])
+    eng = Engine(folders["A"], dtype="float32", max_num_seqs=2, kv_block_size=16, num_kv_blocks=3)
+    prompt = random_tokens(40, cfg["vocab_size"], 41)
+    out = eng.generate([prompt], SamplingParams.greedy(30, ignore_eos=True))[0]
+    req = next(iter(eng.requests.values()))
+    assert req.finish_reason == "capacity" and len(out) == 3 * 16 - 40 + 1      # 48 cached tokens, one more chosen
+    assert out == plain.greedy_generate(w, c, prompt, len(out))
+    assert eng.runner.cache.free_blocks() == [3]
+    with pytest.raises(ValueError):                  # a prompt that the whole pool cannot hold is refused at once
+        eng.add_request(random_tokens(60, cfg["vocab_size"], 42), SamplingParams.greedy(2))
+
+
+def test_preemption_in_bfloat16_with_seeded_sampling(folders):
+    """Recomputation after a preemption goes through other kernels than the first pass (a long
+    prompt portion instead of single tokens), so in bfloat16 logits differ by rounding; tokens are
+    compared where the plain model's choice is clear of that, logits everywhere."""
+    from tiny_llm_amd import Engine, SamplingParams
+    cfg, eng_kw, _ = CONFIGS["A"]
+    w, c = read_weights(folders["A"], round_to=torch.bfloat16)
+    prompts = [random_tokens(n, cfg["vocab_size"], 530 + n) for n in (30, 28, 26)]
+    sps = [SamplingParams(max_new_tokens=40, temperature=0.8, top_k=40, top_p=0.95, seed=900 + i, ignore_eos=True)
+           for i in range(3)]
+    tight = Engine(folders["A"], dtype="bfloat16", max_num_seqs=4, kv_block_size=16, num_kv_blocks=9)
+    poison(tight)
+    log = spy_on_steps(tight)
+    out = tight.generate(prompts, sps)
+    assert sum(r.preemptions for r in tight.requests.values()) >= 1
+    assert all(len(o) == 40 for o in out)
+    tight.runner.cache.audit()
+    assert tight.runner.cache.free_blocks() == [9]
+    # a preempted request is recomputed from position 0; what it had generated stays its own
+    worst, n = check_logged_logits(log, {r.req_id: r.tokens for r in tight.requests.values()}, w, c, torch.bfloat16, 2e-2)
+    print(f"preemption in bfloat16: {n} rows , worst rel err {worst:.2e}")
+    assert n == 120
+    refs = [plain.llama_forward(w, c, p + o, act_dtype=torch.bfloat16) for p, o in zip(prompts, out)]
+    for i, (p, o) in enumerate(zip(prompts, out)):
+        for j, tok in enumerate(o):
+            row = refs[i][len(p) + j - 1].float()
+            u = plain.uniform_for(sps[i].seed, len(p) + j)
+            want = plain.sample_token(row, 0.8, 40, 0.95, u)
+            if want != tok:
+                # the engine drew the same uniform number from logits that differ by rounding: the two
+                # tokens are neighbours in the cumulative distribution
+                probs = torch.softmax(row.double() / 0.8, -1)
+                assert float(probs[tok]) > 1e-4
+    agree = sum(plain.sample_token(refs[i][len(p) + j - 1].float(), 0.8, 40, 0.95,
+                                   plain.uniform_for(sps[i].seed, len(p) + j)) == tok
+                for i, (p, o) in enumerate(zip(prompts, out)) for j, tok in enumerate(o))
+    assert agree >= 0.9 * 120
+
+
+def test_sharded_folder_generates_like_the_single_file(folders, tmp_path):
+    from safetensors import safe_open
+    from tiny_llm_amd import Engine, SamplingParams
+    from tiny_llm_amd.weights import save_file
+    cfg, eng_kw, _ = CONFIGS["B"]
+    with safe_open(os.path.join(folders["B"], "model.safetensors"), "pt") as f:
+        names = list(f.keys())
+        weight_map = {}
+        for i in range(2):
+            fname = f"model-{i + 1:05d}-of-00002.safetensors"
+            save_file({n: f.get_tensor(n) for n in names[i::2]}, str(tmp_path / fname))
+            weight_map.update({n: fname for n in names[i::2]})
+    json.dump({"metadata": {}, "weight_map": weight_map}, open(tmp_path / "model.safetensors.index.json", "w"))
+    json.dump(json.load(open(os.path.join(folders["B"], "config.json"))), open(tmp_path / "config.json", "w"))
+    prompts = [random_tokens(n, cfg["vocab_size"], 60 + n) for n in (9, 40)]
+    sp = SamplingParams.greedy(12, ignore_eos=True)
+    a = Engine(folders["B"], dtype="float32", **eng_kw).generate(prompts, sp)
+    b = Engine(str(tmp_path), dtype="float32", **eng_kw).generate(prompts, sp)
+    assert a == b
+
+
+def test_a_step_that_fails_leaves_the_cache_as_it_was(folders):
+    from tiny_llm_amd.config import EngineConfig
+    from tiny_llm_amd.engine.loading import build_runner, load_model
+    from tiny_llm_amd.engine.step import StepEntry
+    cfg, eng_kw, _ = CONFIGS["A"]
+    engine = EngineConfig(dtype="float32", max_cache_tokens=256, max_num_seqs=3, use_graphs=False, **eng_kw)
+    _, dec = load_model(folders["A"], engine)
+    runner = build_runner(dec, engine)
+    a = random_tokens(40, cfg["vocab_size"], 1)
+    first = runner.step([StepEntry("a", a[:20], [19])]).cpu()
+    before = (runner.cache.free_blocks(), runner.cache.free_slots, list(runner.cache.block_table("a", 0)))
+    forward = dec.forward
+
+    def broken(ctx):
+        raise RuntimeError("a kernel refused")
+    dec.forward = broken
+    with pytest.raises(RuntimeError):
+        runner.step([StepEntry("a", a[20:], [19]), StepEntry("b", a[:17], [16])])
+    dec.forward = forward
+    assert (runner.cache.free_blocks(), runner.cache.free_slots, list(runner.cache.block_table("a", 0))) == before
+    assert not runner.cache.has("b") and runner.cache.num_tokens("a") == 20
+    runner.cache.audit()
+    again = runner.step([StepEntry("a", a[20:], [19]), StepEntry("b", a[:20], [19])]).cpu()
+    assert rel_err(again[1], first[0]) < 1e-6
 
 
 def test_command_line_generates_from_prompt_ids(folders):

@@ -101,7 +101,8 @@ def test_lm_head_last_rows_reference_vector():
 @pytest.mark.parametrize("M,K,N", [(127, 255, 353), (1, 64, 251), (7, 176, 64), (130, 96, 517), (64, 2048, 256),
                                    (300, 5632, 136), (9, 5640, 520), (16, 4104, 40), (8, 5640, 524), (3, 2056, 2044),
                                    (5, 9000, 72), (8, 64, 4100), (12, 96, 8200), (16, 72, 12300), (7, 64, 8200),
-                                   (5, 64, 2500), (16, 96, 3302)])
+                                   (5, 64, 2500), (16, 96, 3302), (17, 2048, 32000), (40, 64, 16390),
+                                   (64, 2048, 32000), (33, 128, 128256)])
 def test_linear_sizes(dtype, M, K, N):
     if dtype == torch.bfloat16 and K % 8:
         K = K + 8 - K % 8
@@ -189,7 +190,8 @@ def test_linear_norm(M, K, N):
 
 
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 40, 64])
-@pytest.mark.parametrize("K,N,N2", [(64, 248, 96), (5632, 2048, 516), (176, 64, 40), (96, 520, 1030), (2120, 1000, 72), (64, 4200, 40), (64, 64, 8300), (64, 2600, 3000)])
+@pytest.mark.parametrize("K,N,N2", [(64, 248, 96), (5632, 2048, 516), (176, 64, 40), (96, 520, 1030), (2120, 1000, 72),
+                                    (64, 4200, 40), (64, 64, 8300), (64, 2600, 3000), (72, 2048, 32000), (64, 64, 16390)])
 def test_linear_handoff(M, K, N, N2):
     """A norm handed from the product that writes the residual stream to the product that reads
     it: the first also writes bf16(w * x) and partial sums of x^2, the second applies 1 / rms."""
@@ -763,3 +765,23 @@ def test_sampling_distribution():
     counts = torch.tensor([got.count(i) for i in kept], dtype=torch.float64) / n
     assert set(got) == set(kept)
     assert (counts - probs).abs().max() < 0.015
+
+
+# ------------------------------------------------------------ seeded numbers
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_seeded_numbers_are_the_same_bits_on_host_and_device(dtype):
+    """Random-weights mode: a tensor made on the device equals the one made on the host (which
+    is what a written model folder holds), for matrices, norm weights and the rounding to bfloat16."""
+    from tiny_llm_amd.parts.base import WeightSpec
+    from tiny_llm_amd.weights.loader import random_tensor
+    for spec, std, nstd in ((WeightSpec("model.layers.0.mlp.up_proj.weight", (1031, 517)), 0.02, 0.0),
+                            (WeightSpec("a.weight", (3, 5, 7)), 1.7, 0.0),
+                            (WeightSpec("n.weight", (4099,), role="vector", init="ones"), 0.02, 0.1),
+                            (WeightSpec("n.weight", (33,), role="vector", init="ones"), 0.02, 0.0),
+                            (WeightSpec("big.weight", (3000, 2048)), 0.02, 0.0)):
+        host = random_tensor(spec, 77, std, nstd, dtype=dtype)
+        dev = random_tensor(spec, 77, std, nstd, device=DEV, dtype=dtype)
+        assert dev.dtype == dtype and dev.shape == host.shape
+        assert torch.equal(dev.cpu(), host), spec.name
+    other = random_tensor(WeightSpec("a.weight", (3, 5, 7)), 78, 1.7, 0.0, device=DEV, dtype=dtype)
+    assert not torch.equal(other.cpu(), random_tensor(WeightSpec("a.weight", (3, 5, 7)), 77, 1.7, 0.0, dtype=dtype))

@@ -60,11 +60,11 @@ def make_runner(folder, dtype, block_size, max_tokens, poison=True):
     return runner
 
 
-def replay(runner, steps):
+def replay(runner, steps, use_graph=False):
     from tiny_llm_amd.engine.step import StepEntry
     out = {}
     for s in steps:
-        logits = runner.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]])
+        logits = runner.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]], use_graph=use_graph)
         if logits.shape[0]:
             out[s["step"]] = logits.cpu()
         for rid in s["end"]:
@@ -119,6 +119,28 @@ def test_mixed_with_page_reuse(name, dtype, tmp_path_factory):
         worst = check(out, steps, ref, TOL[dtype])
         print(f"{name} {dtype} mixed seed {seed}: worst rel err {worst:.2e}, pool {peak} tokens")
         assert runner.cache.free_blocks() == [g.pool.num_blocks for g in runner.cache.groups]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_cuttings_as_captured_steps(name, dtype, tmp_path_factory):
+    """The same traces with every step run as a HIP graph of its shape (sizes rounded up, padding
+    tokens, tiles and rows): twice over on one runner, so that the second pass replays what the
+    first captured, with other shapes between the replays."""
+    folder, reqs, ref, eng = material(name, dtype, tmp_path_factory)
+    steps, peak = traces.mixed(reqs, seed=2)
+    runner = make_runner(folder, dtype, eng["kv_block_size"], max(peak, max(r64(len(t)) for t in reqs.values())))
+    for build in (lambda: steps, lambda: traces.portions(reqs), lambda: traces.tail_one_by_one(reqs)):
+        st = build()
+        for again in range(2):
+            out = replay(runner, st, use_graph=True)
+            worst = check(out, st, ref, TOL[dtype])
+            assert runner.cache.free_blocks() == [g.pool.num_blocks for g in runner.cache.groups]
+    captured = [k for k, g in runner._graphs.items() if g.graph is not None]
+    print(f"{name} {dtype}: {len(runner._graphs)} shapes, {len(captured)} captured, "
+          f"{runner.graph_steps} graph steps, {runner.eager_steps} eager, worst {worst:.2e}")
+    assert runner.graph_steps > runner.eager_steps
+    assert not any(g.capture_failed for g in runner._graphs.values())
 
 
 def test_first_tokens_and_single_token_request(tmp_path_factory):

@@ -1,0 +1,133 @@
+"""The engine at the layer sizes of TinyLlama 1.1B (hidden 2048, 32 heads over 4 kv heads of 64,
+intermediate 5632, vocabulary 32000; 2 of its 22 layers) with seeded random weights made on the
+device, against the plain implementation run on the same weights made on the host: the four
+cuttings in 32-bit and bfloat16, and generation with graphs across the 512-token context bound."""
+import pytest
+import torch
+
+import plain_llama as plain
+import traces
+from test_replay_gpu import check, r64, replay
+from util import random_tokens, rel_err
+
+pytestmark = pytest.mark.gpu
+
+SHAPE = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama", "num_hidden_layers": 2, "hidden_size": 2048,
+    "num_attention_heads": 32, "num_key_value_heads": 4, "intermediate_size": 5632, "vocab_size": 32000,
+    "rope_theta": 10000.0, "rms_norm_eps": 1e-5, "max_position_embeddings": 2048, "tie_word_embeddings": False,
+    "hidden_act": "silu", "attention_bias": False, "rope_scaling": None, "initializer_range": 0.02, "eos_token_id": 2,
+}
+LAYERS_FULL = 22
+SEED, STD = 5, 0.02
+SHARPEN = 2.0       # q and k projections times this: attention far from uniform, so a misplaced key shows
+TOL = {"float32": 1e-4, "bfloat16": 2e-2}
+LENGTHS = [330, 137, 540, 64]
+
+_made = {}
+
+
+def host_weights(round_to=None):
+    """The weights `Engine(config=SHAPE, weights_seed=SEED)` makes on the device, made on the host."""
+    key = str(round_to)
+    if key not in _made:
+        from tiny_llm_amd.config import resolve
+        from tiny_llm_amd.models.decoder import Decoder
+        from tiny_llm_amd.weights.loader import random_tensor
+        _, spec = resolve(SHAPE)
+        w = {}
+        for s in Decoder(spec, "float32", "cpu").weight_specs():
+            t = random_tensor(s, SEED, STD, 0.0)
+            if s.name.endswith(("q_proj.weight", "k_proj.weight")):
+                t = t * SHARPEN
+            if round_to is not None and t.dim() >= 2:
+                t = t.to(round_to)
+            w[s.name] = t.double()
+        _made[key] = w
+    return _made[key]
+
+
+def requests():
+    return {f"r{i}": random_tokens(n, SHAPE["vocab_size"], 31 * i + 7) for i, n in enumerate(LENGTHS)}
+
+
+def references(dtype):
+    key = ("ref", dtype)
+    if key not in _made:
+        act = torch.bfloat16 if dtype == "bfloat16" else None
+        w = host_weights(act)
+        _made[key] = {rid: plain.llama_forward(w, SHAPE, toks, act_dtype=act) for rid, toks in requests().items()}
+    return _made[key]
+
+
+def sharpen(decoder):
+    for layer in decoder.layers:
+        m = layer.mixer
+        m.w_qkv[: m.q_size + m.kv_size] *= SHARPEN       # a power of two: exact in both element types
+
+
+def make_runner(dtype, max_tokens):
+    from tiny_llm_amd.config import EngineConfig
+    from tiny_llm_amd.engine.loading import build_runner, random_model
+    engine = EngineConfig(dtype=dtype, kv_block_size=16, max_cache_tokens=max_tokens, max_num_seqs=8,
+                          max_num_batched_tokens=4096, use_graphs=False)
+    _, dec = random_model(SHAPE, engine, seed=SEED, std=STD)
+    sharpen(dec)
+    runner = build_runner(dec, engine)
+    for g in runner.cache.groups:
+        for t in g.tensors.values():
+            t.fill_(float("nan"))
+    return runner
+
+
+def test_device_made_weights_equal_host_made_weights():
+    from tiny_llm_amd.config import EngineConfig
+    from tiny_llm_amd.engine.loading import random_model
+    _, dec = random_model(SHAPE, EngineConfig(dtype="float32"), seed=SEED, std=STD)
+    w = host_weights()
+    m = dec.layers[1].mixer
+    q = w["model.layers.1.self_attn.q_proj.weight"] / SHARPEN
+    assert torch.equal(m.w_qkv[: m.q_size].cpu().double(), q)
+    assert torch.equal(dec.lm_head.weight.cpu().double(), w["lm_head.weight"])
+    assert torch.equal(dec.layers[0].by_role["ffn"].w_down.cpu().double(), w["model.layers.0.mlp.down_proj.weight"])
+    assert torch.equal(dec.final_norm.weight.cpu().double(), w["model.norm.weight"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_four_cuttings_at_the_real_layer_sizes(dtype):
+    reqs, ref = requests(), references(dtype)
+    biggest = max(r64(len(t)) for t in reqs.values())
+    mixed, peak = traces.mixed(reqs, seed=4)
+    assert peak < sum(r64(len(t)) for t in reqs.values())        # pages are used again
+    runner = make_runner(dtype, max(biggest, peak))
+    for name, steps in (("whole", traces.whole(reqs)), ("tail", traces.tail_one_by_one(reqs)),
+                        ("portions", traces.portions(reqs, sizes=(7, 2, 190, 3, 2, 33, 64, 2, 300, 1, 129))),
+                        ("mixed", mixed)):
+        out = replay(runner, steps)
+        worst = check(out, steps, ref, TOL[dtype])
+        print(f"TinyLlama layer sizes (2 of {LAYERS_FULL} layers) {dtype} {name}: worst rel err {worst:.2e}", flush=True)
+        assert runner.cache.free_blocks() == [g.pool.num_blocks for g in runner.cache.groups]
+
+
+@pytest.mark.parametrize("graphs", [True, False])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_generation_across_the_512_bound_at_the_real_layer_sizes(dtype, graphs):
+    """What the throughput measurement runs: prompts of about 500 tokens, decode steps as graphs
+    whose attention splits a request's keys over workgroups once the context passes 512."""
+    from tiny_llm_amd import Engine, SamplingParams
+    from test_engine_gpu import check_logged_logits, poison, spy_on_steps
+    act = torch.bfloat16 if dtype == "bfloat16" else None
+    w = host_weights(act)
+    prompts = [random_tokens(n, SHAPE["vocab_size"], 900 + n) for n in (500, 481, 507, 470)]
+    eng = Engine(config=SHAPE, dtype=dtype, weights_seed=SEED, init_std=STD, kv_block_size=16, max_num_seqs=4,
+                 max_num_batched_tokens=1024, max_cache_tokens=4 * 576, use_graphs=graphs)
+    sharpen(eng.decoder)
+    poison(eng)
+    log = spy_on_steps(eng)
+    out = eng.generate(prompts, SamplingParams.greedy(24, ignore_eos=True))
+    tokens_of = {i: p + o for i, (p, o) in enumerate(zip(prompts, out))}
+    worst, n = check_logged_logits(log, tokens_of, w, SHAPE, act, TOL[dtype])
+    print(f"TinyLlama layer sizes {dtype} graphs={graphs}: {n} rows across 512, worst rel err {worst:.2e}", flush=True)
+    assert n == 4 * 24
+    if graphs:
+        assert sorted({k[2] for k, g in eng.runner._graphs.items() if k[0] == "decode" and g.graph is not None}) == [512, 1024]

@@ -86,6 +86,8 @@ class CacheManager:
         self.states: Dict[Hashable, torch.Tensor] = {}
         self._free_slots: List[int] = list(range(self.max_seqs - 1, -1, -1))
         self.requests: Dict[Hashable, RequestCache] = {}
+        # what the last `reserve_step` changed, until the step commits: (new requests, table lengths before)
+        self._reservation: Optional[tuple] = None
 
     # ------------------------------------------------------------------- tensors
     def elements_per_block(self) -> int:
@@ -203,11 +205,41 @@ class CacheManager:
             raise OutOfBlocks("the step needs more cache blocks than are free: needs "
                               f"{[sum(n[g] for n in needs) for g in range(len(self.groups))]}, "
                               f"free {self.free_blocks()}")
+        lengths = {rid: [len(b) for b in self.requests[rid].blocks] for rid, _ in growing if rid in self.requests}
+        self._reservation = (list(new), lengths, [rid for rid, _ in growing])
         for rid in new:
             self.add_request(rid)
         for rid, new_len in growing:
             self.grow(rid, new_len)
         return before
+
+    def undo_reservation(self) -> None:
+        """The step that the last `reserve_step` was for did not run: requests it admitted leave
+        again and tables it lengthened are cut back, in the reverse of the order in which they were
+        served, so that the cache and its free lists are as they were before.  Does nothing when no
+        reservation is open."""
+        if self._reservation is None:
+            return
+        new, lengths, order = self._reservation
+        self._reservation = None
+        for rid in reversed(order):
+            rc = self.requests.get(rid)
+            if rc is None:
+                continue
+            lens = lengths.get(rid, [0] * len(self.groups))
+            for gi, (g, n) in enumerate(zip(self.groups, lens)):
+                extra = [b for b in rc.blocks[gi][n:] if b != RELEASED]
+                if extra:
+                    g.pool.free(list(reversed(extra)))
+                del rc.blocks[gi][n:]
+        for rid in reversed(new):
+            rc = self.requests.pop(rid, None)
+            if rc is not None:
+                self._free_slots.append(rc.slot)
+
+    def forget_reservation(self) -> None:
+        """The step ran and was committed."""
+        self._reservation = None
 
     def commit(self, req_id, new_len: int) -> None:
         """The step has written positions < new_len.  Gives back what a window has passed."""

@@ -25,7 +25,7 @@ class EngineConfig:
     max_num_batched_tokens: int = 2048  # token budget of one step
     max_model_len: Optional[int] = None  # None = the model's max_position_embeddings
     device: int = 0
-    use_graphs: bool = True            # capture decode-only steps in HIP graphs
+    use_graphs: bool = True            # run steps as HIP graphs, captured per shape of step
     seed: int = 0
 
     def __post_init__(self):

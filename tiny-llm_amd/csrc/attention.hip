@@ -518,6 +518,7 @@ __global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
   const int tile = n_tiles - 1 - item / nkv, kvh = item % nkv;
   const int G = nq / nkv, TW = 16 / G;
   const int req = tile_req[tile], tok0 = tile_tok0[tile], ntok = tile_ntok[tile];
+  if (ntok <= 0) return;      // a padding tile of a step laid out for more tiles than it has (whole workgroup)
   const int32_t* bt = block_tables + (int64_t)req * max_blocks;
 
   // the tokens of a tile are consecutive tokens of one request, so their positions are consecutive

@@ -12,10 +12,10 @@ import itertools
 from typing import Dict, Hashable, List, Mapping, Optional, Sequence, Union
 
 from ..config import EngineConfig
-from ..sampling import Sampler, SamplingParams
+from ..sampling import SamplingParams
 from .loading import build_runner, load_model, random_model
 from .scheduler import Request, Scheduler
-from .step import StepEntry
+from .step import SampleSpec, StepEntry
 
 
 class Engine:
@@ -36,7 +36,6 @@ class Engine:
         self.scheduler = Scheduler(self.runner.cache, self.engine_config.max_num_seqs,
                                    self.engine_config.max_num_batched_tokens, self.runner.max_model_len,
                                    self.eos_token_ids)
-        self.sampler = Sampler(self.decoder.device)
         self._ids = itertools.count()
         self.requests: Dict[Hashable, Request] = {}
         self.steps_run = 0
@@ -72,35 +71,22 @@ class Engine:
 
     # -------------------------------------------------------------------- step
     def step(self) -> List[Request]:
-        """One scheduler decision, one forward pass, one sampling call.  Returns the requests
-        that finished in this step."""
+        """One scheduler decision, one forward pass with the sampler at its end.  Returns the
+        requests that finished in this step."""
         plan = self.scheduler.schedule()
         done = list(plan.finished)
         if not plan.entries:
             return done
-        if all(e.count == 1 and e.samples for e in plan.entries):
-            # decode-only step: model and sampler run as one (captured) unit on the device
-            reqs = [e.request for e in plan.entries]
-            toks = self.runner.decode_step([r.req_id for r in reqs], [r.token_slice(e.start, 1)[0] for r, e in
-                                                                      zip(reqs, plan.entries)],
-                                           [r.params for r in reqs], [r.seed for r in reqs],
-                                           [r.num_tokens for r in reqs], use_graph=self.engine_config.use_graphs)
-            done += self.scheduler.update(plan, {r.req_id: t for r, t in zip(reqs, toks)})
-            self.steps_run += 1
-            return done
-        entries, rows = [], []
+        entries, rows, samples = [], [], []
         for e in plan.entries:
-            toks = e.request.token_slice(e.start, e.count)
-            entries.append(StepEntry(e.request.req_id, toks, [e.count - 1] if e.samples else []))
+            r = e.request
+            entries.append(StepEntry(r.req_id, r.token_slice(e.start, e.count), [e.count - 1] if e.samples else []))
             if e.samples:
-                rows.append(e.request)
-        logits = self.runner.step(entries)
-        sampled = {}
-        if rows:
-            toks = self.sampler(logits, [r.params for r in rows], [r.seed for r in rows],
-                                [r.num_tokens for r in rows])
-            sampled = {r.req_id: t for r, t in zip(rows, toks)}
-        done += self.scheduler.update(plan, sampled)
+                p = r.params
+                rows.append(r)
+                samples.append(SampleSpec(p.temperature if p.do_sample else 0.0, p.top_k, p.top_p, r.seed, r.num_tokens))
+        toks = self.runner.run(entries, samples, use_graph=self.engine_config.use_graphs)
+        done += self.scheduler.update(plan, {r.req_id: t for r, t in zip(rows, toks)})
         self.steps_run += 1
         return done
 

@@ -1,16 +1,25 @@
 """The step function: one batch of (request, its next tokens) through the model.
 
 A step runs only the tokens it is given, against the cache that earlier steps
-left, and returns the logits at the wanted places.  Entries may be portions of
-prompts beside single decoded tokens, cut anywhere.  The reference's runtime needs
-five calls and allows either whole prompts from position 0 or exactly one token per
-request (tiny_llm/pipeline/pipeline.cpp:132-140, 184-190,
+left, and returns the logits at the wanted places (`step`) or the tokens sampled
+from them on the device (`run`).  Entries may be portions of prompts beside single
+decoded tokens, cut anywhere.  The reference's runtime needs five calls and allows
+either whole prompts from position 0 or exactly one token per request
+(tiny_llm/pipeline/pipeline.cpp:132-140, 184-190,
 tiny_llm/runtime/cuda/cuda_runtime.cpp:673, 690); here it is one call for any mix.
 
-Step metadata is built on the host in one pinned int32 buffer and uploaded with
-one copy (the reference uploads a block table per layer with a stream sync each,
-cuda_runtime.cpp:758-773).  Token rows map to requests through `req_of_token`, so
-kernels need no search over sequence separators (tiny_llm/ops/details.hpp:19-36).
+Step metadata is laid out by ONE routine (`Layout`, `fill_metadata`) in one pinned
+int32 buffer and uploaded with one copy (the reference uploads a block table per
+layer with a stream sync each, cuda_runtime.cpp:758-773).  Token rows map to
+requests through `req_of_token`, so kernels need no search over sequence
+separators (tiny_llm/ops/details.hpp:19-36).
+
+A step runs eagerly or as a HIP graph.  A graph is captured per shape of step:
+decode-only steps by (requests, bound on the context), other steps by capacities
+(tokens, requests, wanted rows) to which the step is padded: padding tokens write
+no cache slot, padding query tiles hold no token, padding rows of the output are
+dropped.  Eager and captured steps share the layout routine, the model code and
+the sampler; a captured step only has its sizes rounded up and its buffers static.
 """
 from __future__ import annotations
 
@@ -22,6 +31,7 @@ import numpy as np
 import torch
 
 from ..cache import CacheManager
+from ..kernels import ops
 
 
 @dataclass
@@ -32,8 +42,21 @@ class StepEntry:
 
 
 @dataclass
+class SampleSpec:
+    """How the token of one wanted row is chosen on the device: temperature <= 0 is the first
+    maximum; else temperature -> top-k -> top-p -> multinomial with the uniform number of
+    (seed, counter)."""
+    temperature: float = 0.0
+    top_k: int = 0
+    top_p: float = 1.0
+    seed: int = 0
+    counter: int = 0
+
+
+@dataclass
 class StepContext:
-    """Who is in the batch and where each token sits; device tensors are int32."""
+    """Who is in the batch and where each token sits; device tensors are int32.
+    In a captured step the sizes are capacities and the host copies are not meaningful."""
     num_tokens: int
     num_requests: int
     tokens: torch.Tensor            # [T]
@@ -52,8 +75,9 @@ class StepContext:
     max_q_len: int = 0
     max_seq_len: int = 0
     block_size: int = 0
-
+    static: bool = False            # a captured step: nothing may be built on the host any more
     _tiles: Dict[int, tuple] = field(default_factory=dict)
+    _on_new_width = None            # told when a tile width is asked for the first time
 
     @property
     def decode_only(self) -> bool:
@@ -62,19 +86,16 @@ class StepContext:
     def attention_tiles(self, tokens_per_tile: int):
         """(tile_req, tile_tok0, tile_ntok) int32 device tensors: every request's tokens of this
         step cut into groups of at most `tokens_per_tile` (the query tiles of the MFMA attention
-        kernel).  Built once per width and step."""
+        kernels).  Widths that earlier steps asked for came with the step's upload; a new width is
+        built here, once, and remembered for the steps to come."""
         if tokens_per_tile not in self._tiles:
-            req, tok0, ntok = [], [], []
-            t = 0
-            for r, n in enumerate(self.q_lens):
-                for s in range(0, n, tokens_per_tile):
-                    req.append(r)
-                    tok0.append(t + s)
-                    ntok.append(min(tokens_per_tile, n - s))
-                t += n
-            dev = self.tokens.device
-            packed = torch.tensor([req, tok0, ntok], dtype=torch.int32).to(dev, non_blocking=True)
+            if self.static:
+                raise StepError(f"query tiles of {tokens_per_tile} tokens were not laid out for this captured step")
+            req, tok0, ntok = tile_lists(self.q_lens, tokens_per_tile)
+            packed = torch.tensor([req, tok0, ntok], dtype=torch.int32).to(self.tokens.device, non_blocking=True)
             self._tiles[tokens_per_tile] = (packed[0], packed[1], packed[2])
+            if self._on_new_width is not None:
+                self._on_new_width(tokens_per_tile)
         return self._tiles[tokens_per_tile]
 
 
@@ -82,6 +103,197 @@ class StepError(ValueError):
     pass
 
 
+def tile_lists(q_lens: Sequence[int], width: int):
+    """Every request's tokens cut into groups of at most `width`: (request, first token row, count)."""
+    req, tok0, ntok = [], [], []
+    t = 0
+    for r, n in enumerate(q_lens):
+        for s in range(0, n, width):
+            req.append(r)
+            tok0.append(t + s)
+            ntok.append(min(width, n - s))
+        t += n
+    return req, tok0, ntok
+
+
+# ----------------------------------------------------------------------- layout
+class Layout:
+    """Where every section of a step's metadata lies in its int32 buffer, for given capacities:
+    T tokens, R requests, n_out wanted rows, G cache groups with block tables MB wide, query-tile
+    lists by width, and (optionally) the sampler's per-row arguments.  Sections start on 16 bytes."""
+
+    def __init__(self, T: int, R: int, n_out: int, G: int, MB: int, tile_caps: Dict[int, int], sampling: bool):
+        self.T, self.R, self.n_out, self.G, self.MB = T, R, n_out, G, MB
+        self.tile_caps = dict(tile_caps)
+        self.sampling = sampling
+        self.off: Dict[str, Tuple[int, int]] = {}
+        at = 0
+
+        def add(name, n):
+            nonlocal at
+            self.off[name] = (at, n)
+            at += ((n + 3) // 4) * 4
+
+        for name, n in (("tokens", T), ("positions", T), ("req_of_token", T), ("cu_seqlens", R + 1), ("seq_lens", R),
+                        ("state_slots", R), ("logit_rows", n_out)):
+            add(name, n)
+        for g in range(G):
+            add(f"slots{g}", T)
+        for g in range(G):
+            add(f"tables{g}", R * MB)
+        for w, cap in self.tile_caps.items():
+            add(f"tiles{w}", 3 * cap)
+        if sampling:
+            for name in ("temperature", "top_p", "top_k", "counters"):
+                add(name, n_out)
+            add("seeds", 2 * n_out)         # int64
+        self.total = at
+
+    def sec(self, buf, name: str):
+        o, n = self.off[name]
+        return buf[o:o + n]
+
+    def context(self, dev: torch.Tensor, block_size: int, **host) -> StepContext:
+        """The device views of an uploaded buffer as a StepContext."""
+        T, R, G, MB = self.T, self.R, self.G, self.MB
+        ctx = StepContext(
+            num_tokens=T, num_requests=R, tokens=self.sec(dev, "tokens"), positions=self.sec(dev, "positions"),
+            req_of_token=self.sec(dev, "req_of_token"), cu_seqlens_q=self.sec(dev, "cu_seqlens"),
+            seq_lens=self.sec(dev, "seq_lens"), state_slots=self.sec(dev, "state_slots"),
+            logit_rows=self.sec(dev, "logit_rows") if self.n_out else None,
+            block_tables=[self.sec(dev, f"tables{g}").view(R, MB) for g in range(G)],
+            slot_mappings=[self.sec(dev, f"slots{g}") for g in range(G)], block_size=block_size, **host)
+        for w, cap in self.tile_caps.items():
+            t = self.sec(dev, f"tiles{w}")
+            ctx._tiles[w] = (t[:cap], t[cap:2 * cap], t[2 * cap:3 * cap])
+        return ctx
+
+    def sampler_args(self, dev: torch.Tensor):
+        n = self.n_out
+        return (self.sec(dev, "temperature").view(torch.float32), self.sec(dev, "top_k"),
+                self.sec(dev, "top_p").view(torch.float32), self.sec(dev, "seeds").view(torch.int64),
+                self.sec(dev, "counters"))
+
+
+@dataclass
+class _Row:
+    """One entry of a step, resolved against the cache."""
+    req_id: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int]
+    context_len: int            # tokens cached before the step
+    slot: int
+    tables: List[List[int]]     # per cache group
+
+
+def fill_metadata(host: np.ndarray, lay: Layout, rows: Sequence[_Row], block_size: int,
+                  samples: Optional[Sequence[SampleSpec]] = None, seen: Optional[list] = None) -> None:
+    """Writes the metadata of a step into `host` (int32, at least lay.total long): the ONE routine
+    behind eager steps, captured decode steps and captured mixed steps.
+
+    Capacities beyond the step's own sizes are padded so that the same kernels run unchanged:
+    padding tokens are token 0 at position 0 of request row 0 with cache slot -1 (nothing is
+    stored); padding requests have no tokens (cu_seqlens stays at T); padding query tiles hold no
+    token; padding output rows point at row 0 and are dropped by the caller.
+    `seen` (per group, per request row): block-table rows a static buffer already holds."""
+    T_cap, R_cap, G, MB, bs = lay.T, lay.R, lay.G, lay.MB, block_size
+    R = len(rows)
+    tok, pos, rot = lay.sec(host, "tokens"), lay.sec(host, "positions"), lay.sec(host, "req_of_token")
+    cu, sl, ss, lr = (lay.sec(host, n) for n in ("cu_seqlens", "seq_lens", "state_slots", "logit_rows"))
+    sms = [lay.sec(host, f"slots{g}") for g in range(G)]
+    bts = [lay.sec(host, f"tables{g}").reshape(R_cap, MB) for g in range(G)]
+    t = k = 0
+    q_lens = []
+    for r, row in enumerate(rows):
+        n, c = len(row.tokens), row.context_len
+        tok[t:t + n] = row.tokens
+        cu[r] = t
+        sl[r] = c + n
+        ss[r] = row.slot
+        for w in row.want:
+            lr[k] = t + int(w)
+            k += 1
+        if n == 1:
+            pos[t] = c
+            rot[t] = r
+        else:
+            pos[t:t + n] = np.arange(c, c + n, dtype=np.int32)
+            rot[t:t + n] = r
+        for g in range(G):
+            table = row.tables[g]
+            if len(table) > MB:
+                raise StepError(f"request {row.req_id!r} holds {len(table)} blocks, the table has room for {MB}")
+            last = seen[g][r] if seen is not None else None
+            # a row is rewritten only when it belongs to another admission than last time (the table
+            # object is made when a request is admitted) or has changed length; blocks that a window
+            # has released turn into -1 without a change of length, but they lie before the window
+            # and are never read
+            if last is None or last[0] is not table or last[1] != len(table):
+                bts[g][r, :len(table)] = np.maximum(np.asarray(table, dtype=np.int32), 0)
+                if seen is not None:
+                    seen[g][r] = (table, len(table))
+            if n == 1:
+                sms[g][t] = max(table[c // bs], 0) * bs + c % bs
+            else:
+                p = np.arange(c, c + n, dtype=np.int32)
+                sms[g][t:t + n] = np.maximum(np.asarray(table, dtype=np.int32), 0)[p // bs] * bs + p % bs
+        q_lens.append(n)
+        t += n
+    T = t
+    if T < T_cap:
+        tok[T:T_cap] = 0
+        pos[T:T_cap] = 0
+        rot[T:T_cap] = 0
+        for g in range(G):
+            sms[g][T:T_cap] = -1
+    cu[R:R_cap + 1] = T
+    if R < R_cap:
+        sl[R:R_cap] = 0
+        ss[R:R_cap] = 0
+    if k < lay.n_out:
+        lr[k:lay.n_out] = 0
+    for w, cap in lay.tile_caps.items():
+        req, tok0, ntok = tile_lists(q_lens, w)
+        m = len(req)
+        if m > cap:
+            raise StepError(f"{m} query tiles of {w} tokens, the layout has room for {cap}")
+        sec = lay.sec(host, f"tiles{w}")
+        sec[0:m], sec[cap:cap + m], sec[2 * cap:2 * cap + m] = req, tok0, ntok
+        sec[m:cap], sec[cap + m:2 * cap], sec[2 * cap + m:3 * cap] = 0, 0, 0
+    if lay.sampling:
+        n_out = lay.n_out
+        fl = host.view(np.float32)
+        o_t, o_p = lay.off["temperature"][0], lay.off["top_p"][0]
+        tk, ct = lay.sec(host, "top_k"), lay.sec(host, "counters")
+        sd = host.view(np.int64)[lay.off["seeds"][0] // 2: lay.off["seeds"][0] // 2 + n_out]
+        m = len(samples) if samples is not None else 0
+        if m:
+            fl[o_t:o_t + m] = [s.temperature for s in samples]
+            fl[o_p:o_p + m] = [s.top_p for s in samples]
+            tk[:m] = [s.top_k for s in samples]
+            ct[:m] = [s.counter for s in samples]
+            sd[:m] = [s.seed & 0x7FFFFFFFFFFFFFFF for s in samples]
+        if m < n_out:
+            fl[o_t + m:o_t + n_out] = 0.0
+            fl[o_p + m:o_p + n_out] = 1.0
+            tk[m:], ct[m:], sd[m:] = 0, 0, 0
+
+
+def token_capacity(n: int, limit: int) -> int:
+    """The token count a captured step is padded to: steps of 16 up to 64 (the few-row products'
+    own steps), of 64 up to 1024, of 256 beyond."""
+    step = 16 if n <= 64 else (64 if n <= 1024 else 256)
+    return min(-(-n // step) * step, max(limit, n))
+
+
+def power_of_two_at_least(n: int) -> int:
+    p = 1
+    while p < n:
+        p *= 2
+    return p
+
+
+# ----------------------------------------------------------------------- runner
 class ModelRunner:
     """Owns the decoder's cache views and turns step entries into one forward pass."""
 
@@ -97,21 +309,20 @@ class ModelRunner:
             decoder.caches[i][role] = cache.layer_cache((i, role), readers.get((i, role)))
         for (i, role) in decoder.state_specs():
             decoder.states[i][role] = cache.states[(i, role)]
+        self.workspace = ops.Workspace(self.device, self.max_tokens)
         self._pinned: Optional[torch.Tensor] = None
         self._uploaded: Optional[torch.cuda.Event] = None
-        self._graphs: Dict[Tuple[int, int], "DecodeGraph"] = {}
+        self._graphs: Dict[tuple, "StepGraph"] = {}
+        self._graph_pool = None
+        self._tile_widths: set = set()          # query-tile widths the model's kernels have asked for
+        self.last_logits: Optional[torch.Tensor] = None     # of the last `run` (tests look at it)
+        self.graph_steps = 0
+        self.eager_steps = 0
 
-    # ----------------------------------------------------------------- metadata
-    def _host_buffer(self, n: int) -> torch.Tensor:
-        if self._pinned is None or self._pinned.numel() < n:
-            self._pinned = torch.empty(max(n, 1 << 16), dtype=torch.int32, pin_memory=True)
-        return self._pinned[:n]
-
-    def prepare(self, entries: Sequence[StepEntry]) -> StepContext:
-        """Checks the entries, takes the cache blocks they need (all or nothing) and
-        builds the step metadata on the device."""
+    # ---------------------------------------------------------------- validation
+    def _resolve(self, entries: Sequence[StepEntry]) -> Tuple[List[_Row], int]:
+        """Checks the entries, takes the cache blocks they need (all or nothing)."""
         cm = self.cache
-        bs = cm.block_size
         if not entries:
             raise StepError("a step needs at least one entry")
         seen = set()
@@ -129,110 +340,146 @@ class ModelRunner:
             for w in e.want:
                 if not (0 <= int(w) < n):
                     raise StepError(f"wanted place {w} of request {e.req_id!r} is outside its {n} tokens")
+            c = cm.num_tokens(e.req_id) if cm.has(e.req_id) else 0
+            if c + n > self.max_model_len:
+                raise StepError(f"request {e.req_id!r} would reach {c + n} tokens, "
+                                f"the limit is {self.max_model_len}")
             T += n
         if T > self.max_tokens:
             raise StepError(f"step brings {T} tokens, the budget is {self.max_tokens}")
-
-        for e in entries:
-            c = cm.num_tokens(e.req_id) if cm.has(e.req_id) else 0
-            if c + len(e.tokens) > self.max_model_len:
-                raise StepError(f"request {e.req_id!r} would reach {c + len(e.tokens)} tokens, "
-                                f"the limit is {self.max_model_len}")
         ctx_lens = cm.reserve_step([(e.req_id, len(e.tokens)) for e in entries])
-        new_lens = [c + len(e.tokens) for c, e in zip(ctx_lens, entries)]
+        G = len(cm.groups)
+        rows = [_Row(e.req_id, e.tokens, e.want, c, cm.slot(e.req_id), [cm.block_table(e.req_id, g) for g in range(G)])
+                for e, c in zip(entries, ctx_lens)]
+        return rows, T
 
-        R, G = len(entries), len(cm.groups)
-        max_blocks = max(1, max(-(-n // bs) for n in new_lens))
-        n_out = sum(len(e.want) for e in entries)
-        sizes = [T, T, T, R + 1, R, R, n_out] + [T] * G + [R * max_blocks] * G
-        offs = [0]
-        for s in sizes:
-            offs.append(offs[-1] + ((s + 3) // 4) * 4)   # 16-byte aligned sections
-        if self._uploaded is not None:
-            self._uploaded.synchronize()      # the last step's upload has left the pinned buffer
-        buf = self._host_buffer(offs[-1])
-        host = buf.numpy()
-        host[:offs[-1]] = 0
-        tok, pos, rot = host[offs[0]:], host[offs[1]:], host[offs[2]:]
-        cu, sl, ss, lr = host[offs[3]:], host[offs[4]:], host[offs[5]:], host[offs[6]:]
-        t = 0
-        k = 0
-        q_lens, slots = [], []
-        for r, e in enumerate(entries):
-            n = len(e.tokens)
-            c = ctx_lens[r]
-            tok[t:t + n] = e.tokens
-            pos[t:t + n] = range(c, c + n)
-            rot[t:t + n] = r
-            cu[r] = t
-            sl[r] = new_lens[r]
-            ss[r] = cm.slot(e.req_id)
-            slots.append(cm.slot(e.req_id))
-            for w in e.want:
-                lr[k] = t + int(w)
-                k += 1
-            for g in range(G):
-                table = cm.block_table(e.req_id, g)
-                sm = host[offs[7 + g]:]
-                bt = host[offs[7 + G + g]:]
-                tb = np.maximum(np.asarray(table, dtype=np.int32), 0)   # released blocks are never read
-                bt[r * max_blocks: r * max_blocks + len(table)] = tb
-                p = np.arange(c, c + n, dtype=np.int32)
-                sm[t:t + n] = tb[p // bs] * bs + p % bs
-            q_lens.append(n)
-            t += n
-        cu[R] = T
-        dev = buf.to(self.device, non_blocking=True)
-        self._uploaded = torch.cuda.Event()
-        self._uploaded.record()
-        sec = lambda i, n: dev[offs[i]:offs[i] + n]
-        return StepContext(
-            num_tokens=T, num_requests=R,
-            tokens=sec(0, T), positions=sec(1, T), req_of_token=sec(2, T), cu_seqlens_q=sec(3, R + 1),
-            seq_lens=sec(4, R), state_slots=sec(5, R), logit_rows=sec(6, n_out) if n_out else None,
-            block_tables=[sec(7 + G + g, R * max_blocks).view(R, max_blocks) for g in range(G)],
-            slot_mappings=[sec(7 + g, T) for g in range(G)],
-            q_lens=q_lens, context_lens=ctx_lens, slots_host=slots, max_q_len=max(q_lens),
-            max_seq_len=max(new_lens), block_size=bs)
+    def _host_buffer(self, n: int) -> torch.Tensor:
+        if self._pinned is None or self._pinned.numel() < n:
+            self._pinned = torch.empty(max(n, 1 << 16), dtype=torch.int32, pin_memory=True)
+        return self._pinned[:n]
 
-    # --------------------------------------------------------------------- step
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def _new_width(self, w: int) -> None:
+        self._tile_widths.add(w)
+
+    def _tile_caps(self, T: int, R: int, decode_only: bool) -> Dict[int, int]:
+        """Room for the query tiles of every width the kernels use (none in decode-only steps,
+        where row i is request i)."""
+        if decode_only:
+            return {}
+        return {w: -(-T // w) + R for w in sorted(self._tile_widths)}
+
+    # ------------------------------------------------------------------- eager
+    def prepare(self, entries: Sequence[StepEntry], samples: Optional[Sequence[SampleSpec]] = None):
+        """Reserves cache, lays the step out at its exact sizes and uploads it.
+        Returns (context, layout, device buffer, rows)."""
+        rows, T = self._resolve(entries)
+        try:
+            bs = self.cache.block_size
+            R, G = len(rows), len(self.cache.groups)
+            max_blocks = max(1, max(len(tb) for row in rows for tb in row.tables) if G else 1)
+            n_out = sum(len(r.want) for r in rows)
+            q_lens = [len(r.tokens) for r in rows]
+            decode_only = max(q_lens) == 1
+            tile_caps = {} if decode_only else {w: len(tile_lists(q_lens, w)[0]) for w in sorted(self._tile_widths)}
+            lay = Layout(T, R, n_out, G, max_blocks, tile_caps, samples is not None)
+            if self._uploaded is not None:
+                self._uploaded.synchronize()      # the last step's upload has left the pinned buffer
+            buf = self._host_buffer(lay.total)
+            host = buf.numpy()
+            host[:lay.total] = 0
+            fill_metadata(host, lay, rows, bs, samples)
+            dev = buf.to(self.device, non_blocking=True)
+            self._uploaded = torch.cuda.Event()
+            self._uploaded.record()
+            ctx_lens = [r.context_len for r in rows]
+            ctx = lay.context(dev, bs, q_lens=q_lens, context_lens=ctx_lens, slots_host=[r.slot for r in rows],
+                              max_q_len=max(q_lens), max_seq_len=max(c + n for c, n in zip(ctx_lens, q_lens)))
+            ctx._on_new_width = self._new_width
+            return ctx, lay, dev, rows
+        except BaseException:
+            self.cache.undo_reservation()
+            raise
+
+    def _forward(self, ctx: StepContext) -> torch.Tensor:
+        with ops.use_workspace(self.workspace):
+            return self.decoder.forward(ctx)
+
+    def _commit(self, rows: Sequence[_Row]) -> None:
+        for r in rows:
+            self.cache.commit(r.req_id, r.context_len + len(r.tokens))
+        self.cache.forget_reservation()
+
+    def step(self, entries: Sequence[StepEntry], use_graph: bool = False) -> torch.Tensor:
         """Runs the entries as one batch.  Returns float32 logits [wanted, vocab] on the
-        device, in the order of the entries and of each entry's `want`."""
-        ctx = self.prepare(entries)
-        logits = self.decoder.forward(ctx)
-        for e, c, n in zip(entries, ctx.context_lens, ctx.q_lens):
-            self.cache.commit(e.req_id, c + n)
+        device, in the order of the entries and of each entry's `want`.  If the forward pass
+        raises, the cache is as it was before the call."""
+        if use_graph and self.decoder.graph_safe:
+            return self._graph_step(entries, None)[0]
+        ctx, _, _, rows = self.prepare(entries)
+        try:
+            logits = self._forward(ctx)
+        except BaseException:
+            self.cache.undo_reservation()
+            raise
+        self._commit(rows)
+        self.eager_steps += 1
         return logits
 
-    # ------------------------------------------------------------ decode graphs
-    def decode_step(self, req_ids: Sequence[Hashable], tokens: Sequence[int], params, seeds: Sequence[int],
-                    counters: Sequence[int], use_graph: bool = True) -> List[int]:
-        """One decoded token for each request (its next input token given), sampled on the device.
-        With `use_graph` the whole step (model and sampler) is one HIP graph per batch size,
-        replayed on static buffers; only the metadata upload and the token download remain."""
-        R = len(req_ids)
-        cm = self.cache
-        for rid, t in zip(req_ids, tokens):
-            if not (0 <= int(t) < self.vocab_size):
-                raise StepError(f"token id {t} of request {rid!r} is outside the vocabulary")
-            if (cm.num_tokens(rid) if cm.has(rid) else 0) + 1 > self.max_model_len:
-                raise StepError(f"request {rid!r} would exceed {self.max_model_len} tokens")
-        ctx_lens = cm.reserve_step([(rid, 1) for rid in req_ids])
-        # One graph per batch size and context bound: the bound (a power of two, at least 512) decides
-        # into how many workgroups the attention kernel splits a request's keys, which is fixed at capture.
-        bound = 512
-        while bound < max(ctx_lens) + 1:
-            bound *= 2
-        bound = min(bound, self.max_model_len)
-        dg = self._graphs.get((R, bound))
-        if dg is None:
-            dg = self._graphs[(R, bound)] = DecodeGraph(self, R, bound)
-        toks = dg.run(req_ids, tokens, ctx_lens, params, seeds, counters,
-                      capture=use_graph and self.decoder.graph_safe)
-        for rid, c in zip(req_ids, ctx_lens):
-            cm.commit(rid, c + 1)
-        return toks
+    def run(self, entries: Sequence[StepEntry], samples: Sequence[SampleSpec], use_graph: bool = True) -> List[int]:
+        """Runs the entries and chooses a token for every wanted row on the device (`samples` has
+        one SampleSpec per wanted row, in order).  Returns the tokens.  With `use_graph` the whole
+        step, model and sampler, is a HIP graph per shape of step, replayed on static buffers: only
+        the metadata upload and the token download remain on the host."""
+        n_out = sum(len(e.want) for e in entries)
+        if len(samples) != n_out:
+            raise StepError(f"{n_out} rows are wanted, {len(samples)} sampling settings were given")
+        if use_graph and self.decoder.graph_safe:
+            return self._graph_step(entries, samples)[1]
+        ctx, lay, dev, rows = self.prepare(entries, samples)
+        try:
+            logits = self._forward(ctx)
+            out = torch.empty(n_out, dtype=torch.int32, device=self.device)
+            if n_out:
+                ops.sample(logits, out, *lay.sampler_args(dev))
+        except BaseException:
+            self.cache.undo_reservation()
+            raise
+        self._commit(rows)
+        self.eager_steps += 1
+        self.last_logits = logits
+        return out.cpu().tolist()
+
+    # ------------------------------------------------------------------ graphs
+    def _graph_step(self, entries: Sequence[StepEntry], samples: Optional[Sequence[SampleSpec]]):
+        rows, T = self._resolve(entries)
+        try:
+            R = len(rows)
+            n_out = sum(len(r.want) for r in rows)
+            decode_only = all(len(r.tokens) == 1 for r in rows)
+            new_lens = [r.context_len + len(r.tokens) for r in rows]
+            if decode_only and n_out == R:
+                # exact sizes; the bound on the context (a power of two, at least 512) decides into how
+                # many workgroups the attention kernel splits a request's keys, which is fixed at capture
+                bound = min(max(512, power_of_two_at_least(max(new_lens))), max(self.max_model_len, 1))
+                bound = max(bound, max(new_lens))
+                key = ("decode", R, bound, samples is not None)
+                caps = (R, R, R, 1, bound)
+            else:
+                T_cap = token_capacity(T, self.max_tokens)
+                R_cap = min(power_of_two_at_least(R), max(self.cache.max_seqs, R))
+                # every row may be wanted (replay), or at most one per request (serving)
+                n_cap = R_cap if n_out <= R_cap and samples is not None else T_cap
+                key = ("mixed", T_cap, R_cap, n_cap, samples is not None)
+                caps = (T_cap, R_cap, n_cap, T_cap, self.max_model_len)
+            sg = self._graphs.get(key)
+            if sg is None:
+                sg = self._graphs[key] = StepGraph(self, *caps, sampling=samples is not None)
+            logits, toks = sg.run(rows, samples, n_out)
+        except BaseException:
+            self.cache.undo_reservation()
+            raise
+        self._commit(rows)
+        return logits, toks
 
     def finish(self, req_id) -> None:
         """The request is done: its blocks and its state slot are given back."""
@@ -240,125 +487,118 @@ class ModelRunner:
             self.cache.free_request(req_id)
 
 
-class DecodeGraph:
-    """Static buffers and the captured HIP graph of a decode-only step of `R` requests whose
-    contexts stay within `max_seq_len` tokens.
+class StepGraph:
+    """Static buffers and the captured HIP graph of steps of one shape: capacities of T tokens,
+    R requests and n_out wanted rows, `max_q_len` 1 (decode: row i is request i) or more, contexts
+    within `max_seq_len`.
 
-    The block-table width is fixed at its maximum and the key splits of the attention kernel follow
-    `max_seq_len`, so one capture serves every step of that batch size and context bound.  The
-    first run of a size executes eagerly (kernels configure themselves, the allocator warms up);
-    the second is captured; later ones are replayed.  No memset node is recorded: buffers are
-    written by kernels and by the upload only."""
+    The block-table width is fixed at its maximum.  The first run of a shape executes eagerly on the
+    static buffers (kernels configure themselves, the workspace grows, the tile widths the kernels
+    ask for become known); the second is captured; later ones are replayed.  No memset node is
+    recorded: buffers are written by kernels and by the upload only.  A shape whose capture fails
+    (a part asks for something that was not laid out) keeps running eagerly."""
 
-    def __init__(self, runner: ModelRunner, R: int, max_seq_len: int):
-        self.runner, self.R = runner, R
-        cm = runner.cache
-        dev = runner.device
-        bs = cm.block_size
-        self.G = len(cm.groups)
-        self.MB = -(-runner.max_model_len // bs)
-        G, MB = self.G, self.MB
-        # int32 sections: tokens, positions, req_of_token, cu_seqlens, seq_lens, state_slots, logit_rows,
-        # slot mappings, block tables, then sampling: temperature(f32) top_p(f32) top_k counters seeds(i64)
-        sizes = [R, R, R, R + 1, R, R, R] + [R] * G + [R * MB] * G + [R, R, R, R, 2 * R]
-        offs = [0]
-        for n in sizes:
-            offs.append(offs[-1] + ((n + 3) // 4) * 4)
-        self.offs = offs
-        self.host = torch.zeros(offs[-1], dtype=torch.int32, pin_memory=True)
-        self.dev = torch.zeros(offs[-1], dtype=torch.int32, device=dev)
-        self.np = self.host.numpy()
-        sec = lambda i, n: self.dev[offs[i]:offs[i] + n]
-        self.np[offs[2]:offs[2] + R] = np.arange(R)
-        self.np[offs[3]:offs[3] + R + 1] = np.arange(R + 1)
-        self.np[offs[6]:offs[6] + R] = np.arange(R)
-        self.ctx = StepContext(
-            num_tokens=R, num_requests=R, tokens=sec(0, R), positions=sec(1, R), req_of_token=sec(2, R),
-            cu_seqlens_q=sec(3, R + 1), seq_lens=sec(4, R), state_slots=sec(5, R), logit_rows=sec(6, R),
-            block_tables=[sec(7 + G + g, R * MB).view(R, MB) for g in range(G)],
-            slot_mappings=[sec(7 + g, R) for g in range(G)],
-            q_lens=[1] * R, context_lens=[0] * R, slots_host=[0] * R, max_q_len=1,
-            max_seq_len=max_seq_len, block_size=bs)
-        s0 = 7 + 2 * G
-        self.temperature = sec(s0, R).view(torch.float32)
-        self.top_p = sec(s0 + 1, R).view(torch.float32)
-        self.top_k = sec(s0 + 2, R)
-        self.counters = sec(s0 + 3, R)
-        self.seeds = sec(s0 + 4, 2 * R).view(torch.int64)
-        self.s0 = s0
-        self.out = torch.zeros(R, dtype=torch.int32, device=dev)
-        self.out_host = torch.zeros(R, dtype=torch.int32, pin_memory=True)
+    def __init__(self, runner: ModelRunner, T: int, R: int, n_out: int, max_q_len: int, max_seq_len: int,
+                 sampling: bool):
+        self.runner = runner
+        self.T, self.R, self.n_out = T, R, n_out
+        self.max_q_len, self.max_seq_len, self.sampling = max_q_len, max_seq_len, sampling
         self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.capture_failed = False
         self.runs = 0
-        self._tables = [[None] * R for _ in range(G)]     # (table, its length) last written per row
-        # the attention kernel's query tiles of a decode step never change: one token per request
-        ar = torch.arange(R, dtype=torch.int32, device=dev)
-        one = torch.ones(R, dtype=torch.int32, device=dev)
-        for width in range(1, 17):
-            self.ctx._tiles[width] = (ar, ar, one)
+        self.logits: Optional[torch.Tensor] = None
+        self._build()
+
+    def _build(self) -> None:
+        """(Re)lays the static buffers out for the tile widths known by now."""
+        runner = self.runner
+        cm = runner.cache
+        G = len(cm.groups)
+        MB = -(-runner.max_model_len // cm.block_size)
+        self.layout = Layout(self.T, self.R, self.n_out, G, MB,
+                             runner._tile_caps(self.T, self.R, self.max_q_len == 1), self.sampling)
+        self.widths = set(self.layout.tile_caps)
+        self.host = torch.zeros(self.layout.total, dtype=torch.int32, pin_memory=True)
+        self.dev = torch.zeros(self.layout.total, dtype=torch.int32, device=runner.device)
+        self.np = self.host.numpy()
+        self.ctx = self.layout.context(self.dev, cm.block_size, q_lens=[], context_lens=[], slots_host=[],
+                                       max_q_len=self.max_q_len, max_seq_len=self.max_seq_len)
+        self.seen = [[None] * self.R for _ in range(G)]
+        self.out = torch.zeros(max(self.n_out, 1), dtype=torch.int32, device=runner.device)
+        self.out_host = torch.zeros(max(self.n_out, 1), dtype=torch.int32, pin_memory=True)
+        self.graph = None
 
     def _body(self):
-        from ..kernels import ops
-        logits = self.runner.decoder.forward(self.ctx)
-        ops.sample(logits, self.out, self.temperature, self.top_k, self.top_p, self.seeds, self.counters)
+        self.logits = self.runner._forward(self.ctx)
+        if self.sampling and self.n_out:
+            ops.sample(self.logits, self.out[:self.n_out], *self.layout.sampler_args(self.dev))
 
-    def run(self, req_ids, tokens, ctx_lens, params, seeds, counters, capture: bool) -> List[int]:
-        R, G, MB, offs, h = self.R, self.G, self.MB, self.offs, self.np
-        cm = self.runner.cache
-        bs = cm.block_size
-        h[offs[0]:offs[0] + R] = tokens
-        h[offs[1]:offs[1] + R] = ctx_lens
-        h[offs[4]:offs[4] + R] = np.asarray(ctx_lens, dtype=np.int32) + 1
-        slots = [cm.slot(rid) for rid in req_ids]
-        h[offs[5]:offs[5] + R] = slots
-        for g in range(G):
-            bt = h[offs[7 + G + g]:offs[7 + G + g] + R * MB].reshape(R, MB)
-            sm = h[offs[7 + g]:offs[7 + g] + R]
-            seen = self._tables[g]
-            for r, (rid, c) in enumerate(zip(req_ids, ctx_lens)):
-                table = cm.block_table(rid, g)
-                # a row is rewritten only when it belongs to another admission than last time (the
-                # table object is made when a request is admitted) or has changed length (released
-                # blocks turn into -1 without a change of length, but a decode step never reads
-                # them: they lie before the window)
-                last = seen[r]
-                if last is None or last[0] is not table or last[1] != len(table):
-                    bt[r, :len(table)] = np.maximum(np.asarray(table, dtype=np.int32), 0)
-                    seen[r] = (table, len(table))
-                sm[r] = max(table[c // bs], 0) * bs + c % bs
-        s0 = self.s0
-        fview = self.host.view(torch.float32).numpy()
-        fview[offs[s0]:offs[s0] + R] = [p.temperature if p.do_sample else 0.0 for p in params]
-        fview[offs[s0 + 1]:offs[s0 + 1] + R] = [p.top_p for p in params]
-        h[offs[s0 + 2]:offs[s0 + 2] + R] = [p.top_k for p in params]
-        h[offs[s0 + 3]:offs[s0 + 3] + R] = counters
-        self.host.view(torch.int64).numpy()[offs[s0 + 4] // 2:offs[s0 + 4] // 2 + R] = \
-            [s & 0x7FFFFFFFFFFFFFFF for s in seeds]
-        self.ctx.context_lens = list(ctx_lens)
-        self.ctx.slots_host = slots
+    def run(self, rows: Sequence[_Row], samples, n_out: int):
+        runner = self.runner
+        if self.graph is None and self.max_q_len > 1 and self.widths != runner._tile_widths:
+            self._build()                       # a kernel asked for a tile width this layout lacks
+        fill_metadata(self.np, self.layout, rows, runner.cache.block_size, samples, self.seen)
         self.dev.copy_(self.host, non_blocking=True)
-        if not capture or self.runs == 0:
+        if self.graph is not None:
+            self.graph.replay()
+            runner.graph_steps += 1
+        elif self.runs == 0 or self.capture_failed:
+            # eager on the static buffers; the host copies a part may look at are those of this step
+            self.ctx.static = False
+            self.ctx.q_lens = [len(r.tokens) for r in rows] + [0] * (self.R - len(rows))
+            self.ctx.context_lens = [r.context_len for r in rows] + [0] * (self.R - len(rows))
+            self.ctx.slots_host = [r.slot for r in rows] + [0] * (self.R - len(rows))
+            self.ctx._on_new_width = runner._new_width
+            if self.max_q_len > 1:
+                for w in runner._tile_widths - self.widths:
+                    self.ctx._tiles.pop(w, None)
+            known = set(self.ctx._tiles)
             self._body()
-        elif self.graph is None:
-            torch.cuda.synchronize()
-            # Nothing may be finalised while the stream is capturing: the release of pinned buffers,
-            # graphs or events of an engine that is no longer referenced is not allowed then and
-            # ends the process.  So dead objects are collected now, and the collector rests until
-            # the capture is over (torch.cuda.graph does not collect by itself any more).
-            gc.collect()
-            collecting = gc.isenabled()
-            gc.disable()
-            try:
-                self.graph = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(self.graph):
-                    self._body()
-            finally:
-                if collecting:
-                    gc.enable()
-            self.graph.replay()
+            for w in set(self.ctx._tiles) - known:      # built for this step only: not part of the layout
+                del self.ctx._tiles[w]
+            runner.eager_steps += 1
         else:
-            self.graph.replay()
+            self._capture()
+            runner.graph_steps += 1
         self.runs += 1
-        self.out_host.copy_(self.out, non_blocking=True)
-        torch.cuda.current_stream().synchronize()
-        return self.out_host.tolist()
+        toks: List[int] = []
+        if self.sampling and n_out:
+            self.out_host.copy_(self.out, non_blocking=True)
+            torch.cuda.current_stream().synchronize()
+            toks = self.out_host[:n_out].tolist()
+            runner.last_logits = self.logits[:n_out]
+            return None, toks
+        # the logits live in memory the next replay overwrites: the caller gets a copy
+        return self.logits[:n_out].clone(), toks
+
+    def _capture(self) -> None:
+        runner = self.runner
+        torch.cuda.synchronize()
+        # Nothing may be finalised while the stream is capturing: the release of pinned buffers,
+        # graphs or events of an engine that is no longer referenced is not allowed then and
+        # ends the process.  So dead objects are collected now, and the collector rests until
+        # the capture is over (torch.cuda.graph does not collect by itself any more).
+        gc.collect()
+        collecting = gc.isenabled()
+        gc.disable()
+        self.ctx.static = True
+        self.ctx._on_new_width = None
+        graph = torch.cuda.CUDAGraph()
+        if runner._graph_pool is None:
+            runner._graph_pool = torch.cuda.graph_pool_handle()
+        try:
+            # all graphs of a runner share one memory pool: one runs at a time, and what a step
+            # returns has left the pool (tokens on the host, logits copied) before the next replay
+            with torch.cuda.graph(graph, pool=runner._graph_pool):
+                self._body()
+        except StepError:
+            self.capture_failed = True
+            self.ctx.static = False
+            torch.cuda.synchronize()
+            self._body()
+            return
+        finally:
+            if collecting:
+                gc.enable()
+        self.graph = graph
+        graph.replay()

@@ -87,6 +87,75 @@ def _rows_2d(t: torch.Tensor, name: str) -> None:
         _fail(f"{name} must be 2-D with unit inner stride")
 
 
+# ------------------------------------------------------------- step workspace
+class Workspace:
+    """The buffers a step's kernels pass intermediates through, by name: allocated once at the
+    size of the largest step (`max_rows` rows for row-shaped buffers) and used again by every
+    layer and every step, eager or captured.  A buffer is never freed or moved while the workspace
+    lives (a captured graph holds its address); one that turns out too small is retired, not freed.
+
+    `rotate=n` hands out n buffers in turn under one name, for values that are still read while
+    their successor is written (the norm hand-off between consecutive products)."""
+
+    FIRST_ROWS = 4096       # rows the buffers are first made for when steps may be larger still
+
+    def __init__(self, device, max_rows: int):
+        self.device = torch.device(device)
+        self.max_rows = min(int(max_rows), self.FIRST_ROWS)
+        self._bufs: dict = {}
+        self._turn: dict = {}
+        self._retired: list = []
+
+    def take(self, name: str, shape, dtype: torch.dtype, rotate: int = 1) -> torch.Tensor:
+        shape = tuple(int(s) for s in shape)
+        if rotate > 1:
+            i = self._turn.get(name, 0)
+            self._turn[name] = (i + 1) % rotate
+            name = f"{name}#{i}"
+        n = 1
+        for s in shape:
+            n *= s
+        key = (name, dtype)
+        buf = self._bufs.get(key)
+        if buf is None or buf.numel() < n:
+            if buf is not None:
+                self._retired.append(buf)
+            cap = n
+            if len(shape) == 2 and shape[0] <= self.max_rows:
+                cap = self.max_rows * shape[1]
+            buf = self._bufs[key] = torch.empty(cap, dtype=dtype, device=self.device)
+        return buf[:n].view(shape)
+
+    def nbytes(self) -> int:
+        return sum(b.numel() * b.element_size() for b in list(self._bufs.values()) + self._retired)
+
+
+_workspace: Optional[Workspace] = None
+
+
+class use_workspace:
+    """`with use_workspace(ws):` intermediates of the ops and parts inside come from `ws`."""
+
+    def __init__(self, ws: Optional[Workspace]):
+        self.ws = ws
+
+    def __enter__(self):
+        global _workspace
+        self.prev, _workspace = _workspace, self.ws
+        return self.ws
+
+    def __exit__(self, *exc):
+        global _workspace
+        _workspace = self.prev
+
+
+def scratch(name: str, shape, dtype: torch.dtype, device, rotate: int = 1) -> torch.Tensor:
+    """An uninitialised intermediate: from the step's workspace when one is in use, else fresh."""
+    if _workspace is not None and torch.device(device) == _workspace.device:
+        return _workspace.take(name, shape, dtype, rotate)
+    return torch.empty(tuple(shape), dtype=dtype, device=device)
+
+
 # ------------------------------------------------- sizes, checked when parts are built
 MAX_HEAD_DIM = 256      # the general attention kernel keeps a head's row in one wave's registers
 
@@ -241,8 +310,8 @@ def linear_norm(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: torch
     if M > FUSED_MAX_ROWS or N > FUSED_MAX_COLS:
         if not (x.is_contiguous()):
             _fail("norm input must be contiguous")
-        h = torch.empty((M, K), dtype=torch.bfloat16, device=x.device)
-        inv_rms = torch.empty(M, dtype=torch.float32, device=x.device)
+        h = scratch("norm_operand", (M, K), torch.bfloat16, x.device)
+        inv_rms = scratch("norm_row_factor", (M,), torch.float32, x.device)
         _check(_lib().tl_norm_prescale(_ptr(x), _ptr(norm_weight), _ptr(rows), _ptr(h), _ptr(inv_rms), c_int(M),
                                        c_int(K), c_float(eps), c_int(_dt(norm_weight)), _stream()), "norm_prescale")
         return linear(h, w, out, residual, epilogue, row_scale=inv_rms)
@@ -312,7 +381,7 @@ def _linear_split(a, w, out, residual, swiglu, row_scale, sumsq_in, parts, eps, 
     """Partial products into a workspace, then one kernel that adds them and applies the epilogue."""
     M, K = a.shape
     N = w.shape[0]
-    work = torch.empty(splits * M * N, dtype=torch.float32, device=a.device)
+    work = scratch("splitk_partials", (splits * M * N,), torch.float32, a.device)
     emit_w, emit_op, emit_sq = emit if emit is not None else (None, None, None)
     _check(_lib().tl_linear_splitk(
         _ptr(a, 16), _ptr(w, 16), _ptr(out), _ptr(residual), _ptr(row_scale), _ptr(sumsq_in), c_int(parts),

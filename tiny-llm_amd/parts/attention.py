@@ -73,14 +73,14 @@ class Attention(Mixer):
     # --------------------------------------------------------------------- compute
     def forward(self, h, ctx, cache: LayerCache, state, residual, next_norm=None):
         T = residual.shape[0]
-        qkv = torch.empty((T, self.q_size + 2 * self.kv_size), dtype=self.dtype, device=residual.device)
+        qkv = ops.scratch("qkv", (T, self.q_size + 2 * self.kv_size), self.dtype, residual.device)
         if isinstance(h, LazyNorm):
             h.linear(self.w_qkv, qkv)
         else:
             ops.linear(h, self.w_qkv, qkv)
         tables = self.position.rotary_tables()
         cos, sin, rot = tables if tables is not None else (None, None, 0)
-        attn = torch.empty((T, self.q_size), dtype=self.dtype, device=residual.device)
+        attn = ops.scratch("attention_out", (T, self.q_size), self.dtype, residual.device)
         q = qkv[:, :self.q_size]
         flash = ops.flash_attention_supported(self.dtype, self.num_heads, self.num_kv_heads, self.head_dim)
         group = self.num_heads // self.num_kv_heads
@@ -122,8 +122,8 @@ class Attention(Mixer):
         n_splits = max(1, min(-(-key_tiles // ops.flash_waves(self.head_dim)), room, 16))
         if n_splits == 1:
             return 1, None
-        return n_splits, torch.empty(n_splits * T * self.num_heads * (self.head_dim + 2), dtype=torch.float32,
-                                     device=device)
+        return n_splits, ops.scratch("attention_partials", (n_splits * T * self.num_heads * (self.head_dim + 2),),
+                                     torch.float32, device)
 
 
 register_mixer("attention", Attention)

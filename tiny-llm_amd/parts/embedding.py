@@ -28,7 +28,7 @@ class TokenEmbedding(Embedding):
         self.weight = tensors[f"{self.prefix}.weight"].contiguous()
 
     def forward(self, tokens: torch.Tensor, ctx=None) -> torch.Tensor:
-        out = torch.empty((tokens.numel(), self.hidden_size), dtype=torch.float32, device=tokens.device)
+        out = ops.scratch("residual", (tokens.numel(), self.hidden_size), torch.float32, tokens.device)
         return ops.embedding(tokens, self.weight, out)
 
 

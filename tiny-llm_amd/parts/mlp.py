@@ -47,7 +47,7 @@ class SwiGLU(FeedForward):
 
     def forward(self, h, ctx, residual, next_norm=None):
         T, dev = residual.shape[0], residual.device
-        z = torch.empty((T, self.intermediate_size), dtype=self.dtype, device=dev)
+        z = ops.scratch("ffn_gated", (T, self.intermediate_size), self.dtype, dev)
         if isinstance(h, LazyNorm):
             h.linear(self.w_gate_up, z, epilogue="swiglu")
         else:

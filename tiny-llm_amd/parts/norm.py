@@ -71,14 +71,17 @@ class RMSNorm(Norm):
         and can prepare the norm on the way (`ops.linear_handoff`), or None where that does not apply."""
         if not ops.can_hand_off(n_rows, self.hidden_size, inner, self.dtype):
             return None
-        operand = torch.empty((n_rows, self.hidden_size), dtype=torch.bfloat16, device=device)
-        sumsq = torch.empty((n_rows, ops.handoff_parts(n_rows, self.hidden_size, inner)), dtype=torch.float32,
-                            device=device)
+        # still read by the next product while the product after that writes its own: three in turn
+        operand = ops.scratch("handoff_operand", (n_rows, self.hidden_size), torch.bfloat16, device, rotate=3)
+        sumsq = ops.scratch("handoff_sumsq", (n_rows, ops.handoff_parts(n_rows, self.hidden_size, inner)),
+                            torch.float32, device, rotate=3)
         return self.weight, operand, sumsq
 
     def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         n = x.shape[0] if rows is None else rows.numel()
-        out = torch.empty((n, self.hidden_size), dtype=self.dtype, device=x.device)
+        # two in turn: a block's second norm is computed while nothing reads its first any more, but
+        # the final norm's rows must not alias what a consumer still holds
+        out = ops.scratch("normed", (n, self.hidden_size), self.dtype, x.device, rotate=2)
         return ops.rmsnorm(x, self.weight, self.eps, out, rows)
 
 
