@@ -215,7 +215,13 @@ __global__ void random_normal_kernel(T* __restrict__ out, int64_t n, uint64_t ke
     x *= 0x94D049BB133111EBull;
     x ^= x >> 31;
     const float z = table[x >> (64 - table_bits)];
-    out[i] = from_f32<T>(__fadd_rn(__fmul_rn(scale, z), shift));
+    float v;
+    {
+#pragma clang fp contract(off)      // two roundings, as on the host: never one fused multiply-add
+      const float p = scale * z;
+      v = p + shift;
+    }
+    out[i] = from_f32<T>(v);
   }
 }
 

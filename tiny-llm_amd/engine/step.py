@@ -527,6 +527,7 @@ class StepGraph:
         self.out = torch.zeros(max(self.n_out, 1), dtype=torch.int32, device=runner.device)
         self.out_host = torch.zeros(max(self.n_out, 1), dtype=torch.int32, pin_memory=True)
         self.graph = None
+        self._uploaded: Optional[torch.cuda.Event] = None
 
     def _body(self):
         self.logits = self.runner._forward(self.ctx)
@@ -537,8 +538,12 @@ class StepGraph:
         runner = self.runner
         if self.graph is None and self.max_q_len > 1 and self.widths != runner._tile_widths:
             self._build()                       # a kernel asked for a tile width this layout lacks
+        if self._uploaded is not None:
+            self._uploaded.synchronize()        # the last upload has left the pinned buffer
         fill_metadata(self.np, self.layout, rows, runner.cache.block_size, samples, self.seen)
         self.dev.copy_(self.host, non_blocking=True)
+        self._uploaded = torch.cuda.Event()
+        self._uploaded.record()
         if self.graph is not None:
             self.graph.replay()
             runner.graph_steps += 1
