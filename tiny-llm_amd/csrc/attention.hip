@@ -15,6 +15,8 @@
 // All arithmetic is float32 whatever the cache's element type.  It takes any head
 // size up to 256, any page size, any grouping of query heads.
 #include "common.h"
+#include "no_alloc.h"
+#include <mutex>
 
 namespace {
 
@@ -954,12 +956,12 @@ int tl_flash_waves(int hd) { return flash_waves(hd); }
 // bfloat16 only.  Tiles: tile_req / tile_tok0 / tile_ntok [n_tiles] describe groups of at most
 // 16 / (nq / nkv) consecutive tokens of one request; all three null: tile i is token i of request i.  With n_splits > 1, part_o
 // [n_splits, n_tokens, nq, hd] and part_ml [n_splits, n_tokens, nq, 2] (float32) are scratch.
-int tl_flash_attention(const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
-                       const int32_t* block_tables, int max_blocks, const int32_t* tile_req,
-                       const int32_t* tile_tok0, const int32_t* tile_ntok, const int32_t* positions, void* out,
-                       int64_t out_stride, float* part_o, float* part_ml, int n_tiles, int n_tokens, int nq,
-                       int nkv, int hd, int block_size, float scale, int window, int n_splits,
-                       const float* rope_cos, const float* rope_sin, int fuse_store, hipStream_t stream) {
+static int flash_attention_any(const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
+                               const int32_t* block_tables, int max_blocks, const int32_t* tile_req,
+                               const int32_t* tile_tok0, const int32_t* tile_ntok, const int32_t* positions, void* out,
+                               int64_t out_stride, float* part_o, float* part_ml, int n_tiles, int n_tokens, int nq,
+                               int nkv, int hd, int block_size, float scale, int window, int n_splits,
+                               const float* rope_cos, const float* rope_sin, int fuse_store, hipStream_t stream) {
   if (n_tiles <= 0 || n_tokens <= 0) return TL_OK;
   if (nq <= 0 || nkv <= 0 || nq % nkv || nq / nkv > 16 || hd <= 0 || hd % 16 || hd > 128 || block_size <= 0 ||
       max_blocks <= 0 || window < 0 || n_splits < 1 || nkv > 65535 || n_splits > 65535 || q_stride % 8)
@@ -995,6 +997,70 @@ int tl_flash_attention(const void* q, int64_t q_stride, const void* k_cache, con
   else if (n_splits > 1) TL_COMBINE(2);
 #undef TL_COMBINE
   return tl_launch_status();
+}
+
+int tl_flash_attention(const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
+                       const int32_t* block_tables, int max_blocks, const int32_t* tile_req,
+                       const int32_t* tile_tok0, const int32_t* tile_ntok, const int32_t* positions, void* out,
+                       int64_t out_stride, float* part_o, float* part_ml, int n_tiles, int n_tokens, int nq,
+                       int nkv, int hd, int block_size, float scale, int window, int n_splits,
+                       const float* rope_cos, const float* rope_sin, int fuse_store, hipStream_t stream) {
+  return flash_attention_any(q, q_stride, k_cache, v_cache, block_tables, max_blocks, tile_req, tile_tok0, tile_ntok,
+                             positions, out, out_stride, part_o, part_ml, n_tiles, n_tokens, nq, nkv, hd, block_size,
+                             scale, window, n_splits, rope_cos, rope_sin, fuse_store, stream);
+}
+
+// ------------------------------------------------ the entry point that allocates nothing
+// The partial results of split attention live in a device array that is part of the library
+// itself.  Each GPU holds its own copy at its own address, which the host learns once per device
+// with hipGetSymbolAddress; kernels receive that address like any other buffer.
+static __device__ __align__(256) float scratch[TL_STATIC_SCRATCH_FLOATS];
+
+constexpr int kMaxDevices = 64;
+static float* g_scratch_of_device[kMaxDevices] = {};
+static std::mutex g_scratch_mutex;
+
+// The address of the current device's copy of `scratch` (looked up at the first call on that device).
+static int static_scratch_of_current_device(float** ptr) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return TL_ERR_LAUNCH;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_of_device[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return TL_ERR_LAUNCH;
+    g_scratch_of_device[dev] = (float*)p;
+  }
+  *ptr = g_scratch_of_device[dev];
+  return TL_OK;
+}
+
+int64_t tl_static_scratch_floats(void) { return (int64_t)TL_STATIC_SCRATCH_FLOATS; }
+
+int tl_flash_attention_static(const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
+                              const int32_t* block_tables, int max_blocks, const int32_t* tile_req,
+                              const int32_t* tile_tok0, const int32_t* tile_ntok, const int32_t* positions,
+                              void* out, int64_t out_stride, int n_tiles, int n_tokens, int nq, int nkv, int hd,
+                              int block_size, float scale, int window, int n_splits, const float* rope_cos,
+                              const float* rope_sin, int fuse_store, hipStream_t stream) {
+  if (n_tiles <= 0 || n_tokens <= 0) return TL_OK;
+  if (n_splits < 1 || nq <= 0 || hd <= 0) return TL_ERR_ARG;
+  float* part_o = nullptr;
+  float* part_ml = nullptr;
+  if (n_splits > 1) {
+    const int64_t rows = (int64_t)n_splits * n_tokens * nq;
+    if (rows * (hd + 2) > (int64_t)TL_STATIC_SCRATCH_FLOATS) return TL_ERR_SCRATCH;
+    float* base = nullptr;
+    const int rc = static_scratch_of_current_device(&base);
+    if (rc != TL_OK) return rc;
+    // Every partial that the merge reads is written by this very call (a workgroup without keys
+    // writes a neutral partial), so nothing has to start at zero and what an earlier, larger call
+    // left behind is never read.
+    part_o = base;
+    part_ml = base + rows * hd;
+  }
+  return flash_attention_any(q, q_stride, k_cache, v_cache, block_tables, max_blocks, tile_req, tile_tok0, tile_ntok,
+                             positions, out, out_stride, part_o, part_ml, n_tiles, n_tokens, nq, nkv, hd, block_size,
+                             scale, window, n_splits, rope_cos, rope_sin, fuse_store, stream);
 }
 
 }  // extern "C"

@@ -563,7 +563,7 @@ def flash_attention_supported(dtype: torch.dtype, num_heads: int, num_kv_heads: 
 def flash_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                     tiles, positions: torch.Tensor, out: torch.Tensor, num_heads: int, num_kv_heads: int,
                     head_dim: int, scale: float, window: int = 0, n_splits: int = 1,
-                    scratch: Optional[torch.Tensor] = None, fused_rope=None) -> torch.Tensor:
+                    scratch: Optional[torch.Tensor] = None, fused_rope=None, static_scratch: bool = False) -> torch.Tensor:
     """The same function as `paged_attention` on the matrix cores (bfloat16).  `tiles` =
     (tile_req, tile_tok0, tile_ntok): groups of at most 16 // (heads / kv_heads) consecutive
     tokens of one request; None for a decode step, where row i is the one new token of request i
@@ -572,7 +572,10 @@ def flash_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
 
     fused_rope=(cos, sin), for steps of ONE new token per request: `q` is the first slice of the
     unrotated rows [q heads | k heads | v heads]; the kernel rotates q and the new key over the
-    whole head and writes the new key and value into the caches itself (no `rope_store` before)."""
+    whole head and writes the new key and value into the caches itself (no `rope_store` before).
+
+    static_scratch=True: the partial results go to the device array the library holds itself
+    (`tl_flash_attention_static`: no `scratch` is taken; sizes beyond that array are refused)."""
     tile_req, tile_tok0, tile_ntok = tiles if tiles is not None else (None, None, None)
     _dev(q, k_cache, v_cache, block_tables, tile_req, tile_tok0, tile_ntok, positions, out, scratch)
     _rows_2d(q, "q")
@@ -605,7 +608,7 @@ def flash_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     if not (q.stride(0) % 8 == 0):
         _fail("q rows must be 16-byte aligned")
     part_o = part_ml = None
-    if n_splits > 1:
+    if n_splits > 1 and not static_scratch:
         need = n_splits * T * num_heads * (head_dim + 2)
         if not (scratch is not None and scratch.dtype == torch.float32 and scratch.is_contiguous()
                 and scratch.numel() >= need):
@@ -624,6 +627,18 @@ def flash_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         # q must be the head of a [q | k | v] row
         if not (q.stride(0) >= (num_heads + 2 * num_kv_heads) * head_dim):
             _fail("fused mode needs q inside its qkv rows")
+    if static_scratch:
+        code = _lib().tl_flash_attention_static(
+            _ptr(q, 16), c_int64(q.stride(0)), _ptr(k_cache, 16), _ptr(v_cache, 16), _ptr(block_tables),
+            c_int(block_tables.shape[1]), _ptr(tile_req), _ptr(tile_tok0), _ptr(tile_ntok), _ptr(positions),
+            _ptr(out, 8), c_int64(out.stride(0)), c_int(n_tiles), c_int(T), c_int(num_heads), c_int(num_kv_heads),
+            c_int(head_dim), c_int(k_cache.shape[2]), c_float(scale), c_int(window), c_int(n_splits), _ptr(cos),
+            _ptr(sin), c_int(1 if fused_rope is not None else 0), _stream())
+        if code == 3:
+            _fail(f"split attention over the library's static scratch: {n_splits} splits x {T} tokens x {num_heads} "
+                  f"heads x {head_dim + 2} floats exceed its {STATIC_SCRATCH_FLOATS} floats")
+        _check(code, "flash_attention_static")
+        return out
     _check(_lib().tl_flash_attention(
         _ptr(q, 16), c_int64(q.stride(0)), _ptr(k_cache, 16), _ptr(v_cache, 16), _ptr(block_tables),
         c_int(block_tables.shape[1]), _ptr(tile_req), _ptr(tile_tok0), _ptr(tile_ntok), _ptr(positions),
@@ -632,6 +647,9 @@ def flash_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         c_int(window), c_int(n_splits), _ptr(cos), _ptr(sin), c_int(1 if fused_rope is not None else 0),
         _stream()), "flash_attention")
     return out
+
+
+STATIC_SCRATCH_FLOATS = 1 << 20     # capacity of the library's own scratch array (csrc/no_alloc.h)
 
 
 def flash_waves(head_dim: int) -> int:
