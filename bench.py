@@ -19,7 +19,7 @@ sys.path.insert(0, ROOT)
 HBM_GBS = 8000.0
 PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
 
-# BASELINE.json configs[2]
+# the TinyLlama 1.1B shape
 TINYLLAMA = {
     "architectures": ["LlamaForCausalLM"], "model_type": "llama", "num_hidden_layers": 22, "hidden_size": 2048,
     "num_attention_heads": 32, "num_key_value_heads": 4, "intermediate_size": 5632, "vocab_size": 32000,

@@ -66,23 +66,47 @@ def _hipcc() -> str:
                              "the engine has no path without its HIP kernels")
 
 
-def _writable_dir() -> str:
-    intree = os.path.join(_PKG, "_lib")
+def _intree_dir() -> str:
+    return os.path.join(_PKG, "_lib")
+
+
+def _intree_writable() -> bool:
+    intree = _intree_dir()
     try:
         os.makedirs(intree, exist_ok=True)
         probe = os.path.join(intree, f".probe-{os.getpid()}")
         with open(probe, "w"):
             pass
         os.remove(probe)
-        return intree
+        return True
     except OSError:
-        d = os.path.join(tempfile.gettempdir(), f"tinyllm-amd-{os.getuid()}")
-        os.makedirs(d, exist_ok=True)
-        return d
+        return False
+
+
+def _private_temp_dir() -> str:
+    """A build folder of this user's own under the system's temporary directory: made with mode
+    0700, and refused unless it belongs to this user and nobody else can write to it (another
+    user could otherwise plant a library there that this process would load)."""
+    d = os.path.join(tempfile.gettempdir(), f"tinyllm-amd-{os.getuid()}")
+    try:
+        os.mkdir(d, 0o700)
+    except FileExistsError:
+        pass
+    st = os.lstat(d)
+    import stat as _stat
+    if not _stat.S_ISDIR(st.st_mode) or st.st_uid != os.getuid() or (st.st_mode & 0o022):
+        return tempfile.mkdtemp(prefix="tinyllm-amd-")
+    return d
+
+
+def _writable_dir() -> str:
+    return _intree_dir() if _intree_writable() else _private_temp_dir()
 
 
 def _candidates() -> List[str]:
-    return [os.path.join(_PKG, "_lib"), os.path.join(tempfile.gettempdir(), f"tinyllm-amd-{os.getuid()}")]
+    """Where a built library may lie: in the tree; the private temporary folder only when the tree
+    cannot be written to."""
+    return [_intree_dir()] if _intree_writable() else [_intree_dir(), _private_temp_dir()]
 
 
 def _is_current(lib_path: str) -> bool:
@@ -103,7 +127,8 @@ def build(force: bool = True, verbose: bool = True) -> str:
     if not force and _is_current(lib_path):
         return lib_path
     hipcc = _hipcc()
-    obj_dir = os.path.join(out_dir, "obj")
+    # objects of this build alone: two processes that build at once never link each other's halves
+    obj_dir = os.path.join(out_dir, f"obj.{os.getpid()}")
     os.makedirs(obj_dir, exist_ok=True)
     srcs = sources()
     env = dict(os.environ)
@@ -142,9 +167,13 @@ def build(force: bool = True, verbose: bool = True) -> str:
     p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, env=env, text=True)
     if p.returncode != 0:
         raise KernelLibraryError(f"linking {lib_path} failed:\n{p.stderr[-4000:]}")
-    os.replace(tmp, lib_path)
-    with open(lib_path + ".digest", "w") as f:
-        f.write(_source_digest())
+    import fcntl
+    with open(os.path.join(out_dir, ".lock"), "w") as lock:      # library and stamp change together
+        fcntl.flock(lock, fcntl.LOCK_EX)
+        os.replace(tmp, lib_path)
+        with open(lib_path + ".digest", "w") as f:
+            f.write(_source_digest())
+    shutil.rmtree(obj_dir, ignore_errors=True)
     say(f"built in {time.time() - t0:.0f}s")
     return lib_path
 
