@@ -481,6 +481,247 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
   }
 }
 
+// ====================================================== float32 on the matrix cores
+// attention_f32_kernel: true float32 (v_mfma_f32_16x16x4_f32 for both products, float32 softmax)
+// for every step, prompt portions and decoded tokens alike.  The result of a query row does not
+// depend, to the bit, on what else is in the batch, on how the tokens were cut into steps or on
+// how the keys are spread over workgroups, because the terms are always combined in ONE tree:
+//   * keys in tiles of 64 at absolute positions 64 t .. 64 t + 63; a tile gives (m, l, O) from scratch:
+//     m the largest score, l = sum exp2(s - m), O = sum exp2(s - m) v (scores in units of log2 e);
+//   * the tiles of a chunk of 8 (512 keys) are merged in ascending order, starting from "nothing";
+//   * the chunks are merged in ascending order, starting from "nothing".
+// `merge_f32` is the one merge; a tile or chunk that holds no visible key merges as an exact no-op,
+// so skipping it changes nothing.  A workgroup (four waves) owns 16 query rows of one request and
+// kv head (tokens times the heads of the group, as in the bfloat16 kernels) and either walks all
+// chunks itself (gridDim.z == 1) or owns chunk blockIdx.z and leaves its (m, l, O) in `part` for
+// attention_f32_combine_kernel.  Its waves take the tiles of a chunk in turn; a wave reads keys
+// straight into the first product's operands and stages values through an LDS area of its own.
+constexpr int A32_WAVES = 4, A32_THREADS = A32_WAVES * TL_WAVE, A32_CHUNK = 8;
+constexpr int A32_VW = 64, A32_VS = A32_VW + 4;      // value columns staged at a time, row stride in LDS
+
+__device__ __forceinline__ void merge_f32(float& M, float& L, float m, float l, float& wa, float& wb) {
+  const float Mn = fmaxf(M, m);
+  wa = __builtin_amdgcn_exp2f(M - Mn);
+  wb = __builtin_amdgcn_exp2f(m - Mn);
+  const float lb = l * wb;
+  L = __builtin_fmaf(L, wa, lb);
+  M = Mn;
+}
+__device__ __forceinline__ float merge_f32_value(float O, float o, float wa, float wb) {
+  const float ob = o * wb;
+  return __builtin_fmaf(O, wa, ob);
+}
+
+template <int HDT>
+__global__ __launch_bounds__(A32_THREADS) void attention_f32_kernel(
+    const float* __restrict__ q, int64_t q_stride, const float* __restrict__ k_cache,
+    const float* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int max_blocks,
+    const int32_t* __restrict__ tile_req, const int32_t* __restrict__ tile_tok0,
+    const int32_t* __restrict__ tile_ntok, const int32_t* __restrict__ positions, float* __restrict__ out,
+    int64_t out_stride, float* __restrict__ part, int nq, int nkv, int block_size, float scale, int window,
+    int n_tokens) {
+  constexpr int HD = HDT * 16;
+  constexpr int PS = HD + 4;                       // row stride of a tile's O in LDS
+  constexpr int EPT = 16 * HD / A32_THREADS;       // output elements a thread merges (= HDT)
+  extern __shared__ __attribute__((aligned(16))) float smem32[];
+  float* Vl_all = smem32;                                          // [waves][64][A32_VS]
+  float* Po = smem32 + A32_WAVES * FA_KT * A32_VS;                 // [8 tiles][16 rows][PS]
+  float* Pml = Po + A32_CHUNK * 16 * PS;                           // [8 tiles][16 rows][2]
+
+  const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
+  const int l16 = lane % 16, kk = lane / 16;
+  const int tile = blockIdx.x, kvh = blockIdx.y;
+  const int G = nq / nkv, TW = 16 / G;
+  const int req = tile_req ? tile_req[tile] : tile, tok0 = tile_req ? tile_tok0[tile] : tile;
+  const int ntok = tile_req ? tile_ntok[tile] : 1;
+  if (ntok <= 0) return;                           // a padding tile (whole workgroup)
+  const int32_t* bt = block_tables + (int64_t)req * max_blocks;
+  float* Vl = Vl_all + wave * FA_KT * A32_VS;
+
+  // this lane's query row (the second operand's column l16)
+  const int tok_local = l16 / G, hh = l16 % G;
+  const bool row_valid = tok_local < TW && tok_local < ntok;
+  const int tok = tok0 + (row_valid ? tok_local : 0);
+  const int pos = row_valid ? positions[tok] : -1;
+  const int row_lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
+  const int hi = row_max_i32(pos), lo = row_min_i32(row_valid ? row_lo : 0x7fffffff);
+  const int kv_end = hi + 1, kv_begin = lo;
+  const int first_tile = kv_begin / FA_KT, last_tile = (kv_end + FA_KT - 1) / FA_KT;
+  const int c_first = gridDim.z > 1 ? (int)blockIdx.z : first_tile / A32_CHUNK;
+  const int c_last = gridDim.z > 1 ? (int)blockIdx.z + 1 : (last_tile + A32_CHUNK - 1) / A32_CHUNK;
+
+  f32x4 qf[HDT];
+  {
+    const float* qrow = q + (int64_t)tok * q_stride + (int64_t)(kvh * G + hh) * HD;
+#pragma unroll
+    for (int g4 = 0; g4 < HDT; ++g4)
+      qf[g4] = row_valid ? *(const f32x4*)(qrow + g4 * 16 + kk * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const float c_log2 = scale * 1.44269504088896341f;
+
+  // the elements this thread merges: e = tid + 256 u -> (row e / HD, dim e % HD)
+  float Mrun[EPT], Lrun[EPT], Orun[EPT];
+#pragma unroll
+  for (int u = 0; u < EPT; ++u) {
+    Mrun[u] = kNegBig;
+    Lrun[u] = 0.f;
+    Orun[u] = 0.f;
+  }
+
+  for (int c = c_first; c < c_last; ++c) {
+    const int t_lo = max(c * A32_CHUNK, first_tile), t_hi = min((c + 1) * A32_CHUNK, last_tile);
+    for (int t = t_lo + wave; t < t_hi; t += A32_WAVES) {
+      const int kb = t * FA_KT;
+      // ---- scores S^T = K Q^T: lane (l16, kk) of subtile st holds keys kb + 16 st + 4 kk + r of row l16
+      f32x4 sc[4];
+#pragma unroll
+      for (int st = 0; st < 4; ++st) {
+        const int key = kb + st * 16 + l16;
+        const bool in_range = key < kv_end;
+        const int jb = min(key / block_size, max_blocks - 1);
+        const int64_t blk = max(bt[in_range ? jb : 0], 0);
+        const float* krow = k_cache + ((blk * nkv + kvh) * block_size + (key - (key / block_size) * block_size)) * HD;
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int g4 = 0; g4 < HDT; ++g4) {
+          const f32x4 kf = in_range ? *(const f32x4*)(krow + g4 * 16 + kk * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[e], qf[g4][e], acc, 0, 0, 0);
+        }
+        sc[st] = acc;
+      }
+      // ---- the tile's softmax from scratch
+      float m_t = -INFINITY;
+#pragma unroll
+      for (int st = 0; st < 4; ++st)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int key = kb + st * 16 + kk * 4 + r;
+          const bool vis = row_valid && key <= pos && key >= row_lo;
+          sc[st][r] = vis ? sc[st][r] * c_log2 : -INFINITY;
+          m_t = fmaxf(m_t, sc[st][r]);
+        }
+      m_t = fmaxf(max_over_rows(m_t), kNegBig);
+      float l_t = 0.f;
+#pragma unroll
+      for (int st = 0; st < 4; ++st)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          sc[st][r] = __builtin_amdgcn_exp2f(sc[st][r] - m_t);
+          l_t += sc[st][r];
+        }
+      l_t = sum_over_rows(l_t);
+      // ---- O^T = V^T P^T, the values staged 64 columns at a time (lane = key row)
+      f32x4 o[HDT];
+#pragma unroll
+      for (int dt = 0; dt < HDT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      {
+        const int key = kb + lane;
+        const bool in_range = key >= kv_begin && key < kv_end;
+        const int jb = min(key / block_size, max_blocks - 1);
+        const int64_t blk = max(bt[in_range ? jb : 0], 0);
+        const float* vrow = v_cache + ((blk * nkv + kvh) * block_size + (key - (key / block_size) * block_size)) * HD;
+#pragma unroll
+        for (int dh = 0; dh < (HD + A32_VW - 1) / A32_VW; ++dh) {
+          constexpr int full = A32_VW / 4;
+          const int chunks = min(full, (HD - dh * A32_VW) / 4);
+          if (dh > 0) {       // this wave's reads of the columns staged before are done
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+          }
+#pragma unroll
+          for (int ch = 0; ch < full; ++ch)
+            if (ch < chunks) {
+              // rows outside the request's keys are zeroed: stale pages may hold anything, and 0 * NaN is NaN
+              const f32x4 v = in_range ? *(const f32x4*)(vrow + dh * A32_VW + ch * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
+              *(f32x4*)(&Vl[lane * A32_VS + ch * 4]) = v;
+            }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+          for (int dl = 0; dl < A32_VW / 16; ++dl) {
+            const int dt = dh * (A32_VW / 16) + dl;
+            if (dt < HDT) {
+#pragma unroll
+              for (int st = 0; st < 4; ++st)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                  const float vf = Vl[(st * 16 + kk * 4 + r) * A32_VS + dl * 16 + l16];
+                  o[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf, sc[st][r], o[dt], 0, 0, 0);
+                }
+            }
+          }
+        }
+        // the area is free for the wave's next tile
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      }
+      // ---- the tile's (m, l, O) to its slot: lane (l16, kk) holds row l16, dims 16 dt + 4 kk + r
+      const int slot = t - c * A32_CHUNK;
+#pragma unroll
+      for (int dt = 0; dt < HDT; ++dt) *(f32x4*)(&Po[(slot * 16 + l16) * PS + dt * 16 + kk * 4]) = o[dt];
+      if (kk == 0) {
+        Pml[(slot * 16 + l16) * 2] = m_t;
+        Pml[(slot * 16 + l16) * 2 + 1] = l_t;
+      }
+    }
+    __syncthreads();
+    // ---- merge the chunk's tiles in ascending order, then the chunk into the running result
+#pragma unroll
+    for (int u = 0; u < EPT; ++u) {
+      const int e = tid + A32_THREADS * u, row = e / HD, d = e % HD;
+      float Mc = kNegBig, Lc = 0.f, Oc = 0.f, wa, wb;
+      for (int t = t_lo; t < t_hi; ++t) {
+        const int slot = t - c * A32_CHUNK;
+        merge_f32(Mc, Lc, Pml[(slot * 16 + row) * 2], Pml[(slot * 16 + row) * 2 + 1], wa, wb);
+        Oc = merge_f32_value(Oc, Po[(slot * 16 + row) * PS + d], wa, wb);
+      }
+      merge_f32(Mrun[u], Lrun[u], Mc, Lc, wa, wb);
+      Orun[u] = merge_f32_value(Orun[u], Oc, wa, wb);
+    }
+    __syncthreads();      // the slots are written again in the next chunk
+  }
+
+#pragma unroll
+  for (int u = 0; u < EPT; ++u) {
+    const int e = tid + A32_THREADS * u, row = e / HD, d = e % HD;
+    const int t_local = row / G, h_local = row % G;
+    if (t_local >= TW || t_local >= ntok) continue;
+    const int t = tok0 + t_local, h = kvh * G + h_local;
+    if (gridDim.z == 1) {
+      out[(int64_t)t * out_stride + (int64_t)h * HD + d] = Lrun[u] > 0.f ? Orun[u] / Lrun[u] : 0.f;
+    } else {
+      float* pr = part + (((int64_t)blockIdx.z * n_tokens + t) * nq + h) * (HD + 2);
+      pr[d] = Orun[u];
+      if (d == 0) {
+        pr[HD] = Mrun[u];
+        pr[HD + 1] = Lrun[u];
+      }
+    }
+  }
+}
+
+// Merges the chunks that attention_f32_kernel left in `part` [chunks][tokens][heads][hd + 2], in
+// ascending order from "nothing": the very sequence of operations of a workgroup that walks the
+// chunks itself.  One wave per (token, head).
+__global__ __launch_bounds__(TL_WAVE) void attention_f32_combine_kernel(const float* __restrict__ part,
+                                                                       float* __restrict__ out, int64_t out_stride,
+                                                                       int n_tokens, int nq, int hd, int n_chunks) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  for (int d = lane; d < hd; d += TL_WAVE) {
+    float M = kNegBig, L = 0.f, O = 0.f, wa, wb;
+    for (int c = 0; c < n_chunks; ++c) {
+      const float* pr = part + (((int64_t)c * n_tokens + t) * nq + h) * (hd + 2);
+      merge_f32(M, L, pr[hd], pr[hd + 1], wa, wb);
+      O = merge_f32_value(O, pr[d], wa, wb);
+    }
+    out[(int64_t)t * out_stride + (int64_t)h * hd + d] = L > 0.f ? O / L : 0.f;
+  }
+}
+
 // flash_prefill_bf16_kernel: the same mathematics arranged for prompt portions.  A workgroup
 // owns up to 8 query tiles (one per wave, 128 rows: for 8 heads per kv head that is 16 tokens) of
 // consecutive tokens of one request, and all eight waves work on the SAME 64-key tile, staged and
@@ -916,6 +1157,48 @@ int tl_paged_attention(const void* q, int64_t q_stride, const void* k_cache, con
                        positions, (bf16_t*)out, out_stride, nq, nkv, hd, block_size, scale, window);
   else
     return TL_ERR_ARG;
+  return tl_launch_status();
+}
+
+// float32 on the matrix cores, for every kind of step.  Tiles as tl_flash_attention (null: tile i
+// is token i of request i).  n_chunks == 1: a workgroup walks all keys of its tile; n_chunks > 1: it
+// must be at least ceil(longest context / 512), chunk c goes to workgroup (., ., c) and `part`
+// [n_chunks, n_tokens, nq, hd + 2] floats is scratch.  Either way the same bits.
+int tl_attention_f32(const float* q, int64_t q_stride, const float* k_cache, const float* v_cache,
+                     const int32_t* block_tables, int max_blocks, const int32_t* tile_req,
+                     const int32_t* tile_tok0, const int32_t* tile_ntok, const int32_t* positions, float* out,
+                     int64_t out_stride, float* part, int n_tiles, int n_tokens, int nq, int nkv, int hd,
+                     int block_size, float scale, int window, int n_chunks, hipStream_t stream) {
+  if (n_tiles <= 0 || n_tokens <= 0) return TL_OK;
+  if (nq <= 0 || nkv <= 0 || nq % nkv || nq / nkv > 16 || hd <= 0 || hd % 16 || hd > 128 || block_size <= 0 ||
+      max_blocks <= 0 || window < 0 || n_chunks < 1 || nkv > 65535 || n_chunks > 65535 || q_stride % 4 ||
+      out_stride % 1)
+    return TL_ERR_ARG;
+  if (n_chunks > 1 && !part) return TL_ERR_ARG;
+  if (!tile_req && (tile_tok0 || tile_ntok || n_tiles != n_tokens)) return TL_ERR_ARG;
+  if (tile_req && (!tile_tok0 || !tile_ntok)) return TL_ERR_ARG;
+  const size_t smem = (size_t)(A32_WAVES * FA_KT * A32_VS + A32_CHUNK * 16 * (hd + 4) + A32_CHUNK * 16 * 2) * sizeof(float);
+#define TL_A32_CASE(HDT)                                                                                          \
+  case HDT: {                                                                                                     \
+    static bool configured = false;                                                                               \
+    if (!configured) {                                                                                            \
+      if (hipFuncSetAttribute((const void*)attention_f32_kernel<HDT>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                              (int)smem) != hipSuccess)                                                           \
+        return TL_ERR_LAUNCH;                                                                                     \
+      configured = true;                                                                                          \
+    }                                                                                                             \
+    hipLaunchKernelGGL(attention_f32_kernel<HDT>, dim3(n_tiles, nkv, n_chunks), dim3(A32_THREADS), smem, stream,  \
+                       q, q_stride, k_cache, v_cache, block_tables, max_blocks, tile_req, tile_tok0, tile_ntok,   \
+                       positions, out, out_stride, part, nq, nkv, block_size, scale, window, n_tokens);           \
+  } break;
+  switch (hd / 16) {
+    TL_A32_CASE(1) TL_A32_CASE(2) TL_A32_CASE(3) TL_A32_CASE(4)
+    TL_A32_CASE(5) TL_A32_CASE(6) TL_A32_CASE(7) TL_A32_CASE(8)
+  }
+#undef TL_A32_CASE
+  if (n_chunks > 1)
+    hipLaunchKernelGGL(attention_f32_combine_kernel, dim3(n_tokens, nq), dim3(TL_WAVE), 0, stream, part, out,
+                       out_stride, n_tokens, nq, hd, n_chunks);
   return tl_launch_status();
 }
 

@@ -18,8 +18,17 @@
 namespace {
 
 // ===================================================================== float32
-constexpr int F_BM = 64, F_BN = 64, F_BK = 16, F_THREADS = 256;
-constexpr int F_KBLOCK = 256;     // the k block of the order of addition (a multiple of F_BK)
+// True float32 on the matrix cores: v_mfma_f32_16x16x4_f32 takes float32 operands and keeps float32
+// sums (no reduced-precision mode).  Both kernels below add the terms of an output element in ONE
+// order, so that a row gives the same bits alone and in any batch, by either kernel:
+//   * k runs in blocks of 256, each block summed from zero, the block sums added in ascending order;
+//   * inside a block, groups of 16 k in ascending order; a group is four matrix instructions, the
+//     e-th of which takes k = 16 group + {0, 4, 8, 12} + e (a lane holds four consecutive k of its row,
+//     one for each of the four instructions);
+//   * operands beyond K are zero.
+constexpr int F_KBLOCK = 256;     // the k block of the order of addition
+constexpr int F_BM = 128, F_BN = 128, F_BK = 16, F_THREADS = 256;
+constexpr int F_LD = F_BK + 4;    // LDS row stride in floats (80 bytes: 16-byte aligned rows)
 
 // silu(g) * u of an interleaved gate|up pair of output columns, as the reference computes it
 // (tiny_llm/ops/cuda/silu.cu:10, arithmetic.cu:13), from the float32 accumulators.
@@ -31,91 +40,125 @@ __device__ __forceinline__ float swiglu_pair_fast(float g, float u) {
   return g * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-1.44269504088896341f * g)) * u;
 }
 
-template <typename TO, bool SWIGLU>
+// Four consecutive k of one row, zero beyond K; VEC: 16-byte aligned rows and K a multiple of 4.
+template <bool VEC>
+__device__ __forceinline__ f32x4 load_k4(const float* __restrict__ row, int k, int K) {
+  f32x4 v = {0.f, 0.f, 0.f, 0.f};
+  if constexpr (VEC) {
+    if (k < K) v = *(const f32x4*)(row + k);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (k + e < K) v[e] = row[k + e];
+  }
+  return v;
+}
+
+// Tiles of 128 rows x 128 columns, four waves of 64 x 64 (4 x 4 matrix tiles of 16 x 16), k in
+// steps of 16 through double-buffered LDS.  The matrix instruction's rows are the output COLUMNS
+// (weights are its first operand), so a lane ends up with four consecutive columns of one row.
+template <bool SWIGLU, bool VEC>
 __global__ __launch_bounds__(F_THREADS) void gemm_f32_kernel(const float* __restrict__ a,
                                                              const float* __restrict__ w,
-                                                             TO* __restrict__ out,
+                                                             float* __restrict__ out,
                                                              const float* __restrict__ residual, int M,
                                                              int N, int K, int64_t lda, int64_t ldo) {
-  __shared__ float As[F_BK][F_BM + 4];
-  __shared__ float Ws[F_BK][F_BN + 4];
-  const int tid = threadIdx.x;
+  __shared__ __attribute__((aligned(16))) float As[2][F_BM * F_LD];
+  __shared__ __attribute__((aligned(16))) float Ws[2][F_BN * F_LD];
+  const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
+  const int wm = wave / 2, wn = wave % 2;
   const int m0 = blockIdx.y * F_BM, n0 = blockIdx.x * F_BN;
-  const int ty = tid / 16, tx = tid % 16;
-  float acc[4][4] = {}, tot[4][4] = {};
-  // each thread stages 4 consecutive k of one row of each operand
-  const int lr = tid / 4, lk = (tid % 4) * 4;
-  for (int k0 = 0; k0 < K; k0 += F_BK) {
-    float av[4], wv[4];
+  const int l16 = lane % 16, kk = lane / 16;
+  // staging: thread = (row tid / 2, k half tid % 2), two groups of four k each
+  const int sr = tid / 2, sk = (tid % 2) * 8;
+  const float* arow = a + (int64_t)min(m0 + sr, M - 1) * lda;
+  const float* wrow = w + (int64_t)min(n0 + sr, N - 1) * K;
+  f32x4 acc[4][4], tot[4][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int k = k0 + lk + i;
-      av[i] = (m0 + lr < M && k < K) ? a[(int64_t)(m0 + lr) * lda + k] : 0.f;
-      wv[i] = (n0 + lr < N && k < K) ? w[(int64_t)(n0 + lr) * K + k] : 0.f;
+  for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+      acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      tot[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
-    __syncthreads();
+  f32x4 ga[2], gw[2];
+  auto fetch = [&](int k0) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      As[lk + i][lr] = av[i];
-      Ws[lk + i][lr] = wv[i];
+    for (int h = 0; h < 2; ++h) {
+      ga[h] = load_k4<VEC>(arow, k0 + sk + 4 * h, K);
+      gw[h] = load_k4<VEC>(wrow, k0 + sk + 4 * h, K);
     }
-    __syncthreads();
+  };
+  auto stage = [&](int buf) {
 #pragma unroll
-    for (int k = 0; k < F_BK; ++k) {
-      float ar[4], wr[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        ar[i] = As[k][ty * 4 + i];
-        wr[i] = Ws[k][tx * 4 + i];
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(ar[i], wr[j], acc[i][j]);
+    for (int h = 0; h < 2; ++h) {
+      *(f32x4*)(&As[buf][sr * F_LD + sk + 4 * h]) = ga[h];
+      *(f32x4*)(&Ws[buf][sr * F_LD + sk + 4 * h]) = gw[h];
     }
-    if ((k0 + F_BK) % F_KBLOCK == 0 || k0 + F_BK >= K) {     // a block of the order of addition ends
+  };
+  fetch(0);
+  stage(0);
+  __syncthreads();
+  const int steps = (K + F_BK - 1) / F_BK;
+  for (int s = 0; s < steps; ++s) {
+    const int buf = s & 1;
+    if (s + 1 < steps) fetch((s + 1) * F_BK);
+    f32x4 wv[4], av[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+    for (int t = 0; t < 4; ++t) {
+      wv[t] = *(const f32x4*)(&Ws[buf][(wn * 64 + t * 16 + l16) * F_LD + kk * 4]);
+      av[t] = *(const f32x4*)(&As[buf][(wm * 64 + t * 16 + l16) * F_LD + kk * 4]);
+    }
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          tot[i][j] += acc[i][j];
-          acc[i][j] = 0.f;
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+          acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv[nt][e], av[mt][e], acc[nt][mt], 0, 0, 0);
+    if (((s + 1) * F_BK) % F_KBLOCK == 0 || s + 1 == steps) {     // a block of the order of addition ends
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) {
+          tot[nt][mt] += acc[nt][mt];
+          acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
     }
+    if (s + 1 < steps) stage(buf ^ 1);
+    __syncthreads();
   }
+  // lane (l16, kk) of tile (nt, mt) holds row m = mt*16 + l16, columns n = nt*16 + 4 kk + r
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = tot[i][j];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int m = m0 + ty * 4 + i;
+  for (int mt = 0; mt < 4; ++mt) {
+    const int m = m0 + wm * 64 + mt * 16 + l16;
     if (m >= M) continue;
-    if constexpr (SWIGLU) {   // columns (2j, 2j+1) = (gate_j, up_j); N is even
 #pragma unroll
-      for (int j = 0; j < 4; j += 2) {
-        const int n = n0 + tx * 4 + j;
-        if (n >= N) continue;
-        out[(int64_t)m * ldo + n / 2] = from_f32<TO>(swiglu_pair(acc[i][j], acc[i][j + 1]));
-      }
-    } else {
+    for (int nt = 0; nt < 4; ++nt) {
+      const int n = n0 + wn * 64 + nt * 16 + kk * 4;
+      const f32x4 v = tot[nt][mt];
+      if constexpr (SWIGLU) {   // columns (2j, 2j+1) = (gate_j, up_j); N is even
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int n = n0 + tx * 4 + j;
-        if (n >= N) continue;
-        float v = acc[i][j];
-        if (residual) v += residual[(int64_t)m * ldo + n];
-        out[(int64_t)m * ldo + n] = from_f32<TO>(v);
+        for (int r = 0; r < 4; r += 2)
+          if (n + r < N) out[(int64_t)m * ldo + (n + r) / 2] = swiglu_pair(v[r], v[r + 1]);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (n + r < N) {
+            const int64_t at = (int64_t)m * ldo + n + r;
+            out[at] = residual ? v[r] + residual[at] : v[r];
+          }
       }
     }
   }
 }
 
-// The same product for few rows (decode steps), where the tiled kernel leaves most of the chip
-// idle.  A workgroup owns 8 output columns; a thread owns one k block of 256 of one column (and the
-// blocks 32, 64, ... further on) and works through it in ascending k for 8 rows at a time; the
-// block sums meet in LDS and are added in ascending order: the order of gemm_f32_kernel, to the bit.
-constexpr int FR_COLS = 8, FR_LANES = 32, FR_THREADS = FR_COLS * FR_LANES, FR_ROWS = 8;
+// The same product for few rows (decode steps): the weights stream once, straight from memory
+// into the matrix instruction's operand registers.  A workgroup owns 16 output columns; its eight
+// waves deal the k blocks of 256 out among themselves (a wave requests a whole block, 16 KB, at
+// once); the block sums meet in LDS and are added in ascending order: the order of
+// gemm_f32_kernel, to the bit.  Rows come in tiles of 16 (up to four).
+constexpr int FR_WAVES = 8, FR_THREADS = FR_WAVES * TL_WAVE, FR_COLS = 16, FR_MAX_MT = 4;
 
 template <bool SWIGLU>
 __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* __restrict__ a,
@@ -123,56 +166,47 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
                                                                    float* __restrict__ out,
                                                                    const float* __restrict__ residual, int M,
                                                                    int N, int K, int64_t lda, int64_t ldo) {
-  extern __shared__ float rows_smem[];
+  extern __shared__ float rows_smem[];      // [m tiles][k blocks][16 rows][16 columns]
   const int nkb = (K + F_KBLOCK - 1) / F_KBLOCK;
-  float* part = rows_smem;                                   // [FR_COLS][nkb][FR_ROWS]
-  float* sums = rows_smem + FR_COLS * nkb * FR_ROWS;         // [FR_COLS][FR_ROWS]
-  const int tid = threadIdx.x, c = tid / FR_LANES, bl = tid % FR_LANES;
+  const int mts = (M + 15) / 16;
+  const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
+  const int l16 = lane % 16, kk = lane / 16;
   const int n0 = blockIdx.x * FR_COLS;
-  const float* wrow = w + (int64_t)min(n0 + c, N - 1) * K;
-  for (int m0 = 0; m0 < M; m0 += FR_ROWS) {
-    const float* arow[FR_ROWS];
+  const float* wrow = w + (int64_t)min(n0 + l16, N - 1) * K;
+  for (int b = wave; b < nkb; b += FR_WAVES) {
+    const int kb = b * F_KBLOCK;
+    f32x4 wv[16];
 #pragma unroll
-    for (int r = 0; r < FR_ROWS; ++r) arow[r] = a + (int64_t)min(m0 + r, M - 1) * lda;
-    for (int b = bl; b < nkb; b += FR_LANES) {
-      float acc[FR_ROWS];
+    for (int g = 0; g < 16; ++g) wv[g] = load_k4<true>(wrow, kb + g * 16 + kk * 4, K);
+    for (int mt = 0; mt < mts; ++mt) {
+      const float* arow = a + (int64_t)min(mt * 16 + l16, M - 1) * lda;
+      f32x4 av[16];
 #pragma unroll
-      for (int r = 0; r < FR_ROWS; ++r) acc[r] = 0.f;
-      const int k_end = min((b + 1) * F_KBLOCK, K);          // K is a multiple of 4
-#pragma unroll 4
-      for (int k = b * F_KBLOCK; k < k_end; k += 4) {
-        const f32x4 wv = *(const f32x4*)(wrow + k);
+      for (int g = 0; g < 16; ++g) av[g] = load_k4<true>(arow, kb + g * 16 + kk * 4, K);
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int r = 0; r < FR_ROWS; ++r) {
-          const f32x4 av = *(const f32x4*)(arow[r] + k);
+      for (int g = 0; g < 16; ++g)
 #pragma unroll
-          for (int e = 0; e < 4; ++e) acc[r] = fmaf(av[e], wv[e], acc[r]);
-        }
-      }
-#pragma unroll
-      for (int r = 0; r < FR_ROWS; ++r) part[(c * nkb + b) * FR_ROWS + r] = acc[r];
+        for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wv[g][e], av[g][e], acc, 0, 0, 0);
+      // lane (l16, kk): row m = l16, columns 4 kk + r
+      *(f32x4*)(&rows_smem[((mt * nkb + b) * 16 + l16) * 16 + kk * 4]) = acc;
     }
-    __syncthreads();
-    if (tid < FR_COLS * FR_ROWS) {
-      const int cc = tid / FR_ROWS, r = tid % FR_ROWS;
-      float t = 0.f;
-      for (int b = 0; b < nkb; ++b) t += part[(cc * nkb + b) * FR_ROWS + r];
-      sums[tid] = t;
-    }
-    __syncthreads();
-    if (tid < FR_COLS * FR_ROWS) {
-      const int cc = tid / FR_ROWS, r = tid % FR_ROWS;
-      const int m = m0 + r, n = n0 + cc;
+  }
+  __syncthreads();
+  for (int e = tid; e < mts * 256; e += FR_THREADS) {
+    const int mt = e / 256, r = (e % 256) / 16, c = e % 16;
+    float t = 0.f;
+    for (int b = 0; b < nkb; ++b) t += rows_smem[((mt * nkb + b) * 16 + r) * 16 + c];
+    const int m = mt * 16 + r, n = n0 + c;
+    if constexpr (SWIGLU) {   // columns (2j, 2j+1) = (gate_j, up_j); N and n0 are even
+      const float u = __shfl_down(t, 1, TL_WAVE);
+      if (m < M && n < N && (c & 1) == 0) out[(int64_t)m * ldo + n / 2] = swiglu_pair(t, u);
+    } else {
       if (m < M && n < N) {
-        if constexpr (SWIGLU) {   // columns (2j, 2j+1) = (gate_j, up_j); N and n0 are even
-          if ((cc & 1) == 0) out[(int64_t)m * ldo + n / 2] = swiglu_pair(sums[tid], sums[tid + FR_ROWS]);
-        } else {
-          const float v = sums[tid];
-          out[(int64_t)m * ldo + n] = residual ? v + residual[(int64_t)m * ldo + n] : v;
-        }
+        const int64_t at = (int64_t)m * ldo + n;
+        out[at] = residual ? t + residual[at] : t;
       }
     }
-    // the next pass writes `part` only after the barrier above and `sums` only after its own first barrier
   }
 }
 
@@ -1147,25 +1181,38 @@ int tl_linear_tile(const void* a, const void* w, void* out, const float* residua
   if (swiglu && ((N & 1) || residual || out_dtype != dtype)) return TL_ERR_ARG;
   if (dtype == 0) {
     if (out_dtype != 0) return TL_ERR_ARG;
-    if (M <= 16 && K % 4 == 0 && K <= 32768 && lda % 4 == 0 && ((uintptr_t)a | (uintptr_t)w) % 16 == 0) {
-      const int nkb = (K + F_KBLOCK - 1) / F_KBLOCK;
-      const size_t smem = (size_t)(FR_COLS * nkb * FR_ROWS + FR_COLS * FR_ROWS) * sizeof(float);   // at most 33 KB
+    const bool vec = K % 4 == 0 && lda % 4 == 0 && ((uintptr_t)a | (uintptr_t)w) % 16 == 0;
+    const int nkb = (K + F_KBLOCK - 1) / F_KBLOCK;
+    const int mts = (M + 15) / 16;
+    const size_t rows_smem = (size_t)mts * nkb * 256 * sizeof(float);
+    if (M <= 16 * FR_MAX_MT && vec && rows_smem <= 96 * 1024) {
+      static bool configured = false;
+      if (!configured) {
+        if (hipFuncSetAttribute((const void*)gemm_f32_rows_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                96 * 1024) != hipSuccess ||
+            hipFuncSetAttribute((const void*)gemm_f32_rows_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                96 * 1024) != hipSuccess)
+          return TL_ERR_LAUNCH;
+        configured = true;
+      }
       dim3 gr((N + FR_COLS - 1) / FR_COLS);
       if (swiglu)
-        hipLaunchKernelGGL((gemm_f32_rows_kernel<true>), gr, dim3(FR_THREADS), smem, stream, (const float*)a,
+        hipLaunchKernelGGL((gemm_f32_rows_kernel<true>), gr, dim3(FR_THREADS), rows_smem, stream, (const float*)a,
                            (const float*)w, (float*)out, residual, M, N, K, lda, ldo);
       else
-        hipLaunchKernelGGL((gemm_f32_rows_kernel<false>), gr, dim3(FR_THREADS), smem, stream, (const float*)a,
+        hipLaunchKernelGGL((gemm_f32_rows_kernel<false>), gr, dim3(FR_THREADS), rows_smem, stream, (const float*)a,
                            (const float*)w, (float*)out, residual, M, N, K, lda, ldo);
       return tl_launch_status();
     }
     dim3 g((N + F_BN - 1) / F_BN, (M + F_BM - 1) / F_BM);
-    if (swiglu)
-      hipLaunchKernelGGL((gemm_f32_kernel<float, true>), g, dim3(F_THREADS), 0, stream, (const float*)a,
-                         (const float*)w, (float*)out, residual, M, N, K, lda, ldo);
-    else
-      hipLaunchKernelGGL((gemm_f32_kernel<float, false>), g, dim3(F_THREADS), 0, stream, (const float*)a,
-                         (const float*)w, (float*)out, residual, M, N, K, lda, ldo);
+#define TL_F32_TILED(SW, VE)                                                                                  \
+  hipLaunchKernelGGL((gemm_f32_kernel<SW, VE>), g, dim3(F_THREADS), 0, stream, (const float*)a, (const float*)w, \
+                     (float*)out, residual, M, N, K, lda, ldo)
+    if (swiglu && vec) TL_F32_TILED(true, true);
+    else if (swiglu) TL_F32_TILED(true, false);
+    else if (vec) TL_F32_TILED(false, true);
+    else TL_F32_TILED(false, false);
+#undef TL_F32_TILED
   } else if (dtype == 1) {
     if (K % 8 || lda % 8) return TL_ERR_ARG;
     if (out_dtype != 0 && out_dtype != 1) return TL_ERR_ARG;

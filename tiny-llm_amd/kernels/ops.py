@@ -554,6 +554,70 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     return out
 
 
+F32_CHUNK_KEYS = 512     # keys per chunk of the float32 attention kernel's fixed merge tree
+
+
+def attention_f32_supported(dtype: torch.dtype, num_heads: int, num_kv_heads: int, head_dim: int) -> bool:
+    """Sizes the float32 matrix-core attention kernel takes; everything else goes to `paged_attention`."""
+    return (dtype == torch.float32 and head_dim % 16 == 0 and head_dim <= 128 and num_kv_heads > 0
+            and num_heads % num_kv_heads == 0 and num_heads // num_kv_heads <= 16)
+
+
+def attention_f32(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                  tiles, positions: torch.Tensor, out: torch.Tensor, num_heads: int, num_kv_heads: int,
+                  head_dim: int, scale: float, window: int = 0, n_chunks: int = 1,
+                  scratch: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The same function as `paged_attention` in true float32 on the matrix cores.  `tiles` as for
+    `flash_attention` (None: row i is the one new token of request i).  n_chunks == 1: one
+    workgroup per tile and kv head walks all keys; n_chunks > 1 (at least ceil(longest context /
+    512)): the chunks of 512 keys go to workgroups of their own and float32 `scratch` of
+    n_chunks * T * heads * (head_dim + 2) elements holds their results.  The bits of a row's result
+    do not depend on n_chunks, on the tiles or on the rest of the batch."""
+    tile_req, tile_tok0, tile_ntok = tiles if tiles is not None else (None, None, None)
+    _dev(q, k_cache, v_cache, block_tables, tile_req, tile_tok0, tile_ntok, positions, out, scratch)
+    _rows_2d(q, "q")
+    _rows_2d(out, "attention output")
+    T = q.shape[0]
+    if not attention_f32_supported(q.dtype, num_heads, num_kv_heads, head_dim):
+        _fail("the float32 matrix-core attention kernel takes float32, head sizes in steps of 16 up to 128, up "
+              "to 16 heads per kv head")
+    if not (q.shape[1] == num_heads * head_dim and tuple(out.shape) == (T, num_heads * head_dim)):
+        _fail("q and the attention output must be [T, heads * head_dim]")
+    if not (k_cache.dtype == v_cache.dtype == out.dtype == torch.float32):
+        _fail("q, caches and output must be float32")
+    if not (k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dim() == 4
+            and k_cache.shape == v_cache.shape and k_cache.shape[1] == num_kv_heads
+            and k_cache.shape[3] == head_dim):
+        _fail("cache must be contiguous [blocks, kv_heads, block, head_dim]")
+    if not (block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()):
+        _fail("block tables must be contiguous int32 [requests, max_blocks]")
+    if not (positions.dtype == torch.int32 and positions.is_contiguous() and positions.numel() == T):
+        _fail("positions must be contiguous int32, one per row")
+    if tiles is None:
+        n_tiles = T
+        if not (block_tables.shape[0] >= T):
+            _fail("without tile arrays every row is a request of its own and needs a block table row")
+    else:
+        n_tiles = tile_req.numel()
+        for t in (tile_req, tile_tok0, tile_ntok):
+            if not (t.dtype == torch.int32 and t.is_contiguous() and t.numel() == n_tiles):
+                _fail("tile arrays must be int32 [tiles]")
+    if not (q.stride(0) % 4 == 0 and n_chunks >= 1):
+        _fail("q rows must be 16-byte aligned and n_chunks positive")
+    if n_chunks > 1:
+        need = n_chunks * T * num_heads * (head_dim + 2)
+        if not (scratch is not None and scratch.dtype == torch.float32 and scratch.is_contiguous()
+                and scratch.numel() >= need):
+            _fail(f"chunked attention needs {need} float32 of scratch")
+    _check(_lib().tl_attention_f32(
+        _ptr(q, 16), c_int64(q.stride(0)), _ptr(k_cache, 16), _ptr(v_cache, 16), _ptr(block_tables),
+        c_int(block_tables.shape[1]), _ptr(tile_req), _ptr(tile_tok0), _ptr(tile_ntok), _ptr(positions),
+        _ptr(out), c_int64(out.stride(0)), _ptr(scratch), c_int(n_tiles), c_int(T), c_int(num_heads),
+        c_int(num_kv_heads), c_int(head_dim), c_int(k_cache.shape[2]), c_float(scale), c_int(window),
+        c_int(n_chunks), _stream()), "attention_f32")
+    return out
+
+
 def flash_attention_supported(dtype: torch.dtype, num_heads: int, num_kv_heads: int, head_dim: int) -> bool:
     """Sizes the MFMA attention kernel takes; everything else goes to `paged_attention`."""
     return (dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 128 and num_kv_heads > 0

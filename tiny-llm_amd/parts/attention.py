@@ -104,6 +104,19 @@ class Attention(Mixer):
             ops.flash_attention(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, attn,
                                 self.num_heads, self.num_kv_heads, self.head_dim, self.scale, self.window,
                                 n_splits, scratch, fused_rope=(cos, sin) if fuse else None)
+        elif ops.attention_f32_supported(self.dtype, self.num_heads, self.num_kv_heads, self.head_dim) \
+                and q.stride(0) % 4 == 0:
+            # true float32 on the matrix cores; one fixed merge tree, so the same bits whatever the batch
+            decode = ctx.max_q_len == 1 and T == ctx.num_requests
+            tiles = None if decode else ctx.attention_tiles(16 // group)
+            n_chunks = -(-ctx.max_seq_len // ops.F32_CHUNK_KEYS) if ctx.max_q_len == 1 else 1
+            scratch = None
+            if n_chunks > 1:
+                scratch = ops.scratch("attention_partials", (n_chunks * T * self.num_heads * (self.head_dim + 2),),
+                                      torch.float32, residual.device)
+            ops.attention_f32(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, attn,
+                              self.num_heads, self.num_kv_heads, self.head_dim, self.scale, self.window, n_chunks,
+                              scratch)
         else:
             ops.paged_attention(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.req_of_token,
                                 ctx.positions, attn, self.num_heads, self.num_kv_heads, self.head_dim,
