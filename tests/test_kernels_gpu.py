@@ -513,7 +513,7 @@ def _paged_case(dtype, lens, q_lens, nq, nkv, hd, bs, window=0, seed=0, boost=No
                                 i32(pos), out, nq, nkv, hd, 1.0 / math.sqrt(hd), window)
             return out.reshape(-1, nq, hd), torch.cat(refs)
         scratch = torch.full((max(1, n_splits * T * nq * (hd + 2)),), float("nan"), device=DEV)
-        if impl == "f32":       # n_splits stands for the number of 512-key chunks given to workgroups of their own
+        if impl == "f32":       # n_splits stands for the number of 256-key chunks given to workgroups of their own
             tiles = None if (n_splits == -1) else (i32(t_req), i32(t_tok0), i32(t_ntok))
             chunks = max(1, abs(n_splits))
             scratch = torch.full((max(1, chunks * T * nq * (hd + 2)),), float("nan"), device=DEV)
@@ -607,7 +607,7 @@ def test_flash_attention_window_edge(window):
 
 
 # ---------------------------------------------- float32 attention on the matrix cores
-@pytest.mark.parametrize("chunks", [1, 2])
+@pytest.mark.parametrize("chunks", [1, 3])
 @pytest.mark.parametrize("nq,nkv,hd,bs", FLASH_SHAPES)
 def test_attention_f32_mixed_batch(nq, nkv, hd, bs, chunks):
     out, ref = _paged_case(torch.float32, lens=[123, 107, 65, 1, 300, 2, 513], q_lens=[123, 40, 1, 1, 1, 2, 257],
@@ -618,17 +618,17 @@ def test_attention_f32_mixed_batch(nq, nkv, hd, bs, chunks):
 
 def test_attention_f32_far_key_window_edge_and_decode_batch():
     for far in (0, 15, 16, 63, 64, 255, 256, 511, 512, 699):
-        for chunks in (1, 2):
+        for chunks in (1, 3):
             out, ref = _paged_case(torch.float32, lens=[700], q_lens=[30 if chunks == 1 else 1], nq=8, nkv=1, hd=64,
                                    bs=16, seed=far, boost=far, impl="f32", n_splits=chunks)
             assert rel(out, ref) < 2e-6, far
     for window in (1, 7, 16, 33, 100, 600):
         out, ref = _paged_case(torch.float32, lens=[190, 40, 64, 130, 1300], q_lens=[190, 1, 5, 70, 2], nq=4, nkv=2,
-                               hd=32, bs=8, window=window, seed=window, impl="f32", n_splits=3)
+                               hd=32, bs=8, window=window, seed=window, impl="f32", n_splits=6)
         assert not torch.isnan(out).any()
         assert rel(out, ref) < 2e-6, window
     lens = [1, 2, 63, 64, 65, 127, 128, 129, 500, 1000, 17, 256, 512, 513, 1024, 1025]
-    for chunks in (1, 3, -3):       # -3: without tile arrays (row i is request i), as a decode step runs
+    for chunks in (1, 5, -5):       # -5: without tile arrays (row i is request i), as a decode step runs
         out, ref = _paged_case(torch.float32, lens=lens, q_lens=[1] * len(lens), nq=32, nkv=4, hd=64, bs=16,
                                seed=5, impl="f32", n_splits=chunks)
         assert rel(out, ref) < 2e-6
@@ -636,16 +636,16 @@ def test_attention_f32_far_key_window_edge_and_decode_batch():
 
 def test_attention_f32_gives_the_same_bits_however_the_work_is_cut():
     """A query row's result, to the bit: alone or in a batch, in tiles of one token or of several,
-    keys walked by one workgroup or chunks of 512 given to several."""
+    keys walked by one workgroup or chunks of 256 given to several."""
     lens, nq, nkv, hd, bs = [1100, 77, 513], 8, 2, 64, 16
     base, _ = _paged_case(torch.float32, lens=lens, q_lens=[300, 77, 1], nq=nq, nkv=nkv, hd=hd, bs=bs, seed=3, impl="f32")
-    for kw in (dict(n_splits=3), dict(tile_tokens=1), dict(tile_tokens=3, n_splits=4), dict(tile_tokens=2, n_splits=1)):
+    for kw in (dict(n_splits=5), dict(tile_tokens=1), dict(tile_tokens=3, n_splits=7), dict(tile_tokens=2, n_splits=1)):
         other, _ = _paged_case(torch.float32, lens=lens, q_lens=[300, 77, 1], nq=nq, nkv=nkv, hd=hd, bs=bs, seed=3,
                                impl="f32", **kw)
         assert torch.equal(other.cpu(), base.cpu()), kw
     # the last rows of the first request alone, as single decoded tokens would come
     tail, _ = _paged_case(torch.float32, lens=lens, q_lens=[1, 1, 1], nq=nq, nkv=nkv, hd=hd, bs=bs, seed=3,
-                          impl="f32", n_splits=-3)
+                          impl="f32", n_splits=-5)
     assert torch.equal(tail.cpu()[0], base.cpu()[299]) and torch.equal(tail.cpu()[1], base.cpu()[376])
 
 

@@ -488,7 +488,7 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
 // how the keys are spread over workgroups, because the terms are always combined in ONE tree:
 //   * keys in tiles of 64 at absolute positions 64 t .. 64 t + 63; a tile gives (m, l, O) from scratch:
 //     m the largest score, l = sum exp2(s - m), O = sum exp2(s - m) v (scores in units of log2 e);
-//   * the tiles of a chunk of 8 (512 keys) are merged in ascending order, starting from "nothing";
+//   * the tiles of a chunk of 4 (256 keys) are merged in ascending order, starting from "nothing";
 //   * the chunks are merged in ascending order, starting from "nothing".
 // `merge_f32` is the one merge; a tile or chunk that holds no visible key merges as an exact no-op,
 // so skipping it changes nothing.  A workgroup (four waves) owns 16 query rows of one request and
@@ -496,7 +496,7 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
 // chunks itself (gridDim.z == 1) or owns chunk blockIdx.z and leaves its (m, l, O) in `part` for
 // attention_f32_combine_kernel.  Its waves take the tiles of a chunk in turn; a wave reads keys
 // straight into the first product's operands and stages values through an LDS area of its own.
-constexpr int A32_WAVES = 4, A32_THREADS = A32_WAVES * TL_WAVE, A32_CHUNK = 8;
+constexpr int A32_WAVES = 4, A32_THREADS = A32_WAVES * TL_WAVE, A32_CHUNK = 4;
 constexpr int A32_VW = 64, A32_VS = A32_VW + 4;      // value columns staged at a time, row stride in LDS
 
 __device__ __forceinline__ void merge_f32(float& M, float& L, float m, float l, float& wa, float& wb) {
@@ -525,8 +525,8 @@ __global__ __launch_bounds__(A32_THREADS) void attention_f32_kernel(
   constexpr int EPT = 16 * HD / A32_THREADS;       // output elements a thread merges (= HDT)
   extern __shared__ __attribute__((aligned(16))) float smem32[];
   float* Vl_all = smem32;                                          // [waves][64][A32_VS]
-  float* Po = smem32 + A32_WAVES * FA_KT * A32_VS;                 // [8 tiles][16 rows][PS]
-  float* Pml = Po + A32_CHUNK * 16 * PS;                           // [8 tiles][16 rows][2]
+  float* Po = smem32 + A32_WAVES * FA_KT * A32_VS;                 // [tiles of a chunk][16 rows][PS]
+  float* Pml = Po + A32_CHUNK * 16 * PS;                           // [tiles of a chunk][16 rows][2]
 
   const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
   const int l16 = lane % 16, kk = lane / 16;
@@ -572,6 +572,20 @@ __global__ __launch_bounds__(A32_THREADS) void attention_f32_kernel(
     const int t_lo = max(c * A32_CHUNK, first_tile), t_hi = min((c + 1) * A32_CHUNK, last_tile);
     for (int t = t_lo + wave; t < t_hi; t += A32_WAVES) {
       const int kb = t * FA_KT;
+      // the first 64 value columns of this lane's key row are requested before anything else
+      constexpr int VPRE = (HD < A32_VW ? HD : A32_VW) / 4;
+      f32x4 vpre[VPRE];
+      const int vkey = kb + lane;
+      const bool v_in_range = vkey >= kv_begin && vkey < kv_end;
+      const float* vrow;
+      {
+        const int jb = min(vkey / block_size, max_blocks - 1);
+        const int64_t blk = max(bt[v_in_range ? jb : 0], 0);
+        vrow = v_cache + ((blk * nkv + kvh) * block_size + (vkey - (vkey / block_size) * block_size)) * HD;
+#pragma unroll
+        for (int ch = 0; ch < VPRE; ++ch)
+          vpre[ch] = v_in_range ? *(const f32x4*)(vrow + ch * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
+      }
       // ---- scores S^T = K Q^T: lane (l16, kk) of subtile st holds keys kb + 16 st + 4 kk + r of row l16
       f32x4 sc[4];
 #pragma unroll
@@ -616,11 +630,7 @@ __global__ __launch_bounds__(A32_THREADS) void attention_f32_kernel(
 #pragma unroll
       for (int dt = 0; dt < HDT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
       {
-        const int key = kb + lane;
-        const bool in_range = key >= kv_begin && key < kv_end;
-        const int jb = min(key / block_size, max_blocks - 1);
-        const int64_t blk = max(bt[in_range ? jb : 0], 0);
-        const float* vrow = v_cache + ((blk * nkv + kvh) * block_size + (key - (key / block_size) * block_size)) * HD;
+        const bool in_range = v_in_range;
 #pragma unroll
         for (int dh = 0; dh < (HD + A32_VW - 1) / A32_VW; ++dh) {
           constexpr int full = A32_VW / 4;
@@ -634,7 +644,9 @@ __global__ __launch_bounds__(A32_THREADS) void attention_f32_kernel(
           for (int ch = 0; ch < full; ++ch)
             if (ch < chunks) {
               // rows outside the request's keys are zeroed: stale pages may hold anything, and 0 * NaN is NaN
-              const f32x4 v = in_range ? *(const f32x4*)(vrow + dh * A32_VW + ch * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
+              f32x4 v;
+              if (dh == 0) v = vpre[ch < VPRE ? ch : 0];
+              else v = in_range ? *(const f32x4*)(vrow + dh * A32_VW + ch * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
               *(f32x4*)(&Vl[lane * A32_VS + ch * 4]) = v;
             }
           __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -1162,7 +1174,7 @@ int tl_paged_attention(const void* q, int64_t q_stride, const void* k_cache, con
 
 // float32 on the matrix cores, for every kind of step.  Tiles as tl_flash_attention (null: tile i
 // is token i of request i).  n_chunks == 1: a workgroup walks all keys of its tile; n_chunks > 1: it
-// must be at least ceil(longest context / 512), chunk c goes to workgroup (., ., c) and `part`
+// must be at least ceil(longest context / 256), chunk c goes to workgroup (., ., c) and `part`
 // [n_chunks, n_tokens, nq, hd + 2] floats is scratch.  Either way the same bits.
 int tl_attention_f32(const float* q, int64_t q_stride, const float* k_cache, const float* v_cache,
                      const int32_t* block_tables, int max_blocks, const int32_t* tile_req,

@@ -154,30 +154,38 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f32_kernel(const float* __rest
 }
 
 // The same product for few rows (decode steps): the weights stream once, straight from memory
-// into the matrix instruction's operand registers.  A workgroup owns 16 output columns; its eight
-// waves deal the k blocks of 256 out among themselves (a wave requests a whole block, 16 KB, at
-// once); the block sums meet in LDS and are added in ascending order: the order of
-// gemm_f32_kernel, to the bit.  Rows come in tiles of 16 (up to four).
-constexpr int FR_WAVES = 8, FR_THREADS = FR_WAVES * TL_WAVE, FR_COLS = 16, FR_MAX_MT = 4;
+// into the matrix instruction's operand registers.  A workgroup owns 16 output columns (8 where
+// 16 would leave compute units without work: the matrix tile's other 8 rows then repeat them and
+// are dropped); its eight waves deal the k blocks of 256 out among themselves, a wave requests a
+// whole block (16 KB) at once and the next one before it multiplies; the block sums meet in LDS and
+// are added in ascending order: the order of gemm_f32_kernel, to the bit.  Rows come in tiles of
+// 16 (up to four).
+constexpr int FR_WAVES = 8, FR_THREADS = FR_WAVES * TL_WAVE, FR_MAX_MT = 4;
 
-template <bool SWIGLU>
+template <bool SWIGLU, int COLS>
 __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* __restrict__ a,
                                                                    const float* __restrict__ w,
                                                                    float* __restrict__ out,
                                                                    const float* __restrict__ residual, int M,
                                                                    int N, int K, int64_t lda, int64_t ldo) {
-  extern __shared__ float rows_smem[];      // [m tiles][k blocks][16 rows][16 columns]
+  extern __shared__ float rows_smem[];      // [m tiles][k blocks][16 rows][COLS columns]
   const int nkb = (K + F_KBLOCK - 1) / F_KBLOCK;
   const int mts = (M + 15) / 16;
   const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
   const int l16 = lane % 16, kk = lane / 16;
-  const int n0 = blockIdx.x * FR_COLS;
-  const float* wrow = w + (int64_t)min(n0 + l16, N - 1) * K;
+  const int n0 = blockIdx.x * COLS;
+  const float* wrow = w + (int64_t)min(n0 + l16 % COLS, N - 1) * K;
+  f32x4 wv[16], wnext[16];
+  if (wave < nkb) {
+#pragma unroll
+    for (int g = 0; g < 16; ++g) wv[g] = load_k4<true>(wrow, wave * F_KBLOCK + g * 16 + kk * 4, K);
+  }
   for (int b = wave; b < nkb; b += FR_WAVES) {
     const int kb = b * F_KBLOCK;
-    f32x4 wv[16];
+    if (b + FR_WAVES < nkb) {
 #pragma unroll
-    for (int g = 0; g < 16; ++g) wv[g] = load_k4<true>(wrow, kb + g * 16 + kk * 4, K);
+      for (int g = 0; g < 16; ++g) wnext[g] = load_k4<true>(wrow, kb + FR_WAVES * F_KBLOCK + g * 16 + kk * 4, K);
+    }
     for (int mt = 0; mt < mts; ++mt) {
       const float* arow = a + (int64_t)min(mt * 16 + l16, M - 1) * lda;
       f32x4 av[16];
@@ -189,14 +197,16 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
 #pragma unroll
         for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wv[g][e], av[g][e], acc, 0, 0, 0);
       // lane (l16, kk): row m = l16, columns 4 kk + r
-      *(f32x4*)(&rows_smem[((mt * nkb + b) * 16 + l16) * 16 + kk * 4]) = acc;
+      if (kk * 4 < COLS) *(f32x4*)(&rows_smem[((mt * nkb + b) * 16 + l16) * COLS + kk * 4]) = acc;
     }
+#pragma unroll
+    for (int g = 0; g < 16; ++g) wv[g] = wnext[g];
   }
   __syncthreads();
-  for (int e = tid; e < mts * 256; e += FR_THREADS) {
-    const int mt = e / 256, r = (e % 256) / 16, c = e % 16;
+  for (int e = tid; e < mts * 16 * COLS; e += FR_THREADS) {
+    const int mt = e / (16 * COLS), r = (e % (16 * COLS)) / COLS, c = e % COLS;
     float t = 0.f;
-    for (int b = 0; b < nkb; ++b) t += rows_smem[((mt * nkb + b) * 16 + r) * 16 + c];
+    for (int b = 0; b < nkb; ++b) t += rows_smem[((mt * nkb + b) * 16 + r) * COLS + c];
     const int m = mt * 16 + r, n = n0 + c;
     if constexpr (SWIGLU) {   // columns (2j, 2j+1) = (gate_j, up_j); N and n0 are even
       const float u = __shfl_down(t, 1, TL_WAVE);
@@ -1184,24 +1194,29 @@ int tl_linear_tile(const void* a, const void* w, void* out, const float* residua
     const bool vec = K % 4 == 0 && lda % 4 == 0 && ((uintptr_t)a | (uintptr_t)w) % 16 == 0;
     const int nkb = (K + F_KBLOCK - 1) / F_KBLOCK;
     const int mts = (M + 15) / 16;
-    const size_t rows_smem = (size_t)mts * nkb * 256 * sizeof(float);
+    // 8 columns a workgroup where that still is one round of workgroups over the 256 compute units
+    // (a workgroup fills a compute unit: more than 256 of them would run in two rounds)
+    const int cols = (N + 7) / 8 <= 256 ? 8 : 16;
+    const size_t rows_smem = (size_t)mts * nkb * 16 * cols * sizeof(float);
     if (M <= 16 * FR_MAX_MT && vec && rows_smem <= 96 * 1024) {
       static bool configured = false;
       if (!configured) {
-        if (hipFuncSetAttribute((const void*)gemm_f32_rows_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                96 * 1024) != hipSuccess ||
-            hipFuncSetAttribute((const void*)gemm_f32_rows_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                96 * 1024) != hipSuccess)
-          return TL_ERR_LAUNCH;
+        const void* kernels[4] = {(const void*)gemm_f32_rows_kernel<true, 16>, (const void*)gemm_f32_rows_kernel<false, 16>,
+                                  (const void*)gemm_f32_rows_kernel<true, 8>, (const void*)gemm_f32_rows_kernel<false, 8>};
+        for (const void* k : kernels)
+          if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024) != hipSuccess)
+            return TL_ERR_LAUNCH;
         configured = true;
       }
-      dim3 gr((N + FR_COLS - 1) / FR_COLS);
-      if (swiglu)
-        hipLaunchKernelGGL((gemm_f32_rows_kernel<true>), gr, dim3(FR_THREADS), rows_smem, stream, (const float*)a,
-                           (const float*)w, (float*)out, residual, M, N, K, lda, ldo);
-      else
-        hipLaunchKernelGGL((gemm_f32_rows_kernel<false>), gr, dim3(FR_THREADS), rows_smem, stream, (const float*)a,
-                           (const float*)w, (float*)out, residual, M, N, K, lda, ldo);
+      dim3 gr((N + cols - 1) / cols);
+#define TL_F32_ROWS(SW, CO)                                                                                   \
+  hipLaunchKernelGGL((gemm_f32_rows_kernel<SW, CO>), gr, dim3(FR_THREADS), rows_smem, stream, (const float*)a, \
+                     (const float*)w, (float*)out, residual, M, N, K, lda, ldo)
+      if (swiglu && cols == 16) TL_F32_ROWS(true, 16);
+      else if (swiglu) TL_F32_ROWS(true, 8);
+      else if (cols == 16) TL_F32_ROWS(false, 16);
+      else TL_F32_ROWS(false, 8);
+#undef TL_F32_ROWS
       return tl_launch_status();
     }
     dim3 g((N + F_BN - 1) / F_BN, (M + F_BM - 1) / F_BM);

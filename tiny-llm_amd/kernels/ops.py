@@ -554,7 +554,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     return out
 
 
-F32_CHUNK_KEYS = 512     # keys per chunk of the float32 attention kernel's fixed merge tree
+F32_CHUNK_KEYS = 256     # keys per chunk of the float32 attention kernel's fixed merge tree
 
 
 def attention_f32_supported(dtype: torch.dtype, num_heads: int, num_kv_heads: int, head_dim: int) -> bool:
@@ -570,7 +570,7 @@ def attention_f32(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
     """The same function as `paged_attention` in true float32 on the matrix cores.  `tiles` as for
     `flash_attention` (None: row i is the one new token of request i).  n_chunks == 1: one
     workgroup per tile and kv head walks all keys; n_chunks > 1 (at least ceil(longest context /
-    512)): the chunks of 512 keys go to workgroups of their own and float32 `scratch` of
+    256)): the chunks of 256 keys go to workgroups of their own and float32 `scratch` of
     n_chunks * T * heads * (head_dim + 2) elements holds their results.  The bits of a row's result
     do not depend on n_chunks, on the tiles or on the rest of the batch."""
     tile_req, tile_tok0, tile_ntok = tiles if tiles is not None else (None, None, None)
