@@ -1,10 +1,15 @@
-"""Decode and prefill throughput of the TinyLlama-1.1B shape with random weights.
+"""Decode and prefill throughput with random weights, on one GPU.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-A step is one decode step of the whole serving path (scheduler, step function, sampling)
-at batch 8 with 512-token prompts.  One JSON line is printed: decoded tokens per second,
-the 2,048-token prefill, the HBM roofline of the decode step, and decode at batch 1 and 64.
+A step is one decode step of the whole serving path (scheduler, step function, sampling).  The
+headline is the TinyLlama-1.1B shape in bfloat16 at batch 8 with 512-token prompts.  ONE JSON line is
+printed: decoded tokens per second, the 2,048-token prefill (whole and in portions of 512), the HBM
+roofline of the decode step, decode at batch 1 and 64; the same in true float32; the machine's peaks
+as measured on the spot (a streaming kernel, a loop of matrix instructions); and two soak workloads
+at larger shapes (a mixed batch of 16 requests with prompts cut into portions of 512 at the
+Llama-3-8B shape; 64 requests of 1,024 tokens that nearly fill the cache at the Llama-2-13B shape).
+`--only` picks a part (for profiling).
 """
 import argparse
 import json
@@ -19,16 +24,22 @@ sys.path.insert(0, ROOT)
 HBM_GBS = 8000.0
 PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
 
-# the TinyLlama 1.1B shape
-TINYLLAMA = {
-    "architectures": ["LlamaForCausalLM"], "model_type": "llama", "num_hidden_layers": 22, "hidden_size": 2048,
-    "num_attention_heads": 32, "num_key_value_heads": 4, "intermediate_size": 5632, "vocab_size": 32000,
-    "rope_theta": 10000.0, "rms_norm_eps": 1e-5, "max_position_embeddings": 2048, "tie_word_embeddings": False,
-    "hidden_act": "silu", "attention_bias": False, "rope_scaling": None, "initializer_range": 0.02,
-    "eos_token_id": 2,
-}
+
+def llama(layers, hidden, heads, kv_heads, inter, vocab, theta, max_pos):
+    return {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "num_hidden_layers": layers,
+            "hidden_size": hidden, "num_attention_heads": heads, "num_key_value_heads": kv_heads,
+            "intermediate_size": inter, "vocab_size": vocab, "rope_theta": theta, "rms_norm_eps": 1e-5,
+            "max_position_embeddings": max_pos, "tie_word_embeddings": False, "hidden_act": "silu",
+            "attention_bias": False, "rope_scaling": None, "initializer_range": 0.02, "eos_token_id": 2}
+
+
+TINYLLAMA = llama(22, 2048, 32, 4, 5632, 32000, 10000.0, 2048)       # the TinyLlama 1.1B shape
+LLAMA3_8B = llama(32, 4096, 32, 8, 14336, 128256, 500000.0, 8192)
+LLAMA2_13B = llama(40, 5120, 40, 40, 13824, 32000, 10000.0, 4096)
 PROMPT_LEN = 512
 PREFILL_TOKENS = 2048
+ELT = {"bf16": 2, "fp32": 4}
+TORCH_NAME = {"bf16": "bfloat16", "fp32": "float32"}
 
 
 def model_numbers(cfg, elt_bytes):
@@ -42,97 +53,255 @@ def model_numbers(cfg, elt_bytes):
     return matmul_params, weight_bytes, kv_bytes_per_token, (L, H, I, V, nq, nkv, hd)
 
 
-def run(args):
-    import torch
-    from tiny_llm_amd import Engine, SamplingParams
+def prefill_flops(cfg, tokens):
+    matmul_params, _, _, (L, H, I, V, nq, nkv, hd) = model_numbers(cfg, 2)
+    return 2.0 * tokens * matmul_params + L * nq * 2.0 * tokens * tokens * hd + 2.0 * V * H
 
-    dtype = "bfloat16" if args.dtype == "bf16" else "float32"
-    elt = 2 if args.dtype == "bf16" else 4
+
+def gen_tokens(n, vocab, seed):
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+# --------------------------------------------------------------- measured peaks
+def measure_peaks():
+    """GB/s of a streaming read and of a copy over 2 GiB, TFLOP/s of matrix-instruction loops."""
+    import torch
+    from tiny_llm_amd.kernels import ops
+    dev = "cuda:0"
+    sink = torch.zeros(4, dtype=torch.float32, device=dev)
+    src = torch.ones(1 << 29, dtype=torch.float32, device=dev)       # 2 GiB: far beyond every cache
+    dst = torch.empty_like(src)
+    nbytes = src.numel() * 4
+
+    def timed(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / reps
+
+    read = max(nbytes / timed(lambda: ops.peak_stream(src, None, sink, blocks), 5) for blocks in (2048, 4096, 8192))
+    copy = max(2 * nbytes / timed(lambda: ops.peak_stream(src, dst, sink, blocks), 5) for blocks in (2048, 4096, 8192))
+    del src, dst
+    out = {"hbm_read_GBs": round(read / 1e9, 1), "hbm_copy_GBs": round(copy / 1e9, 1)}
+    for name, dt in (("bf16", torch.bfloat16), ("fp32", torch.float32)):
+        flops = ops.peak_mfma(sink, dt, 20000, 2048)
+        t = timed(lambda: ops.peak_mfma(sink, dt, 20000, 2048), 3)
+        out[f"mfma_{name}_TFLOPs"] = round(flops / t / 1e12, 1)
+    return out
+
+
+# ------------------------------------------------------------------- one model
+class Bench:
+    def __init__(self, cfg, dtype, max_batch, total_new, block_size, budget=4096, extra_tokens=PREFILL_TOKENS,
+                 prompt_len=PROMPT_LEN, max_cache_tokens=None):
+        import torch
+        from tiny_llm_amd import Engine
+        self.torch = torch
+        self.cfg, self.dtype = cfg, dtype
+        self.V = cfg["vocab_size"]
+        blocks = (max_batch * (prompt_len + total_new) + extra_tokens) // block_size + max_batch + 8
+        if max_cache_tokens is not None:
+            blocks = max_cache_tokens // block_size
+        self.engine = Engine(config=cfg, dtype=TORCH_NAME[dtype], kv_block_size=block_size, max_num_seqs=max_batch,
+                             max_num_batched_tokens=budget, weights_seed=0, num_kv_blocks=blocks)
+        self.sync = torch.cuda.synchronize
+
+    def close(self):
+        self.engine = None
+        import gc
+        gc.collect()
+        self.torch.cuda.empty_cache()
+
+    def decode(self, batch, steps, warmup, prompt_len=PROMPT_LEN):
+        """Prefills `batch` prompts (untimed), then times `steps` decode steps.
+        Returns (seconds, cached tokens read per step summed over the batch)."""
+        from tiny_llm_amd import SamplingParams
+        eng = self.engine
+        params = SamplingParams.greedy(warmup + steps + 1, ignore_eos=True)
+        ids = [eng.add_request(gen_tokens(prompt_len, self.V, 1000 + i), params) for i in range(batch)]
+        while any(eng.requests[i].num_computed < prompt_len for i in ids):
+            eng.step()
+        for _ in range(warmup):
+            eng.step()
+        ctx0 = sum(eng.requests[i].num_tokens for i in ids)
+        self.sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            eng.step()
+        self.sync()
+        dt = time.perf_counter() - t0
+        ctx1 = sum(eng.requests[i].num_tokens for i in ids)
+        for i in ids:
+            eng.abort(i)
+        return dt, (ctx0 + ctx1) / 2.0
+
+    def prefill(self, reps, tokens=PREFILL_TOKENS, budget=None):
+        """Best of `reps` prefills of one prompt (after one untimed), its last logits sampled; with
+        `budget` the prompt is cut into portions of that many tokens (one step each)."""
+        from tiny_llm_amd import SamplingParams
+        eng = self.engine
+        old = eng.scheduler.budget
+        if budget is not None:
+            eng.scheduler.budget = budget
+        times = []
+        for r in range(reps + 1):
+            rid = eng.add_request(gen_tokens(tokens, self.V, 77 + r), SamplingParams.greedy(1, ignore_eos=True))
+            self.sync()
+            t0 = time.perf_counter()
+            while eng.requests[rid].status != "finished":
+                eng.step()
+            self.sync()
+            times.append(time.perf_counter() - t0)
+        eng.scheduler.budget = old
+        return min(times[1:])
+
+    def soak(self, prompt_lens, new_tokens, budget):
+        """All requests at once through the scheduler: prompts in portions under `budget` tokens a
+        step beside decoded tokens.  Returns (seconds, steps, preemptions)."""
+        from tiny_llm_amd import SamplingParams
+        eng = self.engine
+        eng.scheduler.budget = budget
+        ids = [eng.add_request(gen_tokens(n, self.V, 5000 + i), SamplingParams.greedy(new_tokens, ignore_eos=True))
+               for i, n in enumerate(prompt_lens)]
+        self.sync()
+        steps = 0
+        t0 = time.perf_counter()
+        while eng.has_unfinished():
+            eng.step()
+            steps += 1
+        self.sync()
+        dt = time.perf_counter() - t0
+        assert all(len(eng.requests[i].output) == new_tokens for i in ids)
+        return dt, steps, sum(eng.requests[i].preemptions for i in ids)
+
+
+def tinyllama_figures(args, dtype, peaks):
+    """Decode at batch 8 / 1 / 64 and the 2,048-token prefill at the TinyLlama shape in `dtype`."""
+    elt = ELT[dtype]
     cfg = dict(TINYLLAMA)
-    layers_full = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
     matmul_params, weight_bytes, kv_per_tok, (L, H, I, V, nq, nkv, hd) = model_numbers(cfg, elt)
+    steps, warmup = args.steps, args.warmup
+    if dtype == "fp32":
+        steps, warmup = min(steps, 64), min(warmup, 8)       # the 32-bit path is for checking: a shorter run
+    b = Bench(cfg, dtype, max(args.batch, 64), warmup + steps + 1, args.block_size)
+    out = {}
+    if args.only in ("all", "headline", "fp32", "prefill"):
+        pf = b.prefill(3)
+        flops = prefill_flops(cfg, PREFILL_TOKENS)
+        out["prefill"] = {"value": round(PREFILL_TOKENS / pf, 1), "tokens": PREFILL_TOKENS, "ms": round(pf * 1e3, 3),
+                          "frac": round(flops / pf / (PEAK_TFLOPS[dtype] * 1e12), 4)}
+        if peaks:
+            out["prefill"]["frac_measured"] = round(flops / pf / (peaks[f"mfma_{dtype}_TFLOPs"] * 1e12), 4)
+        pc = b.prefill(2, budget=512)
+        out["prefill_chunked_512"] = {"value": round(PREFILL_TOKENS / pc, 1), "ms": round(pc * 1e3, 3), "steps": 4}
+    if args.only != "prefill":
+        dt, ctx_tokens = b.decode(args.batch, steps, warmup)
+        out["ms_per_step"] = dt / steps * 1e3
+        out["value"] = args.batch * steps / dt
+        achieved = (weight_bytes + ctx_tokens * kv_per_tok) / (dt / steps) / 1e9
+        out["roofline"] = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
+                           "frac": round(achieved / HBM_GBS, 4)}
+        if peaks:
+            out["roofline"]["frac_measured"] = round(achieved / peaks["hbm_read_GBs"], 4)
+        out["points"] = {}
+        if args.only in ("all", "headline", "fp32"):
+            for n in (1, 64):
+                d, _ = b.decode(n, steps, warmup)
+                out["points"][f"decode_b{n}"] = round(n * steps / d, 1)
+    out["sizes"] = (L, H, I, V, nq, nkv, hd)
+    out["steps"], out["warmup"] = steps, warmup
+    b.close()
+    return out
 
-    def gen_tokens(n, seed):
-        g = torch.Generator().manual_seed(seed)
-        return torch.randint(0, V, (n,), generator=g).tolist()
 
-    total_new = args.warmup + args.steps + 1
-    max_batch = max(args.batch, 64)
-    engine = Engine(config=cfg, dtype=dtype, kv_block_size=args.block_size, max_num_seqs=max_batch,
-                    max_num_batched_tokens=max(PREFILL_TOKENS, 4096), weights_seed=0,
-                    num_kv_blocks=(max_batch * (PROMPT_LEN + total_new) + PREFILL_TOKENS) // args.block_size + max_batch + 8)
-    sync = torch.cuda.synchronize
+def soak_llama3_8b(args):
+    """16 requests, seeded prompt lengths 128..4096, prompts in portions of 512, 128 tokens each."""
+    import random
+    cfg = dict(LLAMA3_8B)
+    layers_full = cfg["num_hidden_layers"]
+    if args.soak_layers:
+        cfg["num_hidden_layers"] = min(layers_full, args.soak_layers)
+    rng = random.Random(8)
+    lens = [rng.randint(128, 4096) for _ in range(16)]
+    new = 128
+    b = Bench(cfg, "bf16", 16, new, 16, budget=512, max_cache_tokens=sum(-(-(n + new) // 16) * 16 for n in lens) + 1024)
+    b.soak(lens[:2], 4, 512)                                  # warm-up: kernels configure themselves
+    dt, steps, pre = b.soak(lens, new, 512)
+    b.close()
+    total = sum(lens) + 16 * new
+    return {"model": "Llama-3-8B shape", "dtype": "bf16", "layers": cfg["num_hidden_layers"], "layers_full": layers_full,
+            "requests": 16, "prompt_tokens": sum(lens), "decode_tokens": 16 * new, "chunk": 512, "steps": steps,
+            "seconds": round(dt, 3), "tokens_per_s": round(total / dt, 1), "decode_tokens_per_s": round(16 * new / dt, 1),
+            "preemptions": pre}
 
-    def decode_run(batch, steps, warmup):
-        """Prefills `batch` prompts (untimed), then times `steps` decode steps."""
-        params = SamplingParams.greedy(warmup + steps + 1, ignore_eos=True)
-        ids = [engine.add_request(gen_tokens(PROMPT_LEN, 1000 + i), params) for i in range(batch)]
-        while any(engine.requests[i].num_computed < PROMPT_LEN for i in ids):
-            engine.step()
-        for _ in range(warmup):
-            engine.step()
-        ctx0 = sum(engine.requests[i].num_tokens for i in ids)
-        sync()
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            engine.step()
-        sync()
-        dt = time.perf_counter() - t0
-        ctx1 = sum(engine.requests[i].num_tokens for i in ids)
-        for i in ids:
-            engine.abort(i)
-        avg_ctx_tokens = (ctx0 + ctx1) / 2.0          # cached tokens read per step, summed over the batch
-        return dt, avg_ctx_tokens
 
-    def prefill_run(reps):
-        times = []
-        for r in range(reps + 1):
-            rid = engine.add_request(gen_tokens(PREFILL_TOKENS, 77 + r), SamplingParams.greedy(1, ignore_eos=True))
-            sync()
-            t0 = time.perf_counter()
-            engine.step()
-            sync()
-            times.append(time.perf_counter() - t0)
-            assert engine.requests[rid].status == "finished"
-        return min(times[1:])
+def soak_llama2_13b(args):
+    """64 requests of 1,024 prompt tokens, 256 greedy tokens each; the cache pool holds them with little to spare."""
+    cfg = dict(LLAMA2_13B)
+    layers_full = cfg["num_hidden_layers"]
+    if args.soak_layers:
+        cfg["num_hidden_layers"] = min(layers_full, args.soak_layers)
+    n_req, prompt, new = 64, 1024, 256
+    pool_tokens = n_req * (prompt + new) + 64 * 16           # one spare page a request
+    b = Bench(cfg, "bf16", n_req, new, 16, budget=2048, max_cache_tokens=pool_tokens)
+    b.soak([prompt] * 2, 4, 2048)
+    dt, steps, pre = b.soak([prompt] * n_req, new, 2048)
+    _, _, kv_per_tok, _ = model_numbers(cfg, 2)
+    b.close()
+    return {"model": "Llama-2-13B shape", "dtype": "bf16", "layers": cfg["num_hidden_layers"], "layers_full": layers_full,
+            "requests": n_req, "prompt_tokens": n_req * prompt, "decode_tokens": n_req * new, "steps": steps,
+            "seconds": round(dt, 3), "tokens_per_s": round(n_req * (prompt + new) / dt, 1),
+            "decode_tokens_per_s": round(n_req * new / dt, 1), "preemptions": pre,
+            "cache_pool_GB": round(pool_tokens * kv_per_tok / 1e9, 1), "cache_pool_fill": round(n_req * (prompt + new) / pool_tokens, 3)}
 
-    # prefill of one 2,048-token prompt in one step, its last logits sampled
-    pf_tokens = PREFILL_TOKENS
-    pf_s = prefill_run(3) if args.only in ("all", "prefill") else float("nan")
-    if args.only == "prefill":
-        print(json.dumps({"prefill_tok_s": round(pf_tokens / pf_s, 1), "ms": round(pf_s * 1e3, 3)}), flush=True)
+
+def run(args):
+    peaks = measure_peaks() if args.only in ("all", "peaks", "headline", "fp32") else None
+    if args.only == "peaks":
+        print(json.dumps({"measured_peaks": peaks}), flush=True)
         return
-    pf_flops = 2.0 * pf_tokens * matmul_params + L * nq * 2.0 * pf_tokens * pf_tokens * hd + 2.0 * V * H
-    pf_frac = pf_flops / pf_s / (PEAK_TFLOPS[args.dtype] * 1e12)
-
-    dt, ctx_tokens = decode_run(args.batch, args.steps, args.warmup)
-    ms_per_step = dt / args.steps * 1e3
-    value = args.batch * args.steps / dt
-    bytes_per_step = weight_bytes + ctx_tokens * kv_per_tok
-    achieved = bytes_per_step / (dt / args.steps) / 1e9
-
-    points = {}
-    for b in ((1, 64) if args.only == "all" else ()):
-        d, _ = decode_run(b, args.steps, args.warmup)
-        points[f"decode_b{b}"] = round(b * args.steps / d, 1)
-
+    if args.only in ("llama3_8b", "llama2_13b"):
+        fn = soak_llama3_8b if args.only == "llama3_8b" else soak_llama2_13b
+        print(json.dumps({args.only: fn(args)}), flush=True)
+        return
+    main_dtype = "fp32" if args.only == "fp32" else args.dtype
+    fig = tinyllama_figures(args, main_dtype, peaks)
+    if args.only == "prefill":
+        print(json.dumps({"prefill_tok_s": fig["prefill"]["value"], "ms": fig["prefill"]["ms"],
+                          "chunked_512": fig["prefill_chunked_512"]}), flush=True)
+        return
+    L, H, I, V, nq, nkv, hd = fig["sizes"]
     line = {
         "metric": "decode tok/s at batch 8, TinyLlama 1.1B shape (prefill tok/s at 2,048 tokens and batch 1/64 beside it)",
-        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": args.dtype, "data": "synthetic: uniform-random token ids, random weights N(0, 0.02)",
-        "config": {"model": "TinyLlama-1.1B shape", "layers": L, "layers_full": layers_full, "hidden": H,
+        "value": round(fig["value"], 1), "unit": "tokens/s", "n_gpus": 1, "steps": fig["steps"], "warmup": fig["warmup"],
+        "ms_per_step": round(fig["ms_per_step"], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": main_dtype, "data": "synthetic: uniform-random token ids, random weights N(0, 0.02)",
+        "config": {"model": "TinyLlama-1.1B shape", "layers": L, "layers_full": TINYLLAMA["num_hidden_layers"], "hidden": H,
                    "heads": nq, "kv_heads": nkv, "head_dim": hd, "intermediate": I, "vocab": V,
-                   "context": cfg["max_position_embeddings"], "global_batch": args.batch, "seq_len": PROMPT_LEN,
-                   "decode_tokens": args.steps, "kv_block_size": args.block_size, "parallelism": "single GPU"},
-        "prefill": {"value": round(pf_tokens / pf_s, 1), "tokens": pf_tokens, "ms": round(pf_s * 1e3, 3),
-                    "frac": round(pf_frac, 4)},
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_GBS, 4)},
-        "points": points,
+                   "context": TINYLLAMA["max_position_embeddings"], "global_batch": args.batch, "seq_len": PROMPT_LEN,
+                   "decode_tokens": fig["steps"], "kv_block_size": args.block_size, "parallelism": "single GPU"},
+        "prefill": fig.get("prefill"), "roofline": fig["roofline"], "points": fig["points"],
     }
+    if "prefill_chunked_512" in fig:
+        line["prefill_chunked_512"] = fig["prefill_chunked_512"]
+    if peaks:
+        line["measured_peaks"] = peaks
+    if args.only == "all":
+        f32 = tinyllama_figures(args, "fp32", peaks)
+        line["fp32"] = {"decode_b8": round(f32["value"], 1), "ms_per_step_b8": round(f32["ms_per_step"], 4),
+                        "decode_b1": f32["points"]["decode_b1"], "decode_b64": f32["points"]["decode_b64"],
+                        "steps": f32["steps"], "prefill": f32["prefill"], "prefill_chunked_512": f32["prefill_chunked_512"],
+                        "roofline_b8": f32["roofline"]}
+        line["workloads"] = {"llama3_8b_mixed16": soak_llama3_8b(args), "llama2_13b_64x1024": soak_llama2_13b(args)}
     print(json.dumps(line), flush=True)
 
 
@@ -143,10 +312,14 @@ def main():
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
-    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration (0: all)")
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the TinyLlama shape has (0: all)")
+    ap.add_argument("--soak-layers", type=int, default=0, help="fewer layers for the two larger shapes (0: all)")
     ap.add_argument("--block-size", type=int, default=16)
-    ap.add_argument("--only", default="all", choices=["all", "decode", "prefill"],
-                    help="profiling aid: time only the decode batch or only the prefill")
+    ap.add_argument("--only", default="all",
+                    choices=["all", "headline", "decode", "prefill", "fp32", "peaks", "llama3_8b", "llama2_13b"],
+                    help="all: everything in one line; headline: the bfloat16 TinyLlama figures only; decode / prefill: "
+                         "one of them (profiling); fp32: the float32 figures as the headline; peaks / llama3_8b / "
+                         "llama2_13b: that part alone")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         if int(os.environ.get("RANK", "0")) == 0:

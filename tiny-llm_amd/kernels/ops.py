@@ -807,3 +807,26 @@ def random_normal(out: torch.Tensor, table: torch.Tensor, key: int, scale: float
                                    c_int(n.bit_length() - 1), c_float(scale), c_float(shift), c_int(_dt(out)),
                                    _stream()), "random_normal")
     return out
+
+
+# ------------------------------------------------------------- measured peaks
+def peak_stream(src: torch.Tensor, dst: Optional[torch.Tensor], sink: torch.Tensor, blocks: int = 2048) -> None:
+    """Streams through `src` (and copies it to `dst` if given): the kernel the measurement
+    program times for the memory bandwidth the machine gives."""
+    _dev(src, dst, sink)
+    nbytes = src.numel() * src.element_size()
+    if not (src.is_contiguous() and nbytes % 16 == 0 and sink.dtype == torch.float32 and sink.numel() >= 1):
+        _fail("the source must be contiguous with a multiple of 16 bytes, the sink float32")
+    if dst is not None and not (dst.is_contiguous() and dst.numel() * dst.element_size() >= nbytes):
+        _fail("the destination must be contiguous and at least as large as the source")
+    _check(_lib().tl_peak_stream(_ptr(src, 16), _ptr(dst, 16), _ptr(sink), c_int64(nbytes), c_int(0 if dst is None else 1),
+                                 c_int(blocks), _stream()), "peak_stream")
+
+
+def peak_mfma(sink: torch.Tensor, dtype: torch.dtype, iters: int, blocks: int = 1024) -> float:
+    """Launches a loop of independent matrix instructions on registers; returns its flops."""
+    _dev(sink)
+    flops = ctypes.c_double(0.0)
+    _check(_lib().tl_peak_mfma(_ptr(sink), c_int(_DT[dtype]), c_int(iters), c_int(blocks), ctypes.byref(flops), _stream()),
+           "peak_mfma")
+    return float(flops.value)
