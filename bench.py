@@ -124,20 +124,25 @@ class Bench:
         Returns (seconds, cached tokens read per step summed over the batch)."""
         from tiny_llm_amd import SamplingParams
         eng = self.engine
-        params = SamplingParams.greedy(warmup + steps + 1, ignore_eos=True)
+        params = SamplingParams.greedy(warmup + steps + 64, ignore_eos=True)      # nobody ends inside the run
         ids = [eng.add_request(gen_tokens(prompt_len, self.V, 1000 + i), params) for i in range(batch)]
-        while any(eng.requests[i].num_computed < prompt_len for i in ids):
+        reqs = [eng.requests[i] for i in ids]
+        while any(r.num_computed < prompt_len for r in reqs):
             eng.step()
-        for _ in range(warmup):
-            eng.step()
-        ctx0 = sum(eng.requests[i].num_tokens for i in ids)
+        run0 = eng.steps_run
+        while eng.steps_run - run0 < warmup:
+            eng.step(max_decode_steps=warmup - (eng.steps_run - run0))
+        ctx0 = sum(r.num_tokens for r in reqs)
+        run0, out0 = eng.steps_run, sum(len(r.output) for r in reqs)
         self.sync()
         t0 = time.perf_counter()
-        for _ in range(steps):
-            eng.step()
+        # exactly `steps` decode steps (the engine chains several of them on the device per call)
+        while eng.steps_run - run0 < steps:
+            eng.step(max_decode_steps=steps - (eng.steps_run - run0))
         self.sync()
         dt = time.perf_counter() - t0
-        ctx1 = sum(eng.requests[i].num_tokens for i in ids)
+        assert eng.steps_run - run0 == steps and sum(len(r.output) for r in reqs) - out0 == steps * batch
+        ctx1 = sum(r.num_tokens for r in reqs)
         for i in ids:
             eng.abort(i)
         return dt, (ctx0 + ctx1) / 2.0
@@ -192,7 +197,7 @@ def tinyllama_figures(args, dtype, peaks):
     steps, warmup = args.steps, args.warmup
     if dtype == "fp32":
         steps, warmup = min(steps, 64), min(warmup, 8)       # the 32-bit path is for checking: a shorter run
-    b = Bench(cfg, dtype, max(args.batch, 64), warmup + steps + 1, args.block_size)
+    b = Bench(cfg, dtype, max(args.batch, 64), warmup + steps + 80, args.block_size)
     out = {}
     if args.only in ("all", "headline", "fp32", "prefill"):
         pf = b.prefill(3)

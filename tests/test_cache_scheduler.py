@@ -400,3 +400,40 @@ def test_reservation_of_a_step_that_did_not_run_is_undone():
     cm.undo_reservation()
     cm.undo_reservation()                               # nothing open: nothing happens
     cm.audit()
+
+
+def test_runs_of_decode_steps_end_where_a_decision_is_due():
+    """How long a run of chained decode steps may be: up to the first request's end by length, never
+    beside a prompt portion or while somebody waits, never beyond the free cache blocks."""
+    cm, s = make_sched(num_blocks=12, block_size=4, max_seqs=2, budget=64, max_len=40, eos=9)
+    s.add(req("a", 6, max_new=20))
+    s.add(req("b", 3, max_new=7))
+    run_plan(cm, s, s.schedule())                          # prompts; one token each
+    p = s.schedule()
+    assert all(e.count == 1 and e.samples for e in p.entries)
+    assert s.burst_length(p, 16) == 6                      # b has 6 of its 7 tokens to go
+    assert s.burst_length(p, 4) == 4 and s.burst_length(p, 1) == 1
+    s.add(req("c", 5))
+    assert s.burst_length(p, 16) == 1                      # somebody waits: decide step by step
+    s.waiting.clear()
+    # the run's blocks are taken at once; its tokens are applied step by step: b ends by eos at step 3
+    k = 6
+    cm.reserve_step([(e.request.req_id, k) for e in p.entries])
+    for e in p.entries:
+        cm.commit(e.request.req_id, e.start + k)
+    by_step = [[7, 7], [7, 7], [7, 9], [7, 1], [7, 2], [7, 3]]
+    done = s.update_burst(p, by_step)
+    a, b = p.entries[0].request, p.entries[1].request
+    assert [r.req_id for r in done] == ["b"] and b.finish_reason == "stop" and b.output == [7, 7, 7, 9]
+    assert a.output == [7] * 7 and a.num_computed == 6 + 6 and a.status == "running"
+    assert not cm.has("b") and cm.num_tokens("a") == 12
+    cm.audit()
+    # not more steps than blocks: a holds 3 blocks (12 tokens), 9 are free
+    p = s.schedule()
+    assert s.burst_length(p, 32) == 13                     # 13 more tokens end its 20
+    cm2, s2 = make_sched(num_blocks=4, block_size=4, max_seqs=2, budget=64, max_len=400)
+    s2.add(req("x", 6, max_new=200))
+    run_plan(cm2, s2, s2.schedule())
+    p2 = s2.schedule()
+    assert s2.burst_length(p2, 10) == 10                   # 6 + 10 = 16 tokens: the pool's 4 blocks
+    assert s2.burst_length(p2, 11) == 1                    # one more does not fit: step by step (and preemption rules)

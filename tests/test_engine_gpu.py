@@ -285,7 +285,8 @@ def test_graph_replays_against_the_plain_model(dtype, graphs, folders):
     prompts = [random_tokens(n, cfg["vocab_size"], 300 + n) for n in (40, 3, 17, 64, 9, 77, 30)]
     sp = [SamplingParams.greedy(n, ignore_eos=True) for n in (50, 20, 35, 8, 44, 12, 25)]     # batch sizes change as they end
     sp[2] = SamplingParams(max_new_tokens=35, temperature=0.9, top_k=20, top_p=0.9, seed=5, ignore_eos=True)
-    eng = Engine(folders["A"], dtype=dtype, max_num_seqs=3, max_num_batched_tokens=32, use_graphs=graphs, **eng_kw)
+    eng = Engine(folders["A"], dtype=dtype, max_num_seqs=3, max_num_batched_tokens=32, use_graphs=graphs,
+                 decode_burst=1, **eng_kw)       # single steps: the logits of every one are looked at
     poison(eng)
     log = spy_on_steps(eng)
     out = eng.generate(prompts, sp)
@@ -320,7 +321,7 @@ def test_decoding_past_the_first_context_bucket(dtype, graphs, tmp_path_factory)
     w, c = read_weights(folder, round_to=act)
     prompts = [random_tokens(n, cfg["vocab_size"], 700 + n) for n in (497, 490, 505)]
     eng = Engine(folder, dtype=dtype, max_num_seqs=4, max_num_batched_tokens=512, use_graphs=graphs,
-                 max_cache_tokens=3 * 576, **eng_kw)
+                 max_cache_tokens=3 * 576, decode_burst=1, **eng_kw)
     poison(eng)
     log = spy_on_steps(eng)
     out = eng.generate(prompts, SamplingParams.greedy(44, ignore_eos=True))
@@ -341,6 +342,36 @@ def test_decoding_past_the_first_context_bucket(dtype, graphs, tmp_path_factory)
 
 
 _folders = {}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_runs_of_decode_steps_chained_on_the_device(dtype, folders):
+    """Decode steps that the device chains by itself (the sampled token fed back, positions, cache
+    slots and sampling counters moved on by a kernel) give the tokens of single steps: across page
+    edges, with requests ending by length and by an end-of-sequence token inside a run, with
+    seeded sampling, and with requests joining and leaving between runs."""
+    from tiny_llm_amd import Engine, SamplingParams
+    cfg, eng_kw, _ = CONFIGS["A"]
+    prompts = [random_tokens(n, cfg["vocab_size"], 800 + n) for n in (40, 3, 17, 64, 9, 30)]
+    sps = [SamplingParams.greedy(n, ignore_eos=True) for n in (70, 33, 50, 21, 64, 45)]
+    sps[2] = SamplingParams(max_new_tokens=50, temperature=0.9, top_k=20, top_p=0.9, seed=5, ignore_eos=True)
+    sps[4] = SamplingParams.greedy(64)                  # may end early: eos is chosen below among its tokens
+    outs = {}
+    for burst in (1, 16, 5):
+        eng = Engine(folders["A"], dtype=dtype, max_num_seqs=4, max_num_batched_tokens=64, decode_burst=burst, **eng_kw)
+        poison(eng)
+        if burst != 1:
+            eng.scheduler.eos_token_id = outs[1][4][37]         # request 4 draws it in the middle of a run
+        outs[burst] = eng.generate(prompts, sps)
+        eng.runner.cache.audit()
+        assert eng.runner.cache.free_blocks() == [g.pool.num_blocks for g in eng.runner.cache.groups]
+        if burst != 1:
+            assert any(g.runs > 20 and g.feeds_next for g in eng.runner._graphs.values())
+    eos = outs[1][4][37]
+    cut = outs[1][4].index(eos) + 1
+    want = [o if i != 4 else o[:cut] for i, o in enumerate(outs[1])]
+    assert outs[16] == want and outs[5] == want
+    assert [len(o) for o in want] == [70, 33, 50, 21, cut, 45]
 
 
 def test_collector_rests_while_a_step_is_captured(folders, monkeypatch):
@@ -419,7 +450,7 @@ def test_preemption_in_bfloat16_with_seeded_sampling(folders):
     prompts = [random_tokens(n, cfg["vocab_size"], 530 + n) for n in (30, 28, 26)]
     sps = [SamplingParams(max_new_tokens=40, temperature=0.8, top_k=40, top_p=0.95, seed=900 + i, ignore_eos=True)
            for i in range(3)]
-    tight = Engine(folders["A"], dtype="bfloat16", max_num_seqs=4, kv_block_size=16, num_kv_blocks=9)
+    tight = Engine(folders["A"], dtype="bfloat16", max_num_seqs=4, kv_block_size=16, num_kv_blocks=9, decode_burst=1)
     poison(tight)
     log = spy_on_steps(tight)
     out = tight.generate(prompts, sps)

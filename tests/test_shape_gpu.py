@@ -120,7 +120,7 @@ def test_generation_across_the_512_bound_at_the_real_layer_sizes(dtype, graphs):
     w = host_weights(act)
     prompts = [random_tokens(n, SHAPE["vocab_size"], 900 + n) for n in (500, 481, 507, 470)]
     eng = Engine(config=SHAPE, dtype=dtype, weights_seed=SEED, init_std=STD, kv_block_size=16, max_num_seqs=4,
-                 max_num_batched_tokens=1024, max_cache_tokens=4 * 576, use_graphs=graphs)
+                 max_num_batched_tokens=1024, max_cache_tokens=4 * 576, use_graphs=graphs, decode_burst=1)
     sharpen(eng.decoder)
     poison(eng)
     log = spy_on_steps(eng)

@@ -225,6 +225,43 @@ __global__ void random_normal_kernel(T* __restrict__ out, int64_t n, uint64_t ke
   }
 }
 
+// ------------------------------------------------- a decode step feeds the next
+// After a decode step's sampler: the chosen token of every request becomes its next input, its
+// position, cached length and sampling counter go up by one, and its cache slot is looked up in
+// the block table for the new position.  A run of decode steps can then be replayed back to back
+// without the host in between; `history` [history_steps, R] keeps what each step chose.
+struct AdvanceArgs {
+  int32_t* tokens;
+  int32_t* positions;
+  int32_t* seq_lens;
+  int32_t* counters;
+  const int32_t* sampled;
+  int32_t* history;
+  int32_t* step;           // how many steps have run since the host last wrote the metadata
+  int R, G, MB, block_size, history_steps;
+  int32_t* slots[4];
+  const int32_t* tables[4];
+};
+
+__global__ void decode_advance_kernel(const AdvanceArgs a) {
+  const int s = *a.step;
+  __syncthreads();          // every thread has read the step before thread 0 moves it on
+  for (int r = threadIdx.x; r < a.R; r += blockDim.x) {
+    const int tok = a.sampled[r];
+    if (s < a.history_steps) a.history[(int64_t)s * a.R + r] = tok;
+    a.tokens[r] = tok;
+    const int p = a.positions[r] + 1;
+    a.positions[r] = p;
+    a.seq_lens[r] += 1;
+    a.counters[r] += 1;
+    for (int g = 0; g < a.G; ++g) {
+      const int blk = max(a.tables[g][(int64_t)r * a.MB + min(p / a.block_size, a.MB - 1)], 0);
+      a.slots[g][r] = blk * a.block_size + p % a.block_size;
+    }
+  }
+  if (threadIdx.x == 0) *a.step = s + 1;
+}
+
 }  // namespace
 
 #define TL_DISPATCH_T(dtype, ...)                 \
@@ -320,6 +357,24 @@ int tl_random_normal(void* out, int64_t n, uint64_t key, const float* table, int
   else
     hipLaunchKernelGGL(random_normal_kernel<bf16_t>, dim3(blocks), dim3(kThreads), 0, stream, (bf16_t*)out, n, key,
                        table, table_bits, scale, shift);
+  return tl_launch_status();
+}
+
+// One workgroup: R requests, G <= 4 cache groups with block tables [R, MB].
+int tl_decode_advance(int32_t* tokens, int32_t* positions, int32_t* seq_lens, int32_t* counters,
+                      const int32_t* sampled, int32_t* history, int32_t* step, int R, int G, int MB, int block_size,
+                      int history_steps, int32_t* const* slots, const int32_t* const* tables, hipStream_t stream) {
+  if (R <= 0) return TL_OK;
+  if (G < 0 || G > 4 || MB <= 0 || block_size <= 0 || history_steps < 0 || !tokens || !positions || !seq_lens ||
+      !counters || !sampled || !history || !step)
+    return TL_ERR_ARG;
+  AdvanceArgs a{tokens, positions, seq_lens, counters, sampled, history, step, R, G, MB, block_size, history_steps, {}, {}};
+  for (int g = 0; g < G; ++g) {
+    if (!slots[g] || !tables[g]) return TL_ERR_ARG;
+    a.slots[g] = slots[g];
+    a.tables[g] = tables[g];
+  }
+  hipLaunchKernelGGL(decode_advance_kernel, dim3(1), dim3(kThreads), 0, stream, a);
   return tl_launch_status();
 }
 

@@ -70,9 +70,11 @@ class Engine:
         return self.scheduler.has_work()
 
     # -------------------------------------------------------------------- step
-    def step(self) -> List[Request]:
-        """One scheduler decision, one forward pass with the sampler at its end.  Returns the
-        requests that finished in this step."""
+    def step(self, max_decode_steps: Optional[int] = None) -> List[Request]:
+        """One scheduler decision and one forward pass with the sampler at its end, or, where every
+        request decodes and nothing has to be decided for a while, a run of up to `decode_burst`
+        such steps that the device chains by itself (`max_decode_steps` bounds the run for this
+        call).  Returns the requests that finished."""
         plan = self.scheduler.schedule()
         done = list(plan.finished)
         if not plan.entries:
@@ -85,6 +87,17 @@ class Engine:
                 p = r.params
                 rows.append(r)
                 samples.append(SampleSpec(p.temperature if p.do_sample else 0.0, p.top_k, p.top_p, r.seed, r.num_tokens))
+        if self.engine_config.use_graphs and self.engine_config.decode_burst > 1:
+            # a run of decode steps without the host in between, where nothing has to be decided
+            most = self.engine_config.decode_burst
+            if max_decode_steps is not None:
+                most = max(1, min(most, max_decode_steps))
+            k = self.scheduler.burst_length(plan, most)
+            by_step = self.runner.run_burst(entries, samples, k) if k > 1 else None
+            if by_step is not None:
+                done += self.scheduler.update_burst(plan, by_step)
+                self.steps_run += k
+                return done
         toks = self.runner.run(entries, samples, use_graph=self.engine_config.use_graphs)
         done += self.scheduler.update(plan, {r.req_id: t for r, t in zip(rows, toks)})
         self.steps_run += 1

@@ -251,6 +251,43 @@ class Scheduler:
             slots_left -= 1
         return StepPlan(entries, preempted, finished)
 
+    def burst_length(self, plan: StepPlan, most: int) -> int:
+        """How many decode steps the plan's requests can run back to back without a decision in
+        between: every entry decodes, nobody waits for admission, and the run ends where the
+        first request reaches its `max_new_tokens` or the model's length, where it would need
+        cache blocks that are not free, or after `most` steps.  (A request that draws an end-of-
+        sequence token inside the run is finished there when the run is over; what it was given
+        after that token is dropped.)"""
+        if most < 2 or self.waiting or plan.preempted or not plan.entries:
+            return 1
+        k = most
+        for e in plan.entries:
+            req = e.request
+            if e.count != 1 or not e.samples:
+                return 1
+            k = min(k, req.params.max_new_tokens - len(req.output), self.max_model_len - req.num_tokens)
+        if k < 2:
+            return 1
+        need = [0] * len(self.cache.groups)
+        for e in plan.entries:
+            for g, n in enumerate(self.cache.blocks_needed(e.request.req_id, e.request.num_computed + k)):
+                need[g] += n
+        if any(n > f for n, f in zip(need, self.cache.free_blocks())):
+            return 1
+        return k
+
+    def update_burst(self, plan: StepPlan, tokens_by_step: Sequence[Sequence[int]]) -> List[Request]:
+        """After a run of decode steps: each step's tokens as `update` would take them; a request
+        that finished at one step takes no part in the later ones."""
+        done: List[Request] = []
+        live = list(range(len(plan.entries)))
+        for k, toks in enumerate(tokens_by_step):
+            entries = [plan.entries[i] for i in live]
+            step_plan = StepPlan([Scheduled(e.request, e.start + k, 1, True) for e in entries], [], [])
+            done += self.update(step_plan, {plan.entries[i].request.req_id: toks[i] for i in live})
+            live = [i for i in live if plan.entries[i].request.status == RUNNING]
+        return done
+
     # ------------------------------------------------------------------ results
     def update(self, plan: StepPlan, sampled: Dict[Hashable, int]) -> List[Request]:
         """After the step ran: advances every scheduled request, appends sampled tokens,

@@ -147,6 +147,7 @@ class Layout:
             for name in ("temperature", "top_p", "top_k", "counters"):
                 add(name, n_out)
             add("seeds", 2 * n_out)         # int64
+            add("burst_step", 1)            # decode steps run on the device since this upload
         self.total = at
 
     def sec(self, buf, name: str):
@@ -277,6 +278,7 @@ def fill_metadata(host: np.ndarray, lay: Layout, rows: Sequence[_Row], block_siz
             fl[o_t + m:o_t + n_out] = 0.0
             fl[o_p + m:o_p + n_out] = 1.0
             tk[m:], ct[m:], sd[m:] = 0, 0, 0
+        lay.sec(host, "burst_step")[0] = 0
 
 
 def token_capacity(n: int, limit: int) -> int:
@@ -320,8 +322,9 @@ class ModelRunner:
         self.eager_steps = 0
 
     # ---------------------------------------------------------------- validation
-    def _resolve(self, entries: Sequence[StepEntry]) -> Tuple[List[_Row], int]:
-        """Checks the entries, takes the cache blocks they need (all or nothing)."""
+    def _resolve(self, entries: Sequence[StepEntry], reserve: int = 0) -> Tuple[List[_Row], int]:
+        """Checks the entries, takes the cache blocks they need (all or nothing); `reserve`: blocks
+        for that many positions per request instead of for the tokens it brings."""
         cm = self.cache
         if not entries:
             raise StepError("a step needs at least one entry")
@@ -341,13 +344,13 @@ class ModelRunner:
                 if not (0 <= int(w) < n):
                     raise StepError(f"wanted place {w} of request {e.req_id!r} is outside its {n} tokens")
             c = cm.num_tokens(e.req_id) if cm.has(e.req_id) else 0
-            if c + n > self.max_model_len:
-                raise StepError(f"request {e.req_id!r} would reach {c + n} tokens, "
+            if c + max(n, reserve) > self.max_model_len:
+                raise StepError(f"request {e.req_id!r} would reach {c + max(n, reserve)} tokens, "
                                 f"the limit is {self.max_model_len}")
             T += n
         if T > self.max_tokens:
             raise StepError(f"step brings {T} tokens, the budget is {self.max_tokens}")
-        ctx_lens = cm.reserve_step([(e.req_id, len(e.tokens)) for e in entries])
+        ctx_lens = cm.reserve_step([(e.req_id, max(len(e.tokens), reserve)) for e in entries])
         G = len(cm.groups)
         rows = [_Row(e.req_id, e.tokens, e.want, c, cm.slot(e.req_id), [cm.block_table(e.req_id, g) for g in range(G)])
                 for e, c in zip(entries, ctx_lens)]
@@ -449,6 +452,37 @@ class ModelRunner:
         self.last_logits = logits
         return out.cpu().tolist()
 
+    def run_burst(self, entries: Sequence[StepEntry], samples: Sequence[SampleSpec], steps: int):
+        """`steps` decode steps back to back without the host in between: every entry is one
+        decoded token whose logits are wanted; after each step the device turns the step's metadata
+        into the next one's (`ops.decode_advance`: sampled token in, position and counter up, cache
+        slot looked up), so only the first step's metadata is uploaded and only the tokens of all
+        steps come back, once.  Cache blocks for all `steps` positions are taken up front.
+        Returns the tokens by step, [steps][entries], or None if these steps cannot run as a burst
+        (no captured graph of this shape yet, too many cache groups): the caller then runs one step."""
+        if steps < 2 or not self.decoder.graph_safe or len(self.cache.groups) > 4:
+            return None
+        if not all(len(e.tokens) == 1 and len(e.want) == 1 for e in entries) or len(samples) != len(entries):
+            return None
+        cm = self.cache
+        new_max = max((cm.num_tokens(e.req_id) if cm.has(e.req_id) else 0) for e in entries) + steps
+        R = len(entries)
+        bound = min(max(512, power_of_two_at_least(new_max)), max(self.max_model_len, 1))
+        sg = self._graphs.get(("decode", R, bound, True))
+        if sg is None or sg.graph is None or new_max > bound or steps > sg.history_steps:
+            return None
+        rows, _ = self._resolve(entries, reserve=steps)
+        try:
+            toks = sg.burst(rows, samples, steps)
+        except BaseException:
+            self.cache.undo_reservation()
+            raise
+        for r in rows:
+            self.cache.commit(r.req_id, r.context_len + steps)
+        self.cache.forget_reservation()
+        self.graph_steps += steps
+        return toks
+
     # ------------------------------------------------------------------ graphs
     def _graph_step(self, entries: Sequence[StepEntry], samples: Optional[Sequence[SampleSpec]]):
         rows, T = self._resolve(entries)
@@ -526,13 +560,44 @@ class StepGraph:
         self.seen = [[None] * self.R for _ in range(G)]
         self.out = torch.zeros(max(self.n_out, 1), dtype=torch.int32, device=runner.device)
         self.out_host = torch.zeros(max(self.n_out, 1), dtype=torch.int32, pin_memory=True)
+        # a decode step with its sampler ends by preparing the next one on the device (bursts)
+        self.feeds_next = self.max_q_len == 1 and self.sampling and self.n_out == self.R == self.T and G <= 4
+        self.history_steps = self.BURST_STEPS if self.feeds_next else 0
+        if self.feeds_next:
+            self.history = torch.zeros(self.history_steps * self.R, dtype=torch.int32, device=runner.device)
+            self.history_host = torch.zeros(self.history_steps * self.R, dtype=torch.int32, pin_memory=True)
         self.graph = None
         self._uploaded: Optional[torch.cuda.Event] = None
+
+    BURST_STEPS = 32        # most decode steps a burst may hold
 
     def _body(self):
         self.logits = self.runner._forward(self.ctx)
         if self.sampling and self.n_out:
             ops.sample(self.logits, self.out[:self.n_out], *self.layout.sampler_args(self.dev))
+        if self.feeds_next:
+            lay, ctx = self.layout, self.ctx
+            ops.decode_advance(ctx.tokens, ctx.positions, ctx.seq_lens, lay.sec(self.dev, "counters"), self.out,
+                               self.history, lay.sec(self.dev, "burst_step"), ctx.slot_mappings,
+                               ctx.block_tables, ctx.block_size)
+
+    def burst(self, rows: Sequence[_Row], samples, steps: int) -> List[List[int]]:
+        """Uploads the first step's metadata and replays the captured step `steps` times; each
+        replay leaves the next step's metadata behind.  Returns the tokens by step."""
+        runner = self.runner
+        if self._uploaded is not None:
+            self._uploaded.synchronize()
+        fill_metadata(self.np, self.layout, rows, runner.cache.block_size, samples, self.seen)
+        self.dev.copy_(self.host, non_blocking=True)
+        for _ in range(steps):
+            self.graph.replay()
+        n = steps * self.R
+        self.history_host[:n].copy_(self.history[:n], non_blocking=True)
+        torch.cuda.current_stream().synchronize()
+        self._uploaded = None
+        self.runs += steps
+        flat = self.history_host[:n].tolist()
+        return [flat[k * self.R:(k + 1) * self.R] for k in range(steps)]
 
     def run(self, rows: Sequence[_Row], samples, n_out: int):
         runner = self.runner

@@ -830,3 +830,32 @@ def peak_mfma(sink: torch.Tensor, dtype: torch.dtype, iters: int, blocks: int = 
     _check(_lib().tl_peak_mfma(_ptr(sink), c_int(_DT[dtype]), c_int(iters), c_int(blocks), ctypes.byref(flops), _stream()),
            "peak_mfma")
     return float(flops.value)
+
+
+def decode_advance(tokens: torch.Tensor, positions: torch.Tensor, seq_lens: torch.Tensor, counters: torch.Tensor,
+                   sampled: torch.Tensor, history: torch.Tensor, step: torch.Tensor, slot_mappings, block_tables,
+                   block_size: int) -> None:
+    """Turns the metadata of a decode step into that of the next one on the device: the sampled
+    token of each request becomes its input, position, cached length and sampling counter go up by
+    one, the cache slot is looked up for the new position.  history [steps, R] records the tokens,
+    `step` (one int32) counts the steps since the host last wrote the metadata."""
+    R = tokens.numel()
+    G = len(slot_mappings)
+    ints = [tokens, positions, seq_lens, counters, sampled, history, step, *slot_mappings, *block_tables]
+    _dev(*ints)
+    for t in ints:
+        if not (t.dtype == torch.int32 and t.is_contiguous()):
+            _fail("decode_advance takes contiguous int32 tensors")
+    if not (G == len(block_tables) and G <= 4):
+        _fail("decode_advance takes up to four cache groups")
+    if not (all(t.numel() == R for t in (positions, seq_lens, counters, *slot_mappings)) and sampled.numel() >= R
+            and step.numel() >= 1 and history.numel() % R == 0):
+        _fail("decode_advance: one element per request in every per-request tensor")
+    if not all(bt.dim() == 2 and bt.shape[0] == R and bt.shape[1] == block_tables[0].shape[1] for bt in block_tables):
+        _fail("block tables must be [requests, max_blocks] of one width")
+    slots_arr = (c_void_p * 4)(*[t.data_ptr() for t in slot_mappings], *[0] * (4 - G))
+    tables_arr = (c_void_p * 4)(*[t.data_ptr() for t in block_tables], *[0] * (4 - G))
+    _check(_lib().tl_decode_advance(_ptr(tokens), _ptr(positions), _ptr(seq_lens), _ptr(counters), _ptr(sampled),
+                                    _ptr(history), _ptr(step), c_int(R), c_int(G),
+                                    c_int(block_tables[0].shape[1] if G else 1), c_int(block_size),
+                                    c_int(history.numel() // R), slots_arr, tables_arr, _stream()), "decode_advance")
