@@ -497,7 +497,7 @@ def _paged_case(dtype, lens, q_lens, nq, nkv, hd, bs, window=0, seed=0, boost=No
                               hd, 1.0 / math.sqrt(hd), window)
     else:
         # query tiles of at most 16 // (nq / nkv) tokens, as the step context builds them
-        per = (16 // (nq // nkv)) * (8 if impl == "prefill" else 1)
+        per = (16 // (nq // nkv)) * ((8 if impl == "prefill" else 4) if impl.startswith("prefill") else 1)
         if tile_tokens is not None:
             per = tile_tokens
         t_req, t_tok0, t_ntok, t = [], [], [], 0
@@ -508,9 +508,11 @@ def _paged_case(dtype, lens, q_lens, nq, nkv, hd, bs, window=0, seed=0, boost=No
                 t_ntok.append(min(per, ql - s0))
             t += ql
         T = q.shape[0]
-        if impl == "prefill":
+        if impl.startswith("prefill"):
+            scratch = torch.full((max(1, n_splits * T * nq * (hd + 2)),), float("nan"), device=DEV)
             ops().flash_prefill(q.to(DEV), kc.to(DEV), vc.to(DEV), bt.to(DEV), (i32(t_req), i32(t_tok0), i32(t_ntok)),
-                                i32(pos), out, nq, nkv, hd, 1.0 / math.sqrt(hd), window)
+                                i32(pos), out, nq, nkv, hd, 1.0 / math.sqrt(hd), window, 8 if impl == "prefill" else 4,
+                                n_splits, scratch)
             return out.reshape(-1, nq, hd), torch.cat(refs)
         scratch = torch.full((max(1, n_splits * T * nq * (hd + 2)),), float("nan"), device=DEV)
         if impl == "f32":       # n_splits stands for the number of 256-key chunks given to workgroups of their own
@@ -566,27 +568,30 @@ def test_flash_attention_mixed_batch(nq, nkv, hd, bs, n_splits):
     assert rel(out, ref) < 8e-3
 
 
+@pytest.mark.parametrize("impl,n_splits", [("prefill", 1), ("prefill4", 1), ("prefill4", 3), ("prefill", 2)])
 @pytest.mark.parametrize("nq,nkv,hd,bs", FLASH_SHAPES)
-def test_flash_prefill_mixed_batch(nq, nkv, hd, bs):
+def test_flash_prefill_mixed_batch(nq, nkv, hd, bs, impl, n_splits):
     out, ref = _paged_case(torch.bfloat16, lens=[123, 107, 65, 1, 300, 2, 513], q_lens=[123, 40, 1, 1, 1, 2, 257],
-                           nq=nq, nkv=nkv, hd=hd, bs=bs, seed=hd + bs, impl="prefill")
+                           nq=nq, nkv=nkv, hd=hd, bs=bs, seed=hd + bs, impl=impl, n_splits=n_splits)
     assert not torch.isnan(out).any()
     assert rel(out, ref) < 8e-3
 
 
 @pytest.mark.parametrize("window", [1, 7, 16, 33, 100])
 def test_flash_prefill_window_edge(window):
-    out, ref = _paged_case(torch.bfloat16, lens=[190, 40, 64, 130], q_lens=[190, 1, 5, 70], nq=4, nkv=2, hd=32,
-                           bs=8, window=window, seed=window, impl="prefill")
-    assert not torch.isnan(out).any()
-    assert rel(out, ref) < 8e-3
+    for n_splits in (1, 2):
+        out, ref = _paged_case(torch.bfloat16, lens=[190, 40, 64, 130], q_lens=[190, 1, 5, 70], nq=4, nkv=2, hd=32,
+                               bs=8, window=window, seed=window, impl="prefill", n_splits=n_splits)
+        assert not torch.isnan(out).any()
+        assert rel(out, ref) < 8e-3
 
 
 def test_flash_prefill_far_key_among_hundreds():
     for far in (0, 15, 16, 63, 64, 255, 256, 511, 699):
-        out, ref = _paged_case(torch.bfloat16, lens=[700], q_lens=[30], nq=8, nkv=1, hd=64, bs=16, seed=far,
-                               boost=far, impl="prefill")
-        assert rel(out, ref) < 8e-3, far
+        for impl, n_splits in (("prefill", 1), ("prefill4", 1), ("prefill4", 4)):
+            out, ref = _paged_case(torch.bfloat16, lens=[700], q_lens=[30], nq=8, nkv=1, hd=64, bs=16, seed=far,
+                                   boost=far, impl=impl, n_splits=n_splits)
+            assert rel(out, ref) < 8e-3, far
 
 
 @pytest.mark.parametrize("n_splits", [1, 2, 7])

@@ -742,16 +742,16 @@ __global__ __launch_bounds__(TL_WAVE) void attention_f32_combine_kernel(const fl
 // with one query tile each rather than four with two: the workgroup with the most keys sets the
 // kernel's duration, and its time per key tile is the work of one wave.
 constexpr int FP_RT = 1;                      // query tiles (of 16 rows) per wave
-constexpr int FP_WAVES = 8, FP_THREADS = FP_WAVES * TL_WAVE;
-constexpr int FP_TILES = FP_WAVES * FP_RT;    // query tiles per workgroup
+// waves (query tiles) of a workgroup: 8, or 4 where 8 would leave compute units without work
 
-template <int HDT>
-__global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
+template <int HDT, int WAVES>
+__global__ __launch_bounds__(WAVES * TL_WAVE) void flash_prefill_bf16_kernel(
     const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ tile_req, const int32_t* __restrict__ tile_tok0,
     const int32_t* __restrict__ tile_ntok, const int32_t* __restrict__ positions, bf16_t* __restrict__ out,
-    int64_t out_stride, int n_tiles, int nq, int nkv, int block_size, int bs_shift, float scale, int window) {
+    int64_t out_stride, float* __restrict__ part_o, float* __restrict__ part_ml, int n_tiles, int n_tokens,
+    int n_splits, int nq, int nkv, int block_size, int bs_shift, float scale, int window) {
   constexpr int HD = HDT * 16;
   constexpr int KS = (HD + 31) / 32;
   constexpr int KP = KS * 32 + 8;
@@ -768,7 +768,7 @@ __global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
   // of them are resident at once when they fit, workgroup i beside workgroup i + half on the same
   // compute unit, and so every compute unit gets about the same number of key tiles.
   const int total = n_tiles * nkv, half = total / 2;
-  const int L = blockIdx.x;
+  const int L = blockIdx.x % total, split = blockIdx.x / total;      // n_splits workgroups share a tile's keys
   const int item = L < half ? L : total - 1 - (L - half);
   const int tile = n_tiles - 1 - item / nkv, kvh = item % nkv;
   const int G = nq / nkv, TW = 16 / G;
@@ -780,7 +780,12 @@ __global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
   const int pos_first = positions[tok0], pos_last = pos_first + ntok - 1;
   const int kv_end = pos_last + 1;
   const int kv_begin = (window > 0 && pos_first + 1 > window) ? pos_first + 1 - window : 0;
-  const int first_tile = kv_begin / FA_KT, last_tile = (kv_end + FA_KT - 1) / FA_KT;
+  int first_tile = kv_begin / FA_KT, last_tile = (kv_end + FA_KT - 1) / FA_KT;
+  if (n_splits > 1) {       // this workgroup's share of the key tiles (possibly none)
+    const int per = (last_tile - first_tile + n_splits - 1) / n_splits;
+    first_tile = min(first_tile + split * per, last_tile);
+    last_tile = min(first_tile + per, last_tile);
+  }
 
   // this lane's query rows, one per query tile of its wave
   bool row_valid[FP_RT];
@@ -847,7 +852,7 @@ __global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
 
   // staging registers: thread = (key row `lane`, chunk group `wave`); the rows of the next tile are
   // requested while the current tile is being worked on
-  constexpr int KC = (KS * 4 + FP_WAVES - 1) / FP_WAVES, VC = (HD / 8 + FP_WAVES - 1) / FP_WAVES;
+  constexpr int KC = (KS * 4 + WAVES - 1) / WAVES, VC = (HD / 8 + WAVES - 1) / WAVES;
   bf16x8 k_stage[KC], v_stage[VC];
   auto fetch_tile = [&](int kt_idx) {
     const int j = kt_idx * FA_KT + lane;
@@ -862,13 +867,13 @@ __global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
     const bf16_t* vp = v_cache + row_off;
 #pragma unroll
     for (int ci = 0; ci < KC; ++ci) {
-      const int c = ci * FP_WAVES + wave;
+      const int c = ci * WAVES + wave;
       bf16x8 z = {};
       k_stage[ci] = (in_range && c * 8 < HD) ? *(const bf16x8*)(kp + c * 8) : z;
     }
 #pragma unroll
     for (int ci = 0; ci < VC; ++ci) {
-      const int c = ci * FP_WAVES + wave;
+      const int c = ci * WAVES + wave;
       bf16x8 z = {};
       v_stage[ci] = (in_range && c < HD / 8) ? *(const bf16x8*)(vp + c * 8) : z;
     }
@@ -879,12 +884,12 @@ __global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
     bf16_t* Vl = Vbuf[buf];
 #pragma unroll
     for (int ci = 0; ci < KC; ++ci) {
-      const int c = ci * FP_WAVES + wave;
+      const int c = ci * WAVES + wave;
       if (c < KS * 4) *(bf16x8*)(Kl + lane * KP + c * 8) = k_stage[ci];
     }
 #pragma unroll
     for (int ci = 0; ci < VC; ++ci) {
-      const int c = ci * FP_WAVES + wave;
+      const int c = ci * WAVES + wave;
       if (c < HD / 8) *(bf16x8*)(Vl + lane * VS + c * 8) = v_stage[ci];
     }
   };
@@ -1020,6 +1025,16 @@ __global__ __launch_bounds__(FP_THREADS) void flash_prefill_bf16_kernel(
   for (int rt = 0; rt < FP_RT; ++rt) {
     if (!row_valid[rt]) continue;
     const float l = l_acc[rt][0];         // every element of the lane's column holds the row's sum
+    if (n_splits > 1) {       // unnormalised, for flash_combine_kernel
+      const int64_t at = ((int64_t)split * n_tokens + tok[rt]) * nq + head;
+#pragma unroll
+      for (int dt = 0; dt < HDT; ++dt) *(f32x4*)(part_o + at * HD + dt * 16 + g * 4) = o[rt][dt];
+      if (g == 0) {
+        part_ml[at * 2] = m_run[rt];
+        part_ml[at * 2 + 1] = l;
+      }
+      continue;
+    }
     const float inv = l > 0.f ? 1.f / l : 0.f;
     bf16_t* orow = out + (int64_t)tok[rt] * out_stride + (int64_t)head * HD + g * 4;
 #pragma unroll
@@ -1215,13 +1230,21 @@ int tl_attention_f32(const float* q, int64_t q_stride, const float* k_cache, con
 }
 
 // bfloat16 only, for steps that hold prompt portions.  Tiles describe groups of at most
-// 8 * (16 / (nq / nkv)) consecutive tokens of one request.
+// tile_waves * (16 / (nq / nkv)) consecutive tokens of one request; tile_waves is 8, or 4 for steps
+// with so few tiles that workgroups of eight waves would leave compute units without work.
 int tl_flash_prefill(const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
                      const int32_t* block_tables, int max_blocks, const int32_t* tile_req,
                      const int32_t* tile_tok0, const int32_t* tile_ntok, const int32_t* positions, void* out,
-                     int64_t out_stride, int n_tiles, int nq, int nkv, int hd, int block_size, float scale,
-                     int window, hipStream_t stream) {
+                     int64_t out_stride, float* part_o, float* part_ml, int n_tiles, int n_tokens, int nq, int nkv,
+                     int hd, int block_size, float scale, int window, int tile_waves, int n_splits,
+                     hipStream_t stream) {
   if (n_tiles <= 0) return TL_OK;
+  if (tile_waves != 8 && tile_waves != 4) return TL_ERR_ARG;
+  // n_splits > 1: the key tiles of a query tile are shared out over that many workgroups, whose
+  // results (part_o [n_splits, n_tokens, nq, hd], part_ml [n_splits, n_tokens, nq, 2]) a second kernel merges
+  if (n_splits < 1 || n_splits > 64 || n_tokens <= 0 || (n_splits > 1 && (!part_o || !part_ml)) ||
+      (int64_t)n_tiles * nkv * n_splits > 0x7fffffff)
+    return TL_ERR_ARG;
   if (nq <= 0 || nkv <= 0 || nq % nkv || nq / nkv > 16 || hd <= 0 || hd % 16 || hd > 128 || block_size <= 0 ||
       max_blocks <= 0 || window < 0 || nkv > 65535 || (int64_t)n_tiles * nkv > 0x7fffffff || q_stride % 8 ||
       out_stride % 4)
@@ -1229,18 +1252,31 @@ int tl_flash_prefill(const void* q, int64_t q_stride, const void* k_cache, const
   int bs_shift = -1;      // log2 of the page size where it is a power of two
   for (int sh = 0; sh < 31; ++sh)
     if ((1 << sh) == block_size) bs_shift = sh;
-#define TL_PREFILL_CASE(HDT)                                                                                      \
-  case HDT:                                                                                                       \
-    hipLaunchKernelGGL(flash_prefill_bf16_kernel<HDT>, dim3(n_tiles * nkv), dim3(FP_THREADS), 0, stream,          \
-                       (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,  \
-                       max_blocks, tile_req, tile_tok0, tile_ntok, positions, (bf16_t*)out, out_stride, n_tiles,  \
-                       nq, nkv, block_size, bs_shift, scale, window);                                             \
+#define TL_PREFILL_LAUNCH(HDT, W)                                                                                 \
+  hipLaunchKernelGGL((flash_prefill_bf16_kernel<HDT, W>), dim3(n_tiles * nkv * n_splits), dim3(W * TL_WAVE), 0,   \
+                     stream, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,          \
+                     block_tables, max_blocks, tile_req, tile_tok0, tile_ntok, positions, (bf16_t*)out,           \
+                     out_stride, part_o, part_ml, n_tiles, n_tokens, n_splits, nq, nkv, block_size, bs_shift,     \
+                     scale, window)
+#define TL_PREFILL_CASE(HDT)                        \
+  case HDT:                                         \
+    if (tile_waves == 8) TL_PREFILL_LAUNCH(HDT, 8); \
+    else TL_PREFILL_LAUNCH(HDT, 4);                 \
     break;
   switch (hd / 16) {
     TL_PREFILL_CASE(1) TL_PREFILL_CASE(2) TL_PREFILL_CASE(3) TL_PREFILL_CASE(4)
     TL_PREFILL_CASE(5) TL_PREFILL_CASE(6) TL_PREFILL_CASE(7) TL_PREFILL_CASE(8)
   }
 #undef TL_PREFILL_CASE
+#undef TL_PREFILL_LAUNCH
+#define TL_COMBINE(B)                                                                                          \
+  hipLaunchKernelGGL(flash_combine_kernel<B>, dim3(n_tokens, nq), dim3(TL_WAVE), 0, stream, part_o, part_ml, \
+                     (bf16_t*)out, out_stride, n_tokens, nq, hd, n_splits)
+  if (n_splits > 8) TL_COMBINE(16);
+  else if (n_splits > 4) TL_COMBINE(8);
+  else if (n_splits > 2) TL_COMBINE(4);
+  else if (n_splits > 1) TL_COMBINE(2);
+#undef TL_COMBINE
   return tl_launch_status();
 }
 

@@ -503,8 +503,10 @@ class ModelRunner:
                 R_cap = min(power_of_two_at_least(R), max(self.cache.max_seqs, R))
                 # every row may be wanted (replay), or at most one per request (serving)
                 n_cap = R_cap if n_out <= R_cap and samples is not None else T_cap
-                key = ("mixed", T_cap, R_cap, n_cap, samples is not None)
-                caps = (T_cap, R_cap, n_cap, T_cap, self.max_model_len)
+                # the bound on the context decides whether attention shares a tile's keys out
+                bound = max(min(max(512, power_of_two_at_least(max(new_lens))), max(self.max_model_len, 1)), max(new_lens))
+                key = ("mixed", T_cap, R_cap, n_cap, bound, samples is not None)
+                caps = (T_cap, R_cap, n_cap, T_cap, bound)
             sg = self._graphs.get(key)
             if sg is None:
                 sg = self._graphs[key] = StepGraph(self, *caps, sampling=samples is not None)

@@ -730,12 +730,35 @@ _WAVES: dict = {}
 PREFILL_TILES = 8     # query tiles (of 16 rows) one workgroup of the prefill attention kernel owns
 
 
+def prefill_key_splits(num_tokens: int, max_seq_len: int, num_heads: int, num_kv_heads: int, tile_waves: int) -> int:
+    """Over how many workgroups `flash_prefill` shares the key tiles of a query tile out: 1 unless the
+    step has few query tiles (at most two workgroups a compute unit) and contexts of 8 key tiles and more;
+    then one split per 8 key tiles of the longest context, at most 4."""
+    tiles = -(-num_tokens // (tile_waves * (16 // (num_heads // num_kv_heads))))
+    key_tiles = -(-max_seq_len // 64)
+    if tiles * num_kv_heads > 512 or key_tiles < 16:
+        return 1
+    return max(1, min(4, key_tiles // 8, 1024 // max(1, tiles * num_kv_heads)))
+
+
+def prefill_tile_waves(num_tokens: int, num_heads: int, num_kv_heads: int) -> int:
+    """Waves (query tiles of 16 rows) per workgroup of `flash_prefill` for a step of `num_tokens`:
+    eight, or four where eight would give fewer workgroups than the chip has compute units."""
+    per_tile = PREFILL_TILES * (16 // (num_heads // num_kv_heads))
+    return 8 if -(-num_tokens // per_tile) * num_kv_heads >= 256 else 4
+
+
 def flash_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                   tiles, positions: torch.Tensor, out: torch.Tensor, num_heads: int, num_kv_heads: int,
-                  head_dim: int, scale: float, window: int = 0) -> torch.Tensor:
+                  head_dim: int, scale: float, window: int = 0, tile_waves: int = 8, n_splits: int = 1,
+                  scratch: Optional[torch.Tensor] = None) -> torch.Tensor:
     """`flash_attention` arranged for prompt portions: `tiles` are groups of at most
-    PREFILL_TILES * (16 // (heads / kv_heads)) consecutive tokens of one request, and a key or value
-    row is staged once per such group."""
+    tile_waves * (16 // (heads / kv_heads)) consecutive tokens of one request, and a key or value
+    row is staged once per such group.  tile_waves is PREFILL_TILES (8), or 4 for steps with few
+    tokens, where workgroups of eight waves would leave compute units without work
+    (`prefill_tile_waves`).  n_splits > 1 shares a group's key tiles out over that many workgroups
+    (few query rows over long contexts: a portion late in a long prompt) and needs float32 `scratch`
+    of n_splits * T * heads * (head_dim + 2) elements for their results, which a second kernel merges."""
     tile_req, tile_tok0, tile_ntok = tiles
     _dev(q, k_cache, v_cache, block_tables, tile_req, tile_tok0, tile_ntok, positions, out)
     _rows_2d(q, "q")
@@ -762,11 +785,22 @@ def flash_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
             _fail("tile arrays must be int32 [tiles]")
     if not (q.stride(0) % 8 == 0 and out.stride(0) % 4 == 0):
         _fail("q and output rows must be vector aligned")
+    part_o = part_ml = None
+    if n_splits > 1:
+        need = n_splits * T * num_heads * (head_dim + 2)
+        _dev(scratch)
+        if not (scratch is not None and scratch.dtype == torch.float32 and scratch.is_contiguous()
+                and scratch.numel() >= need):
+            _fail(f"split attention needs {need} float32 of scratch")
+        part_o = scratch[:n_splits * T * num_heads * head_dim]
+        part_ml = scratch[n_splits * T * num_heads * head_dim:]
     _check(_lib().tl_flash_prefill(
         _ptr(q, 16), c_int64(q.stride(0)), _ptr(k_cache, 16), _ptr(v_cache, 16), _ptr(block_tables),
         c_int(block_tables.shape[1]), _ptr(tile_req), _ptr(tile_tok0), _ptr(tile_ntok), _ptr(positions),
-        _ptr(out, 8), c_int64(out.stride(0)), c_int(n_tiles), c_int(num_heads), c_int(num_kv_heads),
-        c_int(head_dim), c_int(k_cache.shape[2]), c_float(scale), c_int(window), _stream()), "flash_prefill")
+        _ptr(out, 8), c_int64(out.stride(0)), _ptr(part_o, 16), _ptr(part_ml), c_int(n_tiles), c_int(T),
+        c_int(num_heads), c_int(num_kv_heads),
+        c_int(head_dim), c_int(k_cache.shape[2]), c_float(scale), c_int(window), c_int(tile_waves), c_int(n_splits),
+        _stream()), "flash_prefill")
     return out
 
 

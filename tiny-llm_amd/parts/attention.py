@@ -92,9 +92,17 @@ class Attention(Mixer):
                            cache.v if cache.write else None, self.num_heads, self.num_kv_heads, self.head_dim, rot)
         if flash and ctx.max_q_len > 1:
             # prompt portions: many query rows share each staged key tile
-            tiles = ctx.attention_tiles(ops.PREFILL_TILES * (16 // group))
+            waves = ops.prefill_tile_waves(T, self.num_heads, self.num_kv_heads)
+            tiles = ctx.attention_tiles(waves * (16 // group))
+            # a portion late in a long prompt: few query rows, many keys; the keys are shared out
+            n_splits = ops.prefill_key_splits(T, ctx.max_seq_len, self.num_heads, self.num_kv_heads, waves)
+            scratch = None
+            if n_splits > 1:
+                scratch = ops.scratch("attention_partials", (n_splits * T * self.num_heads * (self.head_dim + 2),),
+                                      torch.float32, residual.device)
             ops.flash_prefill(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, attn,
-                              self.num_heads, self.num_kv_heads, self.head_dim, self.scale, self.window)
+                              self.num_heads, self.num_kv_heads, self.head_dim, self.scale, self.window, waves,
+                              n_splits, scratch)
         elif flash:
             # decoding: one token per request, its keys split over the waves of a workgroup (and over
             # workgroups when the context is long)
