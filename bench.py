@@ -269,7 +269,78 @@ def soak_llama2_13b(args):
             "cache_pool_GB": round(pool_tokens * kv_per_tok / 1e9, 1), "cache_pool_fill": round(n_req * (prompt + new) / pool_tokens, 3)}
 
 
+def host_time(args):
+    """Wall time of a step against the time its captured graph takes on the GPU (events around every
+    replay): decode at batch 64, 8 and 1, and mixed steps of 64 tokens (8 decoded tokens beside 56 of a
+    prompt).  What is left is the host's share: scheduling, metadata, upload, download."""
+    import torch
+    from tiny_llm_amd import SamplingParams
+    spans = []
+    replay = torch.cuda.CUDAGraph.replay
+
+    def timed(self):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        replay(self)
+        e1.record()
+        spans.append((e0, e1))
+
+    torch.cuda.CUDAGraph.replay = timed
+    out = {}
+    try:
+        b = Bench(dict(TINYLLAMA), "bf16", 64, 400, args.block_size, budget=4096)
+        eng = b.engine
+        for batch in (64, 8, 1):
+            ids = [eng.add_request(gen_tokens(PROMPT_LEN, b.V, 1000 + i), SamplingParams.greedy(300, ignore_eos=True))
+                   for i in range(batch)]
+            reqs = [eng.requests[i] for i in ids]
+            while any(r.num_computed < PROMPT_LEN for r in reqs):
+                eng.step()
+            for _ in range(4):
+                eng.step()
+            spans.clear()
+            run0 = eng.steps_run
+            b.sync()
+            t0 = time.perf_counter()
+            while eng.steps_run - run0 < 128:
+                eng.step(max_decode_steps=128 - (eng.steps_run - run0))
+            b.sync()
+            wall = (time.perf_counter() - t0) / 128 * 1e3
+            gpu = sum(a.elapsed_time(c) for a, c in spans) / len(spans)
+            out[f"decode_b{batch}"] = {"wall_ms": round(wall, 4), "gpu_ms": round(gpu, 4), "host_ms": round(wall - gpu, 4),
+                                       "steps_per_call": eng.engine_config.decode_burst}
+            for i in ids:
+                eng.abort(i)
+        eng.scheduler.budget = 64
+        ids = [eng.add_request(gen_tokens(100, b.V, 2000 + i), SamplingParams.greedy(400, ignore_eos=True)) for i in range(8)]
+        while any(eng.requests[i].num_computed < 100 for i in ids):
+            eng.step()
+        for trial in range(2):          # the first pass captures the graphs of these shapes of step, the second is timed
+            long_id = eng.add_request(gen_tokens(1800, b.V, 77 + trial), SamplingParams.greedy(2, ignore_eos=True))
+            for _ in range(4):
+                eng.step()
+            spans.clear()
+            b.sync()
+            t0 = time.perf_counter()
+            n = 0
+            while eng.requests[long_id].num_computed < 1700:
+                eng.step()
+                n += 1
+            b.sync()
+            wall = (time.perf_counter() - t0) / n * 1e3
+            gpu = sum(a.elapsed_time(c) for a, c in spans) / max(1, len(spans))
+            eng.abort(long_id)
+        out["mixed_64_tokens"] = {"wall_ms": round(wall, 4), "gpu_ms": round(gpu, 4), "ratio": round(wall / gpu, 3), "steps": n}
+        b.close()
+    finally:
+        torch.cuda.CUDAGraph.replay = replay
+    return out
+
+
 def run(args):
+    if args.only == "host":
+        print(json.dumps({"host_time": host_time(args)}), flush=True)
+        return
     peaks = measure_peaks() if args.only in ("all", "peaks", "headline", "fp32") else None
     if args.only == "peaks":
         print(json.dumps({"measured_peaks": peaks}), flush=True)
@@ -321,10 +392,10 @@ def main():
     ap.add_argument("--soak-layers", type=int, default=0, help="fewer layers for the two larger shapes (0: all)")
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--only", default="all",
-                    choices=["all", "headline", "decode", "prefill", "fp32", "peaks", "llama3_8b", "llama2_13b"],
+                    choices=["all", "headline", "decode", "prefill", "fp32", "peaks", "llama3_8b", "llama2_13b", "host"],
                     help="all: everything in one line; headline: the bfloat16 TinyLlama figures only; decode / prefill: "
                          "one of them (profiling); fp32: the float32 figures as the headline; peaks / llama3_8b / "
-                         "llama2_13b: that part alone")
+                         "llama2_13b: that part alone; host: a step's wall time against its time on the GPU")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         if int(os.environ.get("RANK", "0")) == 0:
