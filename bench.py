@@ -249,6 +249,22 @@ def soak_llama3_8b(args):
             "preemptions": pre}
 
 
+def prefill_llama3_8b(args):
+    """Whole prompts of 4,096 and 8,192 tokens at the Llama-3-8B shape, one step each."""
+    cfg = dict(LLAMA3_8B)
+    layers_full = cfg["num_hidden_layers"]
+    if args.soak_layers:
+        cfg["num_hidden_layers"] = min(layers_full, args.soak_layers)
+    b = Bench(cfg, "bf16", 1, 1, 16, budget=8192, max_cache_tokens=8192 + 256)
+    out = {"model": "Llama-3-8B shape", "dtype": "bf16", "layers": cfg["num_hidden_layers"], "layers_full": layers_full}
+    for tokens in (4096, 8192):
+        dt = b.prefill(2, tokens=tokens, budget=tokens)
+        out[f"tokens_{tokens}"] = {"ms": round(dt * 1e3, 2), "value": round(tokens / dt, 1),
+                                   "frac": round(prefill_flops(cfg, tokens) / dt / (PEAK_TFLOPS["bf16"] * 1e12), 4)}
+    b.close()
+    return out
+
+
 def soak_llama2_13b(args):
     """64 requests of 1,024 prompt tokens, 256 greedy tokens each; the cache pool holds them with little to spare."""
     cfg = dict(LLAMA2_13B)
@@ -345,8 +361,8 @@ def run(args):
     if args.only == "peaks":
         print(json.dumps({"measured_peaks": peaks}), flush=True)
         return
-    if args.only in ("llama3_8b", "llama2_13b"):
-        fn = soak_llama3_8b if args.only == "llama3_8b" else soak_llama2_13b
+    if args.only in ("llama3_8b", "llama2_13b", "llama3_8b_prefill"):
+        fn = {"llama3_8b": soak_llama3_8b, "llama2_13b": soak_llama2_13b, "llama3_8b_prefill": prefill_llama3_8b}[args.only]
         print(json.dumps({args.only: fn(args)}), flush=True)
         return
     main_dtype = "fp32" if args.only == "fp32" else args.dtype
@@ -377,7 +393,8 @@ def run(args):
                         "decode_b1": f32["points"]["decode_b1"], "decode_b64": f32["points"]["decode_b64"],
                         "steps": f32["steps"], "prefill": f32["prefill"], "prefill_chunked_512": f32["prefill_chunked_512"],
                         "roofline_b8": f32["roofline"]}
-        line["workloads"] = {"llama3_8b_mixed16": soak_llama3_8b(args), "llama2_13b_64x1024": soak_llama2_13b(args)}
+        line["workloads"] = {"llama3_8b_mixed16": soak_llama3_8b(args), "llama3_8b_prefill": prefill_llama3_8b(args),
+                             "llama2_13b_64x1024": soak_llama2_13b(args)}
     print(json.dumps(line), flush=True)
 
 
@@ -392,7 +409,7 @@ def main():
     ap.add_argument("--soak-layers", type=int, default=0, help="fewer layers for the two larger shapes (0: all)")
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--only", default="all",
-                    choices=["all", "headline", "decode", "prefill", "fp32", "peaks", "llama3_8b", "llama2_13b", "host"],
+                    choices=["all", "headline", "decode", "prefill", "fp32", "peaks", "llama3_8b", "llama3_8b_prefill", "llama2_13b", "host"],
                     help="all: everything in one line; headline: the bfloat16 TinyLlama figures only; decode / prefill: "
                          "one of them (profiling); fp32: the float32 figures as the headline; peaks / llama3_8b / "
                          "llama2_13b: that part alone; host: a step's wall time against its time on the GPU")

@@ -354,6 +354,28 @@ def test_linear_row_alone_equals_row_in_batch_fp32(K, N):
         assert rel(full, ref) < 1e-5
 
 
+def test_linear_fp32_tile_shapes_give_the_same_bits():
+    """The float32 product picks 128 x 128 tiles for 1100 x 2100 outputs, 64 x 64 tiles for a
+    512-row slice of them and the few-row kernel for a single row: one order of addition in all."""
+    g = torch.Generator().manual_seed(77)
+    K, N = 520, 2100
+    a = torch.randn(1100, K, generator=g).to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(DEV)
+    res = torch.randn(1100, N, generator=g).to(DEV)
+    def run(rows, residual):
+        x = a[rows].contiguous()
+        out = torch.empty(x.shape[0], N, device=DEV)
+        ops().linear(x, w, out, res[rows].contiguous() if residual else None)
+        return out
+    for residual in (False, True):
+        full = run(slice(0, 1100), residual)
+        assert torch.equal(full[100:612], run(slice(100, 612), residual))
+        assert torch.equal(full[5:6], run(slice(5, 6), residual))
+        assert torch.equal(full[1000:1100], run(slice(1000, 1100), residual))
+        ref = a.double() @ w.double().T + (res.double() if residual else 0)
+        assert rel(full, ref) < 1e-5
+
+
 def test_linear_refuses_bad_inner_size_in_bf16():
     from tiny_llm_amd.kernels import KernelError
     a = torch.zeros(4, 12, dtype=torch.bfloat16, device=DEV)

@@ -27,7 +27,7 @@ namespace {
 //     one for each of the four instructions);
 //   * operands beyond K are zero.
 constexpr int F_KBLOCK = 256;     // the k block of the order of addition
-constexpr int F_BM = 128, F_BN = 128, F_BK = 16, F_THREADS = 256;
+constexpr int F_BK = 16, F_THREADS = 256;
 constexpr int F_LD = F_BK + 4;    // LDS row stride in floats (80 bytes: 16-byte aligned rows)
 
 // silu(g) * u of an interleaved gate|up pair of output columns, as the reference computes it
@@ -54,46 +54,56 @@ __device__ __forceinline__ f32x4 load_k4(const float* __restrict__ row, int k, i
   return v;
 }
 
-// Tiles of 128 rows x 128 columns, four waves of 64 x 64 (4 x 4 matrix tiles of 16 x 16), k in
-// steps of 16 through double-buffered LDS.  The matrix instruction's rows are the output COLUMNS
-// (weights are its first operand), so a lane ends up with four consecutive columns of one row.
-template <bool SWIGLU, bool VEC>
+// Tiles of 32 T rows x 32 T columns, four waves of 16 T x 16 T (T x T matrix tiles of 16 x 16), k in
+// steps of 16 through double-buffered LDS.  T = 4 (128 x 128) where that gives the chip enough
+// tiles, T = 2 (64 x 64) where it does not (a portion of 512 tokens times 2048 columns is 64 tiles
+// of 128 x 128 for 256 compute units); the order in which an output element is added up is the
+// same for every T.  The matrix instruction's rows are the output COLUMNS (weights are its first
+// operand), so a lane ends up with four consecutive columns of one row.
+template <bool SWIGLU, bool VEC, int T>
 __global__ __launch_bounds__(F_THREADS) void gemm_f32_kernel(const float* __restrict__ a,
                                                              const float* __restrict__ w,
                                                              float* __restrict__ out,
                                                              const float* __restrict__ residual, int M,
                                                              int N, int K, int64_t lda, int64_t ldo) {
-  __shared__ __attribute__((aligned(16))) float As[2][F_BM * F_LD];
-  __shared__ __attribute__((aligned(16))) float Ws[2][F_BN * F_LD];
+  constexpr int BT = 32 * T;        // rows and columns of the workgroup's tile
+  constexpr int PIECES = BT / 64;   // 16-byte pieces of each operand per thread and k step
+  static_assert(T == 2 || T == 4, "tiles of 64 x 64 or 128 x 128");
+  __shared__ __attribute__((aligned(16))) float As[2][BT * F_LD];
+  __shared__ __attribute__((aligned(16))) float Ws[2][BT * F_LD];
   const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
   const int wm = wave / 2, wn = wave % 2;
-  const int m0 = blockIdx.y * F_BM, n0 = blockIdx.x * F_BN;
+  const int m0 = blockIdx.y * BT, n0 = blockIdx.x * BT;
   const int l16 = lane % 16, kk = lane / 16;
-  // staging: thread = (row tid / 2, k half tid % 2), two groups of four k each
-  const int sr = tid / 2, sk = (tid % 2) * 8;
-  const float* arow = a + (int64_t)min(m0 + sr, M - 1) * lda;
-  const float* wrow = w + (int64_t)min(n0 + sr, N - 1) * K;
-  f32x4 acc[4][4], tot[4][4];
+  // staging: piece h of a thread is row (h * 256 + tid) / 4 of the tile, four k from 4 * (tid % 4)
+  const int sr = tid / 4, sk = (tid % 4) * 4;
+  const float *arow[PIECES], *wrow[PIECES];
 #pragma unroll
-  for (int nt = 0; nt < 4; ++nt)
+  for (int h = 0; h < PIECES; ++h) {
+    arow[h] = a + (int64_t)min(m0 + h * 64 + sr, M - 1) * lda;
+    wrow[h] = w + (int64_t)min(n0 + h * 64 + sr, N - 1) * K;
+  }
+  f32x4 acc[T][T], tot[T][T];
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
+  for (int nt = 0; nt < T; ++nt)
+#pragma unroll
+    for (int mt = 0; mt < T; ++mt) {
       acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
       tot[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
-  f32x4 ga[2], gw[2];
+  f32x4 ga[PIECES], gw[PIECES];
   auto fetch = [&](int k0) {
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      ga[h] = load_k4<VEC>(arow, k0 + sk + 4 * h, K);
-      gw[h] = load_k4<VEC>(wrow, k0 + sk + 4 * h, K);
+    for (int h = 0; h < PIECES; ++h) {
+      ga[h] = load_k4<VEC>(arow[h], k0 + sk, K);
+      gw[h] = load_k4<VEC>(wrow[h], k0 + sk, K);
     }
   };
   auto stage = [&](int buf) {
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      *(f32x4*)(&As[buf][sr * F_LD + sk + 4 * h]) = ga[h];
-      *(f32x4*)(&Ws[buf][sr * F_LD + sk + 4 * h]) = gw[h];
+    for (int h = 0; h < PIECES; ++h) {
+      *(f32x4*)(&As[buf][(h * 64 + sr) * F_LD + sk]) = ga[h];
+      *(f32x4*)(&Ws[buf][(h * 64 + sr) * F_LD + sk]) = gw[h];
     }
   };
   fetch(0);
@@ -103,24 +113,24 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f32_kernel(const float* __rest
   for (int s = 0; s < steps; ++s) {
     const int buf = s & 1;
     if (s + 1 < steps) fetch((s + 1) * F_BK);
-    f32x4 wv[4], av[4];
+    f32x4 wv[T], av[T];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      wv[t] = *(const f32x4*)(&Ws[buf][(wn * 64 + t * 16 + l16) * F_LD + kk * 4]);
-      av[t] = *(const f32x4*)(&As[buf][(wm * 64 + t * 16 + l16) * F_LD + kk * 4]);
+    for (int t = 0; t < T; ++t) {
+      wv[t] = *(const f32x4*)(&Ws[buf][(wn * 16 * T + t * 16 + l16) * F_LD + kk * 4]);
+      av[t] = *(const f32x4*)(&As[buf][(wm * 16 * T + t * 16 + l16) * F_LD + kk * 4]);
     }
 #pragma unroll
     for (int e = 0; e < 4; ++e)
 #pragma unroll
-      for (int nt = 0; nt < 4; ++nt)
+      for (int nt = 0; nt < T; ++nt)
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt)
+        for (int mt = 0; mt < T; ++mt)
           acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv[nt][e], av[mt][e], acc[nt][mt], 0, 0, 0);
     if (((s + 1) * F_BK) % F_KBLOCK == 0 || s + 1 == steps) {     // a block of the order of addition ends
 #pragma unroll
-      for (int nt = 0; nt < 4; ++nt)
+      for (int nt = 0; nt < T; ++nt)
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt) {
+        for (int mt = 0; mt < T; ++mt) {
           tot[nt][mt] += acc[nt][mt];
           acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
@@ -130,12 +140,12 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f32_kernel(const float* __rest
   }
   // lane (l16, kk) of tile (nt, mt) holds row m = mt*16 + l16, columns n = nt*16 + 4 kk + r
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt) {
-    const int m = m0 + wm * 64 + mt * 16 + l16;
+  for (int mt = 0; mt < T; ++mt) {
+    const int m = m0 + wm * 16 * T + mt * 16 + l16;
     if (m >= M) continue;
 #pragma unroll
-    for (int nt = 0; nt < 4; ++nt) {
-      const int n = n0 + wn * 64 + nt * 16 + kk * 4;
+    for (int nt = 0; nt < T; ++nt) {
+      const int n = n0 + wn * 16 * T + nt * 16 + kk * 4;
       const f32x4 v = tot[nt][mt];
       if constexpr (SWIGLU) {   // columns (2j, 2j+1) = (gate_j, up_j); N is even
 #pragma unroll
@@ -1219,10 +1229,21 @@ int tl_linear_tile(const void* a, const void* w, void* out, const float* residua
 #undef TL_F32_ROWS
       return tl_launch_status();
     }
-    dim3 g((N + F_BN - 1) / F_BN, (M + F_BM - 1) / F_BM);
-#define TL_F32_TILED(SW, VE)                                                                                  \
-  hipLaunchKernelGGL((gemm_f32_kernel<SW, VE>), g, dim3(F_THREADS), 0, stream, (const float*)a, (const float*)w, \
-                     (float*)out, residual, M, N, K, lda, ldo)
+    // 128 x 128 tiles, or 64 x 64 where those take fewer rounds of workgroups over the 256 compute
+    // units even at 0.6 of the larger tile's rate (it fetches twice the operand bytes per flop)
+    const int64_t big = ceil_div64(N, 128) * ceil_div64(M, 128), small = ceil_div64(N, 64) * ceil_div64(M, 64);
+    const bool use_small = (double)ceil_div64(small, 256) / (4 * 0.6) < (double)ceil_div64(big, 256);
+    const int bt = use_small ? 64 : 128;
+    dim3 g((N + bt - 1) / bt, (M + bt - 1) / bt);
+#define TL_F32_TILED(SW, VE)                                                                                        \
+  do {                                                                                                              \
+    if (use_small)                                                                                                  \
+      hipLaunchKernelGGL((gemm_f32_kernel<SW, VE, 2>), g, dim3(F_THREADS), 0, stream, (const float*)a,              \
+                         (const float*)w, (float*)out, residual, M, N, K, lda, ldo);                                \
+    else                                                                                                            \
+      hipLaunchKernelGGL((gemm_f32_kernel<SW, VE, 4>), g, dim3(F_THREADS), 0, stream, (const float*)a,              \
+                         (const float*)w, (float*)out, residual, M, N, K, lda, ldo);                                \
+  } while (0)
     if (swiglu && vec) TL_F32_TILED(true, true);
     else if (swiglu) TL_F32_TILED(true, false);
     else if (vec) TL_F32_TILED(false, true);
