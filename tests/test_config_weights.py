@@ -281,6 +281,40 @@ def test_tied_head_is_not_stored_and_shares_the_table(tmp_path):
     assert 0.03 < float(norm.std()) < 0.3 and abs(float(norm.mean()) - 1) < 0.1
 
 
+@pytest.mark.parametrize("cfg", [TINY_A, TINY_B])
+def test_all_resident_weights_lie_in_one_slab(cfg, tmp_path):
+    """Every tensor a part holds after loading is a view of ONE allocation, at a 256-byte boundary;
+    a tied head is the embedding's view, not a second copy; nothing is left outside; and the values
+    are the file's (fused, interleaved or as they came)."""
+    folder = write_random_model(str(tmp_path), cfg, seed=4, norm_std=0.1)
+    f = SafetensorsFile(os.path.join(folder, "model.safetensors"))
+    dec = _specs(cfg)
+    load_weights(dec, folder)
+    slab = dec.weight_slab
+    lo, hi = slab.buffer.data_ptr(), slab.buffer.data_ptr() + slab.buffer.numel()
+    held, seen = 0, set()
+    for part in dec.parts():
+        for name, t in vars(part).items():
+            if not isinstance(t, torch.Tensor):
+                continue
+            assert lo <= t.data_ptr() and t.data_ptr() + t.numel() * t.element_size() <= hi, (part.prefix, name)
+            assert (t.data_ptr() - lo) % 256 == 0
+            if t.data_ptr() not in seen:
+                seen.add(t.data_ptr())
+                held += t.numel() * t.element_size()
+    assert slab.outside == 0
+    stored = sum(f.get(n).numel() * 4 for n in f.names())       # float32 on this path
+    assert held == stored and slab.used >= held and slab.buffer.numel() < stored + 256 * (len(f.names()) + 64)
+    if cfg.get("tie_word_embeddings"):
+        assert dec.lm_head.weight.data_ptr() == dec.embedding.weight.data_ptr()
+    layer = dec.layers[1]
+    q, k, v = (f.get(f"model.layers.1.self_attn.{n}_proj.weight") for n in "qkv")
+    assert torch.equal(layer.by_role["mixer"].w_qkv, torch.cat([q, k, v]))
+    gate, up = f.get("model.layers.1.mlp.gate_proj.weight"), f.get("model.layers.1.mlp.up_proj.weight")
+    assert torch.equal(layer.by_role["ffn"].w_gate_up[0::2], gate) and torch.equal(layer.by_role["ffn"].w_gate_up[1::2], up)
+    assert torch.equal(dec.final_norm.weight, f.get("model.norm.weight"))
+
+
 def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     folder = write_random_model(str(tmp_path), TINY_A, seed=5)
     path = os.path.join(folder, "model.safetensors")

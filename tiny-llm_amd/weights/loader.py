@@ -100,13 +100,82 @@ def check_against(specs: Sequence[WeightSpec], available: Mapping[str, Tuple[tor
     return source
 
 
-def _bind_all(decoder, fetch: Callable[[WeightSpec], torch.Tensor]) -> None:
-    cache: Dict[str, torch.Tensor] = {}
-    for part in decoder.parts():
+class WeightSlab:
+    """ONE device allocation that holds every resident weight, each at a 256-byte boundary, as the
+    reference places all weights in one static arena (tiny_llm/runtime/cuda/cuda_runtime.cpp:139-145).
+    Parts make their resident tensors in `bind` (fused, interleaved or as they came); `adopt` moves
+    what a part holds into the slab and hands the part views of it."""
+    ALIGN = 256
+
+    def __init__(self, nbytes: int, device):
+        self.buffer = torch.empty(max(int(nbytes), self.ALIGN), dtype=torch.uint8, device=device)
+        self.used = 0
+        self.outside = 0        # bytes of part tensors that found no room (a part that makes more than it was given)
+
+    def place(self, t: torch.Tensor) -> torch.Tensor:
+        n = t.numel() * t.element_size()
+        start = -(-self.used // self.ALIGN) * self.ALIGN
+        if n == 0 or start + n > self.buffer.numel():
+            self.outside += n
+            return t
+        view = self.buffer[start:start + n].view(t.dtype).view(t.shape)
+        view.copy_(t)
+        self.used = start + n
+        return view
+
+    def adopt(self, part, shared: Dict[Tuple[int, int], torch.Tensor], alive: Iterable[torch.Tensor]) -> None:
+        """Moves the tensors `part` holds on the slab's device into the slab.  `alive`: fetched
+        tensors that a later part will receive again (a tied head); what becomes of them is kept in
+        `shared`, so that the later part gets the same view and not a second copy."""
+        alive_keys = {(t.data_ptr(), t.numel() * t.element_size()) for t in alive}
+        here: Dict[Tuple[int, int], torch.Tensor] = {}      # one tensor under two names of this part
+        for attr, val in list(vars(part).items()):
+            if not (isinstance(val, torch.Tensor) and val.device == self.buffer.device and val.is_contiguous()):
+                continue
+            key = (val.data_ptr(), val.numel() * val.element_size())
+            known = shared.get(key, here.get(key))
+            if known is not None and known.dtype == val.dtype:
+                setattr(part, attr, known.view(val.shape))
+                continue
+            view = self.place(val)
+            setattr(part, attr, view)
+            here[key] = view
+            if key in alive_keys:
+                shared[key] = view
+
+
+def _bind_all(decoder, make: Callable[[WeightSpec], torch.Tensor], source_name: Callable[[WeightSpec], str],
+              dtype_of: Callable[[WeightSpec], torch.dtype]) -> None:
+    """Every part receives the tensors it declared (`make` builds one on the decoder's device, of
+    type `dtype_of`; specs with one `source_name` share it) and binds them; what it then holds moves
+    into the decoder's weight slab."""
+    specs = decoder.weight_specs()
+    uses: Dict[str, int] = {}
+    sizes: Dict[Tuple[str, torch.dtype], int] = {}
+    for s in specs:
+        uses[source_name(s)] = uses.get(source_name(s), 0) + 1
+        n = 1
+        for d in s.shape:
+            n *= int(d)
+        sizes[(source_name(s), dtype_of(s))] = n * torch.empty((), dtype=dtype_of(s)).element_size()
+    parts = decoder.parts()
+    total = sum(-(-b // WeightSlab.ALIGN) * WeightSlab.ALIGN for b in sizes.values()) + WeightSlab.ALIGN * len(parts)
+    slab = WeightSlab(total, decoder.device)
+    cache: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
+    shared: Dict[Tuple[int, int], torch.Tensor] = {}
+    for part in parts:
         tensors = {}
         for s in part.weights():
-            tensors[s.name] = fetch(s, cache)
+            key = (source_name(s), dtype_of(s))
+            t = cache.get(key)
+            if t is None:
+                t = make(s)
+                if uses[source_name(s)] > 1:
+                    cache[key] = t
+            tensors[s.name] = t
         part.bind(tensors)
+        slab.adopt(part, shared, cache.values())
+    decoder.weight_slab = slab
 
 
 class Checkpoint:
@@ -164,16 +233,13 @@ def load_weights(decoder, source) -> None:
     source_of = check_against(specs, available, ckpt.folder or "the checkpoint",
                               getattr(decoder.spec, "ignorable_tensors", ()))
 
-    def fetch(s: WeightSpec, cache):
-        src = source_of[s.name]
-        stored = available[src][0]
-        dt = target_dtype(s, stored, decoder.dtype)
-        key = (src, dt)
-        if key not in cache:
-            cache[key] = ckpt.get(src).to(device=decoder.device, dtype=dt, non_blocking=False).contiguous()
-        return cache[key]
+    def dtype_of(s: WeightSpec) -> torch.dtype:
+        return target_dtype(s, available[source_of[s.name]][0], decoder.dtype)
 
-    _bind_all(decoder, fetch)
+    def make(s: WeightSpec) -> torch.Tensor:
+        return ckpt.get(source_of[s.name]).to(device=decoder.device, dtype=dtype_of(s), non_blocking=False).contiguous()
+
+    _bind_all(decoder, make, lambda s: source_of[s.name], dtype_of)
 
 
 # ------------------------------------------------------------------ random weights
@@ -255,15 +321,17 @@ def init_random_weights(decoder, seed: int = 0, std: float = 0.02, norm_std: flo
     `write_random_model` would store for the same seed, rounded to the engine's types."""
     dev = decoder.device
 
-    def fetch(s: WeightSpec, cache):
-        name = s.alias_of if s.alias_of else s.name
-        dt = target_dtype(s, torch.float32, decoder.dtype)
-        if name not in cache:
-            base = WeightSpec(name, s.shape, s.role, s.init)
-            cache[name] = random_tensor(base, seed, std, norm_std, device=dev, dtype=dt)
-        return cache[name]
+    def source_name(s: WeightSpec) -> str:
+        return s.alias_of if s.alias_of else s.name
 
-    _bind_all(decoder, fetch)
+    def dtype_of(s: WeightSpec) -> torch.dtype:
+        return target_dtype(s, torch.float32, decoder.dtype)
+
+    def make(s: WeightSpec) -> torch.Tensor:
+        base = WeightSpec(source_name(s), s.shape, s.role, s.init)
+        return random_tensor(base, seed, std, norm_std, device=dev, dtype=dtype_of(s))
+
+    _bind_all(decoder, make, source_name, dtype_of)
 
 
 def write_random_model(folder: str, config: Mapping, seed: int = 0, std: Optional[float] = None,
