@@ -260,8 +260,8 @@ def test_linear_two_part_launch(M, K, N):
     assert rel(two, one.double()) < 1e-6
 
 
-@pytest.mark.parametrize("M", [17, 64, 65, 200, 512])
-@pytest.mark.parametrize("K,N", [(5632, 2048), (2048, 4100), (1096, 518)])
+@pytest.mark.parametrize("M", [17, 50, 64, 65, 200, 512])
+@pytest.mark.parametrize("K,N", [(5632, 2048), (2048, 4100), (1096, 518), (2048, 2046), (256, 2560), (4096, 6144)])
 def test_linear_split_k(M, K, N):
     """Products with few output tiles split their inner size over workgroups and add the parts up
     in a second kernel, which also applies every epilogue and both sides of the norm hand-off."""
@@ -272,7 +272,12 @@ def test_linear_split_k(M, K, N):
     scale = torch.rand(M, generator=g) + 0.5
     ref = a.double() @ w.double().T
     splits = ops().split_k(M, N, K)
-    if M > 64 or N * K >= (8 << 20):
+    few_tiles = -(-M // 128) * -(-N // 128) < 160
+    if M <= 64:      # few rows: small weight matrices stay with the few-row kernel, large or deep ones are split
+        must_split = K % 64 == 0 and (N * K > (17 << 20) or (N * K > (6 << 20) and (K > 4096 or M > 28)) or M >= 56)
+    else:
+        must_split = K >= 512 and few_tiles
+    if must_split:
         assert splits > 1                     # these sizes are here because they are split
     out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
     ops().linear(a.to(DEV), w.to(DEV), out)

@@ -594,6 +594,107 @@ static int launch_gemm_bf16_any(const bf16_t* a, const bf16_t* w, TO* out, const
   return launch_gemm_bf16_tile<TO, SWIGLU>(whole, a, w, out, residual, row_scale, M, N, K, lda, ldo, k_per_split, stream);
 }
 
+// ------------------------------------------------- split k for few rows: one round trip
+// At most 64 rows, the inner size split over workgroups: a workgroup's share of both operands
+// (64 rows of activations and 128 weight rows, up to 384 k) is small enough for LDS, so ALL of it is
+// requested at once, straight into LDS (global_load_lds_dwordx4: no registers in between, every load
+// of the workgroup in flight together), and the kernel is one round trip to memory long.  The tiled
+// kernel above walks the same share in k steps of 64 and pays a round trip for each.
+// LDS holds slabs of 64 k: [slab][A: 8 groups of 8 rows | W: 16 groups of 8 rows][8 rows x 128 bytes];
+// one load instruction of a wave fills one group (1 KB, lane i -> bytes 16 i); the 16-byte chunk c of
+// row r stands at position c ^ (r % 8), so that the fragment reads of 32 rows do not collide.
+// Result: float32 partial products [split, M, N] for splitk_reduce_kernel.  K must be a multiple of 64.
+constexpr int O_BM = 64, O_BN = 128, O_WAVES = 8, O_THREADS = O_WAVES * TL_WAVE, O_SLAB_K = 64, O_MAX_SLABS = 6;
+constexpr int O_GROUPS = (O_BM + O_BN) / 8, O_GROUP_BYTES = 8 * O_SLAB_K * 2, O_SLAB_BYTES = O_GROUPS * O_GROUP_BYTES;
+typedef __attribute__((address_space(3))) void* tl_lds_ptr;
+typedef const __attribute__((address_space(1))) void* tl_global_ptr;
+
+__global__ __launch_bounds__(O_THREADS) void gemm_oneshot_bf16_kernel(const bf16_t* __restrict__ a,
+                                                                      const bf16_t* __restrict__ w,
+                                                                      float* __restrict__ partial, int M, int N, int K,
+                                                                      int64_t lda, int slabs_per_split) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char oneshot_smem[];
+  const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
+  const int n0 = blockIdx.x * O_BN, split = blockIdx.y;
+  const int nslabs = K / O_SLAB_K, s0 = split * slabs_per_split, s1 = min(nslabs, s0 + slabs_per_split);
+  const int mine = s1 - s0;                       // at least one: the grid has no empty split
+  // requests: of every slab wave v fills group v (8 activation rows) and groups 8 + v and 16 + v
+  // (16 weight rows); a lane's three addresses move on by 64 k from slab to slab
+  static_assert(O_BM / 8 == O_WAVES && O_BN / 8 == 2 * O_WAVES, "one activation group and two weight groups a wave");
+  const int wv = __builtin_amdgcn_readfirstlane(wave);
+  const int lrow = lane / 8, lchunk = (lane % 8) ^ lrow;
+  const int64_t k_first = (int64_t)s0 * O_SLAB_K + lchunk * 8;
+  const bf16_t* src[3] = {a + (int64_t)min(wv * 8 + lrow, M - 1) * lda + k_first,
+                          w + (int64_t)min(n0 + wv * 8 + lrow, N - 1) * K + k_first,
+                          w + (int64_t)min(n0 + (O_WAVES + wv) * 8 + lrow, N - 1) * K + k_first};
+  for (int sl = 0; sl < mine; ++sl) {
+    unsigned char* sb = oneshot_smem + sl * O_SLAB_BYTES + wv * O_GROUP_BYTES;
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
+      __builtin_amdgcn_global_load_lds((tl_global_ptr)src[j], (tl_lds_ptr)(sb + j * O_WAVES * O_GROUP_BYTES), 16, 0, 0);
+      src[j] += O_SLAB_K;
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);             // vmcnt(0): this wave's requests have landed
+  __syncthreads();                                // and everybody's
+  // wave (wm, wn) owns rows wm*32.., columns wn*32..; result transposed (rows of the instruction are
+  // output columns), so a lane ends up with four consecutive columns of one row
+  const int wm = wave / 4, wn = wave % 4;
+  const int r8 = lane % 8;
+  const int lane_off = ((lane % 32) / 8) * O_GROUP_BYTES + r8 * 128;
+  const int a_off = (wm * 32 / 8) * O_GROUP_BYTES + lane_off;
+  const int w_off = (O_BM / 8 + wn * 32 / 8) * O_GROUP_BYTES + lane_off;
+  f32x16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+  for (int sl = 0; sl < mine; ++sl) {
+    const unsigned char* sb = oneshot_smem + sl * O_SLAB_BYTES;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const int pos = ((2 * ks + lane / 32) ^ r8) * 16;
+      const bf16x8 fa = *(const bf16x8*)(sb + a_off + pos);
+      const bf16x8 fw = *(const bf16x8*)(sb + w_off + pos);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw, fa, acc, 0, 0, 0);
+    }
+  }
+  float* out = partial + (int64_t)split * M * N;
+  const int m = wm * 32 + lane % 32;
+  if (m < M) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int n = n0 + wn * 32 + q * 8 + (lane / 32) * 4;
+      if ((N % 4 == 0) && n + 3 < N) {
+        *(f32x4*)(out + (int64_t)m * N + n) = f32x4{acc[q * 4 + 0], acc[q * 4 + 1], acc[q * 4 + 2], acc[q * 4 + 3]};
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (n + e < N) out[(int64_t)m * N + n + e] = acc[q * 4 + e];
+      }
+    }
+  }
+}
+
+// Whether and how the one-round-trip kernel takes a split product: slabs of 64 k per split (0: not
+// this kernel).  As many splits as make about one round of workgroups over the 256 compute units;
+// not where that needs more than 384 k a workgroup (wide products: they keep the tiled kernel).
+static int oneshot_plan(int M, int N, int K, int* slabs_per_split) {
+  *slabs_per_split = 0;
+  if (M <= 16 || M > O_BM || K % O_SLAB_K || K < 4 * O_SLAB_K) return 1;
+  // measured: small weight matrices with few rows are faster in the few-row kernel (one launch)
+  const int64_t weights = (int64_t)N * K;
+  if ((weights <= ((int64_t)6 << 20) && M < 56) || (weights <= ((int64_t)17 << 20) && K <= 4096 && M <= 28)) return 1;
+  const int tiles = (N + O_BN - 1) / O_BN, nslabs = K / O_SLAB_K;
+  const int room = 256 / tiles;                  // splits that still make one round
+  if (room < 2) return 1;
+  int per = (nslabs + room - 1) / room;
+  if (per < 2) per = 2;
+  if (per > O_MAX_SLABS) return 1;
+  const int splits = (nslabs + per - 1) / per;
+  if (splits < 2) return 1;
+  *slabs_per_split = per;
+  return splits;
+}
+
 // ------------------------------------------------------------ split k: the second kernel
 // Adds up the partial products [splits, M, N] of a product whose inner size was split over
 // workgroups and applies what the product's own epilogue would have: row factor (given, or from
@@ -697,6 +798,13 @@ __global__ __launch_bounds__(R_THREADS) void splitk_reduce_kernel(const ReduceAr
 static int splitk_plan(int M, int N, int K, int* tile, int* k_per_split) {
   *tile = 0;
   *k_per_split = 0;
+  int slabs;
+  const int one = oneshot_plan(M, N, K, &slabs);
+  if (one > 1) {
+    *tile = -1;                                   // the one-round-trip kernel
+    *k_per_split = slabs * O_SLAB_K;
+    return one;
+  }
   if (M <= 16 || K < 8 * B_BK) return 1;
   const int bm = M <= 64 ? 64 : 128, bn = 128;
   const int64_t wgs = (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
@@ -1354,8 +1462,23 @@ int tl_linear_splitk(const void* a, const void* w, void* out, const float* resid
   int tile, kps;
   const int splits = splitk_plan(M, N, K, &tile, &kps);
   if (splits < 2) return TL_ERR_ARG;
-  int rc = launch_gemm_bf16_any<float, false>((const bf16_t*)a, (const bf16_t*)w, workspace, nullptr, nullptr, M, N, K,
-                                              lda, N, tile, kps, stream);
+  int rc = TL_OK;
+  if (tile < 0) {
+    const int slabs = kps / O_SLAB_K;
+    const size_t smem = (size_t)slabs * O_SLAB_BYTES;
+    static int configured = 0;
+    if (configured < (int)smem) {
+      if (hipFuncSetAttribute((const void*)gemm_oneshot_bf16_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              O_MAX_SLABS * O_SLAB_BYTES) != hipSuccess)
+        return TL_ERR_LAUNCH;
+      configured = O_MAX_SLABS * O_SLAB_BYTES;
+    }
+    hipLaunchKernelGGL(gemm_oneshot_bf16_kernel, dim3((N + O_BN - 1) / O_BN, splits), dim3(O_THREADS), smem, stream,
+                       (const bf16_t*)a, (const bf16_t*)w, workspace, M, N, K, lda, slabs);
+  } else {
+    rc = launch_gemm_bf16_any<float, false>((const bf16_t*)a, (const bf16_t*)w, workspace, nullptr, nullptr, M, N, K, lda,
+                                            N, tile, kps, stream);
+  }
   if (rc != TL_OK) return rc;
   ReduceArgs p{workspace, splits, M, N, out, ldo, residual, row_scale, in_sumsq, in_parts, in_width, in_eps, emit_w,
                emit_w_dtype == 0 ? 1 : 0, (bf16_t*)emit_operand, emit_sumsq};
