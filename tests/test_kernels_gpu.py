@@ -274,7 +274,8 @@ def test_linear_split_k(M, K, N):
     splits = ops().split_k(M, N, K)
     few_tiles = -(-M // 128) * -(-N // 128) < 160
     if M <= 64:      # few rows: small weight matrices stay with the few-row kernel, large or deep ones are split
-        must_split = K % 64 == 0 and (N * K > (17 << 20) or (N * K > (6 << 20) and (K > 4096 or M > 28)) or M >= 56)
+        must_split = K % 64 == 0 and (N * K > (17 << 20) or (N * K > (6 << 20) and (K > 4096 or M > 28)) or M >= 56) \
+            and not (N > 128 * 128 and M <= 32)
     else:
         must_split = K >= 512 and few_tiles
     if must_split:

@@ -594,20 +594,32 @@ static int launch_gemm_bf16_any(const bf16_t* a, const bf16_t* w, TO* out, const
   return launch_gemm_bf16_tile<TO, SWIGLU>(whole, a, w, out, residual, row_scale, M, N, K, lda, ldo, k_per_split, stream);
 }
 
-// ------------------------------------------------- split k for few rows: one round trip
-// At most 64 rows, the inner size split over workgroups: a workgroup's share of both operands
-// (64 rows of activations and 128 weight rows, up to 384 k) is small enough for LDS, so ALL of it is
-// requested at once, straight into LDS (global_load_lds_dwordx4: no registers in between, every load
-// of the workgroup in flight together), and the kernel is one round trip to memory long.  The tiled
-// kernel above walks the same share in k steps of 64 and pays a round trip for each.
-// LDS holds slabs of 64 k: [slab][A: 8 groups of 8 rows | W: 16 groups of 8 rows][8 rows x 128 bytes];
-// one load instruction of a wave fills one group (1 KB, lane i -> bytes 16 i); the 16-byte chunk c of
-// row r stands at position c ^ (r % 8), so that the fragment reads of 32 rows do not collide.
+// ------------------------------------------- split k for few rows: everything in flight
+// At most 64 rows, the inner size split over workgroups.  A workgroup's share of both operands (64
+// rows of activations and 128 weight rows per 64 k) goes straight into LDS
+// (global_load_lds_dwordx4: no registers in between), as a ring of six slabs of 64 k, so that five
+// slabs (120 KB) are on their way while one is multiplied; a share of up to six slabs is requested
+// at once and the kernel is one round trip to memory long.  The tiled kernel above keeps one k
+// step of 64 in flight and pays a round trip for each.
+// A slab in LDS: [A: 8 groups of 8 rows | W: 16 groups of 8 rows][8 rows x 128 bytes]; one load
+// instruction of a wave fills one group (1 KB, lane i -> bytes 16 i); the 16-byte chunk c of row r
+// stands at position c ^ (r % 8), so that the fragment reads of 32 rows do not collide.
 // Result: float32 partial products [split, M, N] for splitk_reduce_kernel.  K must be a multiple of 64.
-constexpr int O_BM = 64, O_BN = 128, O_WAVES = 8, O_THREADS = O_WAVES * TL_WAVE, O_SLAB_K = 64, O_MAX_SLABS = 6;
+constexpr int O_BM = 64, O_BN = 128, O_WAVES = 8, O_THREADS = O_WAVES * TL_WAVE, O_SLAB_K = 64, O_RING = 6;
 constexpr int O_GROUPS = (O_BM + O_BN) / 8, O_GROUP_BYTES = 8 * O_SLAB_K * 2, O_SLAB_BYTES = O_GROUPS * O_GROUP_BYTES;
 typedef __attribute__((address_space(3))) void* tl_lds_ptr;
 typedef const __attribute__((address_space(1))) void* tl_global_ptr;
+
+// waits until at most 3 * later of this wave's loads are outstanding (three loads a slab)
+__device__ __forceinline__ void oneshot_wait(int later) {
+  switch (later) {
+    case 0: __builtin_amdgcn_s_waitcnt(0x0F70); break;
+    case 1: __builtin_amdgcn_s_waitcnt(0x0F73); break;
+    case 2: __builtin_amdgcn_s_waitcnt(0x0F76); break;
+    case 3: __builtin_amdgcn_s_waitcnt(0x0F79); break;
+    default: __builtin_amdgcn_s_waitcnt(0x0F7C); break;       // 12
+  }
+}
 
 __global__ __launch_bounds__(O_THREADS) void gemm_oneshot_bf16_kernel(const bf16_t* __restrict__ a,
                                                                       const bf16_t* __restrict__ w,
@@ -627,16 +639,15 @@ __global__ __launch_bounds__(O_THREADS) void gemm_oneshot_bf16_kernel(const bf16
   const bf16_t* src[3] = {a + (int64_t)min(wv * 8 + lrow, M - 1) * lda + k_first,
                           w + (int64_t)min(n0 + wv * 8 + lrow, N - 1) * K + k_first,
                           w + (int64_t)min(n0 + (O_WAVES + wv) * 8 + lrow, N - 1) * K + k_first};
-  for (int sl = 0; sl < mine; ++sl) {
-    unsigned char* sb = oneshot_smem + sl * O_SLAB_BYTES + wv * O_GROUP_BYTES;
+  auto request = [&](int sl) {                    // slab sl of this workgroup, into buffer sl % O_RING
+    unsigned char* sb = oneshot_smem + (sl % O_RING) * O_SLAB_BYTES + wv * O_GROUP_BYTES;
 #pragma unroll
     for (int j = 0; j < 3; ++j) {
       __builtin_amdgcn_global_load_lds((tl_global_ptr)src[j], (tl_lds_ptr)(sb + j * O_WAVES * O_GROUP_BYTES), 16, 0, 0);
       src[j] += O_SLAB_K;
     }
-  }
-  __builtin_amdgcn_s_waitcnt(0x0F70);             // vmcnt(0): this wave's requests have landed
-  __syncthreads();                                // and everybody's
+  };
+  for (int sl = 0; sl < min(mine, O_RING - 1); ++sl) request(sl);
   // wave (wm, wn) owns rows wm*32.., columns wn*32..; result transposed (rows of the instruction are
   // output columns), so a lane ends up with four consecutive columns of one row
   const int wm = wave / 4, wn = wave % 4;
@@ -648,7 +659,18 @@ __global__ __launch_bounds__(O_THREADS) void gemm_oneshot_bf16_kernel(const bf16
 #pragma unroll
   for (int r = 0; r < 16; ++r) acc[r] = 0.f;
   for (int sl = 0; sl < mine; ++sl) {
-    const unsigned char* sb = oneshot_smem + sl * O_SLAB_BYTES;
+    // slab sl has landed for this wave once only the slabs requested after it are outstanding;
+    // after the barrier it has landed for everybody, and nobody reads slab sl - 1 any more, whose
+    // buffer the next request takes
+    // (a bare barrier: __syncthreads() would also wait for every outstanding load, the slabs still on
+    // their way included; the counter above is the wait that is needed, and the fragment reads of
+    // the previous slab were consumed by its matrix instructions before any wave gets here)
+    oneshot_wait(min(mine - 1, sl + O_RING - 2) - sl);
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (sl + O_RING - 1 < mine) request(sl + O_RING - 1);
+    const unsigned char* sb = oneshot_smem + (sl % O_RING) * O_SLAB_BYTES;
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
       const int pos = ((2 * ks + lane / 32) ^ r8) * 16;
@@ -674,25 +696,36 @@ __global__ __launch_bounds__(O_THREADS) void gemm_oneshot_bf16_kernel(const bf16
   }
 }
 
-// Whether and how the one-round-trip kernel takes a split product: slabs of 64 k per split (0: not
-// this kernel).  As many splits as make about one round of workgroups over the 256 compute units;
-// not where that needs more than 384 k a workgroup (wide products: they keep the tiled kernel).
+// Whether and how this kernel takes a product of 17 to 64 rows: slabs of 64 k per split (0: not this
+// kernel).  The number of splits with the smallest estimated time: rounds of workgroups over the 256
+// compute units, each as long as a workgroup takes to fetch its share (about 35 GB/s), and the second
+// kernel's reading of the partial sums.
 static int oneshot_plan(int M, int N, int K, int* slabs_per_split) {
   *slabs_per_split = 0;
   if (M <= 16 || M > O_BM || K % O_SLAB_K || K < 4 * O_SLAB_K) return 1;
   // measured: small weight matrices with few rows are faster in the few-row kernel (one launch)
   const int64_t weights = (int64_t)N * K;
-  if ((weights <= ((int64_t)6 << 20) && M < 56) || (weights <= ((int64_t)17 << 20) && K <= 4096 && M <= 28)) return 1;
   const int tiles = (N + O_BN - 1) / O_BN, nslabs = K / O_SLAB_K;
-  const int room = 256 / tiles;                  // splits that still make one round
-  if (room < 2) return 1;
-  int per = (nslabs + room - 1) / room;
-  if (per < 2) per = 2;
-  if (per > O_MAX_SLABS) return 1;
-  const int splits = (nslabs + per - 1) / per;
-  if (splits < 2) return 1;
-  *slabs_per_split = per;
-  return splits;
+  if ((weights <= ((int64_t)6 << 20) && M < 56) || (weights <= ((int64_t)17 << 20) && K <= 4096 && M <= 28) ||
+      (tiles > 128 && M <= 32))
+    return 1;
+  int best = 1, best_per = 0;
+  double best_t = 0.;
+  for (int want = 2; want <= 16; ++want) {
+    const int per = (nslabs + want - 1) / want;
+    if (per < 2) break;
+    const int splits = (nslabs + per - 1) / per;
+    if (splits < 2) continue;
+    const int rounds = (tiles * splits + 255) / 256;
+    const double t = rounds * (2.0 + per * (O_SLAB_BYTES / 35e3)) + 1.5 + splits * (double)M * N * 4 / 3e6;
+    if (best == 1 || t < best_t) {
+      best = splits;
+      best_per = per;
+      best_t = t;
+    }
+  }
+  *slabs_per_split = best_per;
+  return best;
 }
 
 // ------------------------------------------------------------ split k: the second kernel
@@ -798,10 +831,10 @@ __global__ __launch_bounds__(R_THREADS) void splitk_reduce_kernel(const ReduceAr
 static int splitk_plan(int M, int N, int K, int* tile, int* k_per_split) {
   *tile = 0;
   *k_per_split = 0;
-  int slabs;
-  const int one = oneshot_plan(M, N, K, &slabs);
-  if (one > 1) {
-    *tile = -1;                                   // the one-round-trip kernel
+  if (M > 16 && M <= O_BM && K % O_SLAB_K == 0 && K >= 4 * O_SLAB_K) {      // the ring kernel's sizes: it or the few-row kernel
+    int slabs;
+    const int one = oneshot_plan(M, N, K, &slabs);
+    *tile = -1;
     *k_per_split = slabs * O_SLAB_K;
     return one;
   }
@@ -1465,13 +1498,13 @@ int tl_linear_splitk(const void* a, const void* w, void* out, const float* resid
   int rc = TL_OK;
   if (tile < 0) {
     const int slabs = kps / O_SLAB_K;
-    const size_t smem = (size_t)slabs * O_SLAB_BYTES;
-    static int configured = 0;
-    if (configured < (int)smem) {
+    const size_t smem = (size_t)(slabs < O_RING ? slabs : O_RING) * O_SLAB_BYTES;
+    static bool configured = false;
+    if (!configured) {
       if (hipFuncSetAttribute((const void*)gemm_oneshot_bf16_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                              O_MAX_SLABS * O_SLAB_BYTES) != hipSuccess)
+                              O_RING * O_SLAB_BYTES) != hipSuccess)
         return TL_ERR_LAUNCH;
-      configured = O_MAX_SLABS * O_SLAB_BYTES;
+      configured = true;
     }
     hipLaunchKernelGGL(gemm_oneshot_bf16_kernel, dim3((N + O_BN - 1) / O_BN, splits), dim3(O_THREADS), smem, stream,
                        (const bf16_t*)a, (const bf16_t*)w, workspace, M, N, K, lda, slabs);
