@@ -572,37 +572,58 @@ __global__ __launch_bounds__(A32_THREADS) void attention_f32_kernel(
     const int t_lo = max(c * A32_CHUNK, first_tile), t_hi = min((c + 1) * A32_CHUNK, last_tile);
     for (int t = t_lo + wave; t < t_hi; t += A32_WAVES) {
       const int kb = t * FA_KT;
-      // the first 64 value columns of this lane's key row are requested before anything else
+      // Everything the tile needs from memory is requested together, in two rounds (page numbers,
+      // then rows): loads are unconditional, with the index clamped into the table and a row outside
+      // the request's keys read from row 0 of page 0 and zeroed afterwards (stale pages may hold
+      // anything, and 0 * NaN is NaN); a conditional load would become a branch, and every branch
+      // one more round trip in a row.
       constexpr int VPRE = (HD < A32_VW ? HD : A32_VW) / 4;
-      f32x4 vpre[VPRE];
       const int vkey = kb + lane;
       const bool v_in_range = vkey >= kv_begin && vkey < kv_end;
-      const float* vrow;
-      {
-        const int jb = min(vkey / block_size, max_blocks - 1);
-        const int64_t blk = max(bt[v_in_range ? jb : 0], 0);
-        vrow = v_cache + ((blk * nkv + kvh) * block_size + (vkey - (vkey / block_size) * block_size)) * HD;
-#pragma unroll
-        for (int ch = 0; ch < VPRE; ++ch)
-          vpre[ch] = v_in_range ? *(const f32x4*)(vrow + ch * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
-      }
-      // ---- scores S^T = K Q^T: lane (l16, kk) of subtile st holds keys kb + 16 st + 4 kk + r of row l16
-      f32x4 sc[4];
+      bool k_in[4];
+      int page_k[4];
 #pragma unroll
       for (int st = 0; st < 4; ++st) {
         const int key = kb + st * 16 + l16;
-        const bool in_range = key < kv_end;
-        const int jb = min(key / block_size, max_blocks - 1);
-        const int64_t blk = max(bt[in_range ? jb : 0], 0);
-        const float* krow = k_cache + ((blk * nkv + kvh) * block_size + (key - (key / block_size) * block_size)) * HD;
-        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        k_in[st] = key < kv_end;
+        page_k[st] = bt[min(key / block_size, max_blocks - 1)];
+      }
+      const int page_v = bt[min(vkey / block_size, max_blocks - 1)];
+      auto row_of = [&](int page, int key, bool in) {
+        const int64_t off = (((int64_t)max(page, 0) * nkv + kvh) * block_size + (key - (key / block_size) * block_size)) * HD;
+        return in ? off : (int64_t)0;
+      };
+      const float* vrow = v_cache + row_of(page_v, vkey, v_in_range);
+      f32x4 vpre[VPRE];
 #pragma unroll
-        for (int g4 = 0; g4 < HDT; ++g4) {
-          const f32x4 kf = in_range ? *(const f32x4*)(krow + g4 * 16 + kk * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int ch = 0; ch < VPRE; ++ch) vpre[ch] = *(const f32x4*)(vrow + ch * 4);
+      // ---- scores S^T = K Q^T: lane (l16, kk) of subtile st holds keys kb + 16 st + 4 kk + r of row l16
+      f32x4 sc[4];
+      constexpr int STB = HDT <= 4 ? 4 : 2;       // subtiles whose key rows are in registers together
 #pragma unroll
-          for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[e], qf[g4][e], acc, 0, 0, 0);
+      for (int s0 = 0; s0 < 4; s0 += STB) {
+        f32x4 kf[STB][HDT];
+#pragma unroll
+        for (int si = 0; si < STB; ++si) {
+          const float* krow = k_cache + row_of(page_k[s0 + si], kb + (s0 + si) * 16 + l16, k_in[s0 + si]);
+#pragma unroll
+          for (int g4 = 0; g4 < HDT; ++g4) kf[si][g4] = *(const f32x4*)(krow + g4 * 16 + kk * 4);
         }
-        sc[st] = acc;
+#pragma unroll
+        for (int si = 0; si < STB; ++si) {
+          f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int g4 = 0; g4 < HDT; ++g4) {
+            const f32x4 kv = k_in[s0 + si] ? kf[si][g4] : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(kv[e], qf[g4][e], acc, 0, 0, 0);
+          }
+          sc[s0 + si] = acc;
+        }
+      }
+      if (!v_in_range) {
+#pragma unroll
+        for (int ch = 0; ch < VPRE; ++ch) vpre[ch] = f32x4{0.f, 0.f, 0.f, 0.f};
       }
       // ---- the tile's softmax from scratch
       float m_t = -INFINITY;
@@ -646,7 +667,10 @@ __global__ __launch_bounds__(A32_THREADS) void attention_f32_kernel(
               // rows outside the request's keys are zeroed: stale pages may hold anything, and 0 * NaN is NaN
               f32x4 v;
               if (dh == 0) v = vpre[ch < VPRE ? ch : 0];
-              else v = in_range ? *(const f32x4*)(vrow + dh * A32_VW + ch * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
+              else {
+                v = *(const f32x4*)(vrow + dh * A32_VW + ch * 4);
+                if (!in_range) v = f32x4{0.f, 0.f, 0.f, 0.f};
+              }
               *(f32x4*)(&Vl[lane * A32_VS + ch * 4]) = v;
             }
           __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
