@@ -296,27 +296,39 @@ __global__ __launch_bounds__(WM * WN * TL_WAVE) void gemm_bf16_kernel(const bf16
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  // One k step of both operand tiles is AC + WC 16-byte pieces per thread.  Global loads are
-  // unconditional (addresses clamped into the matrix; a piece that lies outside is zeroed when it
-  // is written to LDS): a predicated load becomes a branch, and then the outstanding-load counter
-  // cannot be used to wait for one piece while the next stays in flight.
+  // One k step of both operand tiles is AC + WC 16-byte pieces per thread, fetched with buffer
+  // loads: the address is the tile's first row (the buffer's base, per workgroup) + an offset per
+  // piece that never changes + the k offset, which is one scalar for all lanes, so a k step costs
+  // no address arithmetic; and the buffer ends with the matrix, so rows beyond it read as zero
+  // without a branch.  (A piece beyond K within a row is zeroed when it is written to LDS.)
   constexpr int PIECES = S::AC + S::WC;
   bf16x8 stage[PIECES];
   const int prow = tid / 8, pk = (tid % 8) * 8;            // this thread's row within a pass, k offset
   constexpr int PASS = THREADS / 8;                        // rows per pass
-  auto gload1 = [&](int k0, int p) {
-    const bool is_a = p < S::AC;
-    const int row = (is_a ? m0 + p * PASS : n0 + (p - S::AC) * PASS) + prow, k = k0 + pk;
-    const bf16_t* base = is_a ? a : w;
-    const int64_t ld = is_a ? lda : (int64_t)K;
-    const int lim = is_a ? M : N;
-    stage[p] = *(const bf16x8*)(base + (int64_t)(FULL ? row : min(row, lim - 1)) * ld + (FULL ? k : min(k, K - 8)));
+  auto tile_buffer = [](const bf16_t* first_row, int rows, int64_t ld, int K_) {
+    const int64_t bytes = rows > 0 ? ((int64_t)(rows - 1) * ld + K_) * 2 : 0;
+    return __builtin_amdgcn_make_buffer_rsrc((void*)first_row, 0, (int)(bytes < 0x7fffffff ? bytes : 0x7fffffff), 0x00020000);
   };
-  // FULL: M, N and K are multiples of the tile, so no piece lies outside and nothing is zeroed
+  const __amdgpu_buffer_rsrc_t buf_a = tile_buffer(a + (int64_t)m0 * lda, min(M - m0, BM), lda, K);
+  const __amdgpu_buffer_rsrc_t buf_w = tile_buffer(w + (int64_t)n0 * K, min(N - n0, BN), K, K);
+  int piece_off[PIECES];                                   // bytes from the tile's first row
+#pragma unroll
+  for (int p = 0; p < PIECES; ++p) {
+    const bool is_a = p < S::AC;
+    const int r = (is_a ? p : p - S::AC) * PASS + prow;
+    piece_off[p] = (int)(((int64_t)r * (is_a ? lda : (int64_t)K) + pk) * 2);
+  }
+  typedef int tl_i32x4 __attribute__((ext_vector_type(4)));
+  auto gload1 = [&](int k0, int p) {
+    const tl_i32x4 v = __builtin_bit_cast(
+        tl_i32x4, __builtin_amdgcn_raw_buffer_load_b128(p < S::AC ? buf_a : buf_w, piece_off[p], k0 * 2, 0));
+    stage[p] = __builtin_bit_cast(bf16x8, v);
+  };
+  // FULL: K is a multiple of the k step (and M, N of the tile), so nothing is zeroed
   auto lds_write1 = [&](int buf, int k0, int p) {
     const bool is_a = p < S::AC;
     const int r = (is_a ? p : p - S::AC) * PASS + prow;
-    const bool ok = FULL || ((is_a ? m0 + r < M : n0 + r < N) && k0 + pk < K);
+    const bool ok = FULL || k0 + pk < K;
     bf16x8 z = {};
     bf16_t* dst = is_a ? As + (buf * BM + r) * B_LD + pk : Ws + (buf * BN + r) * B_LD + pk;
     *(bf16x8*)dst = ok ? stage[p] : z;
@@ -494,6 +506,8 @@ static int launch_gemm_bf16_full(const bf16_t* a, const bf16_t* w, TO* out, cons
       return TL_ERR_LAUNCH;
     configured = true;
   }
+  // a tile's rows are addressed with 32-bit byte offsets from its first row
+  if ((int64_t)BM * lda * 2 >= 0x7fffffff || (int64_t)BN * K * 2 >= 0x7fffffff) return TL_ERR_ARG;
   const int64_t splits = k_per_split > 0 ? (K + k_per_split - 1) / k_per_split : 1;
   const int64_t total = (int64_t)((N + BN - 1) / BN) * ((M + BM - 1) / BM) * splits;
   const int64_t grid = (total + B_XCDS - 1) / B_XCDS * B_XCDS;
