@@ -641,7 +641,7 @@ __global__ __launch_bounds__(O_THREADS) void gemm_oneshot_bf16_kernel(const bf16
                                                                       int64_t lda, int slabs_per_split) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char oneshot_smem[];
   const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
-  const int n0 = blockIdx.x * O_BN, split = blockIdx.y;
+  const int n0 = blockIdx.x * O_BN, split = blockIdx.y, m0 = blockIdx.z * O_BM;
   const int nslabs = K / O_SLAB_K, s0 = split * slabs_per_split, s1 = min(nslabs, s0 + slabs_per_split);
   const int mine = s1 - s0;                       // at least one: the grid has no empty split
   // requests: of every slab wave v fills group v (8 activation rows) and groups 8 + v and 16 + v
@@ -650,7 +650,7 @@ __global__ __launch_bounds__(O_THREADS) void gemm_oneshot_bf16_kernel(const bf16
   const int wv = __builtin_amdgcn_readfirstlane(wave);
   const int lrow = lane / 8, lchunk = (lane % 8) ^ lrow;
   const int64_t k_first = (int64_t)s0 * O_SLAB_K + lchunk * 8;
-  const bf16_t* src[3] = {a + (int64_t)min(wv * 8 + lrow, M - 1) * lda + k_first,
+  const bf16_t* src[3] = {a + (int64_t)min(m0 + wv * 8 + lrow, M - 1) * lda + k_first,
                           w + (int64_t)min(n0 + wv * 8 + lrow, N - 1) * K + k_first,
                           w + (int64_t)min(n0 + (O_WAVES + wv) * 8 + lrow, N - 1) * K + k_first};
   auto request = [&](int sl) {                    // slab sl of this workgroup, into buffer sl % O_RING
@@ -694,7 +694,7 @@ __global__ __launch_bounds__(O_THREADS) void gemm_oneshot_bf16_kernel(const bf16
     }
   }
   float* out = partial + (int64_t)split * M * N;
-  const int m = wm * 32 + lane % 32;
+  const int m = m0 + wm * 32 + lane % 32;
   if (m < M) {
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
@@ -716,12 +716,12 @@ __global__ __launch_bounds__(O_THREADS) void gemm_oneshot_bf16_kernel(const bf16
 // kernel's reading of the partial sums.
 static int oneshot_plan(int M, int N, int K, int* slabs_per_split) {
   *slabs_per_split = 0;
-  if (M <= 16 || M > O_BM || K % O_SLAB_K || K < 4 * O_SLAB_K) return 1;
+  if (M <= 16 || K % O_SLAB_K || K < 4 * O_SLAB_K) return 1;
   // measured: small weight matrices with few rows are faster in the few-row kernel (one launch)
   const int64_t weights = (int64_t)N * K;
-  const int tiles = (N + O_BN - 1) / O_BN, nslabs = K / O_SLAB_K;
-  if ((weights <= ((int64_t)6 << 20) && M < 56) || (weights <= ((int64_t)17 << 20) && K <= 4096 && M <= 28) ||
-      (tiles > 128 && M <= 32))
+  const int tiles = ((M + O_BM - 1) / O_BM) * ((N + O_BN - 1) / O_BN), nslabs = K / O_SLAB_K;
+  if (M <= O_BM && ((weights <= ((int64_t)6 << 20) && M < 56) || (weights <= ((int64_t)17 << 20) && K <= 4096 && M <= 28) ||
+                    (tiles > 128 && M <= 32)))
     return 1;
   int best = 1, best_per = 0;
   double best_t = 0.;
@@ -845,7 +845,13 @@ __global__ __launch_bounds__(R_THREADS) void splitk_reduce_kernel(const ReduceAr
 static int splitk_plan(int M, int N, int K, int* tile, int* k_per_split) {
   *tile = 0;
   *k_per_split = 0;
-  if (M > 16 && M <= O_BM && K % O_SLAB_K == 0 && K >= 4 * O_SLAB_K) {      // the ring kernel's sizes: it or the few-row kernel
+  // The ring kernel's sizes.  Up to 64 rows: it or the few-row kernel.  Beyond (tiles of 64 rows side by
+  // side), measured: it beats the k-step loop up to 128 rows on matrices up to 4096 x 6144 and up to 256
+  // rows on small ones; its one accumulator tile a wave is no match for the tiled kernel beyond that.
+  const int64_t weights = (int64_t)N * K;
+  const bool ring_rows = M <= O_BM || (M <= 128 && N <= 6144 && weights <= ((int64_t)26 << 20)) ||
+                         (M <= 256 && weights <= ((int64_t)6 << 20));
+  if (M > 16 && ring_rows && K % O_SLAB_K == 0 && K >= 4 * O_SLAB_K) {
     int slabs;
     const int one = oneshot_plan(M, N, K, &slabs);
     *tile = -1;
@@ -1520,7 +1526,7 @@ int tl_linear_splitk(const void* a, const void* w, void* out, const float* resid
         return TL_ERR_LAUNCH;
       configured = true;
     }
-    hipLaunchKernelGGL(gemm_oneshot_bf16_kernel, dim3((N + O_BN - 1) / O_BN, splits), dim3(O_THREADS), smem, stream,
+    hipLaunchKernelGGL(gemm_oneshot_bf16_kernel, dim3((N + O_BN - 1) / O_BN, splits, (M + O_BM - 1) / O_BM), dim3(O_THREADS), smem, stream,
                        (const bf16_t*)a, (const bf16_t*)w, workspace, M, N, K, lda, slabs);
   } else {
     rc = launch_gemm_bf16_any<float, false>((const bf16_t*)a, (const bf16_t*)w, workspace, nullptr, nullptr, M, N, K, lda,
