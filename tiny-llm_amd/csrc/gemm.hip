@@ -4,13 +4,16 @@
 // residual add that the reference runs as a separate kernel
 // (tiny_llm/ops/cuda/arithmetic.cu:13) is folded into the epilogue.
 //
-//  * gemm_f32_kernel, and gemm_f32_rows_kernel for at most 16 rows: true float32, FMA on the
-//    vector units, no reduced-precision matrix mode.  Both add in ONE order: k ascending inside
-//    blocks of 256, each block from zero, the block sums added in ascending order.  So a row
-//    gives the same bits whether it is computed alone or in a batch, by either kernel.
-//  * gemm_bf16_kernel: bf16 inputs on the MFMA matrix cores
-//    (v_mfma_f32_32x32x16_bf16), float32 accumulation, 256x256, 128x128 or 64x128 tiles with
-//    k steps of 64 staged through double-buffered LDS.
+//  * gemm_f32_kernel (tiles of 128 x 128 or 64 x 64), and gemm_f32_rows_kernel for at most 64 rows:
+//    true float32 on the matrix cores (v_mfma_f32_16x16x4_f32), no reduced-precision mode.  Both add
+//    in ONE order, so a row gives the same bits whether it is computed alone or in a batch, by
+//    either kernel.
+//  * gemm_bf16_kernel: bf16 inputs on the matrix cores (v_mfma_f32_32x32x16_bf16), float32
+//    accumulation, 256 x 256, 256 x 128, 128 x 128 or 64 x 128 tiles with k steps of 64 staged through
+//    double-buffered LDS; optionally over a share of the inner size (split k).
+//  * gemm_oneshot_bf16_kernel: the split product for few rows, operands streamed through a ring of
+//    LDS slabs filled straight from memory; splitk_reduce_kernel adds the parts and applies the epilogue.
+//  * gemm_skinny_bf16_kernel: at most 64 rows (decode steps), weights streamed once into registers.
 #include <type_traits>
 
 #include "common.h"
