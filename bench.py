@@ -322,7 +322,7 @@ def host_time(args):
                 eng.step(max_decode_steps=128 - (eng.steps_run - run0))
             b.sync()
             wall = (time.perf_counter() - t0) / 128 * 1e3
-            gpu = sum(a.elapsed_time(c) for a, c in spans) / len(spans)
+            gpu = sum(a.elapsed_time(c) for a, c in spans) / 128        # a replay may hold several steps
             out[f"decode_b{batch}"] = {"wall_ms": round(wall, 4), "gpu_ms": round(gpu, 4), "host_ms": round(wall - gpu, 4),
                                        "steps_per_call": eng.engine_config.decode_burst}
             for i in ids:

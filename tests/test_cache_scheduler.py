@@ -402,6 +402,41 @@ def test_reservation_of_a_step_that_did_not_run_is_undone():
     cm.audit()
 
 
+def test_a_run_of_steps_is_applied_as_the_steps_one_by_one_would_be():
+    """`update_burst` against `update` called once per step, on random tokens: ends by an
+    end-of-sequence token, by `max_new_tokens` and by the model's length, anywhere in the run."""
+    import copy
+    from tiny_llm_amd.engine.scheduler import Scheduled, StepPlan, RUNNING
+    rng = random.Random(3)
+    for trial in range(60):
+        steps = rng.randint(2, 12)
+        n = rng.randint(1, 5)
+        by_step = [[rng.randint(0, 6) for _ in range(n)] for _ in range(steps)]
+        results = []
+        for burst in (False, True):
+            cm, s = make_sched(num_blocks=200, block_size=4, max_seqs=8, budget=64, max_len=30, eos=(5, 6))
+            r2 = random.Random(trial)
+            for i in range(n):
+                s.add(req(f"r{i}", r2.randint(1, 12), max_new=r2.randint(2, 14), ignore_eos=r2.random() < 0.3))
+            run_plan(cm, s, s.schedule(), token=1)               # prompts; one token each (no eos)
+            p = s.schedule()
+            cm.reserve_step([(e.request.req_id, steps) for e in p.entries])
+            for e in p.entries:
+                cm.commit(e.request.req_id, e.start + steps)
+            if burst:
+                done = s.update_burst(p, by_step)
+            else:
+                done, live = [], list(range(len(p.entries)))
+                for k, toks in enumerate(by_step):
+                    sp = StepPlan([Scheduled(p.entries[i].request, p.entries[i].start + k, 1, True) for i in live], [], [])
+                    done += s.update(sp, {p.entries[i].request.req_id: toks[i] for i in live})
+                    live = [i for i in live if p.entries[i].request.status == RUNNING]
+            results.append(([r.req_id for r in done],
+                            [(e.request.output, e.request.num_computed, e.request.status, e.request.finish_reason)
+                             for e in p.entries]))
+        assert results[0] == results[1], trial
+
+
 def test_runs_of_decode_steps_end_where_a_decision_is_due():
     """How long a run of chained decode steps may be: up to the first request's end by length, never
     beside a prompt portion or while somebody waits, never beyond the free cache blocks."""

@@ -357,7 +357,7 @@ def test_runs_of_decode_steps_chained_on_the_device(dtype, folders):
     sps[2] = SamplingParams(max_new_tokens=50, temperature=0.9, top_k=20, top_p=0.9, seed=5, ignore_eos=True)
     sps[4] = SamplingParams.greedy(64)                  # may end early: eos is chosen below among its tokens
     outs = {}
-    for burst in (1, 16, 5):
+    for burst in (1, 32, 5):
         eng = Engine(folders["A"], dtype=dtype, max_num_seqs=4, max_num_batched_tokens=64, decode_burst=burst, **eng_kw)
         poison(eng)
         if burst != 1:
@@ -367,10 +367,11 @@ def test_runs_of_decode_steps_chained_on_the_device(dtype, folders):
         assert eng.runner.cache.free_blocks() == [g.pool.num_blocks for g in eng.runner.cache.groups]
         if burst != 1:
             assert any(g.runs > 20 and g.feeds_next for g in eng.runner._graphs.values())
+            assert any(g.chain is not None for g in eng.runner._graphs.values())     # four steps a launch
     eos = outs[1][4][37]
     cut = outs[1][4].index(eos) + 1
     want = [o if i != 4 else o[:cut] for i, o in enumerate(outs[1])]
-    assert outs[16] == want and outs[5] == want
+    assert outs[32] == want and outs[5] == want
     assert [len(o) for o in want] == [70, 33, 50, 21, cut, 45]
 
 

@@ -26,7 +26,7 @@ class EngineConfig:
     max_model_len: Optional[int] = None  # None = the model's max_position_embeddings
     device: int = 0
     use_graphs: bool = True            # run steps as HIP graphs, captured per shape of step
-    decode_burst: int = 16             # most decode steps the device chains without the host (1: none)
+    decode_burst: int = 32             # most decode steps the device chains without the host (1: none)
     seed: int = 0
 
     def __post_init__(self):

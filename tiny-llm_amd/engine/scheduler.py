@@ -277,15 +277,35 @@ class Scheduler:
         return k
 
     def update_burst(self, plan: StepPlan, tokens_by_step: Sequence[Sequence[int]]) -> List[Request]:
-        """After a run of decode steps: each step's tokens as `update` would take them; a request
-        that finished at one step takes no part in the later ones."""
+        """After a run of decode steps: what `update` would do with each step's tokens in turn, worked
+        out per request (a request that finishes at one step takes no part in the later ones; what
+        it was given after that step is dropped).  Returns the finished requests in the order in
+        which `update` would have finished them."""
+        steps = len(tokens_by_step)
+        eos = self.eos_token_ids
+        ended = []
+        for i, e in enumerate(plan.entries):
+            req = e.request
+            toks = [int(step[i]) for step in tokens_by_step]
+            # the first step at which `update` would finish the request (1-based), if any
+            by_length = min(req.params.max_new_tokens - len(req.output), self.max_model_len - req.num_tokens)
+            by_length = max(by_length, 1)
+            by_eos = steps + 1
+            if eos and not req.params.ignore_eos:
+                for k, t in enumerate(toks):
+                    if t in eos:
+                        by_eos = k + 1
+                        break
+            take = min(steps, by_length, by_eos)
+            req.output.extend(toks[:take])
+            req.num_computed = e.start + take
+            reason = "stop" if by_eos == take else ("length" if by_length == take else None)
+            if reason:
+                ended.append((take, i, req, reason))
         done: List[Request] = []
-        live = list(range(len(plan.entries)))
-        for k, toks in enumerate(tokens_by_step):
-            entries = [plan.entries[i] for i in live]
-            step_plan = StepPlan([Scheduled(e.request, e.start + k, 1, True) for e in entries], [], [])
-            done += self.update(step_plan, {plan.entries[i].request.req_id: toks[i] for i in live})
-            live = [i for i in live if plan.entries[i].request.status == RUNNING]
+        for _, _, req, reason in sorted(ended, key=lambda x: (x[0], x[1])):
+            self._finish(req, reason)
+            done.append(req)
         return done
 
     # ------------------------------------------------------------------ results

@@ -540,7 +540,9 @@ class StepGraph:
         self.T, self.R, self.n_out = T, R, n_out
         self.max_q_len, self.max_seq_len, self.sampling = max_q_len, max_seq_len, sampling
         self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.chain: Optional[torch.cuda.CUDAGraph] = None      # CHAIN steps of a burst as one graph
         self.capture_failed = False
+        self.chain_failed = False
         self.runs = 0
         self.logits: Optional[torch.Tensor] = None
         self._build()
@@ -569,6 +571,7 @@ class StepGraph:
             self.history = torch.zeros(self.history_steps * self.R, dtype=torch.int32, device=runner.device)
             self.history_host = torch.zeros(self.history_steps * self.R, dtype=torch.int32, pin_memory=True)
         self.graph = None
+        self.chain = None
         self._uploaded: Optional[torch.cuda.Event] = None
 
     BURST_STEPS = 32        # most decode steps a burst may hold
@@ -591,7 +594,14 @@ class StepGraph:
             self._uploaded.synchronize()
         fill_metadata(self.np, self.layout, rows, runner.cache.block_size, samples, self.seen)
         self.dev.copy_(self.host, non_blocking=True)
-        for _ in range(steps):
+        left = steps
+        if left >= self.CHAIN and self.chain is None and not self.chain_failed:
+            left -= self._capture_chain()
+        if self.chain is not None:
+            while left >= self.CHAIN:       # several steps a launch: the gap between two launches is paid once for them
+                self.chain.replay()
+                left -= self.CHAIN
+        for _ in range(left):
             self.graph.replay()
         n = steps * self.R
         self.history_host[:n].copy_(self.history[:n], non_blocking=True)
@@ -642,6 +652,32 @@ class StepGraph:
             return None, toks
         # the logits live in memory the next replay overwrites: the caller gets a copy
         return self.logits[:n_out].clone(), toks
+
+    CHAIN = 4               # decode steps captured as ONE graph for bursts
+
+    def _capture_chain(self) -> int:
+        """Captures CHAIN steps of a burst as one graph (each step's last kernel prepares the next
+        step's metadata, so the body simply repeats) and runs it once.  Returns the steps run."""
+        runner = self.runner
+        torch.cuda.synchronize()
+        gc.collect()                        # as in _capture: nothing may be finalised during a capture
+        collecting = gc.isenabled()
+        gc.disable()
+        graph = torch.cuda.CUDAGraph()
+        try:
+            with torch.cuda.graph(graph, pool=runner._graph_pool):
+                for _ in range(self.CHAIN):
+                    self._body()
+        except StepError:
+            self.chain_failed = True
+            torch.cuda.synchronize()
+            return 0
+        finally:
+            if collecting:
+                gc.enable()
+        self.chain = graph
+        graph.replay()
+        return self.CHAIN
 
     def _capture(self) -> None:
         runner = self.runner
