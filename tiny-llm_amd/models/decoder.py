@@ -65,6 +65,7 @@ class Decoder:
         # cache and state views by role, per plan entry; attached by the runner once the pools exist
         self.caches: List[Dict[str, LayerCache]] = [{} for _ in spec.plan]
         self.states: List[Dict[str, torch.Tensor]] = [{} for _ in spec.plan]
+        self._graph_safe: Optional[bool] = None
 
     # ---------------------------------------------------------------- declarations
     def parts(self) -> List[Part]:
@@ -76,10 +77,13 @@ class Decoder:
 
     @property
     def graph_safe(self) -> bool:
-        """True if every part (and every part's position encoding) may be captured in a HIP graph."""
-        parts = self.parts()
-        parts += [getattr(p, "position", None) for p in parts]
-        return all(p.graph_safe for p in parts if p is not None)
+        """True if every part (and every part's position encoding) may be captured in a HIP graph.
+        (Asked at every step; the parts do not change once the decoder is built.)"""
+        if self._graph_safe is None:
+            parts = self.parts()
+            parts += [getattr(p, "position", None) for p in parts]
+            self._graph_safe = all(p.graph_safe for p in parts if p is not None)
+        return self._graph_safe
 
     def weight_specs(self) -> List[WeightSpec]:
         specs: List[WeightSpec] = []
