@@ -17,6 +17,7 @@
 #include "common.h"
 #include "no_alloc.h"
 #include <mutex>
+#include <type_traits>
 
 namespace {
 
@@ -934,7 +935,11 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_prefill_bf16_kernel(
     }
     const bf16_t* Kl = Kbuf[cur];
     const bf16_t* Vl = Vbuf[cur];
-    if (kt_idx * FA_KT <= wave_hi) {
+    // The whole tile in two compilations, with and without the mask: written as one body with a
+    // uniform condition around the mask, the compiler turns the condition into selects and every
+    // tile pays the mask's 65 vector instructions (of about 200).
+    auto work_on_tile = [&](auto with_mask) {
+      constexpr bool MASK = decltype(with_mask)::value;
       f32x4 sc[FP_RT][4];
 #pragma unroll
       for (int kt = 0; kt < 4; ++kt)
@@ -953,11 +958,10 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_prefill_bf16_kernel(
         }
       bf16x8 pb[FP_RT][2], pl[FP_RT][2];
       const int tile_j0 = kt_idx * FA_KT;
-      const bool no_mask = all_valid && tile_j0 + FA_KT - 1 <= wave_lo_pos && tile_j0 >= wave_hi_lo;
 #pragma unroll
       for (int rt = 0; rt < FP_RT; ++rt) {
         float m_tile = kNegBig;
-        if (no_mask) {
+        if constexpr (!MASK) {
 #pragma unroll
           for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
@@ -1042,6 +1046,14 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_prefill_bf16_kernel(
           for (int rt = 0; rt < FP_RT; ++rt)
             l_acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, lo ? pl[rt][st] : pb[rt][st], l_acc[rt], 0, 0, 0);
         }
+    };
+    if (kt_idx * FA_KT <= wave_hi) {
+      // a key tile that lies wholly between the wave's smallest position and its largest window
+      // start is visible to every row
+      const int tile_j0 = kt_idx * FA_KT;
+      const bool no_mask = all_valid && tile_j0 + FA_KT - 1 <= wave_lo_pos && tile_j0 >= wave_hi_lo;
+      if (no_mask) work_on_tile(std::false_type{});
+      else work_on_tile(std::true_type{});
     }
     __syncthreads();
   }
