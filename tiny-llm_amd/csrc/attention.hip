@@ -879,28 +879,36 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_prefill_bf16_kernel(
   // requested while the current tile is being worked on
   constexpr int KC = (KS * 4 + WAVES - 1) / WAVES, VC = (HD / 8 + WAVES - 1) / WAVES;
   bf16x8 k_stage[KC], v_stage[VC];
-  auto fetch_tile = [&](int kt_idx) {
-    const int j = kt_idx * FA_KT + lane;
-    const bool in_range = j >= kv_begin && j < kv_end;
-    int64_t row_off = 0;
-    if (in_range) {
-      const int jb = bs_shift >= 0 ? j >> bs_shift : j / block_size;     // uniform choice: no division
-      const int64_t blk = bt[jb];
-      row_off = ((blk * nkv + kvh) * block_size + (j - jb * block_size)) * HD;
-    }
-    const bf16_t* kp = k_cache + row_off;
-    const bf16_t* vp = v_cache + row_off;
+  // The page of this thread's key row is looked up one tile further ahead than the row itself is
+  // requested, so that the request does not begin with a dependent round trip to memory.
+  // Rows of a tile outside the request's keys [kv_begin, kv_end) are read from the nearest row
+  // inside instead (finite data of the same request; every score of such a key is masked, and its
+  // probability is an exact zero): so no load is predicated, which would make it a branch.
+  auto key_row = [&](int kt_idx) { return min(max(kt_idx * FA_KT + lane, kv_begin), kv_end - 1); };
+  auto page_of_row = [&](int kt_idx) {
+    const int j = key_row(kt_idx);
+    return bt[bs_shift >= 0 ? j >> bs_shift : j / block_size];     // uniform choice: no division
+  };
+  auto fetch_tile = [&](int kt_idx, int blk) {
+    const int j = key_row(kt_idx);
+    const int jb = bs_shift >= 0 ? j >> bs_shift : j / block_size;
+    // rows of the cache fit 32 bits (checked on the host); only the last product is 64 bits wide
+    const int row = (max(blk, 0) * nkv + kvh) * block_size + (j - jb * block_size);
+    const bf16_t* kp = k_cache + (int64_t)row * HD;
+    const bf16_t* vp = v_cache + (int64_t)row * HD;
 #pragma unroll
     for (int ci = 0; ci < KC; ++ci) {
       const int c = ci * WAVES + wave;
       bf16x8 z = {};
-      k_stage[ci] = (in_range && c * 8 < HD) ? *(const bf16x8*)(kp + c * 8) : z;
+      k_stage[ci] = z;
+      if (c * 8 < HD) k_stage[ci] = *(const bf16x8*)(kp + c * 8);      // uniform: the dims beyond HD stay zero
     }
 #pragma unroll
     for (int ci = 0; ci < VC; ++ci) {
       const int c = ci * WAVES + wave;
       bf16x8 z = {};
-      v_stage[ci] = (in_range && c < HD / 8) ? *(const bf16x8*)(vp + c * 8) : z;
+      v_stage[ci] = z;
+      if (c < HD / 8) v_stage[ci] = *(const bf16x8*)(vp + c * 8);
     }
   };
   // registers -> LDS, both tiles as they are (the reads of V transpose)
@@ -918,11 +926,22 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_prefill_bf16_kernel(
       if (c < HD / 8) *(bf16x8*)(Vl + lane * VS + c * 8) = v_stage[ci];
     }
   };
+  int next_page = 0;      // of the tile that is requested next
   if (first_tile < last_tile) {
-    fetch_tile(first_tile);
+    fetch_tile(first_tile, page_of_row(first_tile));
+    if (first_tile + 1 < last_tile) next_page = page_of_row(first_tile + 1);
     store_tile(0);
-    if (first_tile + 1 < last_tile) fetch_tile(first_tile + 1);
+    if (first_tile + 1 < last_tile) {
+      fetch_tile(first_tile + 1, next_page);
+      if (first_tile + 2 < last_tile) next_page = page_of_row(first_tile + 2);
+    }
   }
+  // Every load so far has arrived before the loop begins: the queries above all.  The compiler's
+  // placement of waits sees a way into the loop on which they are still in flight (around the
+  // block above) and would otherwise wait for ALL loads before the first matrix instruction of
+  // every iteration, just after the next tile's rows have been requested.  The first tile's
+  // rows are needed here anyway; the second tile's are asked for again below.
+  __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0)
   __syncthreads();
 
   for (int kt_idx = first_tile; kt_idx < last_tile; ++kt_idx) {
@@ -931,7 +950,10 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_prefill_bf16_kernel(
     // has finished reading before the last barrier; then the tile after it is requested
     if (kt_idx + 1 < last_tile) {
       store_tile(cur ^ 1);
-      if (kt_idx + 2 < last_tile) fetch_tile(kt_idx + 2);
+      if (kt_idx + 2 < last_tile) {
+        fetch_tile(kt_idx + 2, next_page);
+        if (kt_idx + 3 < last_tile) next_page = page_of_row(kt_idx + 3);
+      }
     }
     const bf16_t* Kl = Kbuf[cur];
     const bf16_t* Vl = Vbuf[cur];

@@ -785,6 +785,8 @@ def flash_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
             _fail("tile arrays must be int32 [tiles]")
     if not (q.stride(0) % 8 == 0 and out.stride(0) % 4 == 0):
         _fail("q and output rows must be vector aligned")
+    if not (k_cache.shape[0] * k_cache.shape[1] * k_cache.shape[2] < 2 ** 31):
+        _fail("the prefill attention kernel counts the rows of a cache in 32 bits")
     part_o = part_ml = None
     if n_splits > 1:
         need = n_splits * T * num_heads * (head_dim + 2)
