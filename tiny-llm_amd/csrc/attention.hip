@@ -95,7 +95,7 @@ __global__ __launch_bounds__(TL_WAVE) void paged_attention_kernel(
 // flash_attn_bf16_kernel: the same function on the matrix cores, for head sizes
 // that are multiples of 16 up to 128 and up to 16 query heads per kv head.
 //
-// A workgroup (eight wave64) owns a tile of 16 query rows that
+// A workgroup (eight wave64, four for heads beyond 64 dims) owns a tile of 16 query rows that
 // share one request and one kv head: `tile_ntok` consecutive tokens times the G query heads of the
 // group, row = token * G + head.  The waves split the 64-key tiles of the request's
 // cache between them (and `n_splits` workgroups split them further for decoding
@@ -109,9 +109,9 @@ __global__ __launch_bounds__(TL_WAVE) void paged_attention_kernel(
 // the B-operand layout of the second product O^T = V^T P^T, and the output
 // accumulator of a lane belongs to that same row.  The probabilities enter the second
 // product as a sum of two bfloat16 terms, so no accuracy is lost against a float32
-// softmax times bfloat16 values.  V is transposed on its way into
-// LDS.  Rows of a tile outside [kv_begin, kv_end) are zeroed:
-// stale pages may hold anything, and 0 * NaN is NaN.
+// softmax times bfloat16 values.  V is staged in LDS as it is and transposed by the reads.
+// Value rows of a tile outside [kv_begin, kv_end) read finite stand-in data: stale pages may hold
+// anything, and 0 * NaN is NaN.
 constexpr int FA_KT = 64;
 constexpr int FA_VPAD = 8;      // padding of a row of the row-major V tile in LDS (elements)
 constexpr float kNegBig = -1.0e30f;   // "no key yet": finite, so exp2(m - m') never sees inf - inf
@@ -199,12 +199,14 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
   // known here: the pages of this lane's rows in it (one value row, four key rows) are requested
   // together with the position.  The index is clamped into the table; an entry that belongs to no
   // key of the request is not used.
-  const int spec_j = (split * WAVES + wave) * FA_KT;
-  const int spec_v = max(bt[min((spec_j + lane) / block_size, max_blocks - 1)], 0);
-  int spec_k[4];
-#pragma unroll
-  for (int kt = 0; kt < 4; ++kt)
-    spec_k[kt] = max(bt[min((spec_j + kt * 16 + (lane % 16)) / block_size, max_blocks - 1)], 0);
+  // One lookup a lane: the page of key row `lane` of the 64-key tile that begins at key j0, as the
+  // table holds it (any arithmetic on it here would make the wave wait for it here).  The lanes
+  // hand the pages of the rows they load to each other.
+  const int bs_shift = (block_size & (block_size - 1)) == 0 ? __builtin_ctz(block_size) : -1;
+  auto page_index = [&](int j) { return bs_shift >= 0 ? j >> bs_shift : j / block_size; };     // uniform choice
+  auto pages_at = [&](int j0) { return bt[min(page_index(j0 + lane), max_blocks - 1)]; };
+  // (of the wave's first tile if the key range begins at 0: known without the positions)
+  int next_pages = pages_at((split * WAVES + wave) * FA_KT);
 
   // this lane's query row
   const int tok_local = r16 / G, hh = r16 % G;
@@ -254,12 +256,13 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
   // A wave reads its 64-key tile by itself, so nothing in this loop waits for another wave.  Keys
   // go straight from memory into MFMA operands (lane (r16, g) holds dims ks*32 + g*8.. of key rows
   // kt*16 + r16: the layout the score product wants); values pass through an LDS area of the wave's
-  // own (lane = key row), stored as they are; the reads for the second product transpose them.
+  // own, [key][dim] as they are; the reads for the second product transpose them.
   constexpr int VCH = HD / 8;
   bf16x8 k_op[4][KS], v_stage[VCH];
+  // rows of the cache fit 32 bits (checked on the host); only the last product is 64 bits wide
   auto row_offset = [&](int j, int blk) {
-    const int jb = j / block_size;
-    return (((int64_t)blk * nkv + kvh) * block_size + (j - jb * block_size)) * HD;
+    const int row = (blk * nkv + kvh) * block_size + (j - page_index(j) * block_size);
+    return (int64_t)row * HD;
   };
   // Fused mode: the new token's key is rotated here, by the lanes that will hold its chunks as
   // operands (in the wave whose tile it falls into), and written to the cache; its value is read
@@ -286,47 +289,53 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
       }
     }
   }
-  // Loads are unconditional, with the address clamped into the caches (a row outside the tile's
-  // key range reads row 0 of page 0 and is zeroed afterwards: stale pages may hold anything, and
-  // 0 * NaN is NaN): a predicated load would become a branch, and the loads could not all be in
-  // flight together.
-  auto page_of = [&](int j) { return max(bt[min(j / block_size, max_blocks - 1)], 0); };
-  auto fetch = [&](int it, bool spec) {
-    const int base = ((it0 + it) * stride + mine) * FA_KT;
-    bf16x8 z = {};
-    bool k_in[4];
+  // Loads are unconditional and nothing is done to what they bring before it is used: a predicated
+  // load would become a branch, and a select on a loaded register makes the wave wait for the load
+  // where the select stands, so that the next tile's rows would not be on their way while this
+  // tile is worked on.  A key row outside the tile's key range reads row 0 of page 0: whatever it
+  // holds reaches that key's scores only, which the mask replaces.  A value row outside the range
+  // must be finite (its probabilities are exact zeros, and 0 * NaN is NaN; stale pages may hold
+  // anything), so it reads finite data that is at hand: HD elements of the query row.  The key
+  // dims beyond HD of the last k step (head sizes that are no multiple of 32) repeat dims of the
+  // row and meet zeros in the query operand.
+  // Values are requested as whole rows (chunk f = c * 64 + lane of the tile's 64 rows x VCH chunks,
+  // so that a load instruction covers 1 KB of consecutive rows): with a row per lane an instruction
+  // touched 64 cache lines for 16 bytes each, and looking those up was what a round of tiles cost.
+  const bf16_t* finite_row = q + (int64_t)tok0 * q_stride + (int64_t)kvh * G * HD;
+  auto tile_base = [&](int it) { return ((it0 + it) * stride + mine) * FA_KT; };
+  auto fetch = [&](int it, int pages_raw) {
+    const int base = tile_base(it);
+    const int pages = max(pages_raw, 0);
     const bf16_t* kp[4];
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt) {
-      const int j = base + kt * 16 + r16;
-      k_in[kt] = j >= kv_begin && j < kv_end;
-      const int64_t off = row_offset(j, spec ? spec_k[kt] : page_of(j));
-      kp[kt] = k_cache + (k_in[kt] ? off : 0);
+      const int row = kt * 16 + r16, j = base + row;
+      const bool k_in = j >= kv_begin && j < kv_end;
+      const int64_t off = row_offset(j, __shfl(pages, row, TL_WAVE));
+      kp[kt] = k_cache + (k_in ? off : 0);
     }
-    const int jv = base + lane;
-    const bool v_in = jv >= kv_begin && jv < kv_end;
-    const int64_t v_off = row_offset(jv, spec ? spec_v : page_of(jv));
-    const bf16_t* vp = v_cache + (v_in ? v_off : 0);
-    if (do_rope && jv == new_pos) vp = new_v;      // not in the cache yet
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) k_op[kt][ks] = *(const bf16x8*)(kp[kt] + min(ks * 32 + g * 8, HD - 8));
 #pragma unroll
-    for (int c = 0; c < VCH; ++c) v_stage[c] = *(const bf16x8*)(vp + c * 8);
-#pragma unroll
-    for (int kt = 0; kt < 4; ++kt)
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks)
-        if (!k_in[kt] || ks * 32 + g * 8 >= HD) k_op[kt][ks] = z;
-#pragma unroll
-    for (int c = 0; c < VCH; ++c)
-      if (!v_in) v_stage[c] = z;
+    for (int c = 0; c < VCH; ++c) {
+      const int f = c * TL_WAVE + lane, row = f / VCH, ch = f % VCH, j = base + row;
+      const bool v_in = j >= kv_begin && j < kv_end;
+      const int64_t off = row_offset(j, __shfl(pages, row, TL_WAVE));
+      const bf16_t* vp = v_in ? v_cache + off : finite_row;
+      if (do_rope && j == new_pos) vp = new_v;      // not in the cache yet
+      v_stage[c] = *(const bf16x8*)(vp + ch * 8);
+    }
   };
-  // The next tile is requested as soon as the registers of this one are free.
+  // The next tile is requested as soon as the registers of this one are free, and its pages are
+  // looked up an iteration before that, so that the request does not begin with a round trip.
+  // (Two tiles in flight per wave, in two register sets, were measured to gain nothing: what a
+  // compute unit can have on its way from memory is the limit, about 40 GB/s.)
   if (iters > 0) {
-    if (it0 == 0) fetch(0, true);
-    else fetch(0, false);
+    if (it0 != 0) next_pages = pages_at(tile_base(0));
+    fetch(0, next_pages);
+    if (iters > 1) next_pages = pages_at(tile_base(1));
   }
 
   for (int it = 0; it < iters; ++it) {
@@ -341,14 +350,18 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
           for (int ks = 0; ks < KS; ++ks)
             if (kt == (new_pos % FA_KT) / 16) k_op[kt][ks] = new_k[ks];
       }
-      if (lane == new_pos % FA_KT) {
 #pragma unroll
-        for (int c = 0; c < VCH; ++c) *(bf16x8*)(fused.v_cache_w + new_off + c * 8) = v_stage[c];
+      for (int c = 0; c < VCH; ++c) {
+        const int f = c * TL_WAVE + lane;
+        if (f / VCH == new_pos % FA_KT) *(bf16x8*)(fused.v_cache_w + new_off + (f % VCH) * 8) = v_stage[c];
       }
     }
-    // values: registers -> this wave's LDS area, as they are (the reads transpose)
+    // values: registers -> this wave's LDS area, [key][dim] as they are (the reads transpose)
 #pragma unroll
-    for (int c = 0; c < VCH; ++c) *(bf16x8*)(Vl + lane * VS + c * 8) = v_stage[c];
+    for (int c = 0; c < VCH; ++c) {
+      const int f = c * TL_WAVE + lane;
+      *(bf16x8*)(Vl + (f / VCH) * VS + (f % VCH) * 8) = v_stage[c];
+    }
     // scores, transposed: sc[kt][r] = S^T[key kt*16 + g*4 + r][row r16]
     f32x4 sc[4];
 #pragma unroll
@@ -358,7 +371,10 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
       for (int ks = 0; ks < KS; ++ks)
         sc[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_op[kt][ks], qf[ks], sc[kt], 0, 0, 0);
     }
-    if (it + 1 < iters) fetch(it + 1, false);
+    if (it + 1 < iters) {
+      fetch(it + 1, next_pages);
+      if (it + 2 < iters) next_pages = pages_at(tile_base(it + 2));
+    }
     // the LDS operations of one wave are carried out in order; the fences keep the compiler from
     // moving the reads of other lanes' rows above the writes
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -1201,7 +1217,10 @@ static int launch_flash_w(const bf16_t* q, int64_t q_stride, const bf16_t* k_cac
   return TL_OK;
 }
 
-constexpr int flash_waves(int) { return 8; }
+// Waves of a flash_attn_bf16_kernel workgroup.  A tile's keys and values are 16 registers per 16
+// dims of the head: with eight waves (256 registers a wave) the heads beyond 64 dims spilled 27 to
+// 74 registers to memory and the kernel took twice the time that four waves take.
+constexpr int flash_waves(int hd) { return hd <= 64 ? 8 : 4; }
 
 template <int HDT>
 static int launch_flash(const bf16_t* q, int64_t q_stride, const bf16_t* k_cache, const bf16_t* v_cache,

@@ -671,6 +671,8 @@ def flash_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                 _fail("tile arrays must be int32 [tiles]")
     if not (q.stride(0) % 8 == 0):
         _fail("q rows must be 16-byte aligned")
+    if not (k_cache.shape[0] * k_cache.shape[1] * k_cache.shape[2] < 2 ** 31):
+        _fail("the attention kernel counts the rows of a cache in 32 bits")
     part_o = part_ml = None
     if n_splits > 1 and not static_scratch:
         need = n_splits * T * num_heads * (head_dim + 2)
