@@ -233,6 +233,43 @@ def test_linear_handoff(M, K, N, N2):
                              rows=torch.arange(65, dtype=torch.int32, device=DEV))
 
 
+@pytest.mark.parametrize("M,K,N,N2", [(65, 64, 128, 200), (300, 256, 1024, 1030), (2048, 64, 8576, 96),
+                                      (512, 512, 2048, 1024), (1000, 136, 320, 16390)])
+def test_linear_handoff_many_rows(M, K, N, N2):
+    """The hand-off of a norm through the tiled kernel: the producer writes the operand and a sum
+    of squares per 64 columns (also when it is launched in two parts), the consumer works the row
+    factor out of the parts in its epilogue."""
+    g = torch.Generator().manual_seed(M + N)
+    z = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w1 = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16)
+    res = torch.randn(M, N, generator=g)
+    w2 = (torch.randn(N2, N, generator=g) / math.sqrt(N)).to(torch.bfloat16)
+    x_ref = z.double() @ w1.double().T + res.double()
+    assert ops().can_hand_off(M, N, K, torch.bfloat16)
+    for nwt in (torch.float32, torch.bfloat16):
+        nw = (1 + 0.1 * torch.randn(N, generator=g)).to(nwt)
+        x = res.clone().to(DEV)
+        operand = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+        sumsq = torch.full((M, ops().handoff_parts(M, N, K)), float("nan"), dtype=torch.float32, device=DEV)
+        ops().linear_handoff(z.to(DEV), w1.to(DEV), x, x, emit=(nw.to(DEV), operand, sumsq))
+        assert rel(x, x_ref) < 1e-5
+        xs = x.cpu().double()
+        assert torch.equal(operand.cpu(), (nw.float() * x.cpu()).to(torch.bfloat16))
+        assert not torch.isnan(sumsq).any()
+        assert rel(sumsq.sum(dim=1), (xs * xs).sum(dim=1)) < 1e-6
+        inv = 1.0 / torch.sqrt((xs * xs).mean(dim=-1, keepdim=True) + 1e-5)
+        c = (operand.cpu().double() @ w2.double().T) * inv
+        out = torch.empty(M, N2, dtype=torch.float32, device=DEV)
+        ops().linear_handoff(operand, w2.to(DEV), out, prepared=(sumsq, 1e-5, N))
+        assert rel(out, c) < 1e-5
+        ob = torch.empty(M, N2, dtype=torch.bfloat16, device=DEV)
+        ops().linear_handoff(operand, w2.to(DEV), ob, prepared=(sumsq, 1e-5, N))
+        assert rel(ob, c) < 6e-3
+        zz = torch.empty(M, N2 // 2, dtype=torch.bfloat16, device=DEV)
+        ops().linear_handoff(operand, w2.to(DEV), zz, epilogue="swiglu", prepared=(sumsq, 1e-5, N))
+        assert rel(zz, plain.silu(c[:, 0::2]) * c[:, 1::2]) < 6e-3
+
+
 @pytest.mark.parametrize("M,K,N", [(2048, 64, 8576), (1000, 136, 16390)])
 def test_linear_two_part_launch(M, K, N):
     """Wide products are launched in two parts (whole rounds of the largest tile, then the rest with
@@ -310,10 +347,9 @@ def test_linear_split_k(M, K, N):
     w2 = (torch.randn(5000, N, generator=g) / math.sqrt(N)).to(torch.bfloat16)
     inv = 1.0 / torch.sqrt((xs * xs).mean(dim=-1, keepdim=True) + 1e-5)
     c = (operand.cpu().double() @ w2.double().T) * inv
-    if M <= 64 or ops().split_k(M, 5000, N) > 1:
-        zz = torch.empty(M, 2500, dtype=torch.bfloat16, device=DEV)
-        ops().linear_handoff(operand, w2.to(DEV), zz, epilogue="swiglu", prepared=(sumsq, 1e-5, N))
-        assert rel(zz, plain.silu(c[:, 0::2]) * c[:, 1::2]) < 6e-3
+    zz = torch.empty(M, 2500, dtype=torch.bfloat16, device=DEV)
+    ops().linear_handoff(operand, w2.to(DEV), zz, epilogue="swiglu", prepared=(sumsq, 1e-5, N))
+    assert rel(zz, plain.silu(c[:, 0::2]) * c[:, 1::2]) < 6e-3
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

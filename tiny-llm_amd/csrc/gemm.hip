@@ -251,13 +251,35 @@ constexpr int B_BK = 64;
 constexpr int B_LD = B_BK + 8;  // LDS row stride in elements: 144 bytes, keeps 16-byte alignment
 constexpr int B_XCDS = 8;
 
+// What the epilogue of the tiled kernel does to a row besides the product: a factor per row
+// (`row_scale`), or a norm handed from product to product as the few-row kernel does it (see
+// SkinnyArgs).  The producer (float32 output, no SiLU-gate, N a multiple of 64, ldo of 4) also writes
+// emit_operand[m, n] = bf16(emit_w[n] * out[m, n]) and, for every 64 columns, the sum of out^2 into
+// emit_sumsq[m, n / 64] (rows of `emit_parts` parts).  The consumer takes such an operand as `a`
+// and in_sumsq [rows, in_parts], and its row factor is 1 / sqrt(sum / in_width + in_eps).
+struct TileNorm {
+  const float* row_scale = nullptr;
+  const void* emit_w = nullptr;
+  int emit_w_is_f32 = 0;
+  bf16_t* emit_operand = nullptr;
+  int64_t emit_ld = 0;                // row stride of the operand
+  float* emit_sumsq = nullptr;
+  int emit_parts = 0;
+  const float* in_sumsq = nullptr;
+  int in_parts = 0, in_width = 0;
+  float in_eps = 0.f;
+  TileNorm() = default;
+  TileNorm(const float* rs) : row_scale(rs) {}
+};
+
 template <int BM, int BN, int WM, int WN>
 struct GemmShape {
   static constexpr int THREADS = WM * WN * TL_WAVE;
   static constexpr int TM = BM / WM, TN = BN / WN;        // a wave's outputs
   static constexpr int MI = TM / 32, NJ = TN / 32;        // as 32 x 32 MFMA tiles
   static constexpr int AC = BM * (B_BK / 8) / THREADS, WC = BN * (B_BK / 8) / THREADS;
-  static constexpr size_t SMEM = (size_t)2 * (BM + BN) * B_LD * sizeof(bf16_t);
+  static constexpr size_t SMEM = (size_t)2 * (BM + BN) * B_LD * sizeof(bf16_t);      // the operand tiles
+  static constexpr size_t SMEM_ALL = SMEM + BM * sizeof(float);                      // and a factor per row behind them
   static_assert(TM % 32 == 0 && TN % 32 == 0 && AC >= 1 && WC >= 1, "tile does not divide");
 };
 
@@ -267,9 +289,8 @@ __global__ __launch_bounds__(WM * WN * TL_WAVE) void gemm_bf16_kernel(const bf16
                                                                       const bf16_t* __restrict__ w,
                                                                       TO* __restrict__ out,
                                                                       const float* __restrict__ residual,
-                                                                      const float* __restrict__ row_scale, int M,
-                                                                      int N, int K, int64_t lda, int64_t ldo,
-                                                                      int k_per_split) {
+                                                                      const TileNorm nm, int M, int N, int K,
+                                                                      int64_t lda, int64_t ldo, int k_per_split) {
   using S = GemmShape<BM, BN, WM, WN>;
   constexpr int MI = S::MI, NJ = S::NJ, THREADS = S::THREADS;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -298,6 +319,20 @@ __global__ __launch_bounds__(WM * WN * TL_WAVE) void gemm_bf16_kernel(const bf16
     for (int j = 0; j < NJ; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // A norm handed over: the factors of this tile's rows are worked out once, here, where the loads
+  // hide behind the main loop (16 threads share a row's parts out), and wait in LDS for the
+  // epilogue; the barriers of the main loop lie in between.
+  float* row_factor = (float*)(smem_raw + S::SMEM);      // [BM]
+  if (nm.in_sumsq) {      // uniform
+    for (int r = tid / 16; r < BM; r += THREADS / 16) {
+      const int64_t at = (int64_t)min(m0 + r, M - 1) * nm.in_parts;
+      float t = 0.f;
+      for (int q = tid % 16; q < nm.in_parts; q += 16) t += nm.in_sumsq[at + q];
+      t = group_sum<16>(t);
+      if (tid % 16 == 0) row_factor[r] = 1.f / sqrtf(t / (float)nm.in_width + nm.in_eps);
+    }
+  }
 
   // One k step of both operand tiles is AC + WC 16-byte pieces per thread, fetched with buffer
   // loads: the address is the tile's first row (the buffer's base, per workgroup) + an offset per
@@ -450,8 +485,11 @@ __global__ __launch_bounds__(WM * WN * TL_WAVE) void gemm_bf16_kernel(const bf16
       const int r = c / 16, col = (c % 16) * 4;
       const int m = m0 + wm * S::TM + i * 32 + r, n = n0 + wn * S::TN + col;
       if (m >= M || n >= N) continue;
+      // the row's factor (1 / rms of a norm left out of the operand): given, or that of a norm handed over
+      float rs = 1.f;
+      if (nm.in_sumsq) rs = row_factor[m - m0];
+      else if (nm.row_scale) rs = nm.row_scale[m];
       const f32x4 s4 = *(const f32x4*)(cstage + r * E_LD + col);
-      const float rs = row_scale ? row_scale[m] : 1.f;   // e.g. 1 / rms of a norm left out of the operand
       float v[4] = {s4[0] * rs, s4[1] * rs, s4[2] * rs, s4[3] * rs};
       if constexpr (SWIGLU) {   // (gate, up, gate, up) -> two outputs; N is even and n a multiple of 4
         const int64_t oz = (int64_t)m * ldo + n / 2;
@@ -478,6 +516,22 @@ __global__ __launch_bounds__(WM * WN * TL_WAVE) void gemm_bf16_kernel(const bf16
         if constexpr (sizeof(TO) == 4) {
           f32x4 sv = {v[0], v[1], v[2], v[3]};
           *(f32x4*)((float*)out + o) = sv;
+          if constexpr (!SWIGLU) {
+            if (nm.emit_operand) {      // uniform; N is a multiple of 64: the 16 lanes of a row are all here or none is
+              float wn[4];
+              if (nm.emit_w_is_f32) {
+                const f32x4 w4 = *(const f32x4*)((const float*)nm.emit_w + n);
+                wn[0] = w4[0]; wn[1] = w4[1]; wn[2] = w4[2]; wn[3] = w4[3];
+              } else {
+                const bf16x4 w4 = *(const bf16x4*)((const bf16_t*)nm.emit_w + n);
+                wn[0] = (float)w4[0]; wn[1] = (float)w4[1]; wn[2] = (float)w4[2]; wn[3] = (float)w4[3];
+              }
+              bf16x4 ev = {(bf16_t)(wn[0] * v[0]), (bf16_t)(wn[1] * v[1]), (bf16_t)(wn[2] * v[2]), (bf16_t)(wn[3] * v[3])};
+              *(bf16x4*)(nm.emit_operand + (int64_t)m * nm.emit_ld + n) = ev;
+              const float sq = group_sum<16>((v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]));
+              if (lane % 16 == 0) nm.emit_sumsq[(int64_t)m * nm.emit_parts + n / 64] = sq;
+            }
+          }
         } else {
           bf16x4 sv = {(bf16_t)v[0], (bf16_t)v[1], (bf16_t)v[2], (bf16_t)v[3]};
           *(bf16x4*)((bf16_t*)out + o) = sv;
@@ -499,29 +553,32 @@ __global__ __launch_bounds__(WM * WN * TL_WAVE) void gemm_bf16_kernel(const bf16
 
 template <int BM, int BN, int WM, int WN, typename TO, bool SWIGLU, bool FULL>
 static int launch_gemm_bf16_full(const bf16_t* a, const bf16_t* w, TO* out, const float* residual,
-                                 const float* row_scale, int M, int N, int K, int64_t lda, int64_t ldo,
+                                 const TileNorm& row_scale, int M, int N, int K, int64_t lda, int64_t ldo,
                                  int k_per_split, hipStream_t stream) {
   using S = GemmShape<BM, BN, WM, WN>;
   static bool configured = false;
   if (!configured) {
     if (hipFuncSetAttribute((const void*)gemm_bf16_kernel<BM, BN, WM, WN, TO, SWIGLU, FULL>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::SMEM) != hipSuccess)
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::SMEM_ALL) != hipSuccess)
       return TL_ERR_LAUNCH;
     configured = true;
   }
   // a tile's rows are addressed with 32-bit byte offsets from its first row
   if ((int64_t)BM * lda * 2 >= 0x7fffffff || (int64_t)BN * K * 2 >= 0x7fffffff) return TL_ERR_ARG;
+  if (row_scale.emit_operand && (SWIGLU || sizeof(TO) != 4 || N % 64 || ldo % 4 || k_per_split > 0)) return TL_ERR_ARG;
+  if (row_scale.in_sumsq && k_per_split > 0) return TL_ERR_ARG;      // a split product has no epilogue of its own
   const int64_t splits = k_per_split > 0 ? (K + k_per_split - 1) / k_per_split : 1;
   const int64_t total = (int64_t)((N + BN - 1) / BN) * ((M + BM - 1) / BM) * splits;
   const int64_t grid = (total + B_XCDS - 1) / B_XCDS * B_XCDS;
   if (grid > 0x7fffffff) return TL_ERR_ARG;
   hipLaunchKernelGGL((gemm_bf16_kernel<BM, BN, WM, WN, TO, SWIGLU, FULL>), dim3((unsigned)grid), dim3(S::THREADS),
-                     S::SMEM, stream, a, w, out, residual, row_scale, M, N, K, lda, ldo, k_per_split);
+                     S::SMEM_ALL, stream, a, w, out, residual, row_scale, M, N, K, lda, ldo, k_per_split);
+  static_assert(sizeof(TileNorm) <= 96, "passed by value");
   return TL_OK;
 }
 
 template <int BM, int BN, int WM, int WN, typename TO, bool SWIGLU>
-static int launch_gemm_bf16(const bf16_t* a, const bf16_t* w, TO* out, const float* residual, const float* row_scale,
+static int launch_gemm_bf16(const bf16_t* a, const bf16_t* w, TO* out, const float* residual, const TileNorm& row_scale,
                             int M, int N, int K, int64_t lda, int64_t ldo, int k_per_split, hipStream_t stream) {
   if (M % BM == 0 && N % BN == 0 && K % B_BK == 0)
     return launch_gemm_bf16_full<BM, BN, WM, WN, TO, SWIGLU, true>(a, w, out, residual, row_scale, M, N, K, lda, ldo,
@@ -560,7 +617,7 @@ static int best_tile(int M, int N, double* cost) {
 
 template <typename TO, bool SWIGLU>
 static int launch_gemm_bf16_tile(int c, const bf16_t* a, const bf16_t* w, TO* out, const float* residual,
-                                 const float* row_scale, int M, int N, int K, int64_t lda, int64_t ldo,
+                                 const TileNorm& row_scale, int M, int N, int K, int64_t lda, int64_t ldo,
                                  int k_per_split, hipStream_t stream) {
   switch (c) {
     case 0:
@@ -584,7 +641,7 @@ static int launch_gemm_bf16_tile(int c, const bf16_t* a, const bf16_t* w, TO* ou
 // workgroups mostly empty (2048 x 11264: 352 tiles of 256 x 256 on 256 compute units).
 template <typename TO, bool SWIGLU>
 static int launch_gemm_bf16_any(const bf16_t* a, const bf16_t* w, TO* out, const float* residual,
-                                const float* row_scale, int M, int N, int K, int64_t lda, int64_t ldo,
+                                const TileNorm& row_scale, int M, int N, int K, int64_t lda, int64_t ldo,
                                 int tile, int k_per_split, hipStream_t stream) {
   if (tile >= 1 && tile <= 4)
     return launch_gemm_bf16_tile<TO, SWIGLU>(tile - 1, a, w, out, residual, row_scale, M, N, K, lda, ldo, k_per_split,
@@ -602,8 +659,15 @@ static int launch_gemm_bf16_any(const bf16_t* a, const bf16_t* w, TO* out, const
         int rc = launch_gemm_bf16_tile<TO, SWIGLU>(0, a, w, out, residual, row_scale, M, n_first, K, lda, ldo, 0, stream);
         if (rc != TL_OK) return rc;
         const int64_t o_off = SWIGLU ? n_first / 2 : n_first;
+        TileNorm rest_norm = row_scale;      // what it emits belongs to columns n_first on (a multiple of 256)
+        if (rest_norm.emit_operand) {
+          rest_norm.emit_w = rest_norm.emit_w_is_f32 ? (const void*)((const float*)rest_norm.emit_w + n_first)
+                                                     : (const void*)((const bf16_t*)rest_norm.emit_w + n_first);
+          rest_norm.emit_operand += n_first;
+          rest_norm.emit_sumsq += n_first / 64;
+        }
         return launch_gemm_bf16_tile<TO, SWIGLU>(rest, a, w + (int64_t)n_first * K, out + o_off,
-                                                 residual ? residual + o_off : nullptr, row_scale, M, N - n_first, K,
+                                                 residual ? residual + o_off : nullptr, rest_norm, M, N - n_first, K,
                                                  lda, ldo, 0, stream);
       }
     }
@@ -1445,18 +1509,19 @@ int tl_linear(const void* a, const void* w, void* out, const float* residual, co
   return tl_linear_tile(a, w, out, residual, row_scale, M, N, K, lda, ldo, dtype, out_dtype, epilogue, 0, stream);
 }
 
-// Few-row (M <= 64) bfloat16 product that takes part in handing a norm from one product to the
-// next (see SkinnyArgs).  Consumer side: in_sumsq [rows of a, in_parts] (a is then the operand a
-// producer wrote; `rows` gathers rows of both).  Producer side (out_dtype 0, epilogue 0): emit_w
-// [N] (element type emit_w_dtype), emit_operand bf16 [M, N], emit_sumsq float [M, tl_handoff_parts(M, N, K)].
-// Either side may be absent.
+// The bfloat16 product that takes part in handing a norm from one product to the next (see
+// SkinnyArgs and TileNorm): the few-row kernel up to 64 rows, the tiled kernel beyond (no row
+// gather then; a producer needs N to be a multiple of 64).  Consumer side: in_sumsq [rows of a,
+// in_parts] (a is then the operand a producer wrote; `rows` gathers rows of both).  Producer side
+// (out_dtype 0, epilogue 0): emit_w [N] (element type emit_w_dtype), emit_operand bf16 [M, N],
+// emit_sumsq float [M, tl_handoff_parts(M, N, K)].  Either side may be absent.
 int tl_linear_handoff(const void* a, const void* w, void* out, const float* residual, const int32_t* rows,
                       const float* in_sumsq, int in_parts, float in_eps, int in_width, const void* emit_w,
                       int emit_w_dtype, void* emit_operand, float* emit_sumsq, int M, int N, int K, int64_t lda,
                       int64_t ldo, int out_dtype, int epilogue, hipStream_t stream) {
   if (M <= 0) return TL_OK;
   const bool swiglu = epilogue == 1;
-  if (M > 64 || N <= 0 || K <= 0 || K % 8 || lda % 8 || lda < K || ldo < (swiglu ? N / 2 : N) || epilogue < 0 ||
+  if (N <= 0 || K <= 0 || K % 8 || lda % 8 || lda < K || ldo < (swiglu ? N / 2 : N) || epilogue < 0 ||
       epilogue > 1 || (out_dtype != 0 && out_dtype != 1))
     return TL_ERR_ARG;
   if (swiglu && ((N & 1) || residual || out_dtype != 1)) return TL_ERR_ARG;
@@ -1464,6 +1529,36 @@ int tl_linear_handoff(const void* a, const void* w, void* out, const float* resi
   const bool emit = emit_operand != nullptr;
   if (emit && (!emit_w || !emit_sumsq || swiglu || out_dtype != 0 || (emit_w_dtype != 0 && emit_w_dtype != 1)))
     return TL_ERR_ARG;
+  if (M > 64) {      // the tiled kernel
+    if (rows || (emit && (N % 64 || ldo % 4))) return TL_ERR_ARG;
+    TileNorm nm;
+    if (emit) {
+      nm.emit_w = emit_w;
+      nm.emit_w_is_f32 = emit_w_dtype == 0 ? 1 : 0;
+      nm.emit_operand = (bf16_t*)emit_operand;
+      nm.emit_ld = N;
+      nm.emit_sumsq = emit_sumsq;
+      nm.emit_parts = N / 64;
+    }
+    if (in_sumsq) {
+      nm.in_sumsq = in_sumsq;
+      nm.in_parts = in_parts;
+      nm.in_width = in_width;
+      nm.in_eps = in_eps;
+    }
+    int rc;
+    if (swiglu)
+      rc = launch_gemm_bf16_any<bf16_t, true>((const bf16_t*)a, (const bf16_t*)w, (bf16_t*)out, residual, nm, M, N, K,
+                                              lda, ldo, 0, 0, stream);
+    else if (out_dtype == 0)
+      rc = launch_gemm_bf16_any<float, false>((const bf16_t*)a, (const bf16_t*)w, (float*)out, residual, nm, M, N, K,
+                                              lda, ldo, 0, 0, stream);
+    else
+      rc = launch_gemm_bf16_any<bf16_t, false>((const bf16_t*)a, (const bf16_t*)w, (bf16_t*)out, residual, nm, M, N, K,
+                                               lda, ldo, 0, 0, stream);
+    if (rc != TL_OK) return rc;
+    return tl_launch_status();
+  }
   SkinnyArgs p{a, (const bf16_t*)w, out, residual, nullptr, rows, nullptr, 0.f, 0, M, N, K, lda, ldo};
   if (emit) {
     p.emit_w = emit_w;
@@ -1483,8 +1578,10 @@ int tl_linear_handoff(const void* a, const void* w, void* out, const float* resi
 }
 
 // How many partial sums of squares per row tl_linear_handoff writes as a producer for these sizes
-// (one per workgroup: per 16 columns, or per 8 where workgroups own 8).
+// (few rows: one per workgroup, per 16 columns, or per 8 where workgroups own 8; beyond: one per 64
+// columns).
 int tl_handoff_parts(int M, int N, int K) {
+  if (M > 64) return (N + 63) / 64;
   if (skinny_half(M, N, K)) return (N + 7) / 8;
   const bool one_tile = M <= 16 && !(M >= 8 && N > 256 * S_COLS && N <= 4 * 256 * S_COLS);
   const int cw = one_tile ? skinny_cols_wg(N) : S_COLS;

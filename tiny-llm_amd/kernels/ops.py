@@ -353,20 +353,21 @@ _SPLITS: dict = {}      # the plan is a pure function of the sizes
 
 def can_hand_off(rows: int, width: int, inner: int, dtype: torch.dtype) -> bool:
     """Whether `linear_handoff` can prepare a norm over `width` columns for `rows` rows, as the
-    epilogue of the product with inner size `inner`."""
+    epilogue of the product with inner size `inner`: the few-row kernel, a product whose inner
+    size is split, or the tiled kernel where the width is a multiple of 64."""
     if dtype != torch.bfloat16 or rows <= 0 or width % 8 or inner % 8:
         return False
-    return rows <= FEW_ROWS or split_k(rows, width, inner) > 1
+    return rows <= FEW_ROWS or split_k(rows, width, inner) > 1 or width % 64 == 0
 
 
 def handoff_parts(rows: int, width: int, inner: int) -> int:
     """How many partial sums of squares per row the product [rows, inner] x [width, inner]^T writes
     when it prepares a norm: one per workgroup in the few-row kernel (16 or 8 columns), per 1024
-    after a split inner size."""
+    after a split inner size, per 64 in the tiled kernel."""
     if split_k(rows, width, inner) > 1:
         return (width + 1023) // 1024
-    if not (rows <= FEW_ROWS):
-        _fail(f"without a split inner size a norm is prepared for at most {FEW_ROWS} rows")
+    if not (rows <= FEW_ROWS or width % 64 == 0):
+        _fail(f"a norm is prepared for at most {FEW_ROWS} rows, with a split inner size or over a multiple of 64 columns")
     key = (rows, width, inner)
     n = _PARTS.get(key)
     if n is None:
@@ -401,7 +402,8 @@ def linear_handoff(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, residual
     and the sums of out^2 over groups of columns.  prepared = (sumsq [R, P], eps, width): `a` is
     such an operand ([R, K]; `rows` picks rows of both) and the product is multiplied by
     1 / sqrt(sum(sumsq[row]) / width + eps): together the two are rmsnorm(out) @ w.T.
-    For at most 64 rows (one launch), or a product whose inner size is split (`split_k`)."""
+    At most 64 rows go to the few-row kernel, a product whose inner size is split (`split_k`) to
+    its two kernels, any other to the tiled kernel (no `rows` then; emitting needs N % 64 == 0)."""
     _dev(a, w, out, residual, rows)
     _rows_2d(a, "linear input")
     _rows_2d(out, "linear output")
@@ -410,8 +412,10 @@ def linear_handoff(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, residual
     N = w.shape[0]
     swiglu = _epilogue(epilogue)
     splits = split_k(M, N, K) if rows is None and M > 16 else 1
-    if not (0 < M <= FEW_ROWS or splits > 1):
-        _fail(f"a norm is handed over for at most {FEW_ROWS} rows or with a split inner size")
+    if not (M > 0):
+        _fail("no rows")
+    if M > FEW_ROWS and splits == 1 and rows is not None:
+        _fail(f"rows are gathered for at most {FEW_ROWS} of them")
     if not (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_contiguous()
             and w.shape[1] == K):
         _fail(f"input and weight must be bfloat16, weight contiguous [N, {K}]")

@@ -29,8 +29,7 @@ class LazyNorm:
 
     def linear(self, w: torch.Tensor, out: torch.Tensor, epilogue: Optional[str] = None) -> torch.Tensor:
         """out = norm(x)[rows] @ w.T (then the epilogue), by the cheapest route there is."""
-        if self.prepared is not None and (self.num_rows <= ops.FEW_ROWS or (
-                self.rows is None and ops.split_k(self.num_rows, w.shape[0], w.shape[1]) > 1)):
+        if self.prepared is not None and (self.num_rows <= ops.FEW_ROWS or self.rows is None):
             operand, sumsq = self.prepared
             return ops.linear_handoff(operand, w, out, epilogue=epilogue, rows=self.rows,
                                       prepared=(sumsq, self.eps, self.x.shape[1]))
