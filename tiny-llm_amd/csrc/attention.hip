@@ -956,7 +956,7 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_prefill_bf16_kernel(
   // placement of waits sees a way into the loop on which they are still in flight (around the
   // block above) and would otherwise wait for ALL loads before the first matrix instruction of
   // every iteration, just after the next tile's rows have been requested.  The first tile's
-  // rows are needed here anyway; the second tile's are asked for again below.
+  // rows are needed here anyway; the second tile's are waited for too, this once.
   __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0)
   __syncthreads();
 
