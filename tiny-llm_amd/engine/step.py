@@ -595,8 +595,6 @@ class StepGraph:
         fill_metadata(self.np, self.layout, rows, runner.cache.block_size, samples, self.seen)
         self.dev.copy_(self.host, non_blocking=True)
         left = steps
-        if left >= self.CHAIN and self.chain is None and not self.chain_failed:
-            left -= self._capture_chain()
         if self.chain is not None:
             while left >= self.CHAIN:       # several steps a launch: the gap between two launches is paid once for them
                 self.chain.replay()
@@ -655,9 +653,11 @@ class StepGraph:
 
     CHAIN = 4               # decode steps captured as ONE graph for bursts
 
-    def _capture_chain(self) -> int:
-        """Captures CHAIN steps of a burst as one graph (each step's last kernel prepares the next
-        step's metadata, so the body simply repeats) and runs it once.  Returns the steps run."""
+    def _capture_chain(self) -> None:
+        """Captures CHAIN decode steps as one graph for runs of steps (each step's last kernel
+        prepares the next step's metadata, so the body simply repeats).  Nothing runs: it is
+        captured together with the single step, so that a shape of step is ready for runs after
+        its second step and no later step of it pays for a capture."""
         runner = self.runner
         torch.cuda.synchronize()
         gc.collect()                        # as in _capture: nothing may be finalised during a capture
@@ -671,13 +671,11 @@ class StepGraph:
         except StepError:
             self.chain_failed = True
             torch.cuda.synchronize()
-            return 0
+            return
         finally:
             if collecting:
                 gc.enable()
         self.chain = graph
-        graph.replay()
-        return self.CHAIN
 
     def _capture(self) -> None:
         runner = self.runner
@@ -710,3 +708,5 @@ class StepGraph:
                 gc.enable()
         self.graph = graph
         graph.replay()
+        if self.feeds_next and self.history_steps >= self.CHAIN and not self.chain_failed:
+            self._capture_chain()       # a shape that runs of decode steps replay
