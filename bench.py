@@ -240,13 +240,18 @@ def soak_llama3_8b(args):
     new = 128
     b = Bench(cfg, "bf16", 16, new, 16, budget=512, max_cache_tokens=sum(-(-(n + new) // 16) * 16 for n in lens) + 1024)
     b.soak(lens[:2], 4, 512)                                  # warm-up: kernels configure themselves
+    # The workload three times over: the first pass meets every shape of step for the first time (a
+    # shape's first step runs eagerly, its second is captured as a graph), the third replays graphs
+    # only and is the one that counts; the first is reported beside it.
+    cold, _, _ = b.soak(lens, new, 512)
+    b.soak(lens, new, 512)
     dt, steps, pre = b.soak(lens, new, 512)
     b.close()
     total = sum(lens) + 16 * new
     return {"model": "Llama-3-8B shape", "dtype": "bf16", "layers": cfg["num_hidden_layers"], "layers_full": layers_full,
             "requests": 16, "prompt_tokens": sum(lens), "decode_tokens": 16 * new, "chunk": 512, "steps": steps,
             "seconds": round(dt, 3), "tokens_per_s": round(total / dt, 1), "decode_tokens_per_s": round(16 * new / dt, 1),
-            "preemptions": pre}
+            "preemptions": pre, "pass": 3, "first_pass_seconds": round(cold, 3)}
 
 
 def prefill_llama3_8b(args):
@@ -275,13 +280,16 @@ def soak_llama2_13b(args):
     pool_tokens = n_req * (prompt + new) + 64 * 16           # one spare page a request
     b = Bench(cfg, "bf16", n_req, new, 16, budget=2048, max_cache_tokens=pool_tokens)
     b.soak([prompt] * 2, 4, 2048)
+    cold, _, _ = b.soak([prompt] * n_req, new, 2048)          # three passes, as above
+    b.soak([prompt] * n_req, new, 2048)
     dt, steps, pre = b.soak([prompt] * n_req, new, 2048)
     _, _, kv_per_tok, _ = model_numbers(cfg, 2)
     b.close()
     return {"model": "Llama-2-13B shape", "dtype": "bf16", "layers": cfg["num_hidden_layers"], "layers_full": layers_full,
             "requests": n_req, "prompt_tokens": n_req * prompt, "decode_tokens": n_req * new, "steps": steps,
             "seconds": round(dt, 3), "tokens_per_s": round(n_req * (prompt + new) / dt, 1),
-            "decode_tokens_per_s": round(n_req * new / dt, 1), "preemptions": pre,
+            "decode_tokens_per_s": round(n_req * new / dt, 1), "preemptions": pre, "pass": 3,
+            "first_pass_seconds": round(cold, 3),
             "cache_pool_GB": round(pool_tokens * kv_per_tok / 1e9, 1), "cache_pool_fill": round(n_req * (prompt + new) / pool_tokens, 3)}
 
 

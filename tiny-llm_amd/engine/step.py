@@ -572,6 +572,7 @@ class StepGraph:
             self.history_host = torch.zeros(self.history_steps * self.R, dtype=torch.int32, pin_memory=True)
         self.graph = None
         self.chain = None
+        self.bursts = 0         # runs of steps this shape has served
         self._uploaded: Optional[torch.cuda.Event] = None
 
     BURST_STEPS = 32        # most decode steps a burst may hold
@@ -606,7 +607,10 @@ class StepGraph:
         torch.cuda.current_stream().synchronize()
         self._uploaded = None
         self.runs += steps
+        self.bursts += 1
         flat = self.history_host[:n].tolist()
+        if self.chain is None and not self.chain_failed:
+            self._capture_chain()       # behind the shape's first run, of whatever length: see there
         return [flat[k * self.R:(k + 1) * self.R] for k in range(steps)]
 
     def run(self, rows: Sequence[_Row], samples, n_out: int):
@@ -655,9 +659,10 @@ class StepGraph:
 
     def _capture_chain(self) -> None:
         """Captures CHAIN decode steps as one graph for runs of steps (each step's last kernel
-        prepares the next step's metadata, so the body simply repeats).  Nothing runs: it is
-        captured together with the single step, so that a shape of step is ready for runs after
-        its second step and no later step of it pays for a capture."""
+        prepares the next step's metadata, so the body simply repeats).  Nothing runs.  It is
+        captured behind the first run of steps of this shape, however short: a shape that is
+        replayed in runs stays, and its later runs pay for no capture; a shape that a batch passes
+        through once (requests ending one after the other) never pays for this one."""
         runner = self.runner
         torch.cuda.synchronize()
         gc.collect()                        # as in _capture: nothing may be finalised during a capture
@@ -708,5 +713,3 @@ class StepGraph:
                 gc.enable()
         self.graph = graph
         graph.replay()
-        if self.feeds_next and self.history_steps >= self.CHAIN and not self.chain_failed:
-            self._capture_chain()       # a shape that runs of decode steps replay
