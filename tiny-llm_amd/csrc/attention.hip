@@ -170,6 +170,21 @@ __device__ __forceinline__ bf16x8 rotate_chunk(const bf16x8 x, const bf16x8 y, i
   return r;
 }
 
+// The same with the 8 angles of the chunk in registers (c8, s8 = cos and sin of the pairs j0 .. j0 + 7).
+template <int HD>
+__device__ __forceinline__ bf16x8 rotate_chunk_regs(const bf16x8 x, const bf16x8 y, int d0, const float* c8,
+                                                    const float* s8) {
+  bf16x8 r;
+  const bool first = d0 < HD / 2;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float a = first ? (float)x[e] : (float)y[e];     // the pair's first-half value
+    const float b = first ? (float)y[e] : (float)x[e];     // and its second-half value
+    r[e] = (bf16_t)(first ? c8[e] * a - s8[e] * b : s8[e] * a + c8[e] * b);
+  }
+  return r;
+}
+
 template <int HDT, int WAVES>
 __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
     const bf16_t* __restrict__ q, int64_t q_stride, const bf16_t* __restrict__ k_cache,
@@ -213,7 +228,23 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
   const bool row_valid = tok_local < ntok;
   const int tok = tok0 + (row_valid ? tok_local : 0);
   const int head = kvh * G + hh;
+  // The kernel begins with two round trips to memory and no more.  First everything whose address
+  // the launch gives: the page lookup above, the position, the raw chunks of the query row (own
+  // and partner dims).  Then what needs the position: the first key tile, the angles and, in the
+  // wave that owns the new token's tile, its page and the raw chunks of its key.  All loads are unconditional (rows
+  // and dims clamped into the tensors, the results masked later): asked for one by one under
+  // their conditions they were seven round trips in a row.
   const int pos = row_valid ? positions[tok] : -1;
+  bf16x8 qx[KS], qy[KS], kx[KS], ky[KS];
+  {
+    const bf16_t* qrow = q + (int64_t)tok * q_stride + (int64_t)head * HD;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int dc = min(ks * 32 + g * 8, HD - 8), dp = (dc + HD / 2) % HD;
+      qx[ks] = *(const bf16x8*)(qrow + dc);
+      if (do_rope) qy[ks] = *(const bf16x8*)(qrow + dp);      // uniform
+    }
+  }
   const int row_lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
 
   // key range of the tile: union over its rows
@@ -228,25 +259,12 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
   const int iters = (last_tile - mine + stride - 1) / stride - it0;      // may be <= 0: no tile
   // fused mode: the one new token of the tile, at position kv_end - 1
   const int new_pos = kv_end - 1;
-  const float* cs = do_rope ? fused.cos_t + (int64_t)new_pos * (HD / 2) : nullptr;
-  const float* sn = do_rope ? fused.sin_t + (int64_t)new_pos * (HD / 2) : nullptr;
+  // (a tile without a valid row has new_pos -1: it reads the angles of position 0 and uses nothing)
+  const float* cs = do_rope ? fused.cos_t + (int64_t)max(new_pos, 0) * (HD / 2) : nullptr;
+  const float* sn = do_rope ? fused.sin_t + (int64_t)max(new_pos, 0) * (HD / 2) : nullptr;
 
-  // query fragments (B operand): row r16, dims ks*32 + g*8 .. +8
-  bf16x8 qf[KS];
-  {
-    const bf16_t* qrow = q + (int64_t)tok * q_stride + (int64_t)head * HD;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const int d = ks * 32 + g * 8;
-      bf16x8 z = {};
-      qf[ks] = z;
-      if (row_valid && d < HD) {
-        const bf16x8 x = *(const bf16x8*)(qrow + d);
-        qf[ks] = do_rope ? rotate_chunk<HD>(x, *(const bf16x8*)(qrow + (d + HD / 2) % HD), d, cs, sn) : x;
-      }
-    }
-  }
-
+  const int new_tile = new_pos / FA_KT;
+  const bool owns_new = do_rope && new_tile % (WAVES * n_splits) == split * WAVES + wave;
   float m_run = kNegBig, l_run = 0.f;
   f32x4 o[HDT];
 #pragma unroll
@@ -264,31 +282,12 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
     const int row = (blk * nkv + kvh) * block_size + (j - page_index(j) * block_size);
     return (int64_t)row * HD;
   };
-  // Fused mode: the new token's key is rotated here, by the lanes that will hold its chunks as
-  // operands (in the wave whose tile it falls into), and written to the cache; its value is read
-  // from the qkv row where the loop would read the cache.
-  const int new_tile = new_pos / FA_KT;
-  const bf16_t* new_v = nullptr;
-  int64_t new_off = 0;
+  // Fused mode: the new token's key is rotated by the lanes that will hold its chunks as operands
+  // (in the wave whose tile it falls into) and written to the cache; its value is read from the
+  // qkv row where the loop would read the cache.  Both happen below, once the first key tile has
+  // been requested.
+  const bf16_t* new_v = do_rope ? q + (int64_t)tok0 * q_stride + fused.v_off + (int64_t)kvh * HD : nullptr;
   bf16x8 new_k[KS];
-  if (do_rope) {
-    new_v = q + (int64_t)tok0 * q_stride + fused.v_off + (int64_t)kvh * HD;
-    if (new_tile % stride == mine) {
-      new_off = row_offset(new_pos, bt[new_pos / block_size]);     // the same for every lane
-      if (r16 == new_pos % 16) {
-        const bf16_t* krow = q + (int64_t)tok0 * q_stride + fused.k_off + (int64_t)kvh * HD;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const int d = ks * 32 + g * 8;
-          if (d < HD) {
-            new_k[ks] = rotate_chunk<HD>(*(const bf16x8*)(krow + d), *(const bf16x8*)(krow + (d + HD / 2) % HD), d,
-                                         cs, sn);
-            *(bf16x8*)(fused.k_cache_w + new_off + d) = new_k[ks];
-          }
-        }
-      }
-    }
-  }
   // Loads are unconditional and nothing is done to what they bring before it is used: a predicated
   // load would become a branch, and a select on a loaded register makes the wave wait for the load
   // where the select stands, so that the next tile's rows would not be on their way while this
@@ -336,6 +335,52 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
     if (it0 != 0) next_pages = pages_at(tile_base(0));
     fetch(0, next_pages);
     if (iters > 1) next_pages = pages_at(tile_base(1));
+  }
+  // the rest of the second round, behind the key tile: this lane's angles (the chunk of dims d and
+  // d + HD/2 shares the pairs j0 .. j0 + 7) and, where this wave owns the new token's tile, its page
+  float c8[KS][8], s8[KS][8];
+  int new_page = 0;
+  if (do_rope) {
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int dc = min(ks * 32 + g * 8, HD - 8), j0 = dc < HD / 2 ? dc : dc - HD / 2;
+      const f32x4 ca = *(const f32x4*)(cs + j0), cb = *(const f32x4*)(cs + j0 + 4);
+      const f32x4 sa = *(const f32x4*)(sn + j0), sb = *(const f32x4*)(sn + j0 + 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        c8[ks][e] = ca[e];
+        c8[ks][4 + e] = cb[e];
+        s8[ks][e] = sa[e];
+        s8[ks][4 + e] = sb[e];
+      }
+    }
+    if (owns_new) {
+      new_page = bt[new_pos / block_size];
+      if (r16 == new_pos % 16) {      // the lanes that will hold the new key's chunks as operands
+        const bf16_t* krow = q + (int64_t)tok0 * q_stride + fused.k_off + (int64_t)kvh * HD;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const int dc = min(ks * 32 + g * 8, HD - 8), dp = (dc + HD / 2) % HD;
+          kx[ks] = *(const bf16x8*)(krow + dc);
+          ky[ks] = *(const bf16x8*)(krow + dp);
+        }
+      }
+    }
+  }
+  const int64_t new_off = owns_new ? row_offset(new_pos, new_page) : 0;      // the same for every lane
+  // query fragments (B operand): row r16, dims ks*32 + g*8 .. +8, rotated in fused mode; and the
+  // new token's key
+  bf16x8 qf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const int d = ks * 32 + g * 8;
+    bf16x8 z = {};
+    qf[ks] = do_rope ? rotate_chunk_regs<HD>(qx[ks], qy[ks], d, c8[ks], s8[ks]) : qx[ks];
+    if (!(row_valid && d < HD)) qf[ks] = z;
+    if (owns_new && r16 == new_pos % 16 && d < HD) {
+      new_k[ks] = rotate_chunk_regs<HD>(kx[ks], ky[ks], d, c8[ks], s8[ks]);
+      *(bf16x8*)(fused.k_cache_w + new_off + d) = new_k[ks];
+    }
   }
 
   for (int it = 0; it < iters; ++it) {
