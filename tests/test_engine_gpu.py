@@ -305,40 +305,43 @@ def test_graph_replays_against_the_plain_model(dtype, graphs, folders):
     eng.runner.cache.audit()
 
 
+@pytest.mark.parametrize("around", [512, 1024])
 @pytest.mark.parametrize("graphs", [True, False])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_decoding_past_the_first_context_bucket(dtype, graphs, tmp_path_factory):
-    """Contexts that grow from below 512 to beyond: the decode graph of the next context bound
-    takes over a live batch, the attention kernel splits the keys of a request over workgroups
-    and merges them, inside a graph and outside.  Logits of every step against the plain model."""
+def test_decoding_past_a_context_bucket(dtype, graphs, around, tmp_path_factory):
+    """Contexts that grow from below a bound on the context (512, 1024) to beyond: the decode
+    graph of the next bound takes over a live batch; beyond 1024 the bfloat16 attention kernel
+    splits the keys of a request over workgroups and a second kernel merges them, inside a graph
+    and outside.  Logits of every step against the plain model."""
     from tiny_llm_amd import Engine, SamplingParams
     cfg, eng_kw, init = CONFIGS["B"]
-    key = ("past512",)
+    cfg = dict(cfg, max_position_embeddings=2048)
+    key = ("past_bound",)
     if key not in _folders:
-        _folders[key] = make_folder(tmp_path_factory.mktemp("past512"), cfg, seed=21, **init)
+        _folders[key] = make_folder(tmp_path_factory.mktemp("past_bound"), cfg, seed=21, **init)
     folder = _folders[key]
     act = torch.bfloat16 if dtype == "bfloat16" else None
     w, c = read_weights(folder, round_to=act)
-    prompts = [random_tokens(n, cfg["vocab_size"], 700 + n) for n in (497, 490, 505)]
+    prompts = [random_tokens(n, cfg["vocab_size"], 700 + n) for n in (around - 15, around - 22, around - 7)]
     eng = Engine(folder, dtype=dtype, max_num_seqs=4, max_num_batched_tokens=512, use_graphs=graphs,
-                 max_cache_tokens=3 * 576, decode_burst=1, **eng_kw)
+                 max_cache_tokens=3 * (around + 64), decode_burst=1, **eng_kw)
     poison(eng)
     log = spy_on_steps(eng)
     out = eng.generate(prompts, SamplingParams.greedy(44, ignore_eos=True))
     tokens_of = {i: p + o for i, (p, o) in enumerate(zip(prompts, out))}
     worst, n = check_logged_logits(log, tokens_of, w, c, act, 1e-4 if dtype == "float32" else 2e-2)
-    print(f"{dtype} graphs={graphs}: {n} rows across the 512 boundary, worst rel err {worst:.2e}")
+    print(f"{dtype} graphs={graphs}: {n} rows across the {around} boundary, worst rel err {worst:.2e}")
     assert n == 3 * 44
     if graphs:
         bounds = sorted({k[2] for k, g in eng.runner._graphs.items() if k[0] == "decode" and g.graph is not None})
-        assert bounds == [512, 1024]
+        assert bounds == [around, 2 * around]
     if dtype == "bfloat16":
-        # the split path was really taken beyond 512 keys
+        # the split path was really taken beyond 1024 keys, and not before
         attn = eng.decoder.layers[0].mixer
 
         class Ctx:
-            max_seq_len = 1024
-        assert attn._splits(Ctx, 3, eng.decoder.device)[0] >= 2
+            max_seq_len = 2 * around
+        assert (attn._splits(Ctx, 3, eng.decoder.device)[0] >= 2) == (around == 1024)
 
 
 _folders = {}

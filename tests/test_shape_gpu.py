@@ -112,8 +112,8 @@ def test_four_cuttings_at_the_real_layer_sizes(dtype):
 @pytest.mark.parametrize("graphs", [True, False])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_generation_across_the_512_bound_at_the_real_layer_sizes(dtype, graphs):
-    """What the throughput measurement runs: prompts of about 500 tokens, decode steps as graphs
-    whose attention splits a request's keys over workgroups once the context passes 512."""
+    """What the throughput measurement runs: prompts of about 500 tokens, decode steps as graphs,
+    the graph of the next bound on the context taking over once the context passes 512."""
     from tiny_llm_amd import Engine, SamplingParams
     from test_engine_gpu import check_logged_logits, poison, spy_on_steps
     act = torch.bfloat16 if dtype == "bfloat16" else None
