@@ -197,7 +197,7 @@ def tinyllama_figures(args, dtype, peaks):
     steps, warmup = args.steps, args.warmup
     if dtype == "fp32":
         steps, warmup = min(steps, 64), min(warmup, 8)       # the 32-bit path is for checking: a shorter run
-    b = Bench(cfg, dtype, max(args.batch, 64), warmup + steps + 80, args.block_size)
+    b = Bench(cfg, dtype, max(args.batch, 64), warmup + steps + 80, args.block_size, prompt_len=args.prompt_len)
     out = {}
     if args.only in ("all", "headline", "fp32", "prefill"):
         pf = b.prefill(3)
@@ -209,7 +209,7 @@ def tinyllama_figures(args, dtype, peaks):
         pc = b.prefill(2, budget=512)
         out["prefill_chunked_512"] = {"value": round(PREFILL_TOKENS / pc, 1), "ms": round(pc * 1e3, 3), "steps": 4}
     if args.only != "prefill":
-        dt, ctx_tokens = b.decode(args.batch, steps, warmup)
+        dt, ctx_tokens = b.decode(args.batch, steps, warmup, prompt_len=args.prompt_len)
         out["ms_per_step"] = dt / steps * 1e3
         out["value"] = args.batch * steps / dt
         achieved = (weight_bytes + ctx_tokens * kv_per_tok) / (dt / steps) / 1e9
@@ -220,7 +220,7 @@ def tinyllama_figures(args, dtype, peaks):
         out["points"] = {}
         if args.only in ("all", "headline", "fp32"):
             for n in (1, 64):
-                d, _ = b.decode(n, steps, warmup)
+                d, _ = b.decode(n, steps, warmup, prompt_len=args.prompt_len)
                 out["points"][f"decode_b{n}"] = round(n * steps / d, 1)
     out["sizes"] = (L, H, I, V, nq, nkv, hd)
     out["steps"], out["warmup"] = steps, warmup
@@ -387,7 +387,7 @@ def run(args):
         "dtype": main_dtype, "data": "synthetic: uniform-random token ids, random weights N(0, 0.02)",
         "config": {"model": "TinyLlama-1.1B shape", "layers": L, "layers_full": TINYLLAMA["num_hidden_layers"], "hidden": H,
                    "heads": nq, "kv_heads": nkv, "head_dim": hd, "intermediate": I, "vocab": V,
-                   "context": TINYLLAMA["max_position_embeddings"], "global_batch": args.batch, "seq_len": PROMPT_LEN,
+                   "context": TINYLLAMA["max_position_embeddings"], "global_batch": args.batch, "seq_len": args.prompt_len,
                    "decode_tokens": fig["steps"], "kv_block_size": args.block_size, "parallelism": "single GPU"},
         "prefill": fig.get("prefill"), "roofline": fig["roofline"], "points": fig["points"],
     }
@@ -412,6 +412,7 @@ def main():
     ap.add_argument("--steps", type=int, default=240)      # with the warm-up: 256 generated tokens a request
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN, help="prompt tokens of the decode runs (the context they begin at)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the TinyLlama shape has (0: all)")
     ap.add_argument("--soak-layers", type=int, default=0, help="fewer layers for the two larger shapes (0: all)")

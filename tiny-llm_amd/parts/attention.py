@@ -135,14 +135,16 @@ class Attention(Mixer):
     def _splits(self, ctx, T: int, device):
         """How many workgroups share one query tile's keys.  The waves of a workgroup take a
         64-key tile each per round trip to memory (the next one is on its way while a tile is
-        worked on); long contexts are split until a wave has two tiles, as far as that keeps the
-        launch within about 256 workgroups (beyond that the splits only queue up).  The partial
-        results of a split are merged by a second kernel, which costs about what a wave's second
-        tile costs: measured on whole decode steps, two tiles a wave and no merge are 1.5 % of the
-        step faster than one tile a wave at contexts of 9 to 16 key tiles."""
+        worked on).  Up to two tiles a wave nothing is split: the partial results of a split are
+        merged by a second kernel, which costs more than a wave's second tile (measured on whole
+        decode steps at contexts of 9 to 16 key tiles: 1.5 % of the step).  Longer contexts are
+        split until a wave has one tile (at 17 to 32 key tiles two tiles a wave with a merge are
+        3 to 5 % of the step slower than one), as far as that keeps the launch within about 256
+        workgroups (beyond that the splits only queue up)."""
         key_tiles = -(-ctx.max_seq_len // 64)
         room = max(1, 256 // max(1, T * self.num_kv_heads))
-        n_splits = max(1, min(-(-key_tiles // (2 * ops.flash_waves(self.head_dim))), room, 16))
+        n_splits = -(-key_tiles // ops.flash_waves(self.head_dim))
+        n_splits = 1 if n_splits <= 2 else max(1, min(n_splits, room, 16))
         if n_splits == 1:
             return 1, None
         return n_splits, ops.scratch("attention_partials", (n_splits * T * self.num_heads * (self.head_dim + 2),),
