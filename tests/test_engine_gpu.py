@@ -310,9 +310,8 @@ def test_graph_replays_against_the_plain_model(dtype, graphs, folders):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_decoding_past_a_context_bucket(dtype, graphs, around, tmp_path_factory):
     """Contexts that grow from below a bound on the context (512, 1024) to beyond: the decode
-    graph of the next bound takes over a live batch; beyond 1024 the bfloat16 attention kernel
-    splits the keys of a request over workgroups and a second kernel merges them, inside a graph
-    and outside.  Logits of every step against the plain model."""
+    graph of the next bound takes over a live batch, and the bfloat16 attention kernel splits the
+    keys of a request over workgroups and a second kernel merges them, inside a graph and outside.  Logits of every step against the plain model."""
     from tiny_llm_amd import Engine, SamplingParams
     cfg, eng_kw, init = CONFIGS["B"]
     cfg = dict(cfg, max_position_embeddings=2048)
@@ -336,12 +335,12 @@ def test_decoding_past_a_context_bucket(dtype, graphs, around, tmp_path_factory)
         bounds = sorted({k[2] for k, g in eng.runner._graphs.items() if k[0] == "decode" and g.graph is not None})
         assert bounds == [around, 2 * around]
     if dtype == "bfloat16":
-        # the split path was really taken beyond 1024 keys, and not before
+        # the split path was really taken beyond the bound
         attn = eng.decoder.layers[0].mixer
 
         class Ctx:
             max_seq_len = 2 * around
-        assert (attn._splits(Ctx, 3, eng.decoder.device)[0] >= 2) == (around == 1024)
+        assert attn._splits(Ctx, 3, eng.decoder.device)[0] >= 2
 
 
 _folders = {}

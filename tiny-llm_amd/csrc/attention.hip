@@ -1262,10 +1262,13 @@ static int launch_flash_w(const bf16_t* q, int64_t q_stride, const bf16_t* k_cac
   return TL_OK;
 }
 
-// Waves of a flash_attn_bf16_kernel workgroup.  A tile's keys and values are 16 registers per 16
-// dims of the head: with eight waves (256 registers a wave) the heads beyond 64 dims spilled 27 to
-// 74 registers to memory and the kernel took twice the time that four waves take.
-constexpr int flash_waves(int hd) { return hd <= 64 ? 8 : 4; }
+// Waves of a flash_attn_bf16_kernel workgroup, for a launch of `groups` query tiles x kv heads.
+// A tile's keys and values are 16 registers per 16 dims of the head: with eight waves (256
+// registers a wave) the heads beyond 64 dims spilled 27 to 74 registers to memory and the kernel
+// took twice the time that four waves take.  Smaller heads take eight waves where the launch has
+// many workgroups anyway, and four (with the keys shared out over twice the workgroups) where it
+// has few: measured on whole decode steps, batch 1 and 8 gain 1 %, batch 64 would lose 2 %.
+static int flash_waves(int hd, int groups) { return hd <= 64 && groups > 64 ? 8 : 4; }
 
 template <int HDT>
 static int launch_flash(const bf16_t* q, int64_t q_stride, const bf16_t* k_cache, const bf16_t* v_cache,
@@ -1274,10 +1277,15 @@ static int launch_flash(const bf16_t* q, int64_t q_stride, const bf16_t* k_cache
                         int64_t out_stride, float* part_o, float* part_ml, int n_tiles, int n_tokens, int nq, int nkv,
                         int block_size, float scale, int window, int n_splits, const FusedRope& fused,
                         hipStream_t stream) {
-  return launch_flash_w<HDT, flash_waves(HDT * 16)>(q, q_stride, k_cache, v_cache, block_tables, max_blocks, tile_req,
-                                                    tile_tok0, tile_ntok, positions, out, out_stride, part_o, part_ml,
-                                                    n_tiles, n_tokens, nq, nkv, block_size, scale, window, n_splits,
-                                                    fused, stream);
+  if constexpr (HDT <= 4) {
+    if (flash_waves(HDT * 16, n_tiles * nkv) == 8)
+      return launch_flash_w<HDT, 8>(q, q_stride, k_cache, v_cache, block_tables, max_blocks, tile_req, tile_tok0,
+                                    tile_ntok, positions, out, out_stride, part_o, part_ml, n_tiles, n_tokens, nq, nkv,
+                                    block_size, scale, window, n_splits, fused, stream);
+  }
+  return launch_flash_w<HDT, 4>(q, q_stride, k_cache, v_cache, block_tables, max_blocks, tile_req, tile_tok0, tile_ntok,
+                                positions, out, out_stride, part_o, part_ml, n_tiles, n_tokens, nq, nkv, block_size,
+                                scale, window, n_splits, fused, stream);
 }
 
 }  // namespace
@@ -1403,8 +1411,8 @@ int tl_flash_prefill(const void* q, int64_t q_stride, const void* k_cache, const
 }
 
 // How many waves of a workgroup of tl_flash_attention share a query tile's keys, a 64-key tile each at
-// a time (the caller sizes n_splits by it).
-int tl_flash_waves(int hd) { return flash_waves(hd); }
+// a time, in a launch of `groups` query tiles x kv heads (the caller sizes n_splits by it).
+int tl_flash_waves(int hd, int groups) { return flash_waves(hd, groups); }
 
 // bfloat16 only.  Tiles: tile_req / tile_tok0 / tile_ntok [n_tiles] describe groups of at most
 // 16 / (nq / nkv) consecutive tokens of one request; all three null: tile i is token i of request i.  With n_splits > 1, part_o

@@ -722,11 +722,13 @@ def flash_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
 STATIC_SCRATCH_FLOATS = 1 << 20     # capacity of the library's own scratch array (csrc/no_alloc.h)
 
 
-def flash_waves(head_dim: int) -> int:
-    """Waves of a `flash_attention` workgroup: each takes one 64-key tile per round trip to memory."""
-    n = _WAVES.get(head_dim)
+def flash_waves(head_dim: int, groups: int = 1 << 20) -> int:
+    """Waves of a `flash_attention` workgroup in a launch of `groups` query tiles x kv heads: each
+    takes one 64-key tile per round trip to memory."""
+    key = (head_dim, min(groups, 1 << 20))
+    n = _WAVES.get(key)
     if n is None:
-        n = _WAVES[head_dim] = int(_lib().tl_flash_waves(c_int(head_dim)))
+        n = _WAVES[key] = int(_lib().tl_flash_waves(c_int(head_dim), c_int(key[1])))
     return n
 
 

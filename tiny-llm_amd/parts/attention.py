@@ -143,7 +143,7 @@ class Attention(Mixer):
         workgroups (beyond that the splits only queue up)."""
         key_tiles = -(-ctx.max_seq_len // 64)
         room = max(1, 256 // max(1, T * self.num_kv_heads))
-        n_splits = -(-key_tiles // ops.flash_waves(self.head_dim))
+        n_splits = -(-key_tiles // ops.flash_waves(self.head_dim, T * self.num_kv_heads))
         n_splits = 1 if n_splits <= 2 else max(1, min(n_splits, room, 16))
         if n_splits == 1:
             return 1, None
