@@ -1380,9 +1380,10 @@ static int launch_skinny(const SkinnyArgs& p, hipStream_t stream) {
     if constexpr (PRO == PRO_NONE) {
       // A workgroup fetches at a rate of its own, and every workgroup fetches all activation rows:
       // the product is fastest with ONE round of workgroups over the 256 compute units, each owning
-      // as many column tiles as that takes (up to four; wider products stay at one).  Below 8 rows
-      // the activations are too few to matter and more workgroups are faster.
-      const int ct = p.M >= 8 ? (p.N + 256 * S_COLS - 1) / (256 * S_COLS) : 1;
+      // as many column tiles as that takes (up to four; wider products stay at one).  (Also with
+      // few rows: timed alone, more workgroups looked faster below 8 rows; whole decode steps are
+      // 1 % faster at 4 rows with one round and equal at 1 and 2.)
+      const int ct = (p.N + 256 * S_COLS - 1) / (256 * S_COLS);
       if (ct == 2) return launch_skinny_tile<1, 2, TO, PRO, SWIGLU>(p, stream);
       if (ct == 3) return launch_skinny_tile<1, 3, TO, PRO, SWIGLU>(p, stream);
       if (ct == 4) return launch_skinny_tile<1, 4, TO, PRO, SWIGLU>(p, stream);
@@ -1583,7 +1584,7 @@ int tl_linear_handoff(const void* a, const void* w, void* out, const float* resi
 int tl_handoff_parts(int M, int N, int K) {
   if (M > 64) return (N + 63) / 64;
   if (skinny_half(M, N, K)) return (N + 7) / 8;
-  const bool one_tile = M <= 16 && !(M >= 8 && N > 256 * S_COLS && N <= 4 * 256 * S_COLS);
+  const bool one_tile = M <= 16 && !(N > 256 * S_COLS && N <= 4 * 256 * S_COLS);
   const int cw = one_tile ? skinny_cols_wg(N) : S_COLS;
   return (N + cw - 1) / cw;
 }
