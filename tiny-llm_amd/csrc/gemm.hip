@@ -1383,13 +1383,18 @@ static int launch_skinny(const SkinnyArgs& p, hipStream_t stream) {
     if constexpr (PRO == PRO_NONE) {
       // A workgroup fetches at a rate of its own, and every workgroup fetches all activation rows:
       // the product is fastest with ONE round of workgroups over the 256 compute units, each owning
-      // as many column tiles as that takes (up to four; wider products stay at one).  (Also with
-      // few rows: timed alone, more workgroups looked faster below 8 rows; whole decode steps are
-      // 1 % faster at 4 rows with one round and equal at 1 and 2.)
+      // as many column tiles as that takes (up to four).  (Also with few rows: timed alone, more
+      // workgroups looked faster below 8 rows; whole decode steps are 1 % faster at 4 rows with
+      // one round and equal at 1 and 2.)  Wider products run several rounds: one column tile below
+      // 8 rows, two from 8 rows on, where the activation rows a workgroup fetches weigh as much as
+      // its weights (whole decode steps at hidden 4096, intermediate 14336, vocabulary 128256:
+      // 3 % faster at 8 rows and 9 % at 16 with two tiles, 2 to 6 % slower at 1 to 6; four tiles
+      // are slower than two at 16 rows).
       const int ct = (p.N + 256 * S_COLS - 1) / (256 * S_COLS);
       if (ct == 2) return launch_skinny_tile<1, 2, TO, PRO, SWIGLU>(p, stream);
       if (ct == 3) return launch_skinny_tile<1, 3, TO, PRO, SWIGLU>(p, stream);
       if (ct == 4) return launch_skinny_tile<1, 4, TO, PRO, SWIGLU>(p, stream);
+      if (ct > 4 && p.M >= 8) return launch_skinny_tile<1, 2, TO, PRO, SWIGLU>(p, stream);
     }
     return launch_skinny_tile<1, 1, TO, PRO, SWIGLU>(p, stream);
   }
