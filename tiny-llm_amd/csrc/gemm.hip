@@ -786,10 +786,11 @@ static int oneshot_plan(int M, int N, int K, int* slabs_per_split) {
   if (M <= 16 || K % O_SLAB_K || K < 4 * O_SLAB_K) return 1;
   // measured on whole decode steps: small weight matrices with few rows are faster in the few-row
   // kernel (one launch); up to 32 rows for matrices of 6 M weights (3 % of a step at 32 rows; from
-  // 36 rows on this kernel is 2 to 7 % of a step faster)
+  // 36 rows on this kernel is 2 to 7 % of a step faster), up to 18 rows for 17 M weights (4096 x 4096:
+  // from 22 rows on this kernel is 1 to 2 % of a step faster)
   const int64_t weights = (int64_t)N * K;
   const int tiles = ((M + O_BM - 1) / O_BM) * ((N + O_BN - 1) / O_BN), nslabs = K / O_SLAB_K;
-  if (M <= O_BM && ((weights <= ((int64_t)6 << 20) && M <= 32) || (weights <= ((int64_t)17 << 20) && K <= 4096 && M <= 28) ||
+  if (M <= O_BM && ((weights <= ((int64_t)6 << 20) && M <= 32) || (weights <= ((int64_t)17 << 20) && K <= 4096 && M <= 18) ||
                     (tiles > 128 && M <= 32)))
     return 1;
   int best = 1, best_per = 0;
