@@ -102,7 +102,8 @@ def test_lm_head_last_rows_reference_vector():
                                    (300, 5632, 136), (9, 5640, 520), (16, 4104, 40), (8, 5640, 524), (3, 2056, 2044),
                                    (5, 9000, 72), (8, 64, 4100), (12, 96, 8200), (16, 72, 12300), (7, 64, 8200),
                                    (5, 64, 2500), (16, 96, 3302), (17, 2048, 32000), (40, 64, 16390),
-                                   (64, 2048, 32000), (33, 128, 128256)])
+                                   (64, 2048, 32000), (33, 128, 128256), (12, 96, 1500), (16, 2048, 2048),
+                                   (10, 64, 20000), (8, 128, 40004), (4, 2048, 1100), (36, 2048, 2560)])
 def test_linear_sizes(dtype, M, K, N):
     if dtype == torch.bfloat16 and K % 8:
         K = K + 8 - K % 8
