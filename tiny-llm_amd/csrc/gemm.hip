@@ -797,7 +797,8 @@ static int oneshot_plan(int M, int N, int K, int* slabs_per_split) {
   double best_t = 0.;
   for (int want = 2; want <= 16; ++want) {
     const int per = (nslabs + want - 1) / want;
-    if (per < 2) break;
+    // measured on whole steps: shares of fewer than four slabs lose to fewer, longer ones
+    if (per < (nslabs >= 8 ? 4 : 2)) break;
     const int splits = (nslabs + per - 1) / per;
     if (splits < 2) continue;
     const int rounds = (tiles * splits + 255) / 256;
