@@ -76,6 +76,7 @@ class StepContext:
     max_seq_len: int = 0
     block_size: int = 0
     static: bool = False            # a captured step: nothing may be built on the host any more
+    logits_all_rows: bool = False   # logit_rows is 0, 1, 2, ...: every token's logits, in order (no gather needed)
     _tiles: Dict[int, tuple] = field(default_factory=dict)
     _on_new_width = None            # told when a tile width is asked for the first time
 
@@ -491,7 +492,7 @@ class ModelRunner:
             n_out = sum(len(r.want) for r in rows)
             decode_only = all(len(r.tokens) == 1 for r in rows)
             new_lens = [r.context_len + len(r.tokens) for r in rows]
-            if decode_only and n_out == R:
+            if decode_only and all(len(r.want) == 1 for r in rows):      # row i of the logits is request i
                 # exact sizes; the bound on the context (a power of two, at least 512) decides into how
                 # many workgroups the attention kernel splits a request's keys, which is fixed at capture
                 bound = min(max(512, power_of_two_at_least(max(new_lens))), max(self.max_model_len, 1))
@@ -561,6 +562,9 @@ class StepGraph:
         self.np = self.host.numpy()
         self.ctx = self.layout.context(self.dev, cm.block_size, q_lens=[], context_lens=[], slots_host=[],
                                        max_q_len=self.max_q_len, max_seq_len=self.max_seq_len)
+        # decode with a wanted row per request: row i of the logits is token i (padding rows, which would
+        # point at row 0, are dropped by the caller either way), so the head needs no gather of rows
+        self.ctx.logits_all_rows = self.max_q_len == 1 and self.n_out == self.R == self.T
         self.seen = [[None] * self.R for _ in range(G)]
         self.out = torch.zeros(max(self.n_out, 1), dtype=torch.int32, device=runner.device)
         self.out_host = torch.zeros(max(self.n_out, 1), dtype=torch.int32, pin_memory=True)

@@ -148,8 +148,9 @@ class Decoder:
         if not wants_logits:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=x.device)
         norm = self.final_norm
+        rows = None if getattr(ctx, "logits_all_rows", False) else ctx.logit_rows
         if lazy_head:
-            h = norm.lazy(x, ctx.logit_rows, prepared=prepared) if prepared is not None else norm.lazy(x, ctx.logit_rows)
+            h = norm.lazy(x, rows, prepared=prepared) if prepared is not None else norm.lazy(x, rows)
         else:
-            h = norm.forward(x, ctx.logit_rows)
+            h = norm.forward(x, rows)
         return self.lm_head.forward(h)
