@@ -1074,7 +1074,7 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
   float* ss_part = (float*)(part + S_WAVES * MT * CT);              // [S_WAVES][MT * 16]
   const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
   const int M = p.M, N = p.N, K = p.K;
-  const int cw = (MT == 1 && !HALF && p.cols_wg > 0) ? p.cols_wg : COLS * CT;      // columns of this workgroup
+  const int cw = (!HALF && p.cols_wg > 0) ? p.cols_wg : COLS * CT;      // columns of this workgroup
   const int n0 = blockIdx.x * cw;
   const int r16 = lane % 16, g = lane / 16;
   const int rr = HALF ? r16 % 8 : r16;             // the weight row / activation row this lane feeds
@@ -1330,7 +1330,7 @@ static int launch_skinny_deep(const SkinnyArgs& p, hipStream_t stream) {
     configured = true;
   }
   constexpr int cols = HALF ? 8 : S_COLS * CT;
-  const int cw = (MT == 1 && !HALF && p.cols_wg > 0) ? p.cols_wg : cols;
+  const int cw = (!HALF && p.cols_wg > 0) ? p.cols_wg : cols;
   dim3 g((p.N + cw - 1) / cw), b(S_THREADS);
   hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, CT, DEEP, TO, PRO, SWIGLU, HALF>), g, b, smem, stream, p);
   return TL_OK;
@@ -1361,10 +1361,10 @@ static int launch_skinny_tile(const SkinnyArgs& p, hipStream_t stream) {
       return launch_skinny_deep<MT, CT, false, TO, PRO, SWIGLU, true>(p, stream);
     }
   }
-  if constexpr (MT * CT == 1) {
+  if constexpr (CT == 1) {
     SkinnyArgs q = p;
     q.cols_wg = skinny_cols_wg(p.N);
-    if constexpr (PRO == PRO_NONE) {
+    if constexpr (MT == 1 && PRO == PRO_NONE) {
       if (p.K > 4096) return launch_skinny_deep<MT, CT, true, TO, PRO, SWIGLU>(q, stream);
     }
     return launch_skinny_deep<MT, CT, false, TO, PRO, SWIGLU>(q, stream);
@@ -1605,7 +1605,8 @@ int tl_linear_handoff(const void* a, const void* w, void* out, const float* resi
 int tl_handoff_parts(int M, int N, int K) {
   if (M > 64) return (N + 63) / 64;
   if (skinny_half(M, N, K)) return (N + 7) / 8;
-  const bool one_tile = M <= 16 && !(N > 256 * S_COLS && N <= 4 * 256 * S_COLS);
+  // one column tile a workgroup (see launch_skinny and launch_skinny_rows): a part per workgroup
+  const bool one_tile = M <= 16 ? !(N > 256 * S_COLS && N <= 4 * 256 * S_COLS) : N < 256 * 32;
   const int cw = one_tile ? skinny_cols_wg(N) : S_COLS;
   return (N + cw - 1) / cw;
 }
