@@ -192,7 +192,8 @@ def test_linear_norm(M, K, N):
 
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 40, 64])
 @pytest.mark.parametrize("K,N,N2", [(64, 248, 96), (5632, 2048, 516), (176, 64, 40), (96, 520, 1030), (2120, 1000, 72),
-                                    (64, 4200, 40), (64, 64, 8300), (64, 2600, 3000), (72, 2048, 32000), (64, 64, 16390)])
+                                    (64, 4200, 40), (64, 64, 8300), (64, 2600, 3000), (72, 2048, 32000), (64, 64, 16390),
+                                    (64, 5120, 72), (72, 10000, 40), (64, 16376, 24)])
 def test_linear_handoff(M, K, N, N2):
     """A norm handed from the product that writes the residual stream to the product that reads
     it: the first also writes bf16(w * x) and partial sums of x^2, the second applies 1 / rms."""

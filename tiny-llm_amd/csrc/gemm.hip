@@ -989,9 +989,8 @@ struct SkinnyArgs {
   const float* in_sumsq = nullptr;
   int in_parts = 0, in_width = 0;
   float in_eps = 0.f;
-  // One row tile: the columns a workgroup owns, even, at most 16 a column tile (0: all of them).
-  // Fewer make one balanced round of workgroups out of a product whose column tiles do not divide
-  // by 256.  With several column tiles the producer of a norm (emit_operand) takes all columns.
+  // The columns a workgroup owns, even, at most 16 a column tile (0: all of them).  Fewer make one
+  // balanced round of workgroups out of a product whose column tiles do not divide by 256.
   int cols_wg = 0;
 };
 
@@ -1306,10 +1305,14 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
           }
           float sq = valid ? v * v : 0.f;
           sq = group_sum<COLS>(sq);
-          // a column group that begins beyond N has no part of its own
-          if (nn == 0 && m < M && n < N) {
-            if (cw == COLS * CT) p.emit_sumsq[(int64_t)m * ((N + COLS - 1) / COLS) + (n0 / COLS + tile % CT)] = sq;
-            else p.emit_sumsq[(int64_t)m * ((N + cw - 1) / cw) + blockIdx.x] = sq;
+          if (nn == 0 && m < M) {
+            if (CT > 1 && cw != COLS * CT) {
+              // a part per workgroup and column tile, empty ones (beyond N) included
+              p.emit_sumsq[(int64_t)m * ((N + cw - 1) / cw * CT) + blockIdx.x * CT + tile % CT] = sq;
+            } else if (n < N) {     // a column group that begins beyond N has no part of its own
+              if (cw == COLS * CT) p.emit_sumsq[(int64_t)m * ((N + COLS - 1) / COLS) + (n0 / COLS + tile % CT)] = sq;
+              else p.emit_sumsq[(int64_t)m * ((N + cw - 1) / cw) + blockIdx.x] = sq;
+            }
           }
         }
       }
@@ -1346,6 +1349,13 @@ static int skinny_cols_wg(int N) {
   if (tiles <= 128 || tiles >= 256) return S_COLS;
   const int cw = (N + 255) / 256;
   return cw + (cw & 1);
+}
+
+// Columns a workgroup owns with `ct` (2 to 4) column tiles: what makes exactly 256 workgroups, where
+// that needs all `ct` tiles (0: all columns of the tiles).
+static int skinny_cols_wg_tiles(int N, int ct) {
+  const int cw = (N + 255) / 256 + ((N + 255) / 256 & 1);
+  return cw > S_COLS * (ct - 1) && cw < S_COLS * ct ? cw : 0;
 }
 
 // 8 columns a workgroup: for at most 8 rows and an inner size that gives every wave at least
@@ -1401,8 +1411,7 @@ static int launch_skinny(const SkinnyArgs& p, hipStream_t stream) {
         // (whole decode steps: 0.3 % faster at hidden 2048, 0.7 to 1.4 % at hidden 4096, where q/k/v went
         // from 192 workgroups to 256)
         SkinnyArgs q = p;
-        const int cw = (p.N + 255) / 256 + ((p.N + 255) / 256 & 1);
-        if (!p.emit_operand && cw > S_COLS * (ct - 1) && cw < S_COLS * ct) q.cols_wg = cw;
+        q.cols_wg = skinny_cols_wg_tiles(p.N, ct);
         if (ct == 2) return launch_skinny_tile<1, 2, TO, PRO, SWIGLU>(q, stream);
         if (ct == 3) return launch_skinny_tile<1, 3, TO, PRO, SWIGLU>(q, stream);
         return launch_skinny_tile<1, 4, TO, PRO, SWIGLU>(q, stream);
@@ -1606,7 +1615,11 @@ int tl_handoff_parts(int M, int N, int K) {
   if (M > 64) return (N + 63) / 64;
   if (skinny_half(M, N, K)) return (N + 7) / 8;
   // one column tile a workgroup (see launch_skinny and launch_skinny_rows): a part per workgroup
-  const bool one_tile = M <= 16 ? !(N > 256 * S_COLS && N <= 4 * 256 * S_COLS) : N < 256 * 32;
+  if (M <= 16 && N > 256 * S_COLS && N <= 4 * 256 * S_COLS) {       // two to four column tiles a workgroup
+    const int ct = (N + 256 * S_COLS - 1) / (256 * S_COLS), cwt = skinny_cols_wg_tiles(N, ct);
+    return cwt ? (N + cwt - 1) / cwt * ct : (N + S_COLS - 1) / S_COLS;
+  }
+  const bool one_tile = M <= 16 || N < 256 * 32;
   const int cw = one_tile ? skinny_cols_wg(N) : S_COLS;
   return (N + cw - 1) / cw;
 }
