@@ -635,10 +635,13 @@ __global__ __launch_bounds__(A32_THREADS) void attention_f32_kernel(
     for (int t = t_lo + wave; t < t_hi; t += A32_WAVES) {
       const int kb = t * FA_KT;
       // Everything the tile needs from memory is requested together, in two rounds (page numbers,
-      // then rows): loads are unconditional, with the index clamped into the table and a row outside
-      // the request's keys read from row 0 of page 0 and zeroed afterwards (stale pages may hold
-      // anything, and 0 * NaN is NaN); a conditional load would become a branch, and every branch
-      // one more round trip in a row.
+      // then rows): loads are unconditional, with the index clamped into the table; a conditional
+      // load would become a branch, and every branch one more round trip in a row.  A key row
+      // outside the request's keys is read from row 0 of page 0 (its scores are masked below,
+      // whatever they are); a value row outside from the query rows of this tile's first token
+      // (finite numbers: its probabilities are exact zeros, and stale pages may hold NaN, for which
+      // 0 * NaN is NaN).  Nothing is selected into loaded registers, which would make the wave wait
+      // for the rows where the select stands.
       constexpr int VPRE = (HD < A32_VW ? HD : A32_VW) / 4;
       const int vkey = kb + lane;
       const bool v_in_range = vkey >= kv_begin && vkey < kv_end;
@@ -655,7 +658,7 @@ __global__ __launch_bounds__(A32_THREADS) void attention_f32_kernel(
         const int64_t off = (((int64_t)max(page, 0) * nkv + kvh) * block_size + (key - (key / block_size) * block_size)) * HD;
         return in ? off : (int64_t)0;
       };
-      const float* vrow = v_cache + row_of(page_v, vkey, v_in_range);
+      const float* vrow = v_in_range ? v_cache + row_of(page_v, vkey, true) : q + (int64_t)tok0 * q_stride + (int64_t)kvh * G * HD;
       f32x4 vpre[VPRE];
 #pragma unroll
       for (int ch = 0; ch < VPRE; ++ch) vpre[ch] = *(const f32x4*)(vrow + ch * 4);
@@ -676,16 +679,12 @@ __global__ __launch_bounds__(A32_THREADS) void attention_f32_kernel(
           f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int g4 = 0; g4 < HDT; ++g4) {
-            const f32x4 kv = k_in[s0 + si] ? kf[si][g4] : f32x4{0.f, 0.f, 0.f, 0.f};
+            const f32x4 kv = kf[si][g4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(kv[e], qf[g4][e], acc, 0, 0, 0);
           }
           sc[s0 + si] = acc;
         }
-      }
-      if (!v_in_range) {
-#pragma unroll
-        for (int ch = 0; ch < VPRE; ++ch) vpre[ch] = f32x4{0.f, 0.f, 0.f, 0.f};
       }
       // ---- the tile's softmax from scratch
       float m_t = -INFINITY;
@@ -713,7 +712,6 @@ __global__ __launch_bounds__(A32_THREADS) void attention_f32_kernel(
 #pragma unroll
       for (int dt = 0; dt < HDT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
       {
-        const bool in_range = v_in_range;
 #pragma unroll
         for (int dh = 0; dh < (HD + A32_VW - 1) / A32_VW; ++dh) {
           constexpr int full = A32_VW / 4;
@@ -726,13 +724,9 @@ __global__ __launch_bounds__(A32_THREADS) void attention_f32_kernel(
 #pragma unroll
           for (int ch = 0; ch < full; ++ch)
             if (ch < chunks) {
-              // rows outside the request's keys are zeroed: stale pages may hold anything, and 0 * NaN is NaN
               f32x4 v;
               if (dh == 0) v = vpre[ch < VPRE ? ch : 0];
-              else {
-                v = *(const f32x4*)(vrow + dh * A32_VW + ch * 4);
-                if (!in_range) v = f32x4{0.f, 0.f, 0.f, 0.f};
-              }
+              else v = *(const f32x4*)(vrow + dh * A32_VW + ch * 4);
               *(f32x4*)(&Vl[lane * A32_VS + ch * 4]) = v;
             }
           __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
