@@ -369,6 +369,42 @@ def test_linear_swiglu_epilogue(dtype, M, K, N):
         ops().linear(a.to(DEV), w.to(DEV), torch.empty(M, N, dtype=dtype, device=DEV), epilogue="swiglu")
 
 
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 40, 64])
+@pytest.mark.parametrize("K,N", [(64, 250), (2048, 2560), (176, 96), (4096, 64), (5120, 520), (2048, 11264), (300, 4100)])
+def test_linear_norm_f32(M, K, N):
+    """Float32, few rows: the norm inside the product's kernel against norm, then product, in double;
+    with the SiLU-gate epilogue and with a residual; and a row gives the same bits alone and in a batch."""
+    g = torch.Generator().manual_seed(M * 7 + N)
+    x = (torch.randn(M, K, generator=g) * 1.7).to(DEV)
+    nw = (1 + 0.1 * torch.randn(K, generator=g)).to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(DEV)
+    res = torch.randn(M, N, generator=g).to(DEV)
+    eps = 1e-5
+    assert ops().linear_norm_f32_ok(M, N, K, K)
+    ref = plain.rms_norm(x.double().cpu(), nw.double().cpu(), eps) @ w.double().cpu().T
+    out = torch.full((M, N), float("nan"), device=DEV)
+    ops().linear_norm_f32(x, nw, eps, w, out)
+    assert rel(out, ref) < 1e-5
+    out_r = torch.empty(M, N, device=DEV)
+    ops().linear_norm_f32(x, nw, eps, w, out_r, residual=res)
+    assert rel(out_r, ref + res.double().cpu()) < 1e-5
+    if N % 2 == 0:
+        z = torch.empty(M, N // 2, device=DEV)
+        ops().linear_norm_f32(x, nw, eps, w, z, epilogue="swiglu")
+        assert rel(z, plain.silu(ref[:, 0::2]) * ref[:, 1::2]) < 1e-5
+    # against the norm's own kernel followed by the plain product: the same function, other rounding
+    h = torch.empty(M, K, device=DEV)
+    ops().rmsnorm(x, nw, eps, h)
+    two = torch.empty(M, N, device=DEV)
+    ops().linear(h, w, two)
+    assert rel(out, two.double().cpu()) < 1e-5
+    m = M // 2
+    alone = torch.empty(1, N, device=DEV)
+    ops().linear_norm_f32(x[m:m + 1].contiguous(), nw, eps, w, alone)
+    assert torch.equal(alone, out[m:m + 1])
+    assert not ops().linear_norm_f32_ok(65, N, K, K)
+
+
 @pytest.mark.parametrize("K,N", [(200, 90), (1000, 72), (5632, 130), (256, 8), (258, 34)])
 def test_linear_row_alone_equals_row_in_batch_fp32(K, N):
     """In float32 a row gives the same bits alone, among a few rows and among many: the tiled kernel

@@ -175,13 +175,21 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f32_kernel(const float* __rest
 // 16 (up to four).
 constexpr int FR_WAVES = 8, FR_THREADS = FR_WAVES * TL_WAVE, FR_MAX_MT = 4;
 
-template <bool SWIGLU, int COLS>
+//
+// NORM: `a` is the float32 residual stream and the product is that of its RMSNorm,
+// ((norm_w * a) @ w.T) / sqrt(mean(a^2) + eps): the rows are multiplied by the norm's weight as they
+// are loaded, their squares are added up on the way (per k block and row in a fixed order, the
+// blocks in ascending order, so a row's factor depends on nothing but the row), and the factor is
+// applied to the block sums' total.  That saves the norm's kernel in front of the product.
+template <bool SWIGLU, int COLS, bool NORM = false>
 __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* __restrict__ a,
                                                                    const float* __restrict__ w,
                                                                    float* __restrict__ out,
                                                                    const float* __restrict__ residual, int M,
-                                                                   int N, int K, int64_t lda, int64_t ldo) {
-  extern __shared__ float rows_smem[];      // [m tiles][k blocks][16 rows][COLS columns]
+                                                                   int N, int K, int64_t lda, int64_t ldo,
+                                                                   const float* __restrict__ norm_w = nullptr,
+                                                                   float eps = 0.f) {
+  extern __shared__ float rows_smem[];      // [m tiles][k blocks][16 rows][COLS columns], NORM: + [m tiles][k blocks][16]
   const int nkb = (K + F_KBLOCK - 1) / F_KBLOCK;
   const int mts = (M + 15) / 16;
   const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
@@ -193,9 +201,13 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
 #pragma unroll
     for (int g = 0; g < 16; ++g) wv[g] = load_k4<true>(wrow, wave * F_KBLOCK + g * 16 + kk * 4, K);
   }
+  float* ss_smem = rows_smem + mts * nkb * 16 * COLS;
   for (int b = wave; b < nkb; b += FR_WAVES) {
     const int kb = b * F_KBLOCK;
-    if (b + FR_WAVES < nkb) {
+    // (NORM keeps the norm's weights in registers beside the rows instead of the next block's
+    // weights; those are requested once this block is done.  The norm's products have the hidden
+    // size as their inner size: one block a wave up to 2048, two at 4096.)
+    if (!NORM && b + FR_WAVES < nkb) {
 #pragma unroll
       for (int g = 0; g < 16; ++g) wnext[g] = load_k4<true>(wrow, kb + FR_WAVES * F_KBLOCK + g * 16 + kk * 4, K);
     }
@@ -204,6 +216,22 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
       f32x4 av[16];
 #pragma unroll
       for (int g = 0; g < 16; ++g) av[g] = load_k4<true>(arow, kb + g * 16 + kk * 4, K);
+      if constexpr (NORM) {
+        float ss = 0.f;
+#pragma unroll
+        for (int g = 0; g < 16; ++g) {
+          const f32x4 nw = load_k4<true>(norm_w, kb + g * 16 + kk * 4, K);      // 4 * K bytes, from the caches
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            ss += av[g][e] * av[g][e];
+            av[g][e] *= nw[e];
+          }
+        }
+        // the four lanes of a row (one per k quarter): every lane gets (s0 + s1) + (s2 + s3)
+        ss += __shfl_xor(ss, 16, TL_WAVE);
+        ss += __shfl_xor(ss, 32, TL_WAVE);
+        if (kk == 0) ss_smem[(mt * nkb + b) * 16 + l16] = ss;
+      }
       f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int g = 0; g < 16; ++g)
@@ -212,14 +240,26 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
       // lane (l16, kk): row m = l16, columns 4 kk + r
       if (kk * 4 < COLS) *(f32x4*)(&rows_smem[((mt * nkb + b) * 16 + l16) * COLS + kk * 4]) = acc;
     }
+    if constexpr (NORM) {
+      if (b + FR_WAVES < nkb) {
 #pragma unroll
-    for (int g = 0; g < 16; ++g) wv[g] = wnext[g];
+        for (int g = 0; g < 16; ++g) wv[g] = load_k4<true>(wrow, kb + FR_WAVES * F_KBLOCK + g * 16 + kk * 4, K);
+      }
+    } else {
+#pragma unroll
+      for (int g = 0; g < 16; ++g) wv[g] = wnext[g];
+    }
   }
   __syncthreads();
   for (int e = tid; e < mts * 16 * COLS; e += FR_THREADS) {
     const int mt = e / (16 * COLS), r = (e % (16 * COLS)) / COLS, c = e % COLS;
     float t = 0.f;
     for (int b = 0; b < nkb; ++b) t += rows_smem[((mt * nkb + b) * 16 + r) * COLS + c];
+    if constexpr (NORM) {
+      float q = 0.f;
+      for (int b = 0; b < nkb; ++b) q += ss_smem[(mt * nkb + b) * 16 + r];
+      t *= 1.f / sqrtf(q / (float)K + eps);
+    }
     const int m = mt * 16 + r, n = n0 + c;
     if constexpr (SWIGLU) {   // columns (2j, 2j+1) = (gate_j, up_j); N and n0 are even
       const float u = __shfl_down(t, 1, TL_WAVE);
@@ -1439,6 +1479,47 @@ static int launch_skinny_out(const SkinnyArgs& p, int out_dtype, bool swiglu, hi
 }  // namespace
 
 extern "C" {
+
+// Float32, at most 64 rows: out = rmsnorm(x; norm_w, eps) @ w.T, then the epilogue of tl_linear_tile
+// (0: + residual, 1: SiLU-gate), the norm inside the product's kernel.  Returns TL_ERR_ARG for sizes
+// that kernel does not take (tl_linear_norm_f32_ok says which).
+int tl_linear_norm_f32_ok(int M, int N, int K, int64_t lda) {
+  const int nkb = (K + F_KBLOCK - 1) / F_KBLOCK, mts = (M + 15) / 16;
+  const int cols = (N + 7) / 8 <= 256 ? 8 : 16;
+  const size_t smem = (size_t)mts * nkb * 16 * (cols + 1) * sizeof(float);
+  return M > 0 && M <= 16 * FR_MAX_MT && K % 4 == 0 && lda % 4 == 0 && smem <= 96 * 1024;
+}
+
+int tl_linear_norm_f32(const float* x, const float* norm_w, float eps, const float* w, float* out,
+                       const float* residual, int M, int N, int K, int64_t lda, int64_t ldo, int epilogue,
+                       hipStream_t stream) {
+  const bool swiglu = epilogue == 1;
+  if (!tl_linear_norm_f32_ok(M, N, K, lda) || N <= 0 || lda < K || ldo < (swiglu ? N / 2 : N) || epilogue < 0 ||
+      epilogue > 1 || ((uintptr_t)x | (uintptr_t)w | (uintptr_t)norm_w) % 16 != 0)
+    return TL_ERR_ARG;
+  if (swiglu && ((N & 1) || residual)) return TL_ERR_ARG;
+  const int nkb = (K + F_KBLOCK - 1) / F_KBLOCK, mts = (M + 15) / 16;
+  const int cols = (N + 7) / 8 <= 256 ? 8 : 16;
+  const size_t smem = (size_t)mts * nkb * 16 * (cols + 1) * sizeof(float);
+  static bool configured = false;
+  if (!configured) {
+    const void* kernels[4] = {(const void*)gemm_f32_rows_kernel<true, 16, true>, (const void*)gemm_f32_rows_kernel<false, 16, true>,
+                              (const void*)gemm_f32_rows_kernel<true, 8, true>, (const void*)gemm_f32_rows_kernel<false, 8, true>};
+    for (const void* k : kernels)
+      if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024) != hipSuccess) return TL_ERR_LAUNCH;
+    configured = true;
+  }
+  dim3 gr((N + cols - 1) / cols);
+#define TL_F32_ROWS_NORM(SW, CO)                                                                                 \
+  hipLaunchKernelGGL((gemm_f32_rows_kernel<SW, CO, true>), gr, dim3(FR_THREADS), smem, stream, x, w, out, residual, M, \
+                     N, K, lda, ldo, norm_w, eps)
+  if (swiglu && cols == 16) TL_F32_ROWS_NORM(true, 16);
+  else if (swiglu) TL_F32_ROWS_NORM(true, 8);
+  else if (cols == 16) TL_F32_ROWS_NORM(false, 16);
+  else TL_F32_ROWS_NORM(false, 8);
+#undef TL_F32_ROWS_NORM
+  return tl_launch_status();
+}
 
 // out = a @ w.T, then an epilogue.  dtype: element type of a and w (0 float32, 1 bfloat16);
 // out_dtype: of out.  lda: row stride of a in elements; ldo: row stride of out and residual.

@@ -332,6 +332,46 @@ def linear_norm(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: torch
                                  _stream()), "linear_norm")
     return out
 
+def linear_norm_f32_ok(rows: int, cols: int, inner: int, row_stride: int) -> bool:
+    """Whether `linear_norm_f32` takes these sizes (few rows, an inner size in whole vectors)."""
+    return bool(_lib().tl_linear_norm_f32_ok(c_int(rows), c_int(cols), c_int(inner), c_int64(row_stride)))
+
+
+def linear_norm_f32(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: torch.Tensor, out: torch.Tensor,
+                    residual: Optional[torch.Tensor] = None, epilogue: Optional[str] = None) -> torch.Tensor:
+    """out = rmsnorm(x; norm_weight, eps) @ w.T, then the epilogue of `linear`, all float32 and for few
+    rows (`linear_norm_f32_ok`): the norm rides in the product's kernel, evaluated as
+    ((norm_weight * x) @ w.T) / rms with the squares added up in one fixed order per row."""
+    _dev(x, norm_weight, w, out, residual)
+    for t, what in ((x, "norm input"), (w, "weight"), (out, "output"), (norm_weight, "norm weight")):
+        if t.dtype != torch.float32:
+            _fail(f"{what} must be float32")
+    if not (x.dim() == 2 and x.stride(1) == 1):
+        _fail("norm input must be [T, K] with contiguous rows")
+    M, K = x.shape
+    N = w.shape[0]
+    swiglu = _epilogue(epilogue)
+    if not (w.dim() == 2 and w.is_contiguous() and w.shape[1] == K):
+        _fail(f"weight must be contiguous [N, {K}]")
+    if not (norm_weight.is_contiguous() and norm_weight.numel() == K):
+        _fail(f"norm weight must have {K} elements")
+    if not linear_norm_f32_ok(M, N, K, x.stride(0)):
+        _fail(f"the float32 product with a norm takes at most {FEW_ROWS} rows and an inner size in whole vectors")
+    _rows_2d(out, "linear output")
+    if swiglu:
+        if not (N % 2 == 0 and tuple(out.shape) == (M, N // 2) and residual is None):
+            _fail(f"the SiLU-gate epilogue writes [{M}, {N // 2}] and takes no residual")
+    elif tuple(out.shape) != (M, N):
+        _fail(f"linear output must be [{M}, {N}]")
+    if residual is not None:
+        if not (residual.dtype == torch.float32 and residual.shape == out.shape and residual.stride() == out.stride()):
+            _fail("residual must be float32 with the output's layout")
+    _check(_lib().tl_linear_norm_f32(_ptr(x, 16), _ptr(norm_weight, 16), c_float(eps), _ptr(w, 16), _ptr(out),
+                                     _ptr(residual), c_int(M), c_int(N), c_int(K), c_int64(x.stride(0)),
+                                     c_int64(out.stride(0)), c_int(swiglu), _stream()), "linear_norm_f32")
+    return out
+
+
 FEW_ROWS = 64   # most rows the few-row product takes
 
 

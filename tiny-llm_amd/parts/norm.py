@@ -29,6 +29,11 @@ class LazyNorm:
 
     def linear(self, w: torch.Tensor, out: torch.Tensor, epilogue: Optional[str] = None) -> torch.Tensor:
         """out = norm(x)[rows] @ w.T (then the epilogue), by the cheapest route there is."""
+        if self.x.dtype == torch.float32 and w.dtype == torch.float32:
+            # true float32: the norm inside the few-row product's kernel, or a kernel of its own before it
+            if self.rows is None and ops.linear_norm_f32_ok(self.x.shape[0], w.shape[0], self.x.shape[1], self.x.stride(0)):
+                return ops.linear_norm_f32(self.x, self.weight, self.eps, w, out, epilogue=epilogue)
+            return ops.linear(self.materialize(), w, out, epilogue=epilogue)
         if self.prepared is not None and (self.num_rows <= ops.FEW_ROWS or self.rows is None):
             operand, sumsq = self.prepared
             return ops.linear_handoff(operand, w, out, epilogue=epilogue, rows=self.rows,
@@ -45,6 +50,7 @@ class LazyNorm:
 
 class RMSNorm(Norm):
     graph_safe = True
+    F32_FUSED_ROWS = 16      # measured on whole steps: beyond, the norm's own kernel is as fast or faster
 
     def __init__(self, prefix, dtype, device, *, hidden_size: int, eps: float, init: str = "ones"):
         super().__init__(prefix, dtype, device)
@@ -60,9 +66,12 @@ class RMSNorm(Norm):
         self.weight = tensors[f"{self.prefix}.weight"].contiguous()
 
     def lazy(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None, prepared=None):
-        """In bfloat16 the norm rides in the consumer's first product (`ops.linear_norm`)."""
+        """The norm rides in the consumer's first product: in bfloat16 always (`ops.linear_norm`), in
+        float32 for at most 16 rows (`ops.linear_norm_f32`; more rows get the norm's own kernel)."""
         if self.dtype == torch.bfloat16 and self.hidden_size % 8 == 0:
             return LazyNorm(self, x, rows, prepared)
+        if self.dtype == torch.float32 and rows is None and x.shape[0] <= self.F32_FUSED_ROWS and self.hidden_size % 4 == 0:
+            return LazyNorm(self, x, None, None)
         return self.forward(x, rows)
 
     def hand_off_buffers(self, n_rows: int, inner: int, device):
