@@ -196,37 +196,48 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
   const int l16 = lane % 16, kk = lane / 16;
   const int n0 = blockIdx.x * COLS;
   const float* wrow = w + (int64_t)min(n0 + l16 % COLS, N - 1) * K;
+  // A k block that lies wholly inside K is loaded without a predicate per load (each would be a
+  // branch of its own, and the waits around branches are placed for the worst case); only the last,
+  // partial block of an inner size that is no multiple of 256 takes the predicated loads.  The loop
+  // body exists once per case (this block whole or not, the next block whole or not).
+  auto load16 = [&](auto whole, f32x4 (&dst)[16], const float* row, int k0) {
+#pragma unroll
+    for (int g = 0; g < 16; ++g) {
+      if constexpr (decltype(whole)::value) dst[g] = *(const f32x4*)(row + k0 + g * 16 + kk * 4);
+      else dst[g] = load_k4<true>(row, k0 + g * 16 + kk * 4, K);
+    }
+  };
   f32x4 wv[16], wnext[16];
   if (wave < nkb) {
-#pragma unroll
-    for (int g = 0; g < 16; ++g) wv[g] = load_k4<true>(wrow, wave * F_KBLOCK + g * 16 + kk * 4, K);
+    if (wave * F_KBLOCK + F_KBLOCK <= K) load16(std::true_type{}, wv, wrow, wave * F_KBLOCK);
+    else load16(std::false_type{}, wv, wrow, wave * F_KBLOCK);
   }
   float* ss_smem = rows_smem + mts * nkb * 16 * COLS;
-  for (int b = wave; b < nkb; b += FR_WAVES) {
+  auto block = [&](auto whole, auto next_whole, int b) {
     const int kb = b * F_KBLOCK;
     // (NORM keeps the norm's weights in registers beside the rows instead of the next block's
     // weights; those are requested once this block is done.  The norm's products have the hidden
     // size as their inner size: one block a wave up to 2048, two at 4096.)
-    if (!NORM && b + FR_WAVES < nkb) {
-#pragma unroll
-      for (int g = 0; g < 16; ++g) wnext[g] = load_k4<true>(wrow, kb + FR_WAVES * F_KBLOCK + g * 16 + kk * 4, K);
-    }
+    // The first row tile's activations are requested BEFORE the next block's weights: loads come
+    // back in the order they were asked for, and the matrix instructions below wait for the
+    // activations; asked for behind the weights they would wait for those as well, and the block
+    // ahead would hide nothing.
+    f32x4 av[16];
+    load16(whole, av, a + (int64_t)min(l16, M - 1) * lda, kb);
+    if (!NORM && b + FR_WAVES < nkb) load16(next_whole, wnext, wrow, kb + FR_WAVES * F_KBLOCK);
     for (int mt = 0; mt < mts; ++mt) {
-      const float* arow = a + (int64_t)min(mt * 16 + l16, M - 1) * lda;
-      f32x4 av[16];
-#pragma unroll
-      for (int g = 0; g < 16; ++g) av[g] = load_k4<true>(arow, kb + g * 16 + kk * 4, K);
+      if (mt > 0) load16(whole, av, a + (int64_t)min(mt * 16 + l16, M - 1) * lda, kb);
       if constexpr (NORM) {
+        f32x4 nw[16];
+        load16(whole, nw, norm_w, kb);      // 4 * K bytes, from the caches
         float ss = 0.f;
 #pragma unroll
-        for (int g = 0; g < 16; ++g) {
-          const f32x4 nw = load_k4<true>(norm_w, kb + g * 16 + kk * 4, K);      // 4 * K bytes, from the caches
+        for (int g = 0; g < 16; ++g)
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             ss += av[g][e] * av[g][e];
-            av[g][e] *= nw[e];
+            av[g][e] *= nw[g][e];
           }
-        }
         // the four lanes of a row (one per k quarter): every lane gets (s0 + s1) + (s2 + s3)
         ss += __shfl_xor(ss, 16, TL_WAVE);
         ss += __shfl_xor(ss, 32, TL_WAVE);
@@ -241,14 +252,17 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
       if (kk * 4 < COLS) *(f32x4*)(&rows_smem[((mt * nkb + b) * 16 + l16) * COLS + kk * 4]) = acc;
     }
     if constexpr (NORM) {
-      if (b + FR_WAVES < nkb) {
-#pragma unroll
-        for (int g = 0; g < 16; ++g) wv[g] = load_k4<true>(wrow, kb + FR_WAVES * F_KBLOCK + g * 16 + kk * 4, K);
-      }
+      if (b + FR_WAVES < nkb) load16(next_whole, wv, wrow, kb + FR_WAVES * F_KBLOCK);
     } else {
 #pragma unroll
       for (int g = 0; g < 16; ++g) wv[g] = wnext[g];
     }
+  };
+  for (int b = wave; b < nkb; b += FR_WAVES) {
+    const bool whole = (b + 1) * F_KBLOCK <= K, next_whole = (b + FR_WAVES + 1) * F_KBLOCK <= K;
+    if (whole && next_whole) block(std::true_type{}, std::true_type{}, b);
+    else if (whole) block(std::true_type{}, std::false_type{}, b);
+    else block(std::false_type{}, std::false_type{}, b);
   }
   __syncthreads();
   for (int e = tid; e < mts * 16 * COLS; e += FR_THREADS) {
