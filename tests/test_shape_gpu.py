@@ -131,3 +131,37 @@ def test_generation_across_the_512_bound_at_the_real_layer_sizes(dtype, graphs):
     assert n == 4 * 24
     if graphs:
         assert sorted({k[2] for k, g in eng.runner._graphs.items() if k[0] == "decode" and g.graph is not None}) == [512, 1024]
+
+
+@pytest.mark.parametrize("n_requests", [20, 40])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decoding_many_requests_at_the_real_layer_sizes(dtype, n_requests):
+    """Decode steps of 20 and 40 rows as graphs: the products take other kernels there than up to 16
+    rows (two row tiles; from 33 rows a split inner size with a second kernel, also for the output
+    head, which gets every row without a gather) and the attention other workgroups.  Every step's
+    logits of every request against the plain implementation."""
+    from tiny_llm_amd import Engine, SamplingParams
+    from test_engine_gpu import check_logged_logits, poison, spy_on_steps
+    act = torch.bfloat16 if dtype == "bfloat16" else None
+    w = host_weights(act)
+    prompts = [random_tokens(9 + (7 * i) % 23, SHAPE["vocab_size"], 400 + i) for i in range(n_requests)]
+    new = 6
+    eng = Engine(config=SHAPE, dtype=dtype, weights_seed=SEED, init_std=STD, kv_block_size=16, max_num_seqs=n_requests,
+                 max_num_batched_tokens=1024, max_cache_tokens=n_requests * 64, use_graphs=True, decode_burst=1)
+    sharpen(eng.decoder)
+    poison(eng)
+    log = spy_on_steps(eng)
+    out = eng.generate(prompts, SamplingParams.greedy(new, ignore_eos=True))
+    tokens_of = {i: p + o for i, (p, o) in enumerate(zip(prompts, out))}
+    worst, n = check_logged_logits(log, tokens_of, w, SHAPE, act, TOL[dtype])
+    print(f"TinyLlama layer sizes {dtype}, {n_requests} requests: {n} rows, worst rel err {worst:.2e}", flush=True)
+    assert n == n_requests * new
+    decode_graphs = [k for k, g in eng.runner._graphs.items() if k[0] == "decode" and g.graph is not None]
+    assert any(k[1] == n_requests for k in decode_graphs)
+    # the same requests with runs of steps chained on the device: the same kernels, so the same tokens
+    del eng
+    chained = Engine(config=SHAPE, dtype=dtype, weights_seed=SEED, init_std=STD, kv_block_size=16,
+                     max_num_seqs=n_requests, max_num_batched_tokens=1024, max_cache_tokens=n_requests * 64,
+                     use_graphs=True)
+    sharpen(chained.decoder)
+    assert chained.generate(prompts, SamplingParams.greedy(new, ignore_eos=True)) == out
