@@ -1,4 +1,4 @@
-"""Shared test material: the two tiny configurations, model folders, comparisons."""
+"""Shared test material: the tiny configurations, model folders, comparisons."""
 import json
 import os
 
@@ -25,13 +25,24 @@ TINY_B = {
     "hidden_act": "silu", "attention_bias": False, "rope_scaling": None, "initializer_range": 0.05,
     "eos_token_id": 5, "torch_dtype": "float32",
 }
+# A third one with heads of 128 and as many kv heads as heads (the shape of attention of the larger Llamas).
+TINY_C = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "num_hidden_layers": 2, "hidden_size": 256, "num_attention_heads": 2, "num_key_value_heads": 2,
+    "head_dim": 128, "intermediate_size": 352, "vocab_size": 333, "rope_theta": 1000000.0,
+    "rms_norm_eps": 1e-5, "max_position_embeddings": 512, "tie_word_embeddings": False,
+    "hidden_act": "silu", "attention_bias": False, "rope_scaling": None, "initializer_range": 0.03,
+    "eos_token_id": 3, "torch_dtype": "float32",
+}
 # engine-side options that go with them
 ENGINE_A = {"kv_block_size": 16}
 ENGINE_B = {"kv_block_size": 8}
+ENGINE_C = {"kv_block_size": 32}
 INIT_A = {"std": 0.02, "norm_std": 0.0}
 INIT_B = {"std": 0.05, "norm_std": 0.1}
+INIT_C = {"std": 0.03, "norm_std": 0.05}
 
-CONFIGS = {"A": (TINY_A, ENGINE_A, INIT_A), "B": (TINY_B, ENGINE_B, INIT_B)}
+CONFIGS = {"A": (TINY_A, ENGINE_A, INIT_A), "B": (TINY_B, ENGINE_B, INIT_B), "C": (TINY_C, ENGINE_C, INIT_C)}
 
 
 def make_folder(tmp_path, cfg, seed=0, std=0.02, norm_std=0.0, dtype="float32", sharpen=4.0):
