@@ -1,7 +1,7 @@
 """A plain, slow Llama: whole sequences, no cache, one function per part.
 
-Written from the reference's formulas (each function cites file:line under
-/root/reference); it shares no code with the engine.  Everything is computed in
+Written from the reference's formulas (each function cites file:line, relative to the
+reference's checkout); it shares no code with the engine.  Everything is computed in
 float64 by default so that it can serve as the truth for the float32 engine;
 `act_dtype=torch.bfloat16` rounds activations at the places where the serving
 path stores bfloat16, which makes the comparison with that path tight.
@@ -42,11 +42,12 @@ def rope_table(max_len: int, dim: int, base: float):
     return cos.to(torch.float32).to(F64), sin.to(torch.float32).to(F64)
 
 
-def rope_table_fast(max_len: int, dim: int, base: float):
-    """Same table as `rope_table`, vectorised (used for long sequences)."""
+def rope_table_fast(max_len: int, dim: int, base: float, position_factor: float = 1.0):
+    """Same table as `rope_table`, vectorised (used for long sequences).  `position_factor`
+    divides the positions first (linear scaling of positions; the reference has none: 1)."""
     half = dim // 2
     inv = torch.tensor([math.pow(base, -float(i) / float(half)) for i in range(half)], dtype=F64)
-    ang = torch.arange(max_len, dtype=F64)[:, None] * inv[None, :]
+    ang = (torch.arange(max_len, dtype=F64) / position_factor)[:, None] * inv[None, :]
     return torch.cos(ang).to(torch.float32).to(F64), torch.sin(ang).to(torch.float32).to(F64)
 
 
@@ -61,6 +62,20 @@ def apply_rope(x: torch.Tensor, positions: Sequence[int], cos: torch.Tensor, sin
         a, b = x[t, :, :half], x[t, :, half:]
         out[t, :, :half] = c * a - s * b
         out[t, :, half:] = s * a + c * b
+    return out
+
+
+def apply_rope_interleaved(x: torch.Tensor, positions: Sequence[int], cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    """The other usual pairing, which the reference does not have: pair i is (x[2i], x[2i + 1]),
+    rotated by the same angles as pair i of `apply_rope`.  Equal to `apply_rope` on a head whose
+    dims are permuted so that the even ones come first (tested)."""
+    T, nh, hd = x.shape
+    out = x.clone()
+    for t in range(T):
+        c, s = cos[int(positions[t])], sin[int(positions[t])]
+        a, b = x[t, :, 0::2], x[t, :, 1::2]
+        out[t, :, 0::2] = c * a - s * b
+        out[t, :, 1::2] = s * a + c * b
     return out
 
 

@@ -367,11 +367,11 @@ def test_step_metadata_layout_and_padding():
 
 def test_static_block_table_rows_are_rewritten_when_they_change():
     import numpy as np
-    from tiny_llm_amd.engine.step import Layout, fill_metadata
+    from tiny_llm_amd.engine.step import Layout, SeenTables, fill_metadata
     bs = 4
     lay = Layout(2, 2, 2, 1, 4, {}, False)
     buf = np.zeros(lay.total, dtype=np.int32)
-    seen = [[None, None]]
+    seen = SeenTables(1, 2)
     rows = _rows([(5, [1], [0]), (2, [1], [0])], bs)
     fill_metadata(buf, lay, rows, bs, None, seen)
     assert lay.sec(buf, "tables0").reshape(2, 4).tolist() == [[3, 4, 0, 0], [6, 0, 0, 0]]
@@ -382,6 +382,115 @@ def test_static_block_table_rows_are_rewritten_when_they_change():
     fill_metadata(buf, lay, rows, bs, None, seen)
     assert lay.sec(buf, "tables0").reshape(2, 4).tolist() == [[3, 4, 20, 0], [3, 0, 0, 0]]
     assert lay.sec(buf, "slots0").tolist() == [20 * 4, 3 * 4]
+
+
+def test_static_rows_after_a_step_that_did_not_run():
+    """A captured step fails and is undone; another request takes the block that was given back;
+    the first request grows again to the SAME length with ANOTHER block.  The static buffer must
+    then hold the real table: the request would otherwise write its new key to one page and read
+    another request's page."""
+    import numpy as np
+    from tiny_llm_amd.engine.step import Layout, SeenTables, _Row, fill_metadata
+    bs = 4
+    cm = CacheManager(full(1), [None], block_size=bs, num_blocks=8, max_seqs=3)
+    cm.reserve_step([("a", 8), ("b", 8)])
+    cm.commit("a", 8), cm.commit("b", 8)
+    cm.forget_reservation()
+    lay = Layout(2, 2, 2, 1, 4, {}, False)
+    buf = np.zeros(lay.total, dtype=np.int32)
+    seen = SeenTables(1, 2, cm.table_epoch)
+
+    def rows_of(ids):
+        before = cm.reserve_step([(r, 1) for r in ids])
+        return [_Row(r, [1], [0], c, cm.slot(r), [cm.block_table(r, 0)]) for r, c in zip(ids, before)]
+
+    rows = rows_of(["a", "b"])                                  # a: [0, 1, 4], b: [2, 3, 5]
+    fill_metadata(buf, lay, rows, bs, None, seen, cm.table_epoch)
+    assert lay.sec(buf, "tables0").reshape(2, 4).tolist() == [[0, 1, 4, 0], [2, 3, 5, 0]]
+    cm.undo_reservation()                                       # the step did not run
+    assert cm.block_table("a", 0) == [0, 1] and cm.free_blocks() == [4]
+    cm.reserve_step([("c", 3)])                                 # somebody else takes block 4
+    cm.commit("c", 3)
+    cm.forget_reservation()
+    assert cm.block_table("c", 0) == [4]
+    rows = rows_of(["a", "b"])                                  # the same lengths, other blocks
+    assert cm.block_table("a", 0) == [0, 1, 5] and cm.block_table("b", 0) == [2, 3, 6]
+    fill_metadata(buf, lay, rows, bs, None, seen, cm.table_epoch)
+    tables = lay.sec(buf, "tables0").reshape(2, 4)
+    assert tables[0, :3].tolist() == cm.block_table("a", 0) and tables[1, :3].tolist() == cm.block_table("b", 0)
+    assert lay.sec(buf, "slots0").tolist() == [5 * bs, 6 * bs]  # and the new keys go where the table says
+    # without an undo in between nothing is forgotten: rows of unchanged tables are not rewritten
+    for r in ("a", "b"):
+        cm.commit(r, 9)
+    cm.forget_reservation()
+    tables[:] = -5
+    rows = rows_of(["a", "b"])
+    fill_metadata(buf, lay, rows, bs, None, seen, cm.table_epoch)
+    assert (lay.sec(buf, "tables0") == -5).all()
+
+
+def test_a_step_that_did_not_run_leaves_the_state_slots_as_they_were():
+    import torch
+    cm = CacheManager(full(1), [StateSpec((3,))], block_size=4, num_blocks=8, max_seqs=3)
+    cm.allocate_tensors(torch.float32, "cpu")
+    cm.reserve_step([("a", 2), ("b", 2)])
+    st = cm.states[0]
+    st[cm.slot("a")] = torch.tensor([1.0, 2.0, 3.0])
+    st[cm.slot("b")] = torch.tensor([4.0, 5.0, 6.0])
+    cm.commit("a", 2), cm.commit("b", 2)
+    cm.forget_reservation()
+    cm.reserve_step([("b", 1), ("c", 4)])
+    st[cm.slot("b")] += 10.0                # the failing step's parts had already written
+    st[cm.slot("c")] += 7.0
+    cm.undo_reservation()
+    assert st[cm.slot("a")].tolist() == [1.0, 2.0, 3.0] and st[cm.slot("b")].tolist() == [4.0, 5.0, 6.0]
+    assert not cm.has("c")
+    cm.reserve_step([("c", 4)])             # a request admitted later starts from zero as ever
+    assert st[cm.slot("c")].tolist() == [0.0, 0.0, 0.0]
+    cm.audit()
+
+
+def test_every_group_has_a_pool_of_its_own_size():
+    """A window group holds, per request, its window and one portion at most: its pool may be much
+    smaller than the full group's, and a long request is still admitted and served."""
+    from tiny_llm_amd.cache.manager import blocks_held_at_most
+    from tiny_llm_amd.config import EngineConfig
+    from tiny_llm_amd.engine.loading import plan_cache_blocks
+    bs, window, budget, max_len = 4, 6, 8, 200
+    kv = CacheSpec.keys_and_values
+    specs = [kv(1, 8), kv(1, 8, "window", window)]
+    assert blocks_held_at_most(specs[0], bs, 100, budget) == 25
+    assert blocks_held_at_most(specs[1], bs, 100, budget) == 4      # 5 + 8 = 13 positions, starting anywhere
+    assert blocks_held_at_most(specs[1], bs, 9, budget) == 3        # a short request holds all it has
+    probe = CacheManager(specs, [None, None], bs, 1, 1)
+    held = probe.blocks_held_at_most(max_len, budget)
+    e = EngineConfig(kv_block_size=bs, max_num_seqs=2, max_num_batched_tokens=budget)
+    assert plan_cache_blocks(e, max_len, [100, 100], None, held) == [2 * 50, 2 * 4]
+    assert plan_cache_blocks(e, max_len, [100, 100], 5500, held) == [45, 3]     # one factor for all groups
+    e2 = EngineConfig(kv_block_size=bs, max_num_seqs=2, max_num_batched_tokens=budget, num_kv_blocks=30)
+    assert plan_cache_blocks(e2, max_len, [100, 100], None, held) == [30, 8]    # given: for a full group
+    cm = CacheManager(specs, [None, None], bs, [30, 4], 2)
+    assert cm.group_blocks == [30, 4] and cm.num_blocks == 30
+    cm.allocate_tensors(__import__("torch").float32, "cpu")
+    assert cm.groups[0].tensors["k"].shape[1] == 30 and cm.groups[1].tensors["k"].shape[1] == 4
+    s = Scheduler(cm, 2, budget, max_len, None)
+    s.add(req("long", 90, max_new=6))      # 23 blocks in the full group, 4 at most in the window group
+    steps = 0
+    while s.has_work():
+        p = s.schedule()
+        assert p.entries and not p.preempted and not p.finished
+        run_plan(cm, s, p)
+        assert cm.groups[1].pool.used_count <= 4
+        steps += 1
+        assert steps < 100
+    assert s.finished[0].finish_reason == "length" and len(s.finished[0].output) == 6
+    assert cm.free_blocks() == [30, 4]
+    # what can never be held is refused when it is added, per group
+    cm2 = CacheManager(specs, [None, None], bs, [30, 3], 2)
+    s2 = Scheduler(cm2, 2, budget, max_len, None)
+    with pytest.raises(ValueError):
+        s2.add(req("too long for the window pool", 90))
+    s2.add(req("short", 9))                # holds 3 blocks in either group
 
 
 def test_reservation_of_a_step_that_did_not_run_is_undone():
@@ -471,4 +580,40 @@ def test_runs_of_decode_steps_end_where_a_decision_is_due():
     run_plan(cm2, s2, s2.schedule())
     p2 = s2.schedule()
     assert s2.burst_length(p2, 10) == 10                   # 6 + 10 = 16 tokens: the pool's 4 blocks
-    assert s2.burst_length(p2, 11) == 1                    # one more does not fit: step by step (and preemption rules)
+    assert s2.burst_length(p2, 11) == 10                   # one more does not fit: the run ends where the blocks end
+    # a running request that the plan leaves out (the budget is below the number of decoding
+    # requests) would sit idle for a whole run: step by step then
+    cm3, s3 = make_sched(num_blocks=40, block_size=4, max_seqs=3, budget=8, max_len=100)
+    for rid in "abc":
+        s3.add(req(rid, 2, max_new=30))
+    run_plan(cm3, s3, s3.schedule())
+    assert s3.burst_length(s3.schedule(), 8) == 8
+    s3.budget = 2
+    p3 = s3.schedule()
+    assert [e.request.req_id for e in p3.entries] == ["a", "b"] and s3.burst_length(p3, 8) == 1
+
+
+def test_runs_of_decode_steps_in_a_window_group():
+    """The blocks of a whole run are taken up front in every group; what the window has passed
+    goes back when the run is committed."""
+    bs, window = 4, 6
+    specs = [CacheSpec.keys_and_values(1, 8), CacheSpec.keys_and_values(1, 8, "window", window)]
+    cm = CacheManager(specs, [None, None], bs, [20, 6], 2)
+    s = Scheduler(cm, 2, 16, 60, None)
+    s.add(req("a", 10, max_new=30))
+    run_plan(cm, s, s.schedule())
+    p = s.schedule()
+    # the window pool has 6 blocks: a holds 2 (positions 5.. of its 10), 4 are free: 16 more positions
+    k = s.burst_length(p, 32)
+    assert k == 18                                          # 10 + 18 = 28 positions: 7 logical blocks, 3 were given
+    cm.reserve_step([(e.request.req_id, k) for e in p.entries])
+    assert cm.free_blocks() == [20 - 7, 0]
+    for e in p.entries:
+        cm.commit(e.request.req_id, e.start + k)
+    cm.forget_reservation()
+    cm.audit()
+    done = s.update_burst(p, [[7]] * k)
+    assert not done and cm.num_tokens("a") == 28
+    # after the commit only the window's blocks are held: positions 23.. -> logical blocks 5 and 6
+    assert [b != RELEASED for b in cm.block_table("a", 1)] == [False] * 5 + [True] * 2
+    assert cm.free_blocks() == [20 - 7, 6 - 2]

@@ -334,13 +334,11 @@ def test_decoding_past_a_context_bucket(dtype, graphs, around, tmp_path_factory)
     if graphs:
         bounds = sorted({k[2] for k, g in eng.runner._graphs.items() if k[0] == "decode" and g.graph is not None})
         assert bounds == [around, 2 * around]
-    if dtype == "bfloat16":
-        # the split path was really taken beyond the bound
-        attn = eng.decoder.layers[0].mixer
-
-        class Ctx:
-            max_seq_len = 2 * around
-        assert attn._splits(Ctx, 3, eng.decoder.device)[0] >= 2
+    # beyond the bound the keys of a request were really shared out: the run itself asked the
+    # workspace for the partial results (bfloat16: over workgroups; float32: chunks of 256 keys)
+    parts = eng.runner.workspace._bufs.get(("attention_partials", torch.float32))
+    heads, hd = cfg["num_attention_heads"], cfg["head_dim"]
+    assert parts is not None and parts.numel() >= 2 * 3 * heads * (hd + 2)
 
 
 _folders = {}
@@ -531,6 +529,135 @@ def test_a_step_that_fails_leaves_the_cache_as_it_was(folders):
     assert rel_err(again[1], first[0]) < 1e-6
 
 
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_float32_logits_have_the_same_bits_alone_and_in_any_batch(name, folders):
+    """In float32 a token's logits must not depend, to the bit, on what else its step holds: decoded
+    alone (1 row: norms ride in the few-row products), beside other decoding requests, beside a
+    prompt portion that makes the step 40 and 200 rows long (the norm as a row factor of the tiled
+    products; attention by tiles), and as a captured step."""
+    from tiny_llm_amd.config import EngineConfig
+    from tiny_llm_amd.engine.loading import build_runner, load_model
+    from tiny_llm_amd.engine.step import StepEntry
+    cfg, eng_kw, _ = CONFIGS[name]
+    engine = EngineConfig(dtype="float32", max_cache_tokens=2048, max_num_seqs=4, max_num_batched_tokens=512,
+                          use_graphs=True, **eng_kw)
+    _, dec = load_model(folders[name], engine)
+    runner = build_runner(dec, engine)
+    V = cfg["vocab_size"]
+    a, other, long = random_tokens(60, V, 1), random_tokens(30, V, 2), random_tokens(400, V, 3)
+    results = []
+    for beside, graph in ((None, False), ("decoding", False), (39, False), (199, False), (39, True), (None, True)):
+        runner.step([StepEntry("a", a[:50], [])])
+        if beside == "decoding":
+            runner.step([StepEntry("o", other[:20], []), StepEntry("p", long[:77], [])])
+        rows = []
+        for at in range(50, 60):
+            ents = [StepEntry("a", [a[at]], [0])]
+            if beside == "decoding":
+                ents = [StepEntry("o", [other[at - 30]], [0])] + ents + [StepEntry("p", [long[at + 27]], [])]
+            elif beside is not None:
+                ents = [StepEntry(f"l{at}", long[:beside], [beside - 1])] + ents
+            out = runner.step(ents, use_graph=graph)
+            rows.append(out[1 if beside is not None else 0].clone())
+            if beside not in (None, "decoding"):
+                runner.finish(f"l{at}")
+        results.append(torch.stack(rows).cpu())
+        for r in ("a", "o", "p"):
+            runner.finish(r)
+    for got in results[1:]:
+        assert torch.equal(got, results[0])
+    runner.cache.audit()
+
+
+def test_captured_shapes_are_bounded_and_come_back(folders):
+    """At most MAX_STEP_SHAPES shapes of step keep their buffers and graphs; the one used longest ago
+    goes, and is simply built and captured again when its shape returns."""
+    from tiny_llm_amd.config import EngineConfig
+    from tiny_llm_amd.engine.loading import build_runner, load_model
+    from tiny_llm_amd.engine.step import StepEntry
+    cfg, eng_kw, _ = CONFIGS["A"]
+    w, c = read_weights(folders["A"])
+    engine = EngineConfig(dtype="float32", max_cache_tokens=512, max_num_seqs=4, **eng_kw)
+    _, dec = load_model(folders["A"], engine)
+    runner = build_runner(dec, engine)
+    runner.MAX_STEP_SHAPES = 2
+    toks = {r: random_tokens(40, cfg["vocab_size"], 70 + i) for i, r in enumerate("abc")}
+    refs = {r: plain.llama_forward(w, c, t) for r, t in toks.items()}
+    at = {r: 0 for r in toks}
+
+    def step(who, n):
+        ents = [StepEntry(r, toks[r][at[r]:at[r] + n], [n - 1]) for r in who]
+        got = runner.step(ents, use_graph=True).cpu()
+        for i, r in enumerate(who):
+            at[r] += n
+            assert rel_err(got[i], refs[r][at[r] - 1]) < 1e-4
+    step("abc", 5)                       # a mixed shape
+    for _ in range(3):
+        step("abc", 1)                   # decode, three requests: eager, captured, replayed
+    for _ in range(3):
+        step("ab", 1)                    # decode, two requests: the mixed shape goes
+    assert len(runner._graphs) == 2 and {k[0] for k in runner._graphs} == {"decode"}
+    for _ in range(3):
+        step("c", 1)                     # decode, one request: the three-request shape goes
+    assert [k[1] for k in runner._graphs] == [2, 1]
+    for _ in range(3):
+        step("abc", 1)                   # and comes back
+    assert [k[1] for k in runner._graphs] == [1, 3] and runner._graphs[("decode", 3, 512, False)].graph is not None
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_captured_step_that_fails_leaves_no_stale_block_table(dtype, folders):
+    """A replayed decode step fails after its tables were laid out and is undone; another request
+    takes the block that went back; the step is run again and the requests grow to the same
+    lengths with other blocks.  The static buffers of the captured step must follow: logits
+    against the plain model, with a poisoned pool."""
+    from tiny_llm_amd.config import EngineConfig
+    from tiny_llm_amd.engine.loading import build_runner, load_model
+    from tiny_llm_amd.engine.step import StepEntry
+    cfg, eng_kw, _ = CONFIGS["A"]
+    act = torch.bfloat16 if dtype == "bfloat16" else None
+    tol = 1e-4 if dtype == "float32" else 2e-2
+    w, c = read_weights(folders["A"], round_to=act)
+    engine = EngineConfig(dtype=dtype, max_cache_tokens=256, max_num_seqs=3, use_graphs=True, **eng_kw)
+    bs = engine.kv_block_size
+    _, dec = load_model(folders["A"], engine)
+    runner = build_runner(dec, engine)
+    for g in runner.cache.groups:
+        for t in g.tensors.values():
+            t.fill_(float("nan"))
+    n0 = 2 * bs - 2
+    toks = {r: random_tokens(n0 + 8, cfg["vocab_size"], 90 + i) for i, r in enumerate("ab")}
+    toks["c"] = random_tokens(5, cfg["vocab_size"], 99)
+    refs = {r: plain.llama_forward(w, c, t, act_dtype=act) for r, t in toks.items()}
+    runner.step([StepEntry(r, toks[r][:n0], []) for r in "ab"], use_graph=True)
+
+    def decode(at):
+        got = runner.step([StepEntry(r, [toks[r][at]], [0]) for r in "ab"], use_graph=True).cpu()
+        for i, r in enumerate("ab"):
+            assert rel_err(got[i], refs[r][at]) < tol, (r, at)
+
+    decode(n0)              # eagerly on the static buffers
+    decode(n0 + 1)          # captured
+    sg = next(g for k, g in runner._graphs.items() if k[0] == "decode" and g.graph is not None)
+    before = {r: list(runner.cache.block_table(r, 0)) for r in "ab"}
+
+    class Refuses:
+        def replay(self):
+            raise RuntimeError("the replay was refused")
+    good, sg.graph = sg.graph, Refuses()
+    with pytest.raises(RuntimeError):
+        decode(n0 + 2)      # starts a new block for both: laid out, then undone
+    sg.graph = good
+    assert {r: list(runner.cache.block_table(r, 0)) for r in "ab"} == before
+    got = runner.step([StepEntry("c", toks["c"], [4])], use_graph=True).cpu()      # takes the block a was given
+    assert rel_err(got[0], refs["c"][4]) < tol
+    for at in range(n0 + 2, n0 + 8):
+        decode(at)
+    assert runner.cache.block_table("a", 0)[2] != runner.cache.block_table("c", 0)[0]
+    assert runner.graph_steps >= 6
+    runner.cache.audit()
+
+
 def test_command_line_generates_from_prompt_ids(folders):
     cfg = CONFIGS["A"][0]
     prompt = random_tokens(12, cfg["vocab_size"], 5)
@@ -634,13 +761,18 @@ def test_toy_stateful_mixer_registers_builds_and_steps(tmp_path):
     try:
         raw = {"architectures": ["ToyForCausalLM"], "hidden_size": 64, "intermediate_size": 96, "vocab_size": 101}
         engine = EngineConfig(dtype="float32", kv_block_size=4, max_cache_tokens=256, max_num_seqs=3,
-                              max_num_batched_tokens=256, use_graphs=False)
+                              max_num_batched_tokens=48, use_graphs=False)
         _, dec = random_model(raw, engine, seed=1, std=0.3)
         runner = build_runner(dec, engine)
         assert [g.entries for g in runner.cache.groups] == [[(0, "mixer"), (3, "mixer")], [(2, "mixer")]]   # full, windowed
+        # the windowed group never holds more of a request than its window and a step's tokens:
+        # (5 - 1 + 48) positions, starting anywhere in a block, for each of 3 requests
+        assert runner.cache.group_blocks == [64, 3 * 14]
+        assert runner.decoder.caches[2]["mixer"].k.shape[0] == 42 and runner.decoder.caches[0]["mixer"].k.shape[0] == 64
         assert runner.decoder.states[1]["mixer"].shape == (3, 64) and runner.decoder.states[0] == {}
         a, b = random_tokens(45, 101, 1), random_tokens(23, 101, 2)
-        whole = runner.step([StepEntry("a", a, list(range(45))), StepEntry("b", b, list(range(23)))]).cpu()
+        whole = torch.cat([runner.step([StepEntry("a", a, list(range(45)))]).cpu(),
+                           runner.step([StepEntry("b", b, list(range(23)))]).cpu()])
         runner.finish("a")
         runner.finish("b")
         got_a, got_b = [], []

@@ -403,6 +403,46 @@ def test_linear_norm_f32(M, K, N):
     ops().linear_norm_f32(x[m:m + 1].contiguous(), nw, eps, w, alone)
     assert torch.equal(alone, out[m:m + 1])
     assert not ops().linear_norm_f32_ok(65, N, K, K)
+    # the norm as two kernels (what steps of more rows take): the same BITS, with every epilogue, also
+    # when the rows sit among many others (the tiled product) and when they are gathered
+    hp, inv = ops().norm_prescale_f32(x, nw, eps)
+    assert rel(hp, (x * nw).double().cpu()) == 0.0
+    two = torch.full((M, N), float("nan"), device=DEV)
+    ops().linear(hp, w, two, row_scale=inv)
+    assert torch.equal(two, out)
+    ops().linear(hp, w, two, residual=res, row_scale=inv)
+    assert torch.equal(two, out_r)
+    if N % 2 == 0:
+        z2 = torch.empty(M, N // 2, device=DEV)
+        ops().linear(hp, w, z2, epilogue="swiglu", row_scale=inv)
+        assert torch.equal(z2, z)
+    many = torch.cat([x, (torch.randn(90, K, generator=g) * 0.3).to(DEV)])[torch.randperm(M + 90, generator=g).to(DEV)]
+    where = torch.tensor([int((many == x[i]).all(dim=1).nonzero()[0]) for i in range(M)], dtype=torch.int32, device=DEV)
+    hm, invm = ops().norm_prescale_f32(many, nw, eps)
+    big = torch.empty(M + 90, N, device=DEV)
+    ops().linear(hm, w, big, row_scale=invm)
+    assert torch.equal(big[where.long()], out)
+    hg, invg = ops().norm_prescale_f32(many, nw, eps, rows=where)
+    ops().linear(hg, w, two, row_scale=invg)
+    assert torch.equal(two, out)
+
+
+@pytest.mark.parametrize("K", [70, 258, 1001])
+def test_norm_prescale_f32_any_inner_size(K):
+    """Inner sizes that are no multiple of 4 (no fused route exists for them): against the plain norm."""
+    g = torch.Generator().manual_seed(K)
+    M, N, eps = 19, 37, 1e-6
+    x = torch.randn(M, K, generator=g).to(DEV)
+    nw = (1 + 0.1 * torch.randn(K, generator=g)).to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(DEV)
+    h, inv = ops().norm_prescale_f32(x, nw, eps)
+    out = torch.empty(M, N, device=DEV)
+    ops().linear(h, w, out, row_scale=inv)
+    assert rel(out, plain.rms_norm(x.double().cpu(), nw.double().cpu(), eps) @ w.double().cpu().T) < 1e-5
+    alone = torch.empty(1, N, device=DEV)
+    h1, inv1 = ops().norm_prescale_f32(x[7:8].contiguous(), nw, eps)
+    ops().linear(h1, w, alone, row_scale=inv1)
+    assert torch.equal(alone, out[7:8])
 
 
 @pytest.mark.parametrize("K,N", [(200, 90), (1000, 72), (5632, 130), (256, 8), (258, 34)])
@@ -519,6 +559,54 @@ def test_rope_store(dtype, hd, nq, nkv, bs):
     assert torch.equal(vc.cpu().double(), exp_v)
     untouched = exp_k == 1.0
     assert torch.equal(kc.cpu().double()[untouched], exp_k[untouched])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hd,rd", [(32, 32), (48, 16), (128, 128)])
+def test_rope_store_interleaved_pairing_and_scaled_positions(dtype, hd, rd):
+    """The part's other pairing, (2i, 2i + 1), and positions divided by a factor, against the plain
+    functions; pairings and scalings that are not built are refused by name."""
+    from tiny_llm_amd.parts.rotary import RotaryEmbedding
+    nq, nkv, bs, T, max_pos = 3, 2, 8, 9, 80
+    rot = RotaryEmbedding("r", dtype, DEV, head_dim=hd, rotary_dim=rd, theta=300.0, max_position=max_pos,
+                          pairing="interleaved", scaling={"kind": "linear", "factor": 4.0})
+    cos, sin, got_rd = rot.rotary_tables()
+    assert got_rd == rd and rot.pairing == "interleaved"
+    pc, ps = plain.rope_table_fast(max_pos, rd, 300.0, position_factor=4.0)
+    assert torch.equal(cos.cpu().double(), pc) and torch.equal(sin.cpu().double(), ps)
+    assert torch.equal(pc[4 * 7], plain.rope_table_fast(max_pos, rd, 300.0)[0][7])      # position 28 has the angles of 7
+    g = torch.Generator().manual_seed(hd)
+    qkv = torch.randn(T, (nq + 2 * nkv) * hd, generator=g).to(dtype)
+    positions = torch.tensor([0, 1, 2, 3, 30, 31, 79, 5, 64], dtype=torch.int32)
+    slots = torch.tensor([0, 1, 2, 3, 3 * bs + 6, 3 * bs + 7, 5 * bs, -1, 2 * bs + 1], dtype=torch.int32)
+    kc = torch.ones(7, nkv, bs, hd, dtype=dtype, device=DEV)
+    vc = torch.ones(7, nkv, bs, hd, dtype=dtype, device=DEV)
+    dq = qkv.clone().to(DEV)
+    ops().rope_store(dq, positions.to(DEV), cos, sin, slots.to(DEV), kc, vc, nq, nkv, hd, rd, pairing="interleaved")
+
+    def ref(x, heads):
+        x = x.reshape(T, heads, hd).clone()
+        x[..., :rd] = plain.apply_rope_interleaved(x[..., :rd], positions.tolist(), pc, ps)
+        return x
+    t = tol(dtype, 1e-6, 4e-3)
+    assert rel(dq[:, :nq * hd].reshape(T, nq, hd), ref(qkv.double()[:, :nq * hd], nq)) < t
+    k_ref = ref(qkv.double()[:, nq * hd:(nq + nkv) * hd], nkv)
+    for i in range(T):
+        sl = int(slots[i])
+        if sl >= 0:
+            assert rel(kc[sl // bs, :, sl % bs], k_ref[i].to(dtype).double()) < t
+            assert torch.equal(vc[sl // bs, :, sl % bs].cpu(), qkv[i, (nq + nkv) * hd:].reshape(nkv, hd))
+    # the two pairings are one rotation under a permutation of the dims (even dims first)
+    x = torch.randn(T, 2, rd, generator=g, dtype=torch.float64)
+    perm = list(range(0, rd, 2)) + list(range(1, rd, 2))
+    assert torch.allclose(plain.apply_rope_interleaved(x, positions.tolist(), pc, ps)[..., perm],
+                          plain.apply_rope(x[..., perm], positions.tolist(), pc, ps), atol=1e-12)
+    with pytest.raises(ValueError, match="pairing"):
+        RotaryEmbedding("r", dtype, DEV, head_dim=hd, theta=1e4, max_position=8, pairing="quarters")
+    with pytest.raises(ValueError, match="scaling"):
+        RotaryEmbedding("r", dtype, DEV, head_dim=hd, theta=1e4, max_position=8, scaling={"kind": "spiral", "factor": 2})
+    with pytest.raises(Exception, match="pairing"):
+        ops().rope_store(dq, positions.to(DEV), cos, sin, slots.to(DEV), kc, vc, nq, nkv, hd, rd, pairing="quarters")
 
 
 def test_rope_invariants():

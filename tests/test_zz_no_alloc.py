@@ -62,12 +62,17 @@ def test_static_scratch_entry_point_matches_the_one_that_takes_scratch():
     outs = {name: torch.full((b[0].shape[0], nq * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
             for name, b in (("big_s", big), ("big_r", big), ("small_s", small), ("small_r", small))}
     scratch = torch.full((limit,), float("nan"), dtype=torch.float32, device=DEV)
+    # a first call on this device looks the array's address up (and loads the code, array included)
+    warm = torch.empty_like(outs["small_s"])
+    assert call(lib, True, small, nq, nkv, hd, bs, 2, warm) == 0
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    # the device's own count of free memory: an allocation made inside the library, which torch's
+    # allocator knows nothing of, would show here
+    free_before = torch.cuda.mem_get_info()[0]
     assert call(lib, True, big, nq, nkv, hd, bs, 5, outs["big_s"]) == 0
     assert call(lib, True, small, nq, nkv, hd, bs, 3, outs["small_s"]) == 0      # smaller, right after
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] >= free_before
     assert call(lib, False, big, nq, nkv, hd, bs, 5, outs["big_r"], scratch) == 0
     assert call(lib, False, small, nq, nkv, hd, bs, 3, outs["small_r"], scratch) == 0
     torch.cuda.synchronize()

@@ -4,8 +4,10 @@ import os
 
 import torch
 
-# Where the reference's checkout lies (its tests' fixtures are read from there, never run).
-REFERENCE = os.environ.get("TINY_LLM_REFERENCE", "/root/reference")
+# Where the reference's checkout lies (its tests' fixtures are read from there, never run): beside
+# this repository unless TINY_LLM_REFERENCE says otherwise.  Tests that need a fixture skip without it.
+REFERENCE = os.environ.get("TINY_LLM_REFERENCE") or os.path.join(
+    os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__)))), "reference")
 REFERENCE_DATA = os.path.join(REFERENCE, "tests", "datas")
 
 # Two tiny configurations of the architecture that differ in every size and option.

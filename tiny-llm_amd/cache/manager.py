@@ -13,6 +13,10 @@ never run out and frees everything when the whole batch is done
   is more than `window` behind the next query; a "full" group when the request ends.
 * Blocks that are given back are used again by later growth, most recently freed first.
 * `grow` is all-or-nothing over all groups, so a step that cannot be held changes nothing.
+* Every group has a pool of its own size: a window group never holds more of a request than
+  its window and the portion in hand, so its pool may be much smaller than a full group's.
+* A step that did not run is undone: tables are cut back, admitted requests leave, and the
+  per-request state that the step's parts may already have written is put back.
 
 Everything here is host bookkeeping; device tensors are only allocated (by
 `allocate_tensors`) and handed to the mixers as views.
@@ -56,10 +60,42 @@ class RequestCache:
     blocks: List[List[int]] = field(default_factory=list)   # per group: logical block -> id or RELEASED
 
 
+def group_specs(cache_specs) -> Tuple[List[CacheSpec], List[List[Hashable]]]:
+    """The groups that owners with these cache specs form, in order of first appearance:
+    (spec of each group, owners of each group)."""
+    if not isinstance(cache_specs, Mapping):
+        cache_specs = {i: c for i, c in enumerate(cache_specs) if c is not None}
+    specs: List[CacheSpec] = []
+    owners: List[List[Hashable]] = []
+    by_key: Dict[Tuple, int] = {}
+    for i, cs in cache_specs.items():
+        key = cs.group_key()
+        if key not in by_key:
+            by_key[key] = len(specs)
+            specs.append(cs)
+            owners.append([])
+        owners[by_key[key]].append(i)
+    return specs, owners
+
+
+def blocks_held_at_most(spec: CacheSpec, block_size: int, total_len: int, portion: int) -> int:
+    """The most blocks a request of `total_len` tokens holds in a group at any time when it is
+    fed in portions of at most `portion` tokens.  A full group keeps every position.  A window
+    group keeps, while a portion runs, the window behind its first token and the portion itself:
+    at most window - 1 + portion positions, which may start anywhere in a block."""
+    whole = -(-max(0, int(total_len)) // block_size)
+    if spec.kind != "window" or spec.window <= 0:
+        return whole
+    span = spec.window - 1 + max(1, int(portion))
+    return min(whole, (span + block_size - 2) // block_size + 1)
+
+
 class CacheManager:
-    def __init__(self, cache_specs, state_specs, block_size: int, num_blocks: int, max_seqs: int):
+    def __init__(self, cache_specs, state_specs, block_size: int, num_blocks, max_seqs: int):
         """cache_specs / state_specs: {owner: spec} for the runs of layers that keep a cache or a
-        state (any hashable owner), or a sequence indexed by owner with None where there is none."""
+        state (any hashable owner), or a sequence indexed by owner with None where there is none.
+        num_blocks: blocks of every group's pool, or one number per group (in the order of
+        `group_specs`)."""
         if not isinstance(cache_specs, Mapping):
             cache_specs = {i: c for i, c in enumerate(cache_specs) if c is not None}
         if not isinstance(state_specs, Mapping):
@@ -67,37 +103,54 @@ class CacheManager:
         if block_size <= 0:
             raise ValueError("block_size must be positive")
         self.block_size = int(block_size)
-        self.num_blocks = int(num_blocks)
         self.max_seqs = int(max_seqs)
+        specs, owners = group_specs(cache_specs)
+        if isinstance(num_blocks, (list, tuple)):
+            if len(num_blocks) != len(specs):
+                raise ValueError(f"{len(num_blocks)} pool sizes for {len(specs)} cache groups")
+            counts = [int(n) for n in num_blocks]
+        else:
+            counts = [int(num_blocks)] * len(specs)
         self.groups: List[CacheGroup] = []
         self.group_of_entry: Dict[Hashable, int] = {}
         self.index_in_group: Dict[Hashable, int] = {}
-        by_key: Dict[Tuple, int] = {}
-        for i, cs in cache_specs.items():
-            key = cs.group_key()
-            if key not in by_key:
-                by_key[key] = len(self.groups)
-                self.groups.append(CacheGroup(cs, [], BlockPool(self.num_blocks)))
-            g = by_key[key]
-            self.group_of_entry[i] = g
-            self.index_in_group[i] = len(self.groups[g].entries)
-            self.groups[g].entries.append(i)
+        for g, (cs, own, n) in enumerate(zip(specs, owners, counts)):
+            self.groups.append(CacheGroup(cs, list(own), BlockPool(n)))
+            for j, i in enumerate(own):
+                self.group_of_entry[i] = g
+                self.index_in_group[i] = j
+        # the largest pool (what a model with one group calls "the" number of blocks)
+        self.num_blocks = max(counts) if counts else (int(num_blocks) if not isinstance(num_blocks, (list, tuple)) else 0)
+        # goes up whenever a request's block table is cut back: what a step buffer remembers of
+        # the tables it holds is worthless then (the same length may come back with other blocks)
+        self.table_epoch = 0
         self.state_specs: Dict[Hashable, StateSpec] = dict(state_specs)
         self.states: Dict[Hashable, torch.Tensor] = {}
         self._free_slots: List[int] = list(range(self.max_seqs - 1, -1, -1))
         self.requests: Dict[Hashable, RequestCache] = {}
-        # what the last `reserve_step` changed, until the step commits: (new requests, table lengths before)
+        # what the last `reserve_step` changed, until the step commits:
+        # (new requests, table lengths before, order of growth, saved state of the step's requests)
         self._reservation: Optional[tuple] = None
 
     # ------------------------------------------------------------------- tensors
-    def elements_per_block(self) -> int:
-        """Cache elements one more block costs, over all groups (every group has `num_blocks`)."""
-        return sum(g.elements_per_block(self.block_size) for g in self.groups)
+    def elements_per_block(self) -> List[int]:
+        """Cache elements one more block costs in each group (all its owners and tensors)."""
+        return [g.elements_per_block(self.block_size) for g in self.groups]
+
+    @property
+    def group_blocks(self) -> List[int]:
+        """Blocks of each group's pool."""
+        return [g.pool.num_blocks for g in self.groups]
+
+    def blocks_held_at_most(self, total_len: int, portion: int) -> List[int]:
+        """Per group: the most blocks a request of `total_len` tokens holds at any time when fed
+        in portions of at most `portion` tokens."""
+        return [blocks_held_at_most(g.spec, self.block_size, total_len, portion) for g in self.groups]
 
     def allocate_tensors(self, dtype: torch.dtype, device) -> None:
         for g in self.groups:
             for t in g.spec.tensors:
-                shape = (len(g.entries), self.num_blocks, *t.page_shape(self.block_size))
+                shape = (len(g.entries), g.pool.num_blocks, *t.page_shape(self.block_size))
                 g.tensors[t.name] = torch.zeros(shape, dtype=dtype, device=device)
         for owner, ss in self.state_specs.items():
             self.states[owner] = torch.zeros((self.max_seqs, *ss.shape), dtype=ss.dtype, device=device)
@@ -206,7 +259,15 @@ class CacheManager:
                               f"{[sum(n[g] for n in needs) for g in range(len(self.groups))]}, "
                               f"free {self.free_blocks()}")
         lengths = {rid: [len(b) for b in self.requests[rid].blocks] for rid, _ in growing if rid in self.requests}
-        self._reservation = (list(new), lengths, [rid for rid, _ in growing])
+        # the state of the requests that are live already, as it is before the step: a part may
+        # have written a request's state by the time the step fails
+        saved = None
+        if self.states:
+            slots = [self.requests[rid].slot for rid, _ in entries if rid in self.requests]
+            if slots:
+                idx = torch.tensor(slots, dtype=torch.long, device=next(iter(self.states.values())).device)
+                saved = (idx, {owner: st.index_select(0, idx) for owner, st in self.states.items()})
+        self._reservation = (list(new), lengths, [rid for rid, _ in growing], saved)
         for rid in new:
             self.add_request(rid)
         for rid, new_len in growing:
@@ -216,12 +277,18 @@ class CacheManager:
     def undo_reservation(self) -> None:
         """The step that the last `reserve_step` was for did not run: requests it admitted leave
         again and tables it lengthened are cut back, in the reverse of the order in which they were
-        served, so that the cache and its free lists are as they were before.  Does nothing when no
-        reservation is open."""
+        served, so that the cache and its free lists are as they were before; the per-request
+        state of the step's requests is put back as it was.  Does nothing when no reservation is open."""
         if self._reservation is None:
             return
-        new, lengths, order = self._reservation
+        new, lengths, order, saved = self._reservation
         self._reservation = None
+        if saved is not None:
+            idx, by_owner = saved
+            for owner, values in by_owner.items():
+                self.states[owner].index_copy_(0, idx, values)
+        if order:
+            self.table_epoch += 1
         for rid in reversed(order):
             rc = self.requests.get(rid)
             if rc is None:

@@ -110,8 +110,9 @@ __global__ void add_residual_kernel(float* __restrict__ x, const T* __restrict__
 
 // ------------------------------------------------------ rotary + cache write
 // qkv row t = [q heads | k heads | v heads], each head `hd` wide.  The first
-// `rot` dims of every q and k head are rotated in the rotate-half pairing
-// (i, i + rot/2) by the angle table row positions[t]; q is rewritten in place,
+// `rot` dims of every q and k head are rotated by the angle table row positions[t]:
+// pair i is the dims (i, i + rot/2) (rotate-half pairing, interleaved == 0) or the
+// dims (2i, 2i + 1) (interleaved pairing); q is rewritten in place,
 // k (rotated) and v go to the cache slot slot_mapping[t] (a negative slot
 // stores nothing).  Cache layout: [block, kv_head, slot_in_block, hd].
 template <typename T>
@@ -119,7 +120,7 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const int32_t* __restrict
                                   const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                   const int32_t* __restrict__ slot_mapping, T* __restrict__ k_cache,
                                   T* __restrict__ v_cache, int nq, int nkv, int hd, int rot,
-                                  int block_size, int64_t row_stride) {
+                                  int block_size, int64_t row_stride, int interleaved) {
   const int t = blockIdx.x;
   const int pos = positions[t];
   const int half = rot / 2;
@@ -135,7 +136,7 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const int32_t* __restrict
     // eight pairs per thread and 16-byte accesses throughout
     const bool aligned = (((uintptr_t)qkv | (uintptr_t)k_cache | (uintptr_t)v_cache | (uintptr_t)cos_t |
                            (uintptr_t)sin_t) & 15) == 0;
-    if (rot == hd && half % 8 == 0 && row_stride % 8 == 0 && aligned) {
+    if (rot == hd && half % 8 == 0 && row_stride % 8 == 0 && aligned && !interleaved) {
       const int chunks = half / 8;
       for (int i = threadIdx.x; i < (nq + nkv) * chunks; i += kThreads) {
         const int head = i / chunks, j = (i - head * chunks) * 8;
@@ -173,18 +174,19 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const int32_t* __restrict
   const int pairs = (nq + nkv) * half;
   for (int i = threadIdx.x; i < pairs; i += kThreads) {
     const int head = i / half, j = i - head * half;
+    const int ia = interleaved ? 2 * j : j, ib = interleaved ? 2 * j + 1 : j + half;
     T* h = row + (int64_t)head * hd;
-    const float a = to_f32(h[j]), b = to_f32(h[j + half]);
+    const float a = to_f32(h[ia]), b = to_f32(h[ib]);
     const float c = cs[j], s = sn[j];
     const T ra = from_f32<T>(c * a - s * b);
     const T rb = from_f32<T>(s * a + c * b);
     if (head < nq) {
-      h[j] = ra;
-      h[j + half] = rb;
+      h[ia] = ra;
+      h[ib] = rb;
     } else if (slot >= 0) {
       T* dst = k_cache + ((blk * nkv + (head - nq)) * block_size + in_blk) * hd;
-      dst[j] = ra;
-      dst[j + half] = rb;
+      dst[ia] = ra;
+      dst[ib] = rb;
     }
   }
   if (slot < 0) return;
@@ -333,15 +335,16 @@ int tl_add_residual(float* x, const void* y, int64_t total, int dtype, hipStream
 
 int tl_rope_store(void* qkv, const int32_t* positions, const float* cos_t, const float* sin_t,
                   const int32_t* slot_mapping, void* k_cache, void* v_cache, int n_tokens, int nq,
-                  int nkv, int hd, int rot, int block_size, int64_t row_stride, int dtype,
+                  int nkv, int hd, int rot, int block_size, int64_t row_stride, int dtype, int interleaved,
                   hipStream_t stream) {
   if (n_tokens <= 0) return TL_OK;
   if (nq < 0 || nkv < 0 || hd <= 0 || rot < 0 || rot > hd || (rot & 1) || block_size <= 0) return TL_ERR_ARG;
+  if (interleaved != 0 && interleaved != 1) return TL_ERR_ARG;
   if (rot > 0 && (!cos_t || !sin_t)) return TL_ERR_ARG;
   if (slot_mapping && (!k_cache || !v_cache)) return TL_ERR_ARG;
   TL_DISPATCH_T(dtype, hipLaunchKernelGGL(rope_store_kernel<T>, dim3(n_tokens), dim3(kThreads), 0, stream,
                                           (T*)qkv, positions, cos_t, sin_t, slot_mapping, (T*)k_cache,
-                                          (T*)v_cache, nq, nkv, hd, rot, block_size, row_stride);)
+                                          (T*)v_cache, nq, nkv, hd, rot, block_size, row_stride, interleaved);)
   return tl_launch_status();
 }
 

@@ -57,6 +57,64 @@ __device__ __forceinline__ f32x4 load_k4(const float* __restrict__ row, int k, i
   return v;
 }
 
+// The factor of a row's RMSNorm from the sum of its squares: ONE expression for every kernel that
+// takes part in a float32 norm, so that they agree to the bit.
+__device__ __forceinline__ float f32_norm_factor(float sumsq, int K, float eps) {
+  return 1.f / sqrtf(sumsq / (float)K + eps);
+}
+
+// The norm in front of a float32 product for any number of rows, as two kernels: this one writes
+// h = norm_w * x (float32) and a row's factor 1 / rms; the product then multiplies its sums by the
+// factor (row_scale).  The squares of a row are added up in the order of gemm_f32_rows_kernel<NORM>:
+// per k block of 256 four chains (chain q takes k = 16 g + 4 q + e for g = 0..15, e = 0..3, in that
+// order, by fused multiply-adds from zero), the chains as (c0 + c1) + (c2 + c3), the blocks in
+// ascending order.  So a row's result has the same bits whether the norm rode in the few-row product
+// or went through here: a row's logits do not depend on how many rows its step had.
+constexpr int FN_THREADS = 256;
+template <bool VEC>
+__global__ __launch_bounds__(FN_THREADS) void norm_prescale_f32_kernel(const float* __restrict__ x,
+                                                                       const float* __restrict__ norm_w,
+                                                                       const int32_t* __restrict__ rows,
+                                                                       float* __restrict__ h,
+                                                                       float* __restrict__ inv_rms, int K,
+                                                                       int64_t lda, float eps) {
+  extern __shared__ float chain_sums[];     // [k blocks][4]
+  const int m = blockIdx.x;
+  const float* row = x + (int64_t)(rows ? rows[m] : m) * lda;
+  float* dst = h + (int64_t)m * K;
+  const int nkb = (K + F_KBLOCK - 1) / F_KBLOCK;
+  for (int c = threadIdx.x; c < nkb * 4; c += FN_THREADS) {
+    const int kb = (c >> 2) * F_KBLOCK, q = c & 3;
+    float ss = 0.f;
+#pragma unroll 4
+    for (int g = 0; g < 16; ++g) {
+      const int k = kb + g * 16 + q * 4;
+      const f32x4 v = load_k4<VEC>(row, k, K), nw = load_k4<VEC>(norm_w, k, K);
+      f32x4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        ss = __builtin_fmaf(v[e], v[e], ss);
+        o[e] = v[e] * nw[e];
+      }
+      if constexpr (VEC) {
+        if (k < K) *(f32x4*)(dst + k) = o;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (k + e < K) dst[k + e] = o[e];
+      }
+    }
+    chain_sums[c] = ss;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float total = 0.f;
+    for (int b = 0; b < nkb; ++b)
+      total += (chain_sums[4 * b] + chain_sums[4 * b + 1]) + (chain_sums[4 * b + 2] + chain_sums[4 * b + 3]);
+    inv_rms[m] = f32_norm_factor(total, K, eps);
+  }
+}
+
 // Tiles of 32 T rows x 32 T columns, four waves of 16 T x 16 T (T x T matrix tiles of 16 x 16), k in
 // steps of 16 through double-buffered LDS.  T = 4 (128 x 128) where that gives the chip enough
 // tiles, T = 2 (64 x 64) where it does not (a portion of 512 tokens times 2048 columns is 64 tiles
@@ -68,7 +126,8 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f32_kernel(const float* __rest
                                                              const float* __restrict__ w,
                                                              float* __restrict__ out,
                                                              const float* __restrict__ residual, int M,
-                                                             int N, int K, int64_t lda, int64_t ldo) {
+                                                             int N, int K, int64_t lda, int64_t ldo,
+                                                             const float* __restrict__ row_scale) {
   constexpr int BT = 32 * T;        // rows and columns of the workgroup's tile
   constexpr int PIECES = BT / 64;   // 16-byte pieces of each operand per thread and k step
   static_assert(T == 2 || T == 4, "tiles of 64 x 64 or 128 x 128");
@@ -149,7 +208,12 @@ __global__ __launch_bounds__(F_THREADS) void gemm_f32_kernel(const float* __rest
 #pragma unroll
     for (int nt = 0; nt < T; ++nt) {
       const int n = n0 + wn * 16 * T + nt * 16 + kk * 4;
-      const f32x4 v = tot[nt][mt];
+      f32x4 v = tot[nt][mt];
+      if (row_scale) {      // the factor of a norm in front (norm_prescale_f32_kernel)
+        const float f = row_scale[m];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[r] *= f;
+      }
       if constexpr (SWIGLU) {   // columns (2j, 2j+1) = (gate_j, up_j); N is even
 #pragma unroll
         for (int r = 0; r < 4; r += 2)
@@ -188,7 +252,8 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
                                                                    const float* __restrict__ residual, int M,
                                                                    int N, int K, int64_t lda, int64_t ldo,
                                                                    const float* __restrict__ norm_w = nullptr,
-                                                                   float eps = 0.f) {
+                                                                   float eps = 0.f,
+                                                                   const float* __restrict__ row_scale = nullptr) {
   extern __shared__ float rows_smem[];      // [m tiles][k blocks][16 rows][COLS columns], NORM: + [m tiles][k blocks][16]
   const int nkb = (K + F_KBLOCK - 1) / F_KBLOCK;
   const int mts = (M + 15) / 16;
@@ -235,7 +300,7 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
         for (int g = 0; g < 16; ++g)
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            ss += av[g][e] * av[g][e];
+            ss = __builtin_fmaf(av[g][e], av[g][e], ss);
             av[g][e] *= nw[g][e];
           }
         // the four lanes of a row (one per k quarter): every lane gets (s0 + s1) + (s2 + s3)
@@ -272,9 +337,12 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
     if constexpr (NORM) {
       float q = 0.f;
       for (int b = 0; b < nkb; ++b) q += ss_smem[(mt * nkb + b) * 16 + r];
-      t *= 1.f / sqrtf(q / (float)K + eps);
+      t *= f32_norm_factor(q, K, eps);
     }
     const int m = mt * 16 + r, n = n0 + c;
+    if constexpr (!NORM) {
+      if (row_scale && m < M) t *= row_scale[m];    // the factor of a norm in front (norm_prescale_f32_kernel)
+    }
     if constexpr (SWIGLU) {   // columns (2j, 2j+1) = (gate_j, up_j); N and n0 are even
       const float u = __shfl_down(t, 1, TL_WAVE);
       if (m < M && n < N && (c & 1) == 0) out[(int64_t)m * ldo + n / 2] = swiglu_pair(t, u);
@@ -1535,10 +1603,29 @@ int tl_linear_norm_f32(const float* x, const float* norm_w, float eps, const flo
   return tl_launch_status();
 }
 
+// Float32, any number of rows: h[m, :] = norm_w * x[rows[m] or m, :] and inv_rms[m] = 1 / rms of that
+// row, for a product that takes inv_rms as its row_scale: together rmsnorm(x) @ w.T with the bits of
+// tl_linear_norm_f32.  h is [n_rows, K] contiguous.
+int tl_norm_prescale_f32(const float* x, const float* norm_w, const int32_t* rows, float* h, float* inv_rms,
+                         int n_rows, int K, int64_t lda, float eps, hipStream_t stream) {
+  if (n_rows <= 0) return TL_OK;
+  if (K <= 0 || lda < K) return TL_ERR_ARG;
+  const int nkb = (K + F_KBLOCK - 1) / F_KBLOCK;
+  const size_t smem = (size_t)nkb * 4 * sizeof(float);
+  if (smem > 48 * 1024) return TL_ERR_ARG;
+  const bool vec = K % 4 == 0 && lda % 4 == 0 && ((uintptr_t)x | (uintptr_t)norm_w | (uintptr_t)h) % 16 == 0;
+  if (vec)
+    hipLaunchKernelGGL(norm_prescale_f32_kernel<true>, dim3(n_rows), dim3(FN_THREADS), smem, stream, x, norm_w, rows, h,
+                       inv_rms, K, lda, eps);
+  else
+    hipLaunchKernelGGL(norm_prescale_f32_kernel<false>, dim3(n_rows), dim3(FN_THREADS), smem, stream, x, norm_w, rows,
+                       h, inv_rms, K, lda, eps);
+  return tl_launch_status();
+}
+
 // out = a @ w.T, then an epilogue.  dtype: element type of a and w (0 float32, 1 bfloat16);
 // out_dtype: of out.  lda: row stride of a in elements; ldo: row stride of out and residual.
-// row_scale (optional, bfloat16 only): every row m of the product is multiplied by row_scale[m]
-// before the epilogue.
+// row_scale (optional): every row m of the product is multiplied by row_scale[m] before the epilogue.
 // epilogue 0: (+ residual[m, n]), out is [M, N].
 // epilogue 1: SiLU-gate of interleaved columns, out[m, j] = silu(c[m, 2j]) * c[m, 2j+1], out is
 //             [M, N/2] of the input's type; N must be even; no residual.
@@ -1547,7 +1634,6 @@ int tl_linear_tile(const void* a, const void* w, void* out, const float* residua
                    int N, int K, int64_t lda, int64_t ldo, int dtype, int out_dtype, int epilogue, int tile,
                    hipStream_t stream) {
   if (M <= 0) return TL_OK;
-  if (row_scale && dtype != 1) return TL_ERR_ARG;   // only the bfloat16 kernels scale rows
   const bool swiglu = epilogue == 1;
   if (N <= 0 || K <= 0 || lda < K || ldo < (swiglu ? N / 2 : N) || epilogue < 0 || epilogue > 1 || tile < 0 ||
       tile > 4)
@@ -1575,7 +1661,7 @@ int tl_linear_tile(const void* a, const void* w, void* out, const float* residua
       dim3 gr((N + cols - 1) / cols);
 #define TL_F32_ROWS(SW, CO)                                                                                   \
   hipLaunchKernelGGL((gemm_f32_rows_kernel<SW, CO>), gr, dim3(FR_THREADS), rows_smem, stream, (const float*)a, \
-                     (const float*)w, (float*)out, residual, M, N, K, lda, ldo)
+                     (const float*)w, (float*)out, residual, M, N, K, lda, ldo, (const float*)nullptr, 0.f, row_scale)
       if (swiglu && cols == 16) TL_F32_ROWS(true, 16);
       else if (swiglu) TL_F32_ROWS(true, 8);
       else if (cols == 16) TL_F32_ROWS(false, 16);
@@ -1593,10 +1679,10 @@ int tl_linear_tile(const void* a, const void* w, void* out, const float* residua
   do {                                                                                                              \
     if (use_small)                                                                                                  \
       hipLaunchKernelGGL((gemm_f32_kernel<SW, VE, 2>), g, dim3(F_THREADS), 0, stream, (const float*)a,              \
-                         (const float*)w, (float*)out, residual, M, N, K, lda, ldo);                                \
+                         (const float*)w, (float*)out, residual, M, N, K, lda, ldo, row_scale);                     \
     else                                                                                                            \
       hipLaunchKernelGGL((gemm_f32_kernel<SW, VE, 4>), g, dim3(F_THREADS), 0, stream, (const float*)a,              \
-                         (const float*)w, (float*)out, residual, M, N, K, lda, ldo);                                \
+                         (const float*)w, (float*)out, residual, M, N, K, lda, ldo, row_scale);                     \
   } while (0)
     if (swiglu && vec) TL_F32_TILED(true, true);
     else if (swiglu) TL_F32_TILED(true, false);

@@ -2,7 +2,7 @@
 and a runner: the one way every front end (generation, replay, bench) builds a model."""
 from __future__ import annotations
 
-from typing import Mapping, Optional
+from typing import Mapping, Optional, Sequence
 
 import torch
 
@@ -48,26 +48,42 @@ def random_model(config: Mapping, engine: EngineConfig, seed: int = 0, std: Opti
     return cfg, dec
 
 
-def plan_cache_blocks(engine: EngineConfig, max_len: int, bytes_per_block: int, free_bytes: Optional[int]) -> int:
-    """How many cache blocks every group gets.  A number in the configuration is taken as it is
-    (`num_kv_blocks`, or `max_cache_tokens` in blocks).  Otherwise: the worst case of
-    `max_num_seqs` requests of `max_len` tokens, which can never run out (the reference's rule,
-    tiny_llm/runtime/cuda/cuda_runtime.cpp:510-515), capped by `cache_memory_fraction` of the
-    device memory that is free once the weights are resident; a smaller pool is what the
-    scheduler's preemption is for."""
+def plan_cache_blocks(engine: EngineConfig, max_len: int, bytes_per_block, free_bytes: Optional[int],
+                      held_at_most: Optional[Sequence[int]] = None):
+    """How many cache blocks each group's pool gets.
+
+    bytes_per_block: one number per cache group (a single number: one group; an int is returned
+    then).  held_at_most: per group the blocks ONE request of `max_len` tokens holds at most (a full
+    group ceil(max_len / block), a window group its window and a step's token budget); None: every
+    group is full.
+
+    A number in the configuration (`num_kv_blocks`, or `max_cache_tokens` in blocks) is what a
+    full group gets; a group that never holds that much gets its own worst case instead.
+    Otherwise every group gets the worst case of `max_num_seqs` requests, which can never run out
+    (the reference's rule, tiny_llm/runtime/cuda/cuda_runtime.cpp:510-515); if that is more than
+    `cache_memory_fraction` of the device memory that is free once the weights are resident, all
+    groups shrink by one factor (each still serves the same number of longest requests); a smaller
+    pool is what the scheduler's preemption is for."""
     bs = engine.kv_block_size
-    if engine.num_kv_blocks is not None:
-        return max(1, int(engine.num_kv_blocks))
-    if engine.max_cache_tokens is not None:
-        return max(1, -(-engine.max_cache_tokens // bs))
-    blocks = engine.max_num_seqs * (-(-max_len // bs))
-    if free_bytes is not None and bytes_per_block > 0:
-        fit = int(free_bytes * engine.cache_memory_fraction) // bytes_per_block
-        if fit < 1:
-            raise MemoryError(f"no device memory for the cache: one block of {bs} tokens takes "
-                              f"{bytes_per_block} bytes, {free_bytes} bytes are free")
-        blocks = min(blocks, fit)
-    return max(1, blocks)
+    single = not isinstance(bytes_per_block, (list, tuple))
+    per_block = [int(bytes_per_block)] if single else [int(b) for b in bytes_per_block]
+    whole = -(-max_len // bs)
+    held = [whole] * len(per_block) if held_at_most is None else [max(1, int(h)) for h in held_at_most]
+    worst = [engine.max_num_seqs * h for h in held]
+    if engine.num_kv_blocks is not None or engine.max_cache_tokens is not None:
+        given = int(engine.num_kv_blocks) if engine.num_kv_blocks is not None else -(-engine.max_cache_tokens // bs)
+        blocks = [max(1, given if h >= whole else min(given, w)) for h, w in zip(held, worst)]
+    else:
+        blocks = list(worst)
+        need = sum(n * b for n, b in zip(blocks, per_block))
+        if free_bytes is not None and need > 0:
+            room = int(free_bytes * engine.cache_memory_fraction)
+            if room < sum(per_block):
+                raise MemoryError(f"no device memory for the cache: one block of {bs} tokens per group takes "
+                                  f"{sum(per_block)} bytes, {free_bytes} bytes are free")
+            if need > room:
+                blocks = [max(1, n * room // need) for n in blocks]
+    return blocks[0] if single else blocks
 
 
 def build_runner(dec: Decoder, engine: EngineConfig) -> ModelRunner:
@@ -76,9 +92,11 @@ def build_runner(dec: Decoder, engine: EngineConfig) -> ModelRunner:
     bs = engine.kv_block_size
     cache_specs, state_specs = dec.cache_specs(), dec.state_specs()
     elt = torch.empty((), dtype=dec.dtype).element_size()
-    per_block = CacheManager(cache_specs, state_specs, bs, 1, 1).elements_per_block() * elt
+    probe = CacheManager(cache_specs, state_specs, bs, 1, 1)
+    per_block = [n * elt for n in probe.elements_per_block()]
     free = torch.cuda.mem_get_info(dec.device)[0] if dec.device.type == "cuda" else None
-    blocks = plan_cache_blocks(engine, max_len, per_block, free)
+    held = probe.blocks_held_at_most(max_len, engine.max_num_batched_tokens)
+    blocks = plan_cache_blocks(engine, max_len, per_block, free, held)
     cache = CacheManager(cache_specs, state_specs, bs, blocks, engine.max_num_seqs)
     cache.allocate_tensors(dec.dtype, dec.device)
     return ModelRunner(dec, cache, engine.max_num_batched_tokens, max_len)

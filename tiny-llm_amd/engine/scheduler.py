@@ -18,8 +18,10 @@ Decisions (all host-side, testable without a GPU):
   token budget are left.
 * Budget: at most `max_num_batched_tokens` tokens per step; a prompt portion is
   `min(remaining, budget left, blocks that fit)`.
-* A waiting request is admitted only when the blocks for all its tokens are free
-  (its first portion may still be shorter: the token budget).
+* A waiting request is admitted only when, in every cache group, the blocks it will
+  hold at most are free: all its tokens in a group that keeps every position, its
+  window and one portion in a group that keeps a window (its first portion may still
+  be shorter: the token budget).
 * When pages run out for a running request, the request admitted last among those
   not yet scheduled in the step (possibly the request itself) is preempted: its
   blocks and slot are given back at once and it returns to the FRONT of the waiting
@@ -126,10 +128,10 @@ class Scheduler:
             raise ValueError("a request needs at least one prompt token")
         if len(req.prompt) > self.max_model_len:
             raise ValueError(f"prompt of {len(req.prompt)} tokens exceeds max_model_len {self.max_model_len}")
-        blocks_alone = -(-len(req.prompt) // self.cache.block_size)
-        if blocks_alone > self.cache.num_blocks:
-            raise ValueError(f"prompt of {len(req.prompt)} tokens cannot fit the cache "
-                             f"({self.cache.num_blocks} blocks of {self.cache.block_size})")
+        alone = self.cache.blocks_held_at_most(len(req.prompt), self.budget)
+        if any(n > have for n, have in zip(alone, self.cache.group_blocks)):
+            raise ValueError(f"prompt of {len(req.prompt)} tokens cannot fit the cache: it holds up to {alone} "
+                             f"blocks of {self.cache.block_size}, the pools have {self.cache.group_blocks}")
         req.status = WAITING
         self.waiting.append(req)
 
@@ -225,14 +227,15 @@ class Scheduler:
             scheduled_ids.add(req.req_id)
             budget -= count
 
-        # Admission, in arrival order, while a slot, the blocks for ALL the request's tokens and some
-        # budget are left; none in a step that preempted (the freed blocks are for those that run).
+        # Admission, in arrival order, while a slot, the blocks the request will hold at most (in a
+        # full group: for ALL its tokens) and some budget are left; none in a step that preempted
+        # (the freed blocks are for those that run).
         slots_left = min(self.cache.free_slots, self.max_num_seqs - len(self.running))
         while self.waiting and budget > 0 and slots_left > 0 and not preempted:
             req = self.waiting[0]
-            need_all = self.cache.blocks_needed(req.req_id, req.num_tokens)
+            need_all = self.cache.blocks_held_at_most(req.num_tokens, self.budget)
             if not self._fits(need_all, taken):
-                if any(n > self.cache.num_blocks for n in need_all):
+                if any(n > have for n, have in zip(need_all, self.cache.group_blocks)):
                     self.waiting.popleft()                 # more than the whole pool: it can never run
                     req.status, req.finish_reason = FINISHED, "capacity"
                     self.finished.append(req)
@@ -253,13 +256,16 @@ class Scheduler:
 
     def burst_length(self, plan: StepPlan, most: int) -> int:
         """How many decode steps the plan's requests can run back to back without a decision in
-        between: every entry decodes, nobody waits for admission, and the run ends where the
-        first request reaches its `max_new_tokens` or the model's length, where it would need
-        cache blocks that are not free, or after `most` steps.  (A request that draws an end-of-
+        between: every entry decodes, every running request is in the plan, nobody waits for
+        admission, and the run ends where the
+        first request reaches its `max_new_tokens` or the model's length, where the requests would
+        need cache blocks that are not free, or after `most` steps.  (A request that draws an end-of-
         sequence token inside the run is finished there when the run is over; what it was given
         after that token is dropped.)"""
         if most < 2 or self.waiting or plan.preempted or not plan.entries:
             return 1
+        if len(plan.entries) != len(self.running):
+            return 1            # a running request the plan left out (no budget) would sit idle for the whole run
         k = most
         for e in plan.entries:
             req = e.request
@@ -268,13 +274,17 @@ class Scheduler:
             k = min(k, req.params.max_new_tokens - len(req.output), self.max_model_len - req.num_tokens)
         if k < 2:
             return 1
-        need = [0] * len(self.cache.groups)
-        for e in plan.entries:
-            for g, n in enumerate(self.cache.blocks_needed(e.request.req_id, e.request.num_computed + k)):
-                need[g] += n
-        if any(n > f for n, f in zip(need, self.cache.free_blocks())):
-            return 1
-        return k
+        # the longest run whose blocks are free now, in every group (all of them are taken up front)
+        free = self.cache.free_blocks()
+        while k >= 2:
+            need = [0] * len(free)
+            for e in plan.entries:
+                for g, n in enumerate(self.cache.blocks_needed(e.request.req_id, e.request.num_computed + k)):
+                    need[g] += n
+            if all(n <= f for n, f in zip(need, free)):
+                return k
+            k -= 1
+        return 1
 
     def update_burst(self, plan: StepPlan, tokens_by_step: Sequence[Sequence[int]]) -> List[Request]:
         """After a run of decode steps: what `update` would do with each step's tokens in turn, worked

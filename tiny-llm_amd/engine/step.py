@@ -24,6 +24,7 @@ the sampler; a captured step only has its sizes rounded up and its buffers stati
 from __future__ import annotations
 
 import gc
+from collections import OrderedDict
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
@@ -188,8 +189,28 @@ class _Row:
     tables: List[List[int]]     # per cache group
 
 
+class SeenTables:
+    """What a static step buffer already holds of the requests' block tables: per cache group and
+    request row the table object and the length that were written last.  A table only ever grows
+    between two admissions, except when a step that did not run is undone: the cache manager's
+    `table_epoch` goes up then, and everything remembered under an older epoch is forgotten (a
+    table cut back and grown again has its old length with other blocks)."""
+
+    def __init__(self, groups: int, rows: int, epoch: int = 0):
+        self.groups, self.rows_per_group = groups, rows
+        self.epoch = epoch
+        self.rows: List[list] = [[None] * rows for _ in range(groups)]
+
+    def at_epoch(self, epoch: int) -> List[list]:
+        if epoch != self.epoch:
+            self.rows = [[None] * self.rows_per_group for _ in range(self.groups)]
+            self.epoch = epoch
+        return self.rows
+
+
 def fill_metadata(host: np.ndarray, lay: Layout, rows: Sequence[_Row], block_size: int,
-                  samples: Optional[Sequence[SampleSpec]] = None, seen: Optional[list] = None) -> None:
+                  samples: Optional[Sequence[SampleSpec]] = None, seen: Optional[SeenTables] = None,
+                  table_epoch: int = 0) -> None:
     """Writes the metadata of a step into `host` (int32, at least lay.total long): the ONE routine
     behind eager steps, captured decode steps and captured mixed steps.
 
@@ -197,8 +218,10 @@ def fill_metadata(host: np.ndarray, lay: Layout, rows: Sequence[_Row], block_siz
     padding tokens are token 0 at position 0 of request row 0 with cache slot -1 (nothing is
     stored); padding requests have no tokens (cu_seqlens stays at T); padding query tiles hold no
     token; padding output rows point at row 0 and are dropped by the caller.
-    `seen` (per group, per request row): block-table rows a static buffer already holds."""
+    `seen`: the block-table rows a static buffer already holds, valid for the cache manager's
+    `table_epoch` under which they were written."""
     T_cap, R_cap, G, MB, bs = lay.T, lay.R, lay.G, lay.MB, block_size
+    seen = seen.at_epoch(table_epoch) if seen is not None else None
     R = len(rows)
     tok, pos, rot = lay.sec(host, "tokens"), lay.sec(host, "positions"), lay.sec(host, "req_of_token")
     cu, sl, ss, lr = (lay.sec(host, n) for n in ("cu_seqlens", "seq_lens", "state_slots", "logit_rows"))
@@ -227,9 +250,9 @@ def fill_metadata(host: np.ndarray, lay: Layout, rows: Sequence[_Row], block_siz
                 raise StepError(f"request {row.req_id!r} holds {len(table)} blocks, the table has room for {MB}")
             last = seen[g][r] if seen is not None else None
             # a row is rewritten only when it belongs to another admission than last time (the table
-            # object is made when a request is admitted) or has changed length; blocks that a window
-            # has released turn into -1 without a change of length, but they lie before the window
-            # and are never read
+            # object is made when a request is admitted) or has changed length (within one epoch a
+            # table only grows); blocks that a window has released turn into -1 without a change of
+            # length, but they lie before the window and are never read
             if last is None or last[0] is not table or last[1] != len(table):
                 bts[g][r, :len(table)] = np.maximum(np.asarray(table, dtype=np.int32), 0)
                 if seen is not None:
@@ -300,6 +323,12 @@ def power_of_two_at_least(n: int) -> int:
 class ModelRunner:
     """Owns the decoder's cache views and turns step entries into one forward pass."""
 
+    # Shapes of step whose static buffers and graphs are kept.  A serving run meets a few dozen
+    # (batch sizes while requests end one after the other, portions, bounds on the context); each
+    # holds a pinned and a device copy of its metadata and up to two graphs.  The shape used
+    # longest ago goes when a new one would exceed the number.
+    MAX_STEP_SHAPES = 64
+
     def __init__(self, decoder, cache: CacheManager, max_num_batched_tokens: int, max_model_len: int):
         self.decoder = decoder
         self.cache = cache
@@ -315,7 +344,8 @@ class ModelRunner:
         self.workspace = ops.Workspace(self.device, self.max_tokens)
         self._pinned: Optional[torch.Tensor] = None
         self._uploaded: Optional[torch.cuda.Event] = None
-        self._graphs: Dict[tuple, "StepGraph"] = {}
+        # captured steps by shape, least recently used first; at most MAX_STEP_SHAPES are kept
+        self._graphs: "OrderedDict[tuple, StepGraph]" = OrderedDict()
         self._graph_pool = None
         self._tile_widths: set = set()          # query-tile widths the model's kernels have asked for
         self.last_logits: Optional[torch.Tensor] = None     # of the last `run` (tests look at it)
@@ -469,7 +499,7 @@ class ModelRunner:
         new_max = max((cm.num_tokens(e.req_id) if cm.has(e.req_id) else 0) for e in entries) + steps
         R = len(entries)
         bound = min(max(512, power_of_two_at_least(new_max)), max(self.max_model_len, 1))
-        sg = self._graphs.get(("decode", R, bound, True))
+        sg = self._step_graph(("decode", R, bound, True))
         if sg is None or sg.graph is None or new_max > bound or steps > sg.history_steps:
             return None
         rows, _ = self._resolve(entries, reserve=steps)
@@ -508,15 +538,23 @@ class ModelRunner:
                 bound = max(min(max(512, power_of_two_at_least(max(new_lens))), max(self.max_model_len, 1)), max(new_lens))
                 key = ("mixed", T_cap, R_cap, n_cap, bound, samples is not None)
                 caps = (T_cap, R_cap, n_cap, T_cap, bound)
-            sg = self._graphs.get(key)
+            sg = self._step_graph(key)
             if sg is None:
                 sg = self._graphs[key] = StepGraph(self, *caps, sampling=samples is not None)
+                while len(self._graphs) > self.MAX_STEP_SHAPES:
+                    self._graphs.popitem(last=False)        # no capture is under way here: it may be released
             logits, toks = sg.run(rows, samples, n_out)
         except BaseException:
             self.cache.undo_reservation()
             raise
         self._commit(rows)
         return logits, toks
+
+    def _step_graph(self, key) -> Optional["StepGraph"]:
+        sg = self._graphs.get(key)
+        if sg is not None:
+            self._graphs.move_to_end(key)
+        return sg
 
     def finish(self, req_id) -> None:
         """The request is done: its blocks and its state slot are given back."""
@@ -565,7 +603,7 @@ class StepGraph:
         # decode with a wanted row per request: row i of the logits is token i (padding rows, which would
         # point at row 0, are dropped by the caller either way), so the head needs no gather of rows
         self.ctx.logits_all_rows = self.max_q_len == 1 and self.n_out == self.R == self.T
-        self.seen = [[None] * self.R for _ in range(G)]
+        self.seen = SeenTables(G, self.R, cm.table_epoch)
         self.out = torch.zeros(max(self.n_out, 1), dtype=torch.int32, device=runner.device)
         self.out_host = torch.zeros(max(self.n_out, 1), dtype=torch.int32, pin_memory=True)
         # a decode step with its sampler ends by preparing the next one on the device (bursts)
@@ -597,7 +635,8 @@ class StepGraph:
         runner = self.runner
         if self._uploaded is not None:
             self._uploaded.synchronize()
-        fill_metadata(self.np, self.layout, rows, runner.cache.block_size, samples, self.seen)
+        fill_metadata(self.np, self.layout, rows, runner.cache.block_size, samples, self.seen,
+                      runner.cache.table_epoch)
         self.dev.copy_(self.host, non_blocking=True)
         left = steps
         if self.chain is not None:
@@ -623,7 +662,8 @@ class StepGraph:
             self._build()                       # a kernel asked for a tile width this layout lacks
         if self._uploaded is not None:
             self._uploaded.synchronize()        # the last upload has left the pinned buffer
-        fill_metadata(self.np, self.layout, rows, runner.cache.block_size, samples, self.seen)
+        fill_metadata(self.np, self.layout, rows, runner.cache.block_size, samples, self.seen,
+                      runner.cache.table_epoch)
         self.dev.copy_(self.host, non_blocking=True)
         self._uploaded = torch.cuda.Event()
         self._uploaded.record()

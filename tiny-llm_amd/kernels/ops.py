@@ -123,6 +123,10 @@ class Workspace:
             cap = n
             if len(shape) == 2 and shape[0] <= self.max_rows:
                 cap = self.max_rows * shape[1]
+            elif buf is not None:
+                # sizes that depend on the batch and on how a context is split creep up in a
+                # serving run: at least double, so that few retired buffers stay behind
+                cap = max(n, 2 * buf.numel())
             buf = self._bufs[key] = torch.empty(cap, dtype=dtype, device=self.device)
         return buf[:n].view(shape)
 
@@ -222,10 +226,10 @@ def linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, residual: Option
     """out = a @ w.T (+ residual).  a [M, K], w [N, K] share an element type; out [M, N] is that
     type or float32; residual float32 with out's strides.  epilogue="swiglu": the N columns are
     interleaved (gate_j, up_j) pairs and out [M, N/2] = silu(gate) * up, computed from the float32
-    accumulators.  row_scale [M] multiplies the rows of the product first (bfloat16 only).
+    accumulators.  row_scale [M] (float32) multiplies the rows of the product first.
     tile: 0 lets the sizes choose the tile of the bfloat16 product for more than 64 rows; 1 to 4
     force 256x256, 256x128, 128x128, 64x128 (tests and tuning)."""
-    _dev(a, w, out, residual)
+    _dev(a, w, out, residual, row_scale)
     _rows_2d(a, "linear input")
     _rows_2d(out, "linear output")
     M, K = a.shape
@@ -254,9 +258,8 @@ def linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, residual: Option
     al = 16 if dt == 1 else 4      # the bfloat16 kernel moves 16-byte vectors
     ao = 16 if (dt == 1 and not swiglu and M > 64) else 4
     if row_scale is not None:
-        if not (dt == 1 and row_scale.dtype == torch.float32 and row_scale.is_contiguous()
-                and row_scale.numel() == M):
-            _fail("row scales go with the bfloat16 product: float32, one per row")
+        if not (row_scale.dtype == torch.float32 and row_scale.is_contiguous() and row_scale.numel() == M):
+            _fail("row scales are float32, one per row")
     if not (0 <= tile <= 4):
         _fail("tile is 0 (by size) or 1 to 4")
     if dt == 1 and tile == 0 and M > 16:
@@ -370,6 +373,28 @@ def linear_norm_f32(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: t
                                      _ptr(residual), c_int(M), c_int(N), c_int(K), c_int64(x.stride(0)),
                                      c_int64(out.stride(0)), c_int(swiglu), _stream()), "linear_norm_f32")
     return out
+
+
+def norm_prescale_f32(x: torch.Tensor, norm_weight: torch.Tensor, eps: float,
+                      rows: Optional[torch.Tensor] = None):
+    """(h, inv_rms) for float32 x: h = norm_weight * x[rows or all] and the rows' factors 1 / rms, so that
+    linear(h, w, out, row_scale=inv_rms) is rmsnorm(x) @ w.T with the very bits of `linear_norm_f32`
+    (one order of addition for the squares in both): a row's result does not depend on the number of
+    rows in its step, which decides between the two routes."""
+    _dev(x, norm_weight, rows)
+    if not (x.dtype == torch.float32 and norm_weight.dtype == torch.float32 and x.dim() == 2 and x.stride(1) == 1):
+        _fail("norm input and weight must be float32, the input [T, K] with contiguous rows")
+    K = x.shape[1]
+    M = x.shape[0] if rows is None else rows.numel()
+    if not (norm_weight.is_contiguous() and norm_weight.numel() == K):
+        _fail(f"norm weight must have {K} elements")
+    if rows is not None and not (rows.dtype == torch.int32 and rows.is_contiguous()):
+        _fail("row index must be contiguous int32")
+    h = scratch("norm_operand_f32", (M, K), torch.float32, x.device)
+    inv_rms = scratch("norm_row_factor", (M,), torch.float32, x.device)
+    _check(_lib().tl_norm_prescale_f32(_ptr(x), _ptr(norm_weight), _ptr(rows), _ptr(h), _ptr(inv_rms), c_int(M),
+                                       c_int(K), c_int64(x.stride(0)), c_float(eps), _stream()), "norm_prescale_f32")
+    return h, inv_rms
 
 
 FEW_ROWS = 64   # most rows the few-row product takes
@@ -530,9 +555,13 @@ def add_residual(x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
 def rope_store(qkv: torch.Tensor, positions: torch.Tensor, cos: Optional[torch.Tensor],
                sin: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor],
                k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
-               num_heads: int, num_kv_heads: int, head_dim: int, rotary_dim: int) -> None:
+               num_heads: int, num_kv_heads: int, head_dim: int, rotary_dim: int, pairing: str = "half") -> None:
     """Rotate q and k of every row of qkv in place by the row's position and
-    store k, v at the row's cache slot.  Caches: [blocks, kv_heads, block, head_dim]."""
+    store k, v at the row's cache slot.  Caches: [blocks, kv_heads, block, head_dim].
+    pairing: which dims of a head make the i-th rotated pair: "half" (i, i + rotary_dim / 2) or
+    "interleaved" (2i, 2i + 1)."""
+    if pairing not in ROPE_PAIRINGS:
+        _fail(f"rotary pairing {pairing!r} is not built; known: {', '.join(ROPE_PAIRINGS)}")
     _dev(qkv, positions, cos, sin, slot_mapping, k_cache, v_cache)
     _rows_2d(qkv, "qkv")
     T = qkv.shape[0]
@@ -560,7 +589,10 @@ def rope_store(qkv: torch.Tensor, positions: torch.Tensor, cos: Optional[torch.T
     _check(_lib().tl_rope_store(_ptr(qkv), _ptr(positions), _ptr(cos), _ptr(sin), _ptr(slot_mapping),
                                 _ptr(k_cache), _ptr(v_cache), c_int(T), c_int(num_heads), c_int(num_kv_heads),
                                 c_int(head_dim), c_int(rotary_dim), c_int(block_size), c_int64(qkv.stride(0)),
-                                c_int(_dt(qkv)), _stream()), "rope_store")
+                                c_int(_dt(qkv)), c_int(ROPE_PAIRINGS.index(pairing)), _stream()), "rope_store")
+
+
+ROPE_PAIRINGS = ("half", "interleaved")     # the rotation kernel's pairings, by the number it takes
 
 
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,

@@ -80,16 +80,18 @@ class Attention(Mixer):
             ops.linear(h, self.w_qkv, qkv)
         tables = self.position.rotary_tables()
         cos, sin, rot = tables if tables is not None else (None, None, 0)
+        pairing = getattr(self.position, "pairing", "half")     # an encoding that says nothing pairs (i, i + rot/2)
         attn = ops.scratch("attention_out", (T, self.q_size), self.dtype, residual.device)
         q = qkv[:, :self.q_size]
         flash = ops.flash_attention_supported(self.dtype, self.num_heads, self.num_kv_heads, self.head_dim)
         group = self.num_heads // self.num_kv_heads
         # decode steps: rotation and cache write ride in the attention kernel
-        fuse = flash and ctx.max_q_len == 1 and cache.write and rot == self.head_dim
+        fuse = flash and ctx.max_q_len == 1 and cache.write and rot == self.head_dim and pairing == "half"
         if not fuse:
             slots = ctx.slot_mappings[cache.group] if cache.write else None
             ops.rope_store(qkv, ctx.positions, cos, sin, slots, cache.k if cache.write else None,
-                           cache.v if cache.write else None, self.num_heads, self.num_kv_heads, self.head_dim, rot)
+                           cache.v if cache.write else None, self.num_heads, self.num_kv_heads, self.head_dim, rot,
+                           pairing)
         if flash and ctx.max_q_len > 1:
             # prompt portions: many query rows share each staged key tile
             waves = ops.prefill_tile_waves(T, self.num_heads, self.num_kv_heads)

@@ -30,10 +30,14 @@ class LazyNorm:
     def linear(self, w: torch.Tensor, out: torch.Tensor, epilogue: Optional[str] = None) -> torch.Tensor:
         """out = norm(x)[rows] @ w.T (then the epilogue), by the cheapest route there is."""
         if self.x.dtype == torch.float32 and w.dtype == torch.float32:
-            # true float32: the norm inside the few-row product's kernel, or a kernel of its own before it
-            if self.rows is None and ops.linear_norm_f32_ok(self.x.shape[0], w.shape[0], self.x.shape[1], self.x.stride(0)):
+            # true float32: the norm inside the few-row product's kernel (measured on whole steps: up
+            # to 16 rows it saves time), or as two kernels that give the same bits: norm_weight * x
+            # and the rows' factors, then the product with the factor applied to its sums
+            if (self.rows is None and self.x.shape[0] <= RMSNorm.F32_FUSED_ROWS
+                    and ops.linear_norm_f32_ok(self.x.shape[0], w.shape[0], self.x.shape[1], self.x.stride(0))):
                 return ops.linear_norm_f32(self.x, self.weight, self.eps, w, out, epilogue=epilogue)
-            return ops.linear(self.materialize(), w, out, epilogue=epilogue)
+            h, inv_rms = ops.norm_prescale_f32(self.x, self.weight, self.eps, self.rows)
+            return ops.linear(h, w, out, epilogue=epilogue, row_scale=inv_rms)
         if self.prepared is not None and (self.num_rows <= ops.FEW_ROWS or self.rows is None):
             operand, sumsq = self.prepared
             return ops.linear_handoff(operand, w, out, epilogue=epilogue, rows=self.rows,
@@ -67,11 +71,12 @@ class RMSNorm(Norm):
 
     def lazy(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None, prepared=None):
         """The norm rides in the consumer's first product: in bfloat16 always (`ops.linear_norm`), in
-        float32 for at most 16 rows (`ops.linear_norm_f32`; more rows get the norm's own kernel)."""
+        float32 for at most 16 rows (`ops.linear_norm_f32`); more rows, or gathered rows, get the
+        norm as a row factor of the product (`ops.norm_prescale_f32`), which gives the same bits."""
         if self.dtype == torch.bfloat16 and self.hidden_size % 8 == 0:
             return LazyNorm(self, x, rows, prepared)
-        if self.dtype == torch.float32 and rows is None and x.shape[0] <= self.F32_FUSED_ROWS and self.hidden_size % 4 == 0:
-            return LazyNorm(self, x, None, None)
+        if self.dtype == torch.float32 and self.weight.dtype == torch.float32:
+            return LazyNorm(self, x, rows, None)
         return self.forward(x, rows)
 
     def hand_off_buffers(self, n_rows: int, inner: int, device):
