@@ -170,16 +170,27 @@ def norm_operand(x: torch.Tensor, w: torch.Tensor, eps: float, act_dtype):
 
 # ------------------------------------------------------------------------- model
 def llama_forward(w: Dict[str, torch.Tensor], cfg: dict, tokens: Sequence[int],
-                  positions: Optional[Sequence[int]] = None, act_dtype=None, window: int = 0) -> torch.Tensor:
+                  positions: Optional[Sequence[int]] = None, act_dtype=None, window: int = 0,
+                  segments: Optional[Sequence[int]] = None, rows: Optional[Sequence[int]] = None) -> torch.Tensor:
     """Logits [T, vocab] of one request's whole token list
-    (layer order: tiny_llm/parser/llama_parser.cpp:181-271)."""
+    (layer order: tiny_llm/parser/llama_parser.cpp:181-271).
+
+    segments: `tokens` holds several requests one after the other, of these lengths: every part
+    but attention works token by token, and attention runs on each request by itself (positions
+    start at 0 in each).  rows: logits of these token rows only (the reference computes the last
+    row of each request only, tiny_llm/ops/cuda/gemm_q1_helper.cu:99-124)."""
     H = cfg["hidden_size"]
     nq = cfg["num_attention_heads"]
     nkv = cfg.get("num_key_value_heads", nq)
     hd = cfg.get("head_dim") or H // nq
     eps = cfg.get("rms_norm_eps", 1e-6)
     T = len(tokens)
-    positions = list(range(T)) if positions is None else list(positions)
+    segments = [T] if segments is None else list(segments)
+    assert sum(segments) == T
+    if positions is None:
+        positions = [p for n in segments for p in range(n)]
+    positions = list(positions)
+    starts = [sum(segments[:i]) for i in range(len(segments))]
     cos, sin = rope_table_fast(max(positions) + 1, hd, cfg.get("rope_theta", 10000.0))
     x = embedding(tokens, w["model.embed_tokens.weight"])
     for i in range(cfg["num_hidden_layers"]):
@@ -191,11 +202,15 @@ def llama_forward(w: Dict[str, torch.Tensor], cfg: dict, tokens: Sequence[int],
         v = _rnd(sc(linear(h, w[f"{p}.self_attn.v_proj.weight"])), act_dtype).view(T, nkv, hd)
         q = _rnd(apply_rope(q, positions, cos, sin), act_dtype)
         k = _rnd(apply_rope(k, positions, cos, sin), act_dtype)
-        o = _rnd(attention_fast(q, k, v, positions, window), act_dtype).reshape(T, nq * hd)
+        o = torch.cat([attention_fast(q[a:a + n], k[a:a + n], v[a:a + n], positions[a:a + n], window)
+                       for a, n in zip(starts, segments)])
+        o = _rnd(o, act_dtype).reshape(T, nq * hd)
         x = x + linear(o, w[f"{p}.self_attn.o_proj.weight"])
         h2, rs2 = norm_operand(x, w[f"{p}.post_attention_layernorm.weight"], eps, act_dtype)
         x = x + swiglu(h2, w[f"{p}.mlp.gate_proj.weight"], w[f"{p}.mlp.up_proj.weight"],
                        w[f"{p}.mlp.down_proj.weight"], act_dtype, rs2)
+    if rows is not None:
+        x = x[list(rows)]
     xn, rsn = norm_operand(x, w["model.norm.weight"], eps, act_dtype)
     head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", False) else w["lm_head.weight"]
     logits = linear(xn, head)

@@ -292,6 +292,14 @@ def test_model_invariants():
     out = plain.greedy_generate(w, TINY_B, toks[:5], 3)
     assert out[0] == int(plain.llama_forward(w, TINY_B, toks[:5])[-1].argmax())
     assert out[1] == int(plain.llama_forward(w, TINY_B, toks[:5] + out[:1])[-1].argmax())
+    # several requests in one call (what tests of large shapes use to stream the weights once) are
+    # the requests one by one; `rows` picks rows of the result
+    a, b, c = toks[:9], toks[9:10], toks[10:]
+    both = plain.llama_forward(w, TINY_B, a + b + c, segments=[9, 1, 14], act_dtype=torch.bfloat16)
+    for got, one in ((both[:9], a), (both[9:10], b), (both[10:], c)):
+        assert torch.equal(got, plain.llama_forward(w, TINY_B, one, act_dtype=torch.bfloat16))
+    picked = plain.llama_forward(w, TINY_B, a + b + c, segments=[9, 1, 14], rows=[8, 9, 23, 0])
+    assert torch.allclose(picked, plain.llama_forward(w, TINY_B, a + b + c, segments=[9, 1, 14])[[8, 9, 23, 0]], atol=1e-12)
 
 
 # ------------------------------------------------------------------- sampling

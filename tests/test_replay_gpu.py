@@ -22,7 +22,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 # the serving path stores bfloat16, so what is left is the order of float32 sums flipping roundings.
 TOL = {"float32": 1e-4, "bfloat16": 2e-2}
 
-LENGTHS = {"A": [70, 133, 33, 200, 97, 64], "B": [1, 9, 40, 100, 150, 57], "C": [40, 130, 75, 200, 64, 9]}
+LENGTHS = {"A": [70, 133, 33, 200, 97, 64], "B": [1, 9, 40, 100, 150, 57], "C": [40, 130, 75, 200, 64, 9],
+           "D": [24, 121, 48, 190, 5, 73]}
 
 
 def requests_for(name, cfg):
@@ -93,7 +94,7 @@ def r64(n):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_whole_tail_portions(name, dtype, tmp_path_factory):
     folder, reqs, ref, eng = material(name, dtype, tmp_path_factory)
     biggest = max(r64(len(t)) for t in reqs.values())
@@ -107,7 +108,7 @@ def test_whole_tail_portions(name, dtype, tmp_path_factory):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_mixed_with_page_reuse(name, dtype, tmp_path_factory):
     folder, reqs, ref, eng = material(name, dtype, tmp_path_factory)
     for seed in (0, 1):
@@ -122,7 +123,7 @@ def test_mixed_with_page_reuse(name, dtype, tmp_path_factory):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_cuttings_as_captured_steps(name, dtype, tmp_path_factory):
     """The same traces with every step run as a HIP graph of its shape (sizes rounded up, padding
     tokens, tiles and rows): twice over on one runner, so that the second pass replays what the

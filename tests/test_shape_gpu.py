@@ -165,3 +165,115 @@ def test_decoding_many_requests_at_the_real_layer_sizes(dtype, n_requests):
                      use_graphs=True)
     sharpen(chained.decoder)
     assert chained.generate(prompts, SamplingParams.greedy(new, ignore_eos=True)) == out
+
+
+# ------------------------------------------------- the larger shapes the measurements run
+# Two layers at the layer sizes of Llama-3-8B and Llama-2-13B: the products and the attention take
+# other kernels there than at TinyLlama's sizes (inner sizes beyond 4096, heads of 128 with four and
+# with one query head per kv head, a vocabulary of 128256).  The weights are made on the device by
+# name (the same bits as on the host, see above) and copied to the host for the plain model.
+LARGE = {
+    "llama3_8b": {
+        "architectures": ["LlamaForCausalLM"], "model_type": "llama", "num_hidden_layers": 2, "hidden_size": 4096,
+        "num_attention_heads": 32, "num_key_value_heads": 8, "intermediate_size": 14336, "vocab_size": 128256,
+        "rope_theta": 500000.0, "rms_norm_eps": 1e-5, "max_position_embeddings": 8192, "tie_word_embeddings": False,
+        "hidden_act": "silu", "attention_bias": False, "rope_scaling": None, "initializer_range": 0.02},
+    "llama2_13b": {
+        "architectures": ["LlamaForCausalLM"], "model_type": "llama", "num_hidden_layers": 2, "hidden_size": 5120,
+        "num_attention_heads": 40, "num_key_value_heads": 40, "intermediate_size": 13824, "vocab_size": 32000,
+        "rope_theta": 10000.0, "rms_norm_eps": 1e-5, "max_position_embeddings": 4096, "tie_word_embeddings": False,
+        "hidden_act": "silu", "attention_bias": False, "rope_scaling": None, "initializer_range": 0.02},
+}
+_large = {}
+
+
+def large_weights(name):
+    """float32 weights by checkpoint name, on the host (q and k sharpened); made once per shape."""
+    if _large.get("name") != name:
+        from tiny_llm_amd.config import resolve
+        from tiny_llm_amd.models.decoder import Decoder
+        from tiny_llm_amd.weights.loader import random_tensor
+        _large.clear()
+        _, spec = resolve(LARGE[name])
+        w = {}
+        for s in Decoder(spec, "float32", "cpu").weight_specs():
+            t = random_tensor(s, SEED, STD, 0.0, device="cuda:0").cpu()
+            if s.name.endswith(("q_proj.weight", "k_proj.weight")):
+                t = t * SHARPEN
+            w[s.name] = t
+        _large.update(name=name, weights=w)
+    return _large["weights"]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["llama3_8b", "llama2_13b"])
+def test_the_larger_layer_sizes(name, dtype):
+    """A prompt of 520 tokens whole and in portions of 512 + 8, forty short requests whose prompts
+    run as one step, then decode steps of 40, 16 and 1 rows (eagerly, captured and replayed): every
+    wanted row against the plain implementation."""
+    from tiny_llm_amd.config import EngineConfig
+    from tiny_llm_amd.engine.loading import build_runner, random_model
+    from tiny_llm_amd.engine.step import StepEntry
+    cfg = LARGE[name]
+    V = cfg["vocab_size"]
+    act = torch.bfloat16 if dtype == "bfloat16" else None
+    w = large_weights(name)
+    if act is not None:
+        w = {k: (t.to(act).float() if t.dim() >= 2 else t) for k, t in w.items()}
+    long = random_tokens(520, V, 77)
+    n_short, n_decode = 40, 9
+    prompt_len = [6 + (5 * i) % 11 for i in range(n_short)]
+    short = [random_tokens(prompt_len[i] + n_decode, V, 500 + i) for i in range(n_short)]
+    long_rows = [0, 1, 63, 64, 255, 511, 512, 513, 514, 515, 516, 517, 518, 519]
+    # one pass of the plain model over all requests: the weights stream once
+    segments = [520] + [len(s) for s in short]
+    starts = [sum(segments[:i]) for i in range(len(segments))]
+    wanted = [(0, p) for p in long_rows] + [(1 + i, p) for i in range(n_short) for p in range(prompt_len[i] - 1, len(short[i]))]
+    ref_rows = plain.llama_forward(w, cfg, long + [t for s in short for t in s], act_dtype=act, segments=segments,
+                                   rows=[starts[s] + p for s, p in wanted])
+    ref = {sp: ref_rows[i] for i, sp in enumerate(wanted)}
+    del ref_rows, w
+
+    engine = EngineConfig(dtype=dtype, kv_block_size=16, max_cache_tokens=n_short * 64 + 576, max_num_seqs=n_short + 1,
+                          max_num_batched_tokens=1024, use_graphs=True)
+    _, dec = random_model(cfg, engine, seed=SEED, std=STD)
+    sharpen(dec)
+    runner = build_runner(dec, engine)
+    for g in runner.cache.groups:
+        for t in g.tensors.values():
+            t.fill_(float("nan"))
+    worst = 0.0
+
+    def compare(got, where, what):
+        nonlocal worst
+        got = got.cpu()
+        assert got.shape[0] == len(where)
+        for i, sp in enumerate(where):
+            assert torch.isfinite(got[i]).all(), (what, sp)
+            e = rel_err(got[i], ref[sp])
+            worst = max(worst, e)
+            assert e < TOL[dtype], f"{name} {dtype} {what}: request {sp[0]} position {sp[1]}: rel err {e:.3e}"
+
+    compare(runner.step([StepEntry("long", long, long_rows)]), [(0, p) for p in long_rows], "whole")
+    runner.finish("long")
+    for graph in (False, True, True):
+        compare(runner.step([StepEntry("long", long[:512], [0, 1, 63, 64, 255, 511])], use_graph=graph),
+                [(0, p) for p in (0, 1, 63, 64, 255, 511)], "portion of 512")
+        compare(runner.step([StepEntry("long", long[512:], list(range(8)))], use_graph=graph),
+                [(0, p) for p in range(512, 520)], "the last 8 tokens")
+        runner.finish("long")
+    compare(runner.step([StepEntry(i, short[i][:prompt_len[i]], [prompt_len[i] - 1]) for i in range(n_short)], use_graph=True),
+            [(1 + i, prompt_len[i] - 1) for i in range(n_short)], "forty prompts")
+    at = 0
+    for live in (40, 16, 1):
+        for i in range(live, n_short):
+            runner.finish(i)
+        for _ in range(3):          # eagerly on the static buffers, captured, replayed
+            ents = [StepEntry(i, [short[i][prompt_len[i] + at]], [0]) for i in range(live)]
+            compare(runner.step(ents, use_graph=True), [(1 + i, prompt_len[i] + at) for i in range(live)],
+                    f"decode step of {live} rows")
+            at += 1
+    assert at == n_decode
+    assert sorted(k[1] for k, g in runner._graphs.items() if k[0] == "decode" and g.graph is not None) == [1, 16, 40]
+    print(f"{name} layer sizes (2 layers) {dtype}: worst rel err {worst:.2e}", flush=True)
+    runner.cache.audit()

@@ -36,15 +36,28 @@ TINY_C = {
     "hidden_act": "silu", "attention_bias": False, "rope_scaling": None, "initializer_range": 0.03,
     "eos_token_id": 3, "torch_dtype": "float32",
 }
+# A fourth whose heads are no multiple of 16 wide (the general attention kernel) and do not add up to
+# the hidden size; pages of four tokens.
+TINY_D = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "num_hidden_layers": 2, "hidden_size": 136, "num_attention_heads": 6, "num_key_value_heads": 2,
+    "head_dim": 40, "intermediate_size": 232, "vocab_size": 409, "rope_theta": 7000.0,
+    "rms_norm_eps": 3e-6, "max_position_embeddings": 384, "tie_word_embeddings": False,
+    "hidden_act": "silu", "attention_bias": False, "rope_scaling": None, "initializer_range": 0.04,
+    "eos_token_id": 7, "torch_dtype": "float32",
+}
 # engine-side options that go with them
 ENGINE_A = {"kv_block_size": 16}
 ENGINE_B = {"kv_block_size": 8}
 ENGINE_C = {"kv_block_size": 32}
+ENGINE_D = {"kv_block_size": 4}
 INIT_A = {"std": 0.02, "norm_std": 0.0}
 INIT_B = {"std": 0.05, "norm_std": 0.1}
 INIT_C = {"std": 0.03, "norm_std": 0.05}
+INIT_D = {"std": 0.04, "norm_std": 0.2}
 
-CONFIGS = {"A": (TINY_A, ENGINE_A, INIT_A), "B": (TINY_B, ENGINE_B, INIT_B), "C": (TINY_C, ENGINE_C, INIT_C)}
+CONFIGS = {"A": (TINY_A, ENGINE_A, INIT_A), "B": (TINY_B, ENGINE_B, INIT_B), "C": (TINY_C, ENGINE_C, INIT_C),
+           "D": (TINY_D, ENGINE_D, INIT_D)}
 
 
 def make_folder(tmp_path, cfg, seed=0, std=0.02, norm_std=0.0, dtype="float32", sharpen=4.0):
