@@ -101,7 +101,9 @@ def test_contexts_of_thousands_of_tokens(name, dtype, tmp_path_factory, monkeypa
     calls = Calls(monkeypatch)
     runner = make_runner(folder, dtype, block_size, budget=LONG)
     assert runner.workspace.max_rows == ops.Workspace.FIRST_ROWS < LONG
-    # 1. a whole prompt of more rows than the workspace was first made for
+    # 1. a whole prompt of more rows than the workspace was first made for (by a small step)
+    runner.step([StepEntry("first", reqs["short"][:SHORT], [])])
+    runner.finish("first")
     some = sorted(set(list(range(0, LONG, 61)) + list(range(LONG - 40, LONG)) + [4095, 4096, 4097]))
     long = reqs["long"]
     w1 = compare(runner.step([StepEntry("long", long, some)]), ref["long"], some, tol, "whole prompt")
