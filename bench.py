@@ -187,6 +187,20 @@ class Bench:
         return dt, steps, sum(eng.requests[i].preemptions for i in ids)
 
 
+def decode_rooflines(cfg, dtype, batch, seconds, ctx_tokens):
+    """A decode step against both of its bounds: the bytes it has to read (every weight once, the cache of
+    the live requests) over the published memory bandwidth, and its flops (two per weight and row, and the
+    attention over the cached keys) over the published matrix peak of its element type.  `bound` names the
+    one that allows less (float32 at batch 64 is bound by the float32 matrix peak, not by memory)."""
+    matmul_params, weight_bytes, kv_per_tok, (L, H, I, V, nq, nkv, hd) = model_numbers(cfg, ELT[dtype])
+    nbytes = weight_bytes + ctx_tokens * kv_per_tok
+    flops = 2.0 * batch * (matmul_params + V * H) + 4.0 * L * nq * hd * ctx_tokens
+    t_mem, t_flop = nbytes / (HBM_GBS * 1e9), flops / (PEAK_TFLOPS[dtype] * 1e12)
+    return {"ms": round(seconds * 1e3, 4), "bound": "hbm" if t_mem >= t_flop else f"{dtype} matrix peak",
+            "hbm_frac": round(t_mem / seconds, 4), "flops_frac": round(t_flop / seconds, 4),
+            "GBs": round(nbytes / seconds / 1e9, 1), "TFLOPs": round(flops / seconds / 1e12, 2)}
+
+
 def tinyllama_figures(args, dtype, peaks):
     """Decode at batch 8 / 1 / 64 and the 2,048-token prefill at the TinyLlama shape in `dtype`."""
     elt = ELT[dtype]
@@ -220,16 +234,18 @@ def tinyllama_figures(args, dtype, peaks):
         out["points"] = {}
         if args.only in ("all", "headline", "fp32"):
             for n in (1, 64):
-                d, _ = b.decode(n, steps, warmup, prompt_len=args.prompt_len)
+                d, ctx_n = b.decode(n, steps, warmup, prompt_len=args.prompt_len)
                 out["points"][f"decode_b{n}"] = round(n * steps / d, 1)
+                out[f"roofline_b{n}"] = decode_rooflines(cfg, dtype, n, d / steps, ctx_n)
     out["sizes"] = (L, H, I, V, nq, nkv, hd)
     out["steps"], out["warmup"] = steps, warmup
     b.close()
     return out
 
 
-def soak_llama3_8b(args):
-    """16 requests, seeded prompt lengths 128..4096, prompts in portions of 512, 128 tokens each."""
+def soak_llama3_8b(args, dtype="bf16"):
+    """16 requests, seeded prompt lengths 128..4096, prompts in portions of 512, 128 tokens each.
+    bfloat16: three passes, the third counts; float32 (the checking path): one pass."""
     import random
     cfg = dict(LLAMA3_8B)
     layers_full = cfg["num_hidden_layers"]
@@ -238,20 +254,23 @@ def soak_llama3_8b(args):
     rng = random.Random(8)
     lens = [rng.randint(128, 4096) for _ in range(16)]
     new = 128
-    b = Bench(cfg, "bf16", 16, new, 16, budget=512, max_cache_tokens=sum(-(-(n + new) // 16) * 16 for n in lens) + 1024)
+    b = Bench(cfg, dtype, 16, new, 16, budget=512, max_cache_tokens=sum(-(-(n + new) // 16) * 16 for n in lens) + 1024)
     b.soak(lens[:2], 4, 512)                                  # warm-up: kernels configure themselves
     # The workload three times over: the first pass meets every shape of step for the first time (a
     # shape's first step runs eagerly, its second is captured as a graph), the third replays graphs
     # only and is the one that counts; the first is reported beside it.
-    cold, _, _ = b.soak(lens, new, 512)
-    b.soak(lens, new, 512)
-    dt, steps, pre = b.soak(lens, new, 512)
+    cold, steps, pre = b.soak(lens, new, 512)
+    dt, passes = cold, 1
+    if dtype == "bf16":
+        b.soak(lens, new, 512)
+        dt, steps, pre = b.soak(lens, new, 512)
+        passes = 3
     b.close()
     total = sum(lens) + 16 * new
-    return {"model": "Llama-3-8B shape", "dtype": "bf16", "layers": cfg["num_hidden_layers"], "layers_full": layers_full,
+    return {"model": "Llama-3-8B shape", "dtype": dtype, "layers": cfg["num_hidden_layers"], "layers_full": layers_full,
             "requests": 16, "prompt_tokens": sum(lens), "decode_tokens": 16 * new, "chunk": 512, "steps": steps,
             "seconds": round(dt, 3), "tokens_per_s": round(total / dt, 1), "decode_tokens_per_s": round(16 * new / dt, 1),
-            "preemptions": pre, "pass": 3, "first_pass_seconds": round(cold, 3)}
+            "preemptions": pre, "pass": passes, "first_pass_seconds": round(cold, 3)}
 
 
 def prefill_llama3_8b(args):
@@ -270,25 +289,29 @@ def prefill_llama3_8b(args):
     return out
 
 
-def soak_llama2_13b(args):
-    """64 requests of 1,024 prompt tokens, 256 greedy tokens each; the cache pool holds them with little to spare."""
+def soak_llama2_13b(args, dtype="bf16"):
+    """64 requests of 1,024 prompt tokens, 256 greedy tokens each; the cache pool holds them with little to spare.
+    bfloat16: three passes, the third counts; float32 (the checking path): one pass."""
     cfg = dict(LLAMA2_13B)
     layers_full = cfg["num_hidden_layers"]
     if args.soak_layers:
         cfg["num_hidden_layers"] = min(layers_full, args.soak_layers)
     n_req, prompt, new = 64, 1024, 256
     pool_tokens = n_req * (prompt + new) + 64 * 16           # one spare page a request
-    b = Bench(cfg, "bf16", n_req, new, 16, budget=2048, max_cache_tokens=pool_tokens)
+    b = Bench(cfg, dtype, n_req, new, 16, budget=2048, max_cache_tokens=pool_tokens)
     b.soak([prompt] * 2, 4, 2048)
-    cold, _, _ = b.soak([prompt] * n_req, new, 2048)          # three passes, as above
-    b.soak([prompt] * n_req, new, 2048)
-    dt, steps, pre = b.soak([prompt] * n_req, new, 2048)
-    _, _, kv_per_tok, _ = model_numbers(cfg, 2)
+    cold, steps, pre = b.soak([prompt] * n_req, new, 2048)    # three passes, as above
+    dt, passes = cold, 1
+    if dtype == "bf16":
+        b.soak([prompt] * n_req, new, 2048)
+        dt, steps, pre = b.soak([prompt] * n_req, new, 2048)
+        passes = 3
+    _, _, kv_per_tok, _ = model_numbers(cfg, ELT[dtype])
     b.close()
-    return {"model": "Llama-2-13B shape", "dtype": "bf16", "layers": cfg["num_hidden_layers"], "layers_full": layers_full,
+    return {"model": "Llama-2-13B shape", "dtype": dtype, "layers": cfg["num_hidden_layers"], "layers_full": layers_full,
             "requests": n_req, "prompt_tokens": n_req * prompt, "decode_tokens": n_req * new, "steps": steps,
             "seconds": round(dt, 3), "tokens_per_s": round(n_req * (prompt + new) / dt, 1),
-            "decode_tokens_per_s": round(n_req * new / dt, 1), "preemptions": pre, "pass": 3,
+            "decode_tokens_per_s": round(n_req * new / dt, 1), "preemptions": pre, "pass": passes,
             "first_pass_seconds": round(cold, 3),
             "cache_pool_GB": round(pool_tokens * kv_per_tok / 1e9, 1), "cache_pool_fill": round(n_req * (prompt + new) / pool_tokens, 3)}
 
@@ -371,7 +394,8 @@ def run(args):
         return
     if args.only in ("llama3_8b", "llama2_13b", "llama3_8b_prefill"):
         fn = {"llama3_8b": soak_llama3_8b, "llama2_13b": soak_llama2_13b, "llama3_8b_prefill": prefill_llama3_8b}[args.only]
-        print(json.dumps({args.only: fn(args)}), flush=True)
+        res = fn(args) if args.only == "llama3_8b_prefill" else fn(args, args.dtype)
+        print(json.dumps({args.only: res}), flush=True)
         return
     main_dtype = "fp32" if args.only == "fp32" else args.dtype
     fig = tinyllama_figures(args, main_dtype, peaks)
@@ -391,6 +415,9 @@ def run(args):
                    "decode_tokens": fig["steps"], "kv_block_size": args.block_size, "parallelism": "single GPU"},
         "prefill": fig.get("prefill"), "roofline": fig["roofline"], "points": fig["points"],
     }
+    for n in (1, 64):
+        if f"roofline_b{n}" in fig:
+            line[f"roofline_b{n}"] = fig[f"roofline_b{n}"]
     if "prefill_chunked_512" in fig:
         line["prefill_chunked_512"] = fig["prefill_chunked_512"]
     if peaks:
@@ -400,9 +427,11 @@ def run(args):
         line["fp32"] = {"decode_b8": round(f32["value"], 1), "ms_per_step_b8": round(f32["ms_per_step"], 4),
                         "decode_b1": f32["points"]["decode_b1"], "decode_b64": f32["points"]["decode_b64"],
                         "steps": f32["steps"], "prefill": f32["prefill"], "prefill_chunked_512": f32["prefill_chunked_512"],
-                        "roofline_b8": f32["roofline"]}
+                        "roofline_b8": f32["roofline"], "roofline_b1": f32["roofline_b1"], "roofline_b64": f32["roofline_b64"]}
         line["workloads"] = {"llama3_8b_mixed16": soak_llama3_8b(args), "llama3_8b_prefill": prefill_llama3_8b(args),
-                             "llama2_13b_64x1024": soak_llama2_13b(args)}
+                             "llama2_13b_64x1024": soak_llama2_13b(args),
+                             "llama3_8b_mixed16_fp32": soak_llama3_8b(args, "fp32"),
+                             "llama2_13b_64x1024_fp32": soak_llama2_13b(args, "fp32")}
     print(json.dumps(line), flush=True)
 
 
