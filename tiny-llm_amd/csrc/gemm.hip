@@ -245,7 +245,7 @@ constexpr int FR_WAVES = 8, FR_THREADS = FR_WAVES * TL_WAVE, FR_MAX_MT = 4;
 // are loaded, their squares are added up on the way (per k block and row in a fixed order, the
 // blocks in ascending order, so a row's factor depends on nothing but the row), and the factor is
 // applied to the block sums' total.  That saves the norm's kernel in front of the product.
-template <bool SWIGLU, int COLS, bool NORM = false>
+template <bool SWIGLU, int COLS, bool NORM = false, bool WIDE = false>
 __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* __restrict__ a,
                                                                    const float* __restrict__ w,
                                                                    float* __restrict__ out,
@@ -253,10 +253,18 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
                                                                    int N, int K, int64_t lda, int64_t ldo,
                                                                    const float* __restrict__ norm_w = nullptr,
                                                                    float eps = 0.f,
-                                                                   const float* __restrict__ row_scale = nullptr) {
+                                                                   const float* __restrict__ row_scale = nullptr,
+                                                                   int tiles_wg = FR_MAX_MT) {
+  // WIDE (more than 16 rows): blockIdx.y picks a group of `tiles_wg` row tiles, so that a product with
+  // few column tiles still gives every compute unit a workgroup with whole matrix tiles (16 columns)
+  // instead of half-used ones (8 columns); the activations of the next row tile are requested before
+  // this one is multiplied, and the registers that takes are those of the next block's weights, which
+  // are requested behind the block's last row tile instead.
+  static_assert(!(NORM && WIDE), "the norm rides in the product of one row tile");
   extern __shared__ float rows_smem[];      // [m tiles][k blocks][16 rows][COLS columns], NORM: + [m tiles][k blocks][16]
   const int nkb = (K + F_KBLOCK - 1) / F_KBLOCK;
-  const int mts = (M + 15) / 16;
+  const int mt0 = WIDE ? blockIdx.y * tiles_wg : 0;                       // first row tile of this workgroup
+  const int mts = WIDE ? min(tiles_wg, (M + 15) / 16 - mt0) : (M + 15) / 16;   // and how many it owns
   const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
   const int l16 = lane % 16, kk = lane / 16;
   const int n0 = blockIdx.x * COLS;
@@ -272,12 +280,23 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
       else dst[g] = load_k4<true>(row, k0 + g * 16 + kk * 4, K);
     }
   };
-  f32x4 wv[16], wnext[16];
+  auto a_row = [&](int mt) { return a + (int64_t)min((mt0 + mt) * 16 + l16, M - 1) * lda; };
+  f32x4 wv[16], wnext[WIDE ? 1 : 16];
   if (wave < nkb) {
     if (wave * F_KBLOCK + F_KBLOCK <= K) load16(std::true_type{}, wv, wrow, wave * F_KBLOCK);
     else load16(std::false_type{}, wv, wrow, wave * F_KBLOCK);
   }
   float* ss_smem = rows_smem + mts * nkb * 16 * COLS;
+  // one row tile of one k block: the block sum of 16 rows x COLS columns goes to LDS
+  auto multiply = [&](f32x4 (&av)[16], int mt, int b) {
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int g = 0; g < 16; ++g)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wv[g][e], av[g][e], acc, 0, 0, 0);
+    // lane (l16, kk): row m = l16, columns 4 kk + r
+    if (kk * 4 < COLS) *(f32x4*)(&rows_smem[((mt * nkb + b) * 16 + l16) * COLS + kk * 4]) = acc;
+  };
   auto block = [&](auto whole, auto next_whole, int b) {
     const int kb = b * F_KBLOCK;
     // (NORM keeps the norm's weights in registers beside the rows instead of the next block's
@@ -288,39 +307,46 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
     // activations; asked for behind the weights they would wait for those as well, and the block
     // ahead would hide nothing.
     f32x4 av[16];
-    load16(whole, av, a + (int64_t)min(l16, M - 1) * lda, kb);
-    if (!NORM && b + FR_WAVES < nkb) load16(next_whole, wnext, wrow, kb + FR_WAVES * F_KBLOCK);
-    for (int mt = 0; mt < mts; ++mt) {
-      if (mt > 0) load16(whole, av, a + (int64_t)min(mt * 16 + l16, M - 1) * lda, kb);
-      if constexpr (NORM) {
-        f32x4 nw[16];
-        load16(whole, nw, norm_w, kb);      // 4 * K bytes, from the caches
-        float ss = 0.f;
-#pragma unroll
-        for (int g = 0; g < 16; ++g)
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            ss = __builtin_fmaf(av[g][e], av[g][e], ss);
-            av[g][e] *= nw[g][e];
-          }
-        // the four lanes of a row (one per k quarter): every lane gets (s0 + s1) + (s2 + s3)
-        ss += __shfl_xor(ss, 16, TL_WAVE);
-        ss += __shfl_xor(ss, 32, TL_WAVE);
-        if (kk == 0) ss_smem[(mt * nkb + b) * 16 + l16] = ss;
+    load16(whole, av, a_row(0), kb);
+    if constexpr (WIDE) {
+      f32x4 av2[16];
+      for (int mt = 0; mt < mts; mt += 2) {
+        if (mt + 1 < mts) load16(whole, av2, a_row(mt + 1), kb);
+        multiply(av, mt, b);
+        if (mt + 1 < mts) {
+          if (mt + 2 < mts) load16(whole, av, a_row(mt + 2), kb);
+          multiply(av2, mt + 1, b);
+        }
       }
-      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int g = 0; g < 16; ++g)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wv[g][e], av[g][e], acc, 0, 0, 0);
-      // lane (l16, kk): row m = l16, columns 4 kk + r
-      if (kk * 4 < COLS) *(f32x4*)(&rows_smem[((mt * nkb + b) * 16 + l16) * COLS + kk * 4]) = acc;
-    }
-    if constexpr (NORM) {
       if (b + FR_WAVES < nkb) load16(next_whole, wv, wrow, kb + FR_WAVES * F_KBLOCK);
     } else {
+      if (!NORM && b + FR_WAVES < nkb) load16(next_whole, wnext, wrow, kb + FR_WAVES * F_KBLOCK);
+      for (int mt = 0; mt < mts; ++mt) {
+        if (mt > 0) load16(whole, av, a_row(mt), kb);
+        if constexpr (NORM) {
+          f32x4 nw[16];
+          load16(whole, nw, norm_w, kb);      // 4 * K bytes, from the caches
+          float ss = 0.f;
 #pragma unroll
-      for (int g = 0; g < 16; ++g) wv[g] = wnext[g];
+          for (int g = 0; g < 16; ++g)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              ss = __builtin_fmaf(av[g][e], av[g][e], ss);
+              av[g][e] *= nw[g][e];
+            }
+          // the four lanes of a row (one per k quarter): every lane gets (s0 + s1) + (s2 + s3)
+          ss += __shfl_xor(ss, 16, TL_WAVE);
+          ss += __shfl_xor(ss, 32, TL_WAVE);
+          if (kk == 0) ss_smem[(mt * nkb + b) * 16 + l16] = ss;
+        }
+        multiply(av, mt, b);
+      }
+      if constexpr (NORM) {
+        if (b + FR_WAVES < nkb) load16(next_whole, wv, wrow, kb + FR_WAVES * F_KBLOCK);
+      } else {
+#pragma unroll
+        for (int g = 0; g < 16; ++g) wv[g] = wnext[g];
+      }
     }
   };
   for (int b = wave; b < nkb; b += FR_WAVES) {
@@ -339,7 +365,7 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
       for (int b = 0; b < nkb; ++b) q += ss_smem[(mt * nkb + b) * 16 + r];
       t *= f32_norm_factor(q, K, eps);
     }
-    const int m = mt * 16 + r, n = n0 + c;
+    const int m = (mt0 + mt) * 16 + r, n = n0 + c;
     if constexpr (!NORM) {
       if (row_scale && m < M) t *= row_scale[m];    // the factor of a norm in front (norm_prescale_f32_kernel)
     }
@@ -1644,28 +1670,45 @@ int tl_linear_tile(const void* a, const void* w, void* out, const float* residua
     const bool vec = K % 4 == 0 && lda % 4 == 0 && ((uintptr_t)a | (uintptr_t)w) % 16 == 0;
     const int nkb = (K + F_KBLOCK - 1) / F_KBLOCK;
     const int mts = (M + 15) / 16;
-    // 8 columns a workgroup where that still is one round of workgroups over the 256 compute units
-    // (a workgroup fills a compute unit: more than 256 of them would run in two rounds)
-    const int cols = (N + 7) / 8 <= 256 ? 8 : 16;
-    const size_t rows_smem = (size_t)mts * nkb * 16 * cols * sizeof(float);
+    // One row tile: 8 columns a workgroup where that still is one round of workgroups over the 256
+    // compute units (a workgroup fills a compute unit: more than 256 of them would run in two rounds).
+    // More row tiles (17 to 64 rows): whole matrix tiles of 16 columns, and the row tiles shared out
+    // over as many groups of workgroups (1, 2 or 4) as it takes to give every compute unit a
+    // workgroup and to fit the block sums into LDS.
+    int cols = (N + 7) / 8 <= 256 ? 8 : 16, groups = 1;
+    if (mts > 1) {
+      cols = 16;
+      const int col_tiles = (N + 15) / 16;
+      // (more groups only while they stay within one round of 256 workgroups: a second, partly filled
+      // round costs as much as a full one)
+      while (groups < mts && (col_tiles * groups * 2 <= 256 || (size_t)((mts + groups - 1) / groups) * nkb * 16 * cols * sizeof(float) > 96 * 1024))
+        groups *= 2;
+    }
+    const int tiles_wg = (mts + groups - 1) / groups;
+    const size_t rows_smem = (size_t)tiles_wg * nkb * 16 * cols * sizeof(float);
     if (M <= 16 * FR_MAX_MT && vec && rows_smem <= 96 * 1024) {
       static bool configured = false;
       if (!configured) {
-        const void* kernels[4] = {(const void*)gemm_f32_rows_kernel<true, 16>, (const void*)gemm_f32_rows_kernel<false, 16>,
-                                  (const void*)gemm_f32_rows_kernel<true, 8>, (const void*)gemm_f32_rows_kernel<false, 8>};
+        const void* kernels[6] = {(const void*)gemm_f32_rows_kernel<true, 16>, (const void*)gemm_f32_rows_kernel<false, 16>,
+                                  (const void*)gemm_f32_rows_kernel<true, 8>, (const void*)gemm_f32_rows_kernel<false, 8>,
+                                  (const void*)gemm_f32_rows_kernel<true, 16, false, true>,
+                                  (const void*)gemm_f32_rows_kernel<false, 16, false, true>};
         for (const void* k : kernels)
           if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024) != hipSuccess)
             return TL_ERR_LAUNCH;
         configured = true;
       }
-      dim3 gr((N + cols - 1) / cols);
-#define TL_F32_ROWS(SW, CO)                                                                                   \
-  hipLaunchKernelGGL((gemm_f32_rows_kernel<SW, CO>), gr, dim3(FR_THREADS), rows_smem, stream, (const float*)a, \
-                     (const float*)w, (float*)out, residual, M, N, K, lda, ldo, (const float*)nullptr, 0.f, row_scale)
-      if (swiglu && cols == 16) TL_F32_ROWS(true, 16);
-      else if (swiglu) TL_F32_ROWS(true, 8);
-      else if (cols == 16) TL_F32_ROWS(false, 16);
-      else TL_F32_ROWS(false, 8);
+      dim3 gr((N + cols - 1) / cols, (mts + tiles_wg - 1) / tiles_wg);
+#define TL_F32_ROWS(SW, CO, WI)                                                                                        \
+  hipLaunchKernelGGL((gemm_f32_rows_kernel<SW, CO, false, WI>), gr, dim3(FR_THREADS), rows_smem, stream, (const float*)a, \
+                     (const float*)w, (float*)out, residual, M, N, K, lda, ldo, (const float*)nullptr, 0.f, row_scale,  \
+                     tiles_wg)
+      if (mts > 1 && swiglu) TL_F32_ROWS(true, 16, true);
+      else if (mts > 1) TL_F32_ROWS(false, 16, true);
+      else if (swiglu && cols == 16) TL_F32_ROWS(true, 16, false);
+      else if (swiglu) TL_F32_ROWS(true, 8, false);
+      else if (cols == 16) TL_F32_ROWS(false, 16, false);
+      else TL_F32_ROWS(false, 8, false);
 #undef TL_F32_ROWS
       return tl_launch_status();
     }
