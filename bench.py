@@ -94,7 +94,34 @@ def measure_peaks():
         flops = ops.peak_mfma(sink, dt, 20000, 2048)
         t = timed(lambda: ops.peak_mfma(sink, dt, 20000, 2048), 3)
         out[f"mfma_{name}_TFLOPs"] = round(flops / t / 1e12, 1)
+    # one all-to-all hand-over of a few floats among 256 resident workgroups inside a launch, and the
+    # time of an empty launch that depends on the one before it in a graph: a decode layer has five
+    # dependent phases, and either way a phase costs microseconds whatever it computes
+    out["handover_in_kernel_us"] = round(ops.peak_handover(256, 2000, 16), 2)
+    out["dependent_launch_us"] = round(dependent_launch_us(), 2)
     return out
+
+
+def dependent_launch_us(n=200):
+    """Microseconds per kernel of a captured chain of `n` tiny kernels, each depending on the one before."""
+    import torch
+    x = torch.zeros(64, device="cuda:0")
+    for _ in range(3):
+        x.add_(1.0)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for _ in range(n):
+            x.add_(1.0)
+    g.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(5):
+        g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / (5 * n)
 
 
 # ------------------------------------------------------------------- one model

@@ -1032,3 +1032,16 @@ def test_seeded_numbers_are_the_same_bits_on_host_and_device(dtype):
         assert torch.equal(dev.cpu(), host), spec.name
     other = random_tensor(WeightSpec("a.weight", (3, 5, 7)), 78, 1.7, 0.0, device=DEV, dtype=dtype)
     assert not torch.equal(other.cpu(), random_tensor(WeightSpec("a.weight", (3, 5, 7)), 77, 1.7, 0.0, dtype=dtype))
+
+
+def test_handover_probe_runs_and_its_waits_are_bounded():
+    """The measurement of a hand-over among resident workgroups: values arrive right, a round takes
+    microseconds; with a wait of one poll the kernel gives up instead of waiting, and still ends."""
+    us = ops().peak_handover(workgroups=256, rounds=200, payload=16)
+    assert 0.2 < us < 200.0
+    assert ops().peak_handover(workgroups=8, rounds=50, payload=300) > 0.0
+    try:
+        ops().peak_handover(workgroups=256, rounds=50, payload=16, spin_limit=1)
+    except ops().KernelError as e:
+        assert "ran out" in str(e)
+    torch.cuda.synchronize()

@@ -2,7 +2,11 @@
 // time, so that a step's rate can be set against a measured peak beside the published one.
 //   * peak_read_kernel / peak_copy_kernel: streaming reads (and writes) of a large buffer;
 //   * peak_mfma_bf16_kernel / peak_mfma_f32_kernel: a loop of independent matrix instructions on
-//     registers (v_mfma_f32_32x32x16_bf16, v_mfma_f32_16x16x4_f32), no memory traffic.
+//     registers (v_mfma_f32_32x32x16_bf16, v_mfma_f32_16x16x4_f32), no memory traffic;
+//   * peak_handover_kernel: what it costs to hand data from every workgroup to every other INSIDE one
+//     launch (write-through stores, a flag per workgroup, loads that go past the caches): the time a
+//     decode step would pay per dependent phase if its kernels were fused into one persistent kernel,
+//     to be set against the time between two dependent launches of a graph.
 #include "common.h"
 
 namespace {
@@ -74,9 +78,75 @@ __global__ __launch_bounds__(P_THREADS) void peak_mfma_f32_kernel(float* __restr
   if (s == 123456.789f) sink[0] = s;
 }
 
+// One round: every workgroup writes `payload` floats with stores that go through to memory, waits
+// until they are acknowledged, raises its flag; one wave per workgroup reads all flags until all are
+// up; every workgroup then reads another workgroup's floats with loads that go past the caches and
+// checks them.  No read-modify-write, no shared counter: the round's cost is the few trips to the
+// point where the caches of the eight dies meet.  Waits are bounded: after `spin_limit` polls a
+// workgroup gives up, says so in *err and everybody leaves.
+constexpr int H_THREADS = 512, H_MAX_WG = 256;
+__global__ __launch_bounds__(H_THREADS) void peak_handover_kernel(unsigned* __restrict__ flags, float* __restrict__ data,
+                                                                   int rounds, int payload, unsigned spin_limit,
+                                                                   int* __restrict__ err, unsigned* __restrict__ wrong) {
+  __shared__ int ok_s;
+  const int nwg = gridDim.x, wg = blockIdx.x;
+  unsigned bad = 0;
+  for (int it = 0; it < rounds; ++it) {
+    float* mine = data + ((size_t)(it & 1) * nwg + wg) * payload;
+    for (int i = threadIdx.x; i < payload; i += H_THREADS)
+      __hip_atomic_store(&mine[i], (float)(it * 7 + wg * 3 + i), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_s_waitcnt(0);          // this wave's stores have been acknowledged
+    __builtin_amdgcn_s_barrier();
+    if (threadIdx.x < TL_WAVE) {
+      const int lane = threadIdx.x;
+      if (lane == 0) __hip_atomic_store(&flags[wg], (unsigned)(it + 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      bool ok = true;
+      unsigned spins = 0;
+      while (true) {
+        bool up = true;
+#pragma unroll
+        for (int j = 0; j < H_MAX_WG / TL_WAVE; ++j) {
+          const int i = lane * (H_MAX_WG / TL_WAVE) + j;
+          if (i < nwg) up &= __hip_atomic_load(&flags[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= (unsigned)(it + 1);
+        }
+        if (__all(up)) break;
+        if (++spins > spin_limit || __hip_atomic_load(err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
+          ok = false;
+          break;
+        }
+      }
+      if (lane == 0) {
+        if (!ok) __hip_atomic_store(err, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ok_s = ok;
+      }
+    }
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (!*(volatile int*)&ok_s) return;
+    const int other = (wg + 77 + it) % nwg;
+    const float* theirs = data + ((size_t)(it & 1) * nwg + other) * payload;
+    for (int i = threadIdx.x; i < payload; i += H_THREADS)
+      if (__hip_atomic_load(&theirs[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != (float)(it * 7 + other * 3 + i)) ++bad;
+  }
+  if (bad) atomicAdd(wrong, bad);
+}
+
 }  // namespace
 
 extern "C" {
+
+// `rounds` hand-overs of `payload` floats a workgroup among `workgroups` (at most 256, one per compute
+// unit at most: all must be resident at once).  flags: `workgroups` zeroed words; data: 2 * workgroups *
+// payload floats; err, wrong: zeroed words (after the launch: 1 if a wait ran out; values read wrong).
+int tl_peak_handover(unsigned* flags, float* data, int workgroups, int rounds, int payload, unsigned spin_limit, int* err,
+                     unsigned* wrong, hipStream_t stream) {
+  if (!flags || !data || !err || !wrong || workgroups <= 0 || workgroups > H_MAX_WG || rounds <= 0 || payload <= 0 ||
+      spin_limit == 0)
+    return TL_ERR_ARG;
+  hipLaunchKernelGGL(peak_handover_kernel, dim3(workgroups), dim3(H_THREADS), 0, stream, flags, data, rounds, payload,
+                     spin_limit, err, wrong);
+  return tl_launch_status();
+}
 
 // mode 0: read `bytes` of src; mode 1: copy them to dst.  Both 16-byte aligned, bytes a multiple of 16.
 int tl_peak_stream(const void* src, void* dst, float* sink, int64_t bytes, int mode, int blocks, hipStream_t stream) {

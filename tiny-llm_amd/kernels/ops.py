@@ -951,6 +951,36 @@ def peak_mfma(sink: torch.Tensor, dtype: torch.dtype, iters: int, blocks: int = 
     return float(flops.value)
 
 
+def peak_handover(workgroups: int = 256, rounds: int = 2000, payload: int = 16, spin_limit: int = 1 << 20) -> float:
+    """Microseconds one hand-over of `payload` floats from every workgroup to every other takes inside ONE
+    launch of `workgroups` resident workgroups (write-through stores, a flag per workgroup, loads past
+    the caches): what a dependent phase would cost a persistent kernel, beside the time between two
+    dependent launches.  Raises if a wait ran out or a value was read wrong."""
+    if not (0 < workgroups <= 256 and rounds > 0 and payload > 0):
+        _fail("1 to 256 workgroups, at least one round and one float")
+    dev = torch.device("cuda", torch.cuda.current_device())
+    flags = torch.zeros(256, dtype=torch.int32, device=dev)
+    data = torch.zeros(2 * workgroups * payload, dtype=torch.float32, device=dev)
+    state = torch.zeros(2, dtype=torch.int32, device=dev)
+
+    def launch():
+        _check(_lib().tl_peak_handover(_ptr(flags), _ptr(data), c_int(workgroups), c_int(rounds), c_int(payload),
+                                       ctypes.c_uint(spin_limit), _ptr(state[0:1]), _ptr(state[1:2]), _stream()),
+               "peak_handover")
+    launch()
+    torch.cuda.synchronize()
+    flags.zero_()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    launch()
+    e1.record()
+    torch.cuda.synchronize()
+    gave_up, wrong = state.cpu().tolist()
+    if gave_up or wrong:
+        _fail(f"hand-over probe: a wait ran out ({gave_up}) or {wrong} values were read wrong")
+    return e0.elapsed_time(e1) * 1e3 / rounds
+
+
 def decode_advance(tokens: torch.Tensor, positions: torch.Tensor, seq_lens: torch.Tensor, counters: torch.Tensor,
                    sampled: torch.Tensor, history: torch.Tensor, step: torch.Tensor, slot_mappings, block_tables,
                    block_size: int) -> None:
