@@ -957,3 +957,53 @@ def test_toy_routed_feed_forward_and_other_position_encoding(dtype):
         EMBEDDINGS.unregister("scaled_embedding")
         HEADS.unregister("capped_head")
         unregister_architecture("Toy2ForCausalLM")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_chained_decode_steps_with_several_cache_groups(dtype):
+    """A toy architecture whose three attention layers keep caches of three kinds (every position;
+    a window of 20; every position with other kv heads): three cache groups with pools of their own
+    sizes.  Runs of decode steps chained on the device, in which the window group's blocks for a
+    whole run are taken up front and given back behind it, give the tokens of single steps."""
+    from tiny_llm_amd import Engine, SamplingParams
+    from tiny_llm_amd.config import (ModelSpec, PartSpec, PlanEntry, pre_norm_layer, register_architecture,
+                                     unregister_architecture)
+
+    def build(cfg):
+        H = cfg["hidden_size"]
+        norm = PartSpec("rmsnorm", {"hidden_size": H, "eps": 1e-5})
+        ffn = PartSpec("swiglu", {"hidden_size": H, "intermediate_size": 96})
+        rope = {"kind": "rotary", "head_dim": 16, "theta": 1000.0, "max_position": 512}
+
+        def attn(kv_heads, window=0):
+            return PartSpec("attention", {"hidden_size": H, "num_heads": 4, "num_kv_heads": kv_heads, "head_dim": 16,
+                                          "window": window, "position": rope})
+        layers = tuple(pre_norm_layer(f"model.layers.{i}", norm, m, norm, ffn)
+                       for i, m in enumerate([attn(2), attn(2, window=20), attn(1)]))
+        sizes = {"vocab_size": cfg["vocab_size"], "hidden_size": H}
+        return ModelSpec("Toy3ForCausalLM", cfg["vocab_size"], H, 512, PartSpec("token_embedding", sizes, "model.embed_tokens"),
+                         layers, (PlanEntry(0), PlanEntry(1), PlanEntry(2)), norm.named("model.norm"),
+                         PartSpec("lm_head", dict(sizes, tied_to="model.embed_tokens"), "lm_head"))
+
+    register_architecture("Toy3ForCausalLM", dict, build)
+    try:
+        raw = {"architectures": ["Toy3ForCausalLM"], "hidden_size": 64, "vocab_size": 211}
+        prompts = [random_tokens(n, 211, 40 + n) for n in (33, 5, 58)]
+        sps = [SamplingParams.greedy(n, ignore_eos=True) for n in (90, 70, 41)]
+        sps[1] = SamplingParams(max_new_tokens=70, temperature=0.8, top_k=30, top_p=0.9, seed=3, ignore_eos=True)
+        outs = {}
+        for burst in (1, 32):
+            eng = Engine(config=raw, dtype=dtype, weights_seed=2, init_std=0.3, kv_block_size=8, max_num_seqs=3,
+                         max_num_batched_tokens=64, max_cache_tokens=3 * 160, decode_burst=burst)
+            cm = eng.runner.cache
+            assert len(cm.groups) == 3 and cm.group_blocks[0] == 60 and cm.group_blocks[1] < 60 and cm.group_blocks[2] == 60
+            poison(eng)
+            outs[burst] = eng.generate(prompts, sps)
+            cm.audit()
+            assert cm.free_blocks() == cm.group_blocks
+            if burst > 1:
+                chained = [g for g in eng.runner._graphs.values() if g.bursts > 0]
+                assert chained and all(g.feeds_next and g.chain is not None for g in chained)
+        assert outs[32] == outs[1] and [len(o) for o in outs[1]] == [90, 70, 41]
+    finally:
+        unregister_architecture("Toy3ForCausalLM")

@@ -232,6 +232,7 @@ __global__ void random_normal_kernel(T* __restrict__ out, int64_t n, uint64_t ke
 // position, cached length and sampling counter go up by one, and its cache slot is looked up in
 // the block table for the new position.  A run of decode steps can then be replayed back to back
 // without the host in between; `history` [history_steps, R] keeps what each step chose.
+constexpr int TL_MAX_CACHE_GROUPS = 16;     // cache groups a model may have and still chain decode steps on the device
 struct AdvanceArgs {
   int32_t* tokens;
   int32_t* positions;
@@ -241,8 +242,8 @@ struct AdvanceArgs {
   int32_t* history;
   int32_t* step;           // how many steps have run since the host last wrote the metadata
   int R, G, MB, block_size, history_steps;
-  int32_t* slots[4];
-  const int32_t* tables[4];
+  int32_t* slots[TL_MAX_CACHE_GROUPS];
+  const int32_t* tables[TL_MAX_CACHE_GROUPS];
 };
 
 __global__ void decode_advance_kernel(const AdvanceArgs a) {
@@ -363,12 +364,12 @@ int tl_random_normal(void* out, int64_t n, uint64_t key, const float* table, int
   return tl_launch_status();
 }
 
-// One workgroup: R requests, G <= 4 cache groups with block tables [R, MB].
+// One workgroup: R requests, G <= 16 cache groups with block tables [R, MB].
 int tl_decode_advance(int32_t* tokens, int32_t* positions, int32_t* seq_lens, int32_t* counters,
                       const int32_t* sampled, int32_t* history, int32_t* step, int R, int G, int MB, int block_size,
                       int history_steps, int32_t* const* slots, const int32_t* const* tables, hipStream_t stream) {
   if (R <= 0) return TL_OK;
-  if (G < 0 || G > 4 || MB <= 0 || block_size <= 0 || history_steps < 0 || !tokens || !positions || !seq_lens ||
+  if (G < 0 || G > TL_MAX_CACHE_GROUPS || MB <= 0 || block_size <= 0 || history_steps < 0 || !tokens || !positions || !seq_lens ||
       !counters || !sampled || !history || !step)
     return TL_ERR_ARG;
   AdvanceArgs a{tokens, positions, seq_lens, counters, sampled, history, step, R, G, MB, block_size, history_steps, {}, {}};

@@ -491,7 +491,7 @@ class ModelRunner:
         steps come back, once.  Cache blocks for all `steps` positions are taken up front.
         Returns the tokens by step, [steps][entries], or None if these steps cannot run as a burst
         (no captured graph of this shape yet, too many cache groups): the caller then runs one step."""
-        if steps < 2 or not self.decoder.graph_safe or len(self.cache.groups) > 4:
+        if steps < 2 or not self.decoder.graph_safe or len(self.cache.groups) > ops.MAX_CACHE_GROUPS:
             return None
         if not all(len(e.tokens) == 1 and len(e.want) == 1 for e in entries) or len(samples) != len(entries):
             return None
@@ -607,7 +607,7 @@ class StepGraph:
         self.out = torch.zeros(max(self.n_out, 1), dtype=torch.int32, device=runner.device)
         self.out_host = torch.zeros(max(self.n_out, 1), dtype=torch.int32, pin_memory=True)
         # a decode step with its sampler ends by preparing the next one on the device (bursts)
-        self.feeds_next = self.max_q_len == 1 and self.sampling and self.n_out == self.R == self.T and G <= 4
+        self.feeds_next = self.max_q_len == 1 and self.sampling and self.n_out == self.R == self.T and G <= ops.MAX_CACHE_GROUPS
         self.history_steps = self.BURST_STEPS if self.feeds_next else 0
         if self.feeds_next:
             self.history = torch.zeros(self.history_steps * self.R, dtype=torch.int32, device=runner.device)

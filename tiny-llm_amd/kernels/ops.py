@@ -981,6 +981,9 @@ def peak_handover(workgroups: int = 256, rounds: int = 2000, payload: int = 16, 
     return e0.elapsed_time(e1) * 1e3 / rounds
 
 
+MAX_CACHE_GROUPS = 16       # cache groups the decode hand-over kernel takes (csrc/elementwise.hip)
+
+
 def decode_advance(tokens: torch.Tensor, positions: torch.Tensor, seq_lens: torch.Tensor, counters: torch.Tensor,
                    sampled: torch.Tensor, history: torch.Tensor, step: torch.Tensor, slot_mappings, block_tables,
                    block_size: int) -> None:
@@ -995,15 +998,15 @@ def decode_advance(tokens: torch.Tensor, positions: torch.Tensor, seq_lens: torc
     for t in ints:
         if not (t.dtype == torch.int32 and t.is_contiguous()):
             _fail("decode_advance takes contiguous int32 tensors")
-    if not (G == len(block_tables) and G <= 4):
-        _fail("decode_advance takes up to four cache groups")
+    if not (G == len(block_tables) and G <= MAX_CACHE_GROUPS):
+        _fail(f"decode_advance takes up to {MAX_CACHE_GROUPS} cache groups")
     if not (all(t.numel() == R for t in (positions, seq_lens, counters, *slot_mappings)) and sampled.numel() >= R
             and step.numel() >= 1 and history.numel() % R == 0):
         _fail("decode_advance: one element per request in every per-request tensor")
     if not all(bt.dim() == 2 and bt.shape[0] == R and bt.shape[1] == block_tables[0].shape[1] for bt in block_tables):
         _fail("block tables must be [requests, max_blocks] of one width")
-    slots_arr = (c_void_p * 4)(*[t.data_ptr() for t in slot_mappings], *[0] * (4 - G))
-    tables_arr = (c_void_p * 4)(*[t.data_ptr() for t in block_tables], *[0] * (4 - G))
+    slots_arr = (c_void_p * MAX_CACHE_GROUPS)(*[t.data_ptr() for t in slot_mappings], *[0] * (MAX_CACHE_GROUPS - G))
+    tables_arr = (c_void_p * MAX_CACHE_GROUPS)(*[t.data_ptr() for t in block_tables], *[0] * (MAX_CACHE_GROUPS - G))
     _check(_lib().tl_decode_advance(_ptr(tokens), _ptr(positions), _ptr(seq_lens), _ptr(counters), _ptr(sampled),
                                     _ptr(history), _ptr(step), c_int(R), c_int(G),
                                     c_int(block_tables[0].shape[1] if G else 1), c_int(block_size),
