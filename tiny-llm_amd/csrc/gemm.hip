@@ -85,16 +85,22 @@ __global__ __launch_bounds__(FN_THREADS) void norm_prescale_f32_kernel(const flo
   const int nkb = (K + F_KBLOCK - 1) / F_KBLOCK;
   for (int c = threadIdx.x; c < nkb * 4; c += FN_THREADS) {
     const int kb = (c >> 2) * F_KBLOCK, q = c & 3;
+    // all sixteen pieces of the chain are requested before the first is used: one round trip, not sixteen
+    f32x4 v[16], nw[16];
+#pragma unroll
+    for (int g = 0; g < 16; ++g) {
+      v[g] = load_k4<VEC>(row, kb + g * 16 + q * 4, K);
+      nw[g] = load_k4<VEC>(norm_w, kb + g * 16 + q * 4, K);
+    }
     float ss = 0.f;
-#pragma unroll 4
+#pragma unroll
     for (int g = 0; g < 16; ++g) {
       const int k = kb + g * 16 + q * 4;
-      const f32x4 v = load_k4<VEC>(row, k, K), nw = load_k4<VEC>(norm_w, k, K);
       f32x4 o;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        ss = __builtin_fmaf(v[e], v[e], ss);
-        o[e] = v[e] * nw[e];
+        ss = __builtin_fmaf(v[g][e], v[g][e], ss);
+        o[e] = v[g][e] * nw[g][e];
       }
       if constexpr (VEC) {
         if (k < K) *(f32x4*)(dst + k) = o;
