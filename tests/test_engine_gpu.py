@@ -673,6 +673,61 @@ def test_command_line_generates_from_prompt_ids(folders):
     assert bad.returncode == 1 and "[Fatal]" in bad.stderr
 
 
+def test_tokens_stream_as_they_are_generated(folders):
+    """`stream` yields every prompt's tokens in order, each once, with the finish reason at the end;
+    together they are what `generate` returns; a bound of one decode step hands over a token at a time."""
+    from tiny_llm_amd import Engine, SamplingParams
+    cfg, eng_kw, _ = CONFIGS["A"]
+    prompts = [random_tokens(n, cfg["vocab_size"], 300 + n) for n in (5, 40, 17)]
+    sp = [SamplingParams.greedy(n, ignore_eos=True) for n in (9, 3, 20)]
+    eng = Engine(folders["A"], dtype="float32", max_num_seqs=4, max_num_batched_tokens=32, **eng_kw)
+    want = eng.generate(prompts, sp)
+    assert [len(o) for o in want] == [9, 3, 20]
+    for bound in (None, 1):
+        got = [[] for _ in prompts]
+        reasons = [None] * 3
+        chunks = [[] for _ in prompts]
+        for i, fresh, reason in eng.stream(prompts, sp, max_decode_steps=bound):
+            assert reasons[i] is None, "tokens after a request's end"
+            got[i] += fresh
+            chunks[i].append(len(fresh))
+            reasons[i] = reason
+        assert got == want and reasons == ["length"] * 3
+        if bound == 1:
+            assert all(c <= 1 for per in chunks for c in per)
+        else:
+            assert max(chunks[2]) > 1               # chained decode steps hand over several tokens at once
+    seen = []
+    assert eng.generate(prompts[:1], sp[0], on_tokens=lambda i, t, r: seen.append((i, list(t), r))) == want[:1]
+    assert [t for _, ts, _ in seen for t in ts] == want[0] and seen[-1][2] == "length"
+    # a request that asks for nothing ends at once, with its reason and no tokens
+    assert list(eng.stream([prompts[0]], SamplingParams.greedy(0))) == [(0, [], "length")]
+
+
+def test_command_line_streams_and_takes_norm_std(tmp_path):
+    """--stream prints the same ids as the plain run; --norm_std reaches the random weights."""
+    from tiny_llm_amd import Engine, SamplingParams
+    cfg = CONFIGS["B"][0]
+    only_config = tmp_path / "only_config"
+    only_config.mkdir()
+    with open(only_config / "config.json", "w") as f:
+        json.dump(cfg, f)
+    prompt = random_tokens(11, cfg["vocab_size"], 31)
+    base = [sys.executable, os.path.join(ROOT, "bin", "tiny_llm"), "--model_path", str(only_config),
+            "--random_weights", "--weights_seed=5", "--norm_std=0.3", "--nodo_sample", "--max_new_tokens=40",
+            "--dtype", "float32", "--ignore_eos", "--kv_block_size=8", "--prompt_ids", ",".join(map(str, prompt))]
+    outs = []
+    for extra in ([], ["--stream"]):
+        proc = subprocess.run(base + extra, capture_output=True, text=True, timeout=300)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        outs.append([int(t) for t in proc.stdout.strip().splitlines()[-1].split()])
+    engine = Engine(config=cfg, dtype="float32", weights_seed=5, norm_std=0.3, kv_block_size=8)
+    want = engine.generate([prompt], SamplingParams.greedy(40, ignore_eos=True))[0]
+    assert outs[0] == want and outs[1] == want
+    flat = Engine(config=cfg, dtype="float32", weights_seed=5, norm_std=0.0, kv_block_size=8)
+    assert flat.generate([prompt], SamplingParams.greedy(40, ignore_eos=True))[0] != want
+
+
 def test_command_line_random_weights_and_prompt_file(tmp_path):
     """--random_weights takes only config.json from the folder and fills the weights on the device
     from --weights_seed, as the Python entry point does for a configuration; --prompt_ids_file

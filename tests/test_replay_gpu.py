@@ -187,15 +187,16 @@ def test_long_decoding(tmp_path_factory):
     assert worst < TOL["float32"]
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_trace_run_program(dtype, tmp_path_factory, tmp_path):
-    """bin/trace_run as a user runs it: JSON steps on stdin, <step>.f32 files, `done <step>` lines."""
+@pytest.mark.parametrize("dtype,graphs", [("float32", False), ("bfloat16", False), ("bfloat16", True)])
+def test_trace_run_program(dtype, graphs, tmp_path_factory, tmp_path):
+    """bin/trace_run as a user runs it: JSON steps on stdin, <step>.f32 files, `done <step>` lines;
+    with --graphs the shapes of step that come again (the decoded tokens' steps) replay captured graphs."""
     folder, reqs, ref, eng = material("A", dtype, tmp_path_factory)
     steps, peak = traces.mixed(reqs, seed=3)
     out_dir = tmp_path / "out"
     proc = subprocess.run(
         [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
-         "--out", str(out_dir), "--max-tokens", str(peak)],
+         "--out", str(out_dir), "--max-tokens", str(peak)] + (["--graphs"] if graphs else []),
         input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=600)
     assert proc.returncode == 0, proc.stderr[-3000:]
     assert [l for l in proc.stdout.splitlines() if l.startswith("done ")] == [f"done {s['step']}" for s in steps]

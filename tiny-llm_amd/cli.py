@@ -31,6 +31,8 @@ FLAGS: Dict[str, Tuple[type, Any, str]] = {
     "random_weights": (bool, False, "Take only config.json from --model_path and fill the weights from --weights_seed"),
     "weights_seed": (int, 0, "Seed of the random weights"),
     "init_std": (float, 0.0, "Standard deviation of the random matrices (0: the configuration's initializer_range)"),
+    "norm_std": (float, 0.0, "Standard deviation of the random norm weights around 1"),
+    "stream": (bool, False, "Print the output as it is generated, not when the request has ended"),
     "ignore_eos": (bool, False, "Keep generating after the end-of-sequence token"),
     "kv_block_size": (int, 16, "Tokens per cache page"),
     "num_kv_blocks": (int, 0, "Cache pages (0: enough for max_num_seqs full-length requests)"),
@@ -124,6 +126,25 @@ def parse_ids(text: str) -> List[int]:
         raise FlagError("without tokenizer.json a prompt must be token ids separated by spaces or commas") from None
 
 
+def _generate_streaming(engine, text: "_Text", prompt: List[int], params) -> List[int]:
+    """Prints one prompt's output as it arrives: after every run of steps the text of all tokens so
+    far is decoded again and what it gained is written (a token alone need not be whole characters)."""
+    ids: List[int] = []
+    shown = ""
+    for _, fresh, _reason in engine.stream([prompt], params):
+        ids += fresh
+        now = text.decode(ids)
+        if now.startswith(shown):
+            sys.stdout.write(now[len(shown):])
+        else:                                   # the tokenizer changed its mind about earlier text
+            sys.stdout.write("\n" + now)
+        sys.stdout.flush()
+        shown = now
+    sys.stdout.write("\n")
+    sys.stdout.flush()
+    return ids
+
+
 def main(argv: List[str] = None) -> int:
     argv = sys.argv[1:] if argv is None else argv
     try:
@@ -147,7 +168,7 @@ def main(argv: List[str] = None) -> int:
             with open(os.path.join(flags["model_path"], "config.json")) as f:
                 raw = json.load(f)
             engine = Engine(config=raw, engine_config=cfg, weights_seed=flags["weights_seed"],
-                            init_std=flags["init_std"] or None)
+                            init_std=flags["init_std"] or None, norm_std=flags["norm_std"])
         else:
             engine = Engine(flags["model_path"], engine_config=cfg)
         text = _Text(flags["model_path"])
@@ -159,6 +180,9 @@ def main(argv: List[str] = None) -> int:
             if flags["prompt_ids_file"]:
                 with open(flags["prompt_ids_file"]) as f:
                     prompts += [parse_ids(line) for line in f if line.strip()]
+            if flags["stream"] and len(prompts) == 1:
+                _generate_streaming(engine, text, prompts[0], params)
+                return 0
             for out in engine.generate(prompts, params):
                 print(text.decode(out))
             return 0
@@ -178,6 +202,10 @@ def main(argv: List[str] = None) -> int:
                 break
             if not buf:
                 print("The prompt is empty. Please re-enter.")
+                continue
+            if flags["stream"]:
+                print("[Output] >", flush=True)
+                _generate_streaming(engine, text, text.encode(buf), params)
                 continue
             out = engine.generate([text.encode(buf)], params)[0]
             print("[Output] >\n" + text.decode(out), flush=True)

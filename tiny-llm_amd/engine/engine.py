@@ -9,7 +9,7 @@ command line's business.
 from __future__ import annotations
 
 import itertools
-from typing import Dict, Hashable, List, Mapping, Optional, Sequence, Union
+from typing import Callable, Dict, Hashable, Iterator, List, Mapping, Optional, Sequence, Tuple, Union
 
 from ..config import EngineConfig
 from ..sampling import SamplingParams
@@ -104,13 +104,41 @@ class Engine:
         return done
 
     # ---------------------------------------------------------------- generate
-    def generate(self, prompt_token_ids: Sequence[Sequence[int]],
-                 params: Union[SamplingParams, Sequence[SamplingParams], None] = None) -> List[List[int]]:
-        """Generated token ids of every prompt (eos, when it ends a request, is part of them,
-        as in tiny_llm/pipeline/pipeline.cpp:216-223)."""
+    def stream(self, prompt_token_ids: Sequence[Sequence[int]],
+               params: Union[SamplingParams, Sequence[SamplingParams], None] = None,
+               max_decode_steps: Optional[int] = None) -> Iterator[Tuple[int, List[int], Optional[str]]]:
+        """Generates for every prompt and yields `(index of the prompt, its new token ids, finish
+        reason or None)` after each step that gave that prompt tokens, in the order of the prompts.
+        A run of chained decode steps hands over all its tokens at once; `max_decode_steps` bounds
+        such a run (1: a token at a time).  A request preempted for want of pages yields nothing
+        twice: what it had generated is kept and recomputed, not sampled again."""
         if params is None or isinstance(params, SamplingParams):
             params = [params or SamplingParams()] * len(prompt_token_ids)
         ids = [self.add_request(p, sp) for p, sp in zip(prompt_token_ids, params)]
-        while self.scheduler.has_work():
-            self.step()
-        return [list(self.requests[i].output) for i in ids]
+        told = [0] * len(ids)
+        closed = [False] * len(ids)
+        while True:
+            for i, rid in enumerate(ids):
+                r = self.requests[rid]
+                fresh = list(r.output[told[i]:])
+                ended = r.status == "finished" and not closed[i]
+                if fresh or ended:
+                    told[i] += len(fresh)
+                    closed[i] = closed[i] or ended
+                    yield i, fresh, (r.finish_reason if ended else None)
+            if not self.scheduler.has_work():
+                return
+            self.step(max_decode_steps)
+
+    def generate(self, prompt_token_ids: Sequence[Sequence[int]],
+                 params: Union[SamplingParams, Sequence[SamplingParams], None] = None,
+                 on_tokens: Optional[Callable[[int, List[int], Optional[str]], None]] = None) -> List[List[int]]:
+        """Generated token ids of every prompt (eos, when it ends a request, is part of them,
+        as in tiny_llm/pipeline/pipeline.cpp:216-223).  `on_tokens(index, new ids, finish reason
+        or None)` is called as tokens arrive (what `stream` yields)."""
+        out: List[List[int]] = [[] for _ in prompt_token_ids]
+        for i, fresh, reason in self.stream(prompt_token_ids, params):
+            out[i] += fresh
+            if on_tokens is not None:
+                on_tokens(i, fresh, reason)
+        return out
