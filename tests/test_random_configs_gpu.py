@@ -1,0 +1,96 @@
+"""Configurations drawn at random (head sizes with and without a matrix-core kernel, any number of
+heads and groups, widths and vocabularies that are no power of two, pages of any size), each
+replayed in three cuttings in both precisions against the plain model.  The four fixed tiny
+configurations cannot hold every combination; this holds a sample of them and a seed names each."""
+import random
+import tempfile
+
+import pytest
+import torch
+
+import plain_llama as plain
+import traces
+from test_replay_gpu import TOL, check, make_runner, r64, replay
+from util import make_folder, random_tokens, read_weights
+
+pytestmark = pytest.mark.gpu
+
+HEAD_SIZES = [16, 32, 48, 64, 80, 96, 112, 128, 24, 40, 72, 144, 160, 256]
+PAGE_SIZES = [1, 2, 4, 8, 16, 32, 64, 3, 5, 12]
+
+
+def random_config(rng: random.Random) -> dict:
+    hd = rng.choice(HEAD_SIZES)
+    kv = rng.choice([1, 1, 2, 2, 3, 4, 5, 8])
+    group = rng.choice([1, 1, 2, 3, 4, 4, 5, 6, 8, 12, 16, 17, 20])
+    if kv * group * hd > 4096:
+        group = max(1, 2048 // (kv * hd))
+    return {
+        "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+        "num_hidden_layers": rng.randint(1, 3), "hidden_size": rng.choice([8, 16, 24]) * rng.randint(2, 40),
+        "num_attention_heads": kv * group, "num_key_value_heads": kv, "head_dim": hd,
+        "intermediate_size": 8 * rng.randint(3, 90), "vocab_size": rng.randint(17, 3000),
+        "rope_theta": rng.choice([10000.0, 500000.0, 1e6, 777.0]), "rms_norm_eps": rng.choice([1e-5, 1e-6, 3e-4]),
+        "max_position_embeddings": 512, "tie_word_embeddings": rng.random() < 0.4, "hidden_act": "silu",
+        "attention_bias": False, "rope_scaling": None, "initializer_range": 0.03, "eos_token_id": 2,
+        "torch_dtype": "float32",
+    }
+
+
+def test_the_sample_covers_what_it_is_for():
+    """The seeds below reach every head size (those with a matrix-core kernel and those without),
+    more than sixteen query heads a kv head, and pages that do not divide 64."""
+    seen_hd, seen_pages, wide_group = set(), set(), False
+    for seed in SEEDS:
+        rng = random.Random(seed)
+        cfg = random_config(rng)
+        seen_hd.add(cfg["head_dim"])
+        seen_pages.add(rng.choice(PAGE_SIZES))
+        wide_group |= cfg["num_attention_heads"] // cfg["num_key_value_heads"] > 16
+    assert seen_hd == set(HEAD_SIZES) and {3, 5, 12} <= seen_pages and wide_group
+
+
+def _pick_seeds(count):
+    """The first seeds that add a head size not seen before, then the next ones up to `count`."""
+    chosen, seen = [], set()
+    for seed in range(400):
+        hd = random_config(random.Random(seed))["head_dim"]
+        if hd not in seen:
+            seen.add(hd)
+            chosen.append(seed)
+    for seed in range(400):
+        if len(chosen) >= count:
+            break
+        if seed not in chosen:
+            chosen.append(seed)
+    return sorted(chosen)
+
+
+SEEDS = sorted(set(_pick_seeds(28)) | {41, 44, 65})      # the three: heads of 112, decoded tokens
+
+
+@pytest.mark.parametrize("seed", SEEDS)
+def test_random_configuration(seed):
+    rng = random.Random(seed)
+    cfg = random_config(rng)
+    page = rng.choice(PAGE_SIZES)
+    lens = [rng.randint(1, 260) for _ in range(5)]
+    print(f"seed {seed}: {cfg['num_hidden_layers']} layers, hidden {cfg['hidden_size']}, "
+          f"{cfg['num_attention_heads']}/{cfg['num_key_value_heads']} heads of {cfg['head_dim']}, "
+          f"intermediate {cfg['intermediate_size']}, vocabulary {cfg['vocab_size']}, page {page}, lengths {lens}", flush=True)
+    with tempfile.TemporaryDirectory() as tmp:
+        folder = make_folder(tmp, cfg, seed=seed, std=0.03, norm_std=0.1, sharpen=2.0)
+        reqs = {f"r{i}": random_tokens(n, cfg["vocab_size"], 100 * i + seed) for i, n in enumerate(lens)}
+        for dtype in ("float32", "bfloat16"):
+            rounded = torch.bfloat16 if dtype == "bfloat16" else None
+            w, c = read_weights(folder, round_to=rounded)
+            ref = {rid: plain.llama_forward(w, c, toks, act_dtype=rounded) for rid, toks in reqs.items()}
+            biggest = max(r64(len(t)) for t in reqs.values())
+            mixed_steps, peak = traces.mixed(reqs, seed=seed)
+            for steps, tokens in ((mixed_steps, peak), (traces.portions(reqs), biggest),
+                                  (traces.tail_one_by_one(reqs), biggest)):
+                if 64 % page:
+                    tokens += 8 * page          # a request's last page may reach beyond its multiple of 64
+                runner = make_runner(folder, dtype, page, tokens)
+                check(replay(runner, steps), steps, ref, TOL[dtype])
+                assert runner.cache.free_blocks() == [g.pool.num_blocks for g in runner.cache.groups]

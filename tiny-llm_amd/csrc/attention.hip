@@ -377,6 +377,9 @@ __global__ __launch_bounds__(WAVES * TL_WAVE) void flash_attn_bf16_kernel(
     bf16x8 z = {};
     qf[ks] = do_rope ? rotate_chunk_regs<HD>(qx[ks], qy[ks], d, c8[ks], s8[ks]) : qx[ks];
     if (!(row_valid && d < HD)) qf[ks] = z;
+    // (the slots beyond HD of the last k step meet zeros of the query operand: they must hold
+    // something finite, since 0 * NaN is NaN and a register nobody wrote may hold anything)
+    new_k[ks] = z;
     if (owns_new && r16 == new_pos % 16 && d < HD) {
       new_k[ks] = rotate_chunk_regs<HD>(kx[ks], ky[ks], d, c8[ks], s8[ks]);
       *(bf16x8*)(fused.k_cache_w + new_off + d) = new_k[ks];
