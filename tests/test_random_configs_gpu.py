@@ -94,3 +94,50 @@ def test_random_configuration(seed):
                 runner = make_runner(folder, dtype, page, tokens)
                 check(replay(runner, steps), steps, ref, TOL[dtype])
                 assert runner.cache.free_blocks() == [g.pool.num_blocks for g in runner.cache.groups]
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_schedule(seed):
+    """Generation through the entry point with everything about the schedule drawn at random (how
+    many requests and how long, pages so few that requests are preempted, token budgets from 4 to
+    2,048, one to sixteen live requests, captured steps or not, runs of chained decode steps or
+    not): every token is the plain model's choice or within rounding of it, every page comes back."""
+    from tiny_llm_amd import Engine, SamplingParams
+    rng = random.Random(9000 + seed)
+    cfg = random_config(rng)
+    cfg["num_hidden_layers"] = rng.randint(1, 2)
+    page = rng.choice(PAGE_SIZES)
+    n = rng.randint(1, 12)
+    lens = [rng.randint(1, 120) for _ in range(n)]
+    news = [rng.randint(1, 70) for _ in range(n)]
+    budget = rng.choice([4, 8, 16, 33, 64, 256, 2048])
+    seqs = rng.choice([1, 2, 3, 4, 8, 16])
+    biggest = max(-(-(l + m) // page) for l, m in zip(lens, news))
+    total = sum(-(-(l + m) // page) for l, m in zip(lens, news))
+    blocks = rng.randint(biggest, max(biggest, total))
+    graphs = rng.random() < 0.7
+    burst = rng.choice([1, 4, 32])
+    dtype = rng.choice(["float32", "float32", "bfloat16"])
+    print(f"seed {seed}: hidden {cfg['hidden_size']}, {cfg['num_attention_heads']}/{cfg['num_key_value_heads']} heads of "
+          f"{cfg['head_dim']}, page {page}, {blocks} of {total} blocks, budget {budget}, {seqs} live, graphs {graphs}, "
+          f"burst {burst}, {dtype}, (prompt, new) {list(zip(lens, news))}", flush=True)
+    with tempfile.TemporaryDirectory() as tmp:
+        folder = make_folder(tmp, cfg, seed=seed, std=0.03, norm_std=0.1, sharpen=2.0)
+        prompts = [random_tokens(n_tok, cfg["vocab_size"], 100 * i + seed) for i, n_tok in enumerate(lens)]
+        eng = Engine(folder, dtype=dtype, kv_block_size=page, num_kv_blocks=blocks, max_num_seqs=seqs,
+                     max_num_batched_tokens=budget, use_graphs=graphs, decode_burst=burst)
+        for g in eng.runner.cache.groups:
+            for t in g.tensors.values():
+                t.fill_(float("nan"))
+        out = eng.generate(prompts, [SamplingParams.greedy(m, ignore_eos=True) for m in news])
+        eng.runner.cache.audit()
+        assert eng.runner.cache.free_blocks() == [g.pool.num_blocks for g in eng.runner.cache.groups]
+        rounded = torch.bfloat16 if dtype == "bfloat16" else None
+        w, c = read_weights(folder, round_to=rounded)
+        tol = 2 * TOL[dtype]
+        for i, (p, o) in enumerate(zip(prompts, out)):
+            assert len(o) == news[i], (i, eng.requests[i].finish_reason)
+            ref = plain.llama_forward(w, c, p + o, act_dtype=rounded)
+            for k, tok in enumerate(o):
+                row = ref[len(p) + k - 1]
+                assert float(row.max() - row[tok]) <= tol * float(row.abs().max()), (i, k)
