@@ -861,8 +861,32 @@ def test_flash_attention_fused_rotation_and_cache_write(nq, nkv, hd, bs, n_split
     """Decode step with rotation and cache write inside the attention kernel == rope_store + attention.
     The long requests give a wave several key tiles in turn (the new token's in the last), the
     window lets a wave's first tile be another than the one whose pages it looked up ahead."""
+    _fused_against_separate(nq, nkv, hd, bs, n_splits, window, nq + hd)
+
+
+def test_flash_attention_fused_rotation_random_sizes():
+    """The same at sizes drawn at random: every head size the kernel takes, 1 to 16 heads a kv head,
+    pages of 1 to 100 tokens, up to 16 key splits, windows from 1 to beyond the longest context.
+    Both ways write the same rows of the cache."""
+    import random
+    for seed in range(120):
+        rng = random.Random(seed)
+        hd = rng.choice([16, 32, 48, 64, 80, 96, 112, 128])
+        nkv = rng.choice([1, 2, 3, 4, 8])
+        group = rng.choice([1, 2, 3, 4, 5, 8, 16])
+        bs = rng.choice([1, 2, 3, 4, 8, 16, 32, 64, 12, 100])
+        n_splits = rng.choice([1, 2, 3, 4, 8, 16])
+        window = rng.choice([0, 0, 1, 2, 16, 64, 65, 150, 300, 1000])
+        try:
+            _fused_against_separate(nkv * group, nkv, hd, bs, n_splits, window, seed)
+        except AssertionError as e:
+            raise AssertionError(f"seed {seed}: {nkv * group}/{nkv} heads of {hd}, page {bs}, {n_splits} splits, "
+                                 f"window {window}") from e
+
+
+def _fused_against_separate(nq, nkv, hd, bs, n_splits, window, seed):
     from tiny_llm_amd.parts.rotary import RotaryEmbedding
-    g = torch.Generator().manual_seed(nq + hd)
+    g = torch.Generator().manual_seed(seed)
     lens = [1, 2, 63, 64, 65, 129, 300, 17, 600, 1100]
     R = len(lens)
     rot = RotaryEmbedding("r", torch.bfloat16, DEV, head_dim=hd, theta=10000.0, max_position=1200)
@@ -894,9 +918,17 @@ def test_flash_attention_fused_rotation_and_cache_write(nq, nkv, hd, bs, n_split
     out2 = torch.empty(R, nq * hd, dtype=torch.bfloat16, device=DEV)
     ops().flash_attention(qkv2[:, :nq * hd], kc2, vc2, bt.to(DEV), tiles, pos, out2, nq, nkv, hd, hd ** -0.5, window,
                           n_splits, scratch, fused_rope=(cos, sin))
-    assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2)      # the same rows, the same bits
+    # The same rows with the same values: the values are copied, the keys rotated by the same
+    # expression in both kernels, whose multiplications and additions the compiler fuses as it likes
+    # in each: once in some ten thousand elements the last bit of a key differs (and then, by as
+    # little, outputs that the key or the query, rotated the same way, enters).  A row lost or
+    # misplaced is off by the size of the values.
+    assert torch.equal(vc1, vc2)
+    k1, k2 = kc1.float(), kc2.float()
+    assert ((k1 - k2).abs() <= k1.abs() * 2.0 ** -7).all() and (k1 != k2).float().mean() < 1e-3
     assert torch.equal(qkv2.cpu(), qkv)                          # the input rows are left as they were
-    assert rel(out2, out1.double()) < 1e-6
+    assert rel(out2, out1.double()) < 1e-2
+    assert (out2 != out1).float().mean() < 0.02
     # without tile arrays: row i is the one new token of request i
     kc3, vc3 = kc.clone().to(DEV), vc.clone().to(DEV)
     out3 = torch.empty(R, nq * hd, dtype=torch.bfloat16, device=DEV)

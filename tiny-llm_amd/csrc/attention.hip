@@ -152,25 +152,10 @@ struct FusedRope {
 };
 
 // Rotate-half of 8 dims starting at d0 (a multiple of 8): own chunk x, partner chunk y = the dims
-// d0 +- HD/2; the expressions are rope_store_kernel's.
-template <int HD>
-__device__ __forceinline__ bf16x8 rotate_chunk(const bf16x8 x, const bf16x8 y, int d0, const float* cs,
-                                               const float* sn) {
-  constexpr int HALF = HD / 2;
-  bf16x8 r;
-  const bool first = d0 < HALF;
-  const int j0 = first ? d0 : d0 - HALF;
-#pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const float c = cs[j0 + e], sv = sn[j0 + e];
-    const float a = first ? (float)x[e] : (float)y[e];     // the pair's first-half value
-    const float b = first ? (float)y[e] : (float)x[e];     // and its second-half value
-    r[e] = (bf16_t)(first ? c * a - sv * b : sv * a + c * b);
-  }
-  return r;
-}
-
-// The same with the 8 angles of the chunk in registers (c8, s8 = cos and sin of the pairs j0 .. j0 + 7).
+// d0 +- HD/2, with the 8 angles of the chunk in registers (c8, s8 = cos and sin of the pairs
+// j0 .. j0 + 7).  The expressions are rope_store_kernel's; how the compiler fuses their
+// multiplications and additions is its own choice in each kernel, so once in some ten thousand
+// elements the two kernels differ in the last bit of a rotated value.
 template <int HD>
 __device__ __forceinline__ bf16x8 rotate_chunk_regs(const bf16x8 x, const bf16x8 y, int d0, const float* c8,
                                                     const float* s8) {
