@@ -141,3 +141,80 @@ def test_random_schedule(seed):
             for k, tok in enumerate(o):
                 row = ref[len(p) + k - 1]
                 assert float(row.max() - row[tok]) <= tol * float(row.abs().max()), (i, k)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_windowed_architecture(seed):
+    """A toy architecture registered here: two to four attention layers, each with a window drawn at
+    random (0: every key) and so with cache groups and pools of their own, either rotary pairing.
+    Generation under a random schedule (as `test_random_schedule`) against the same model run over
+    each finished request whole, in one eager step with a pool that is never short."""
+    from tiny_llm_amd import Engine, SamplingParams
+    from tiny_llm_amd.config import (EngineConfig, ModelSpec, PartSpec, PlanEntry, pre_norm_layer, register_architecture,
+                                     unregister_architecture)
+    from tiny_llm_amd.engine.loading import build_runner, random_model
+    from tiny_llm_amd.engine.step import StepEntry
+    rng = random.Random(seed)
+    hd = rng.choice([16, 32, 48, 64, 40, 128])
+    kv, group = rng.choice([1, 2, 3]), rng.choice([1, 2, 4])
+    hidden = 8 * rng.randint(4, 40)
+    windows = [rng.choice([0, 1, 2, 5, 16, 20, 33, 64, 100]) for _ in range(rng.randint(2, 4))]
+    pairing = rng.choice(["half", "half", "interleaved"])
+    vocab = rng.randint(50, 900)
+    inter = 8 * rng.randint(4, 40)
+
+    def build(cfg):
+        norm = PartSpec("rmsnorm", {"hidden_size": hidden, "eps": 1e-5})
+        ffn = PartSpec("swiglu", {"hidden_size": hidden, "intermediate_size": inter})
+        rope = {"kind": "rotary", "head_dim": hd, "theta": 1000.0, "max_position": 1024, "pairing": pairing}
+        layers = tuple(pre_norm_layer(f"model.layers.{i}", norm, PartSpec("attention", {
+            "hidden_size": hidden, "num_heads": kv * group, "num_kv_heads": kv, "head_dim": hd, "window": w,
+            "position": rope}), norm, ffn) for i, w in enumerate(windows))
+        sizes = {"vocab_size": vocab, "hidden_size": hidden}
+        return ModelSpec("ToyWindowsForCausalLM", vocab, hidden, 1024, PartSpec("token_embedding", sizes, "model.embed_tokens"),
+                         layers, tuple(PlanEntry(i) for i in range(len(windows))), norm.named("model.norm"),
+                         PartSpec("lm_head", dict(sizes, tied_to="model.embed_tokens"), "lm_head"))
+
+    register_architecture("ToyWindowsForCausalLM", dict, build)
+    try:
+        raw = {"architectures": ["ToyWindowsForCausalLM"], "hidden_size": hidden, "vocab_size": vocab}
+        page = rng.choice([1, 2, 4, 8, 16, 32, 3, 12])
+        n = rng.randint(1, 8)
+        lens = [rng.randint(1, 150) for _ in range(n)]
+        news = [rng.randint(1, 80) for _ in range(n)]
+        budget = rng.choice([4, 8, 16, 33, 64, 256, 2048])
+        seqs = rng.choice([1, 2, 3, 4, 8])
+        graphs = rng.random() < 0.7
+        burst = rng.choice([1, 4, 32])
+        dtype = rng.choice(["float32", "float32", "bfloat16"])
+        biggest = r64(max(l + m for l, m in zip(lens, news))) + 64
+        total = sum(r64(l + m) for l, m in zip(lens, news))
+        cache_tokens = rng.randint(biggest, max(total, biggest) + 64)
+        print(f"seed {seed}: hidden {hidden}, {kv * group}/{kv} heads of {hd}, windows {windows}, {pairing}, page {page}, "
+              f"{cache_tokens} cache tokens, budget {budget}, {seqs} live, graphs {graphs}, burst {burst}, {dtype}, "
+              f"(prompt, new) {list(zip(lens, news))}", flush=True)
+        eng = Engine(config=raw, dtype=dtype, weights_seed=seed, init_std=0.2, kv_block_size=page, max_num_seqs=seqs,
+                     max_num_batched_tokens=budget, max_cache_tokens=cache_tokens, use_graphs=graphs, decode_burst=burst)
+        cm = eng.runner.cache
+        assert len(cm.groups) == len(set(windows))
+        for g in cm.groups:
+            for t in g.tensors.values():
+                t.fill_(float("nan"))
+        prompts = [random_tokens(n_tok, vocab, 100 * i + seed) for i, n_tok in enumerate(lens)]
+        out = eng.generate(prompts, [SamplingParams.greedy(m, ignore_eos=True) for m in news])
+        cm.audit()
+        assert cm.free_blocks() == cm.group_blocks
+        whole = EngineConfig(dtype=dtype, kv_block_size=16, max_cache_tokens=biggest, max_num_seqs=2,
+                             max_num_batched_tokens=4096, use_graphs=False)
+        _, dec = random_model(raw, whole, seed=seed, std=0.2)
+        runner = build_runner(dec, whole)
+        tol = 2 * TOL[dtype]
+        for i, (p, o) in enumerate(zip(prompts, out)):
+            assert len(o) == news[i], (i, eng.requests[i].finish_reason)
+            toks = p + o
+            ref = runner.step([StepEntry("w", toks, list(range(len(p) - 1, len(toks) - 1)))]).float().cpu()
+            runner.finish("w")
+            for k, tok in enumerate(o):
+                assert float(ref[k].max() - ref[k][tok]) <= tol * float(ref[k].abs().max()), (i, k)
+    finally:
+        unregister_architecture("ToyWindowsForCausalLM")
