@@ -218,3 +218,57 @@ def test_random_windowed_architecture(seed):
                 assert float(ref[k].max() - ref[k][tok]) <= tol * float(ref[k].abs().max()), (i, k)
     finally:
         unregister_architecture("ToyWindowsForCausalLM")
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_seeded_sampling_is_the_same_under_any_schedule(seed):
+    """float32, requests with sampling settings and seeds drawn at random (some greedy, some ended
+    by an end-of-sequence token): each request alone in whole-prompt steps, then the batch under two
+    random schedules (the second in another order of arrival) give the same tokens, token for token:
+    a row's logits have the same bits whatever surrounds it, and the random numbers follow the
+    request's seed and position, not the step."""
+    from tiny_llm_amd import Engine, SamplingParams
+    rng = random.Random(31000 + seed)
+    cfg = random_config(rng)
+    cfg["num_hidden_layers"] = rng.randint(1, 2)
+    n = rng.randint(1, 10)
+    lens = [rng.randint(1, 100) for _ in range(n)]
+    news = [rng.randint(1, 60) for _ in range(n)]
+    sps = []
+    for i in range(n):
+        if rng.random() < 0.25:
+            sps.append(SamplingParams.greedy(news[i], ignore_eos=True))
+        else:
+            sps.append(SamplingParams(max_new_tokens=news[i], temperature=rng.choice([0.3, 0.7, 1.0, 1.5]),
+                                      top_k=rng.choice([0, 1, 5, 50]), top_p=rng.choice([0.5, 0.9, 0.95, 1.0]),
+                                      seed=rng.getrandbits(40), ignore_eos=rng.random() < 0.7))
+    with tempfile.TemporaryDirectory() as tmp:
+        folder = make_folder(tmp, cfg, seed=seed, std=0.03, norm_std=0.1, sharpen=2.0)
+        prompts = [random_tokens(n_tok, cfg["vocab_size"], 100 * i + seed) for i, n_tok in enumerate(lens)]
+        outs = []
+        for variant in range(3):
+            page = rng.choice(PAGE_SIZES)
+            budget = rng.choice([4, 8, 16, 33, 64, 256, 2048])
+            seqs = rng.choice([1, 2, 3, 4, 8, 16])
+            biggest = max(-(-(l + m) // page) for l, m in zip(lens, news))
+            total = sum(-(-(l + m) // page) for l, m in zip(lens, news))
+            blocks = rng.randint(biggest, max(biggest, total))
+            graphs = rng.random() < 0.7
+            burst = rng.choice([1, 4, 32])
+            if variant == 0:        # each request alone, whole prompts, eagerly
+                page, budget, seqs, graphs, burst = 16, 4096, 1, False, 1
+                blocks = -(-max(l + m for l, m in zip(lens, news)) // 16) + 1
+            print(f"seed {seed} variant {variant}: page {page}, budget {budget}, {seqs} live, {blocks} of {total} blocks, "
+                  f"graphs {graphs}, burst {burst}", flush=True)
+            eng = Engine(folder, dtype="float32", kv_block_size=page, num_kv_blocks=blocks, max_num_seqs=seqs,
+                         max_num_batched_tokens=budget, use_graphs=graphs, decode_burst=burst)
+            order = list(range(n))
+            if variant == 2:
+                rng.shuffle(order)
+            got = eng.generate([prompts[i] for i in order], [sps[i] for i in order])
+            back = [None] * n
+            for j, i in enumerate(order):
+                back[i] = got[j]
+            outs.append(back)
+            eng.runner.cache.audit()
+        assert outs[1] == outs[0] and outs[2] == outs[0]
