@@ -850,10 +850,49 @@ def test_toy_stateful_mixer_registers_builds_and_steps(tmp_path):
         runner.finish("a")
         again = runner.step([StepEntry("c", a, list(range(45)))]).cpu()
         assert rel_err(again, whole[:45]) < 1e-5
+        # As captured steps: the toy mixer runs loops on the host and may not be captured, so a step is
+        # the graph of the stages before it, the toy layer eagerly, the graph of the stages behind it.
+        # Each shape of step: first eagerly, then captured, then replayed; the same logits every time.
+        assert not runner.decoder.graph_safe and runner.graphs_possible
+        assert [(safe, first, last) for safe, first, last in runner.decoder.graph_runs()] == [(True, 0, 2), (False, 2, 3), (True, 3, 7)]
+        runner.finish("c")
+        for rid in ("g0", "g1", "g2", "g3"):
+            got = runner.step([StepEntry(rid, a, list(range(45)))], use_graph=True).cpu()
+            assert rel_err(got, whole[:45]) < 1e-5, rid
+            runner.finish(rid)
+        sg = next(g for k, g in runner._graphs.items() if k[0] == "mixed")
+        assert sg.runs_captured and [g is not None for g in sg.run_graphs] == [True, False, True] and sg.graph is None
+        before = runner.graph_steps
+        runner.step([StepEntry("h", a[:38], [])], use_graph=True)
+        runner.step([StepEntry("i", b[:20], [])], use_graph=True)
+        for t in range(38, 45):       # single tokens of two requests: one shape, captured at its second step
+            ents = [StepEntry("h", [a[t]], [0])] + ([StepEntry("i", [b[t - 18]], [0])] if t - 18 < 23 else [])
+            got = runner.step(ents, use_graph=True).cpu()
+            assert rel_err(got[0], whole[t]) < 1e-5, t
+            if len(ents) == 2:
+                assert rel_err(got[1], whole[45 + t - 18]) < 1e-5, t
+            runner.cache.audit()
+        assert runner.graph_steps - before >= 4
+        runner.finish("h")
+        runner.finish("i")
         # the state matters: another decay, other logits
         dec.layers[1].mixer.decay = 0.9
-        runner.finish("c")
         assert rel_err(runner.step([StepEntry("d", a, list(range(45)))]).cpu(), whole[:45]) > 1e-3
+        # through the entry point: the scheduler's steps, the sampler behind the last run of stages;
+        # the same tokens with graphs and without (runs of chained decode steps need the whole model
+        # in one graph: asked for, they fall back to single steps)
+        from tiny_llm_amd import Engine, SamplingParams
+        prompts = [a[:30], b, a[5:12]]
+        sps = [SamplingParams.greedy(20, ignore_eos=True), SamplingParams.greedy(9, ignore_eos=True),
+               SamplingParams(max_new_tokens=25, temperature=0.9, top_k=20, seed=5, ignore_eos=True)]
+        outs = []
+        for graphs in (False, True):
+            eng = Engine(config=raw, dtype="float32", weights_seed=1, init_std=0.3, kv_block_size=4, max_cache_tokens=256,
+                         max_num_seqs=3, max_num_batched_tokens=16, use_graphs=graphs, decode_burst=32)
+            outs.append(eng.generate(prompts, sps))
+            eng.runner.cache.audit()
+            assert (eng.runner.graph_steps > 20) == graphs
+        assert outs[0] == outs[1] and [len(o) for o in outs[0]] == [20, 9, 25]
     finally:
         MIXERS.unregister("toy_decay")
         unregister_architecture("ToyForCausalLM")

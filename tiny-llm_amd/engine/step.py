@@ -438,6 +438,12 @@ class ModelRunner:
         with ops.use_workspace(self.workspace):
             return self.decoder.forward(ctx)
 
+    @property
+    def graphs_possible(self) -> bool:
+        """Whether a step can run as HIP graphs: as one, if every part may be captured, or as the
+        capturable runs of its stages with the others eagerly between them."""
+        return any(safe for safe, _, _ in self.decoder.graph_runs())
+
     def _commit(self, rows: Sequence[_Row]) -> None:
         for r in rows:
             self.cache.commit(r.req_id, r.context_len + len(r.tokens))
@@ -447,7 +453,7 @@ class ModelRunner:
         """Runs the entries as one batch.  Returns float32 logits [wanted, vocab] on the
         device, in the order of the entries and of each entry's `want`.  If the forward pass
         raises, the cache is as it was before the call."""
-        if use_graph and self.decoder.graph_safe:
+        if use_graph and self.graphs_possible:
             return self._graph_step(entries, None)[0]
         ctx, _, _, rows = self.prepare(entries)
         try:
@@ -467,7 +473,7 @@ class ModelRunner:
         n_out = sum(len(e.want) for e in entries)
         if len(samples) != n_out:
             raise StepError(f"{n_out} rows are wanted, {len(samples)} sampling settings were given")
-        if use_graph and self.decoder.graph_safe:
+        if use_graph and self.graphs_possible:
             return self._graph_step(entries, samples)[1]
         ctx, lay, dev, rows = self.prepare(entries, samples)
         try:
@@ -607,7 +613,8 @@ class StepGraph:
         self.out = torch.zeros(max(self.n_out, 1), dtype=torch.int32, device=runner.device)
         self.out_host = torch.zeros(max(self.n_out, 1), dtype=torch.int32, pin_memory=True)
         # a decode step with its sampler ends by preparing the next one on the device (bursts)
-        self.feeds_next = self.max_q_len == 1 and self.sampling and self.n_out == self.R == self.T and G <= ops.MAX_CACHE_GROUPS
+        self.feeds_next = (self.max_q_len == 1 and self.sampling and self.n_out == self.R == self.T
+                           and G <= ops.MAX_CACHE_GROUPS and runner.decoder.graph_safe)
         self.history_steps = self.BURST_STEPS if self.feeds_next else 0
         if self.feeds_next:
             self.history = torch.zeros(self.history_steps * self.R, dtype=torch.int32, device=runner.device)
@@ -616,11 +623,22 @@ class StepGraph:
         self.chain = None
         self.bursts = 0         # runs of steps this shape has served
         self._uploaded: Optional[torch.cuda.Event] = None
+        # A model with a part that may not be captured: the runs of its stages, one graph for each
+        # capturable run and the place where each run leaves the residual stream for the next.
+        runs = runner.decoder.graph_runs()
+        self.stage_runs = None if len(runs) == 1 and runs[0][0] else runs
+        self.run_graphs: List[Optional[torch.cuda.CUDAGraph]] = [None] * len(runs)
+        self.run_out: List[Optional[torch.Tensor]] = [None] * len(runs)
+        self.runs_captured = False
 
     BURST_STEPS = 32        # most decode steps a burst may hold
 
     def _body(self):
         self.logits = self.runner._forward(self.ctx)
+        self._tail()
+
+    def _tail(self):
+        """Behind the logits: the sampler and, in a decode step that may be chained, the next step's metadata."""
         if self.sampling and self.n_out:
             ops.sample(self.logits, self.out[:self.n_out], *self.layout.sampler_args(self.dev))
         if self.feeds_next:
@@ -628,6 +646,43 @@ class StepGraph:
             ops.decode_advance(ctx.tokens, ctx.positions, ctx.seq_lens, lay.sec(self.dev, "counters"), self.out,
                                self.history, lay.sec(self.dev, "burst_step"), ctx.slot_mappings,
                                ctx.block_tables, ctx.block_size)
+
+    def _stage_run(self, first: int, last: int, x):
+        """Stages first .. last - 1 on the static buffers; the last run ends with the sampler."""
+        runner = self.runner
+        with ops.use_workspace(runner.workspace):
+            y = runner.decoder.run_stages(self.ctx, first, last, x)
+        if last == runner.decoder.num_stages:
+            self.logits = y
+            self._tail()
+        return y
+
+    def _body_in_runs(self, capture: bool) -> None:
+        """The step of a model that holds a part which may not be captured: every capturable run of
+        stages replays its graph (or is captured now and then replayed), the others run eagerly on the
+        same static buffers.  What an eager run leaves has a new address every time, so it is copied
+        to a fixed place, from which the graph behind it reads."""
+        runner = self.runner
+        x = None
+        for k, (safe, first, last) in enumerate(self.stage_runs):
+            if safe and self.run_graphs[k] is None and capture:
+                self.ctx.static = True
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, pool=runner._graph_pool):
+                    self.run_out[k] = self._stage_run(first, last, x)
+                self.run_graphs[k] = graph
+            if safe and self.run_graphs[k] is not None:
+                self.run_graphs[k].replay()
+                x = self.run_out[k]
+                continue
+            self.ctx.static = False
+            y = self._stage_run(first, last, x)
+            if last < runner.decoder.num_stages:
+                if self.run_out[k] is None or self.run_out[k].shape != y.shape or self.run_out[k].dtype != y.dtype:
+                    self.run_out[k] = torch.empty_like(y)
+                self.run_out[k].copy_(y)
+                y = self.run_out[k]
+            x = y
 
     def burst(self, rows: Sequence[_Row], samples, steps: int) -> List[List[int]]:
         """Uploads the first step's metadata and replays the captured step `steps` times; each
@@ -658,7 +713,7 @@ class StepGraph:
 
     def run(self, rows: Sequence[_Row], samples, n_out: int):
         runner = self.runner
-        if self.graph is None and self.max_q_len > 1 and self.widths != runner._tile_widths:
+        if self.graph is None and not self.runs_captured and self.max_q_len > 1 and self.widths != runner._tile_widths:
             self._build()                       # a kernel asked for a tile width this layout lacks
         if self._uploaded is not None:
             self._uploaded.synchronize()        # the last upload has left the pinned buffer
@@ -673,9 +728,7 @@ class StepGraph:
         elif self.runs == 0 or self.capture_failed:
             # eager on the static buffers; the host copies a part may look at are those of this step
             self.ctx.static = False
-            self.ctx.q_lens = [len(r.tokens) for r in rows] + [0] * (self.R - len(rows))
-            self.ctx.context_lens = [r.context_len for r in rows] + [0] * (self.R - len(rows))
-            self.ctx.slots_host = [r.slot for r in rows] + [0] * (self.R - len(rows))
+            self._host_copies(rows)
             self.ctx._on_new_width = runner._new_width
             if self.max_q_len > 1:
                 for w in runner._tile_widths - self.widths:
@@ -685,6 +738,18 @@ class StepGraph:
             for w in set(self.ctx._tiles) - known:      # built for this step only: not part of the layout
                 del self.ctx._tiles[w]
             runner.eager_steps += 1
+        elif self.stage_runs is not None:
+            # graphs for the capturable runs of stages (captured at this shape's second step), the
+            # other runs eagerly between them with this step's host copies
+            self._host_copies(rows)
+            known = set(self.ctx._tiles)
+            if self.runs_captured:
+                self._body_in_runs(capture=False)
+            else:
+                self._capture_runs()
+            for w in set(self.ctx._tiles) - known:
+                del self.ctx._tiles[w]
+            runner.graph_steps += 1
         else:
             self._capture()
             runner.graph_steps += 1
@@ -698,6 +763,36 @@ class StepGraph:
             return None, toks
         # the logits live in memory the next replay overwrites: the caller gets a copy
         return self.logits[:n_out].clone(), toks
+
+    def _host_copies(self, rows: Sequence[_Row]) -> None:
+        """What a part that runs eagerly may read on the host: this step's lengths and slots."""
+        pad = [0] * (self.R - len(rows))
+        self.ctx.q_lens = [len(r.tokens) for r in rows] + pad
+        self.ctx.context_lens = [r.context_len for r in rows] + pad
+        self.ctx.slots_host = [r.slot for r in rows] + pad
+
+    def _capture_runs(self) -> None:
+        """Captures the capturable runs of stages, one graph each, while the step runs."""
+        runner = self.runner
+        torch.cuda.synchronize()
+        collecting = gc.isenabled()
+        gc.disable()                        # as in _capture: nothing may be finalised during a capture
+        self.ctx._on_new_width = None
+        if runner._graph_pool is None:
+            runner._graph_pool = torch.cuda.graph_pool_handle()
+        try:
+            self._body_in_runs(capture=True)
+            self.runs_captured = True
+        except StepError:
+            # a part asked for something that was not laid out: this shape keeps running eagerly
+            self.capture_failed = True
+            self.run_graphs = [None] * len(self.run_graphs)
+            self.ctx.static = False
+            torch.cuda.synchronize()
+            self._body()
+        finally:
+            if collecting:
+                gc.enable()
 
     CHAIN = 4               # decode steps captured as ONE graph for bursts
 

@@ -66,6 +66,7 @@ class Decoder:
         self.caches: List[Dict[str, LayerCache]] = [{} for _ in spec.plan]
         self.states: List[Dict[str, torch.Tensor]] = [{} for _ in spec.plan]
         self._graph_safe: Optional[bool] = None
+        self._graph_runs: Optional[List[tuple]] = None
 
     # ---------------------------------------------------------------- declarations
     def parts(self) -> List[Part]:
@@ -124,27 +125,72 @@ class Decoder:
         return out
 
     # --------------------------------------------------------------------- compute
+    # The pass in stages: stage 0 embeds the tokens, stage 1 + i is entry i of the plan, the last
+    # one is the final norm and the head.  A step runs all of them in one call; a captured step of
+    # a model that holds a part which may not be captured runs them in runs of stages, the
+    # capturable runs as HIP graphs and the others eagerly between them.
+    @property
+    def num_stages(self) -> int:
+        return len(self.spec.plan) + 2
+
+    def stage_graph_safe(self, stage: int) -> bool:
+        if stage == 0:
+            parts = [self.embedding]
+        elif stage == self.num_stages - 1:
+            parts = [self.final_norm, self.lm_head]
+        else:
+            parts = self.layers[self.spec.plan[stage - 1].layer].parts()
+        parts = parts + [getattr(p, "position", None) for p in parts]
+        return all(p.graph_safe for p in parts if p is not None)
+
+    def graph_runs(self) -> List[tuple]:
+        """The stages in runs that may be captured and runs that may not: (capturable, first, last)
+        with stages first .. last - 1, in order."""
+        if self._graph_runs is None:
+            runs: List[tuple] = []
+            for st in range(self.num_stages):
+                safe = self.stage_graph_safe(st)
+                if runs and runs[-1][0] == safe:
+                    runs[-1] = (safe, runs[-1][1], st + 1)
+                else:
+                    runs.append((safe, st, st + 1))
+            self._graph_runs = runs
+        return self._graph_runs
+
     def forward(self, ctx) -> torch.Tensor:
         """Runs the tokens of `ctx` through the plan; float32 logits at ctx.logit_rows."""
-        x = self.embedding.forward(ctx.tokens, ctx)
+        return self.run_stages(ctx, 0, self.num_stages, None)
+
+    def run_stages(self, ctx, first: int, last: int, x: Optional[torch.Tensor]) -> torch.Tensor:
+        """Stages first .. last - 1.  `x` is the residual stream the stage before `first` left (None
+        for stage 0).  Returns the residual stream, or, behind the last stage, the logits.  A norm is
+        handed from one block to the next only inside one call."""
+        n = self.num_stages
+        plan = self.spec.plan
         wants_logits = ctx.logit_rows is not None and ctx.logit_rows.numel() > 0
         # a head that says so may receive the final norm unevaluated and fuse it into its product
         lazy_head = hasattr(self.final_norm, "lazy") and getattr(self.lm_head, "accepts_lazy_norm", False)
-        plan = self.spec.plan
+        if first == 0:
+            x = self.embedding.forward(ctx.tokens, ctx)
         # A block may prepare the norm that reads its result (the next block's first norm, or the
         # final norm) in its last product; `prepared` carries that from one block to the next.
         prepared = None
-        for i, e in enumerate(plan):
-            block = self.layers[e.layer].block
+        for st in range(max(first, 1), min(last, n - 1)):
+            i = st - 1
+            block = self.layers[plan[i].layer].block
             if not hasattr(block, "forward_chained"):
                 x, prepared = block.forward(x, ctx, self.caches[i], self.states[i]), None
                 continue
-            if i + 1 < len(plan):
-                nxt = self.layers[plan[i + 1].layer].block
-                next_norm = getattr(nxt, "first_norm", None) if hasattr(nxt, "forward_chained") else None
-            else:
-                next_norm = self.final_norm if wants_logits and lazy_head else None
+            next_norm = None
+            if st + 1 < last:                    # what reads this block's result runs in this call
+                if i + 1 < len(plan):
+                    nxt = self.layers[plan[i + 1].layer].block
+                    next_norm = getattr(nxt, "first_norm", None) if hasattr(nxt, "forward_chained") else None
+                else:
+                    next_norm = self.final_norm if wants_logits and lazy_head else None
             x, prepared = block.forward_chained(x, ctx, self.caches[i], self.states[i], prepared, next_norm)
+        if last < n:
+            return x
         if not wants_logits:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=x.device)
         norm = self.final_norm
