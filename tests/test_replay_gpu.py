@@ -196,7 +196,7 @@ def test_trace_run_program(dtype, graphs, tmp_path_factory, tmp_path):
     out_dir = tmp_path / "out"
     proc = subprocess.run(
         [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
-         "--out", str(out_dir), "--max-tokens", str(peak)] + (["--graphs"] if graphs else []),
+         "--out", str(out_dir), "--max-tokens", str(peak)] + (["--graphs", "--npy"] if graphs else []),
         input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=600)
     assert proc.returncode == 0, proc.stderr[-3000:]
     assert [l for l in proc.stdout.splitlines() if l.startswith("done ")] == [f"done {s['step']}" for s in steps]
@@ -206,4 +206,6 @@ def test_trace_run_program(dtype, graphs, tmp_path_factory, tmp_path):
         arr = np.fromfile(out_dir / f"{step}.f32", dtype="<f4")
         assert arr.size == len(where) * vocab
         out[step] = torch.from_numpy(arr.reshape(len(where), vocab))
+        if graphs:
+            assert np.array_equal(np.load(out_dir / f"{step}.npy"), arr.reshape(len(where), vocab))
     check(out, steps, ref, TOL[dtype])
