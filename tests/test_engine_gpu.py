@@ -1054,6 +1054,150 @@ def test_toy_routed_feed_forward_and_other_position_encoding(dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_block_arrangement_and_norm(dtype):
+    """Another arrangement of a layer's parts (one norm; mixer and feed-forward both read it and both
+    add to the residual stream) and another norm (mean taken out, gain and bias), both defined here,
+    in a toy architecture with interleaved rotary pairs and scaled positions.  Against a plain
+    float64 model written here from the plain parts; whole, in portions, as captured steps, and in
+    runs of chained decode steps through the entry point (every part says it may be captured)."""
+    from tiny_llm_amd import Engine, SamplingParams
+    from tiny_llm_amd.config import (EngineConfig, LayerSpec, ModelSpec, PartSpec, PlanEntry, register_architecture,
+                                     resolve, unregister_architecture)
+    from tiny_llm_amd.engine.loading import build_runner, random_model
+    from tiny_llm_amd.engine.step import StepEntry
+    from tiny_llm_amd.models.decoder import Decoder
+    from tiny_llm_amd.parts import BLOCKS, NORMS, Block, Norm, WeightSpec, register_block, register_norm
+    from tiny_llm_amd.weights.loader import random_tensor
+
+    class CentredNorm(Norm):
+        graph_safe = True           # device work only, nothing of the step read on the host
+
+        def __init__(self, prefix, dtype, device, *, hidden_size, eps):
+            super().__init__(prefix, dtype, device)
+            self.H, self.eps = hidden_size, eps
+
+        def weights(self):
+            return [WeightSpec(f"{self.prefix}.gain", (self.H,), role="vector", init="around_one"),
+                    WeightSpec(f"{self.prefix}.bias", (self.H,), role="vector")]
+
+        def bind(self, tensors):
+            self.gain, self.bias = tensors[f"{self.prefix}.gain"].float(), tensors[f"{self.prefix}.bias"].float()
+
+        def forward(self, x, rows=None):
+            if rows is not None:
+                x = x[rows.long()]
+            x = x.float()
+            c = x - x.mean(dim=-1, keepdim=True)
+            y = c * torch.rsqrt((c * c).mean(dim=-1, keepdim=True) + self.eps) * self.gain + self.bias
+            return y.to(self.dtype).contiguous()
+
+    class ParallelBlock(Block):
+        roles = {"norm": "norm", "mixer": "mixer", "ffn": "feed_forward"}
+
+        def forward(self, x, ctx, caches, states):
+            p = self._parts
+            h = p["norm"].forward(x)
+            x = p["mixer"].forward(h, ctx, caches.get("mixer"), states.get("mixer"), x)
+            return p["ffn"].forward(h, ctx, x)
+
+    H, V, HD, NQ, NKV, I, EPS, THETA, FACTOR = 72, 131, 24, 4, 2, 104, 1e-5, 300.0, 2.0
+
+    def build(cfg):
+        norm = PartSpec("centred_norm", {"hidden_size": H, "eps": EPS})
+        rope = {"kind": "rotary", "head_dim": HD, "theta": THETA, "max_position": 256, "pairing": "interleaved",
+                "scaling": {"kind": "linear", "factor": FACTOR}}
+        attn = PartSpec("attention", {"hidden_size": H, "num_heads": NQ, "num_kv_heads": NKV, "head_dim": HD, "position": rope})
+        ffn = PartSpec("swiglu", {"hidden_size": H, "intermediate_size": I})
+        layers = tuple(LayerSpec(f"blocks.{i}", "parallel", {"norm": norm.named("ln"), "mixer": attn.named("attn"),
+                                                               "ffn": ffn.named("mlp")}) for i in range(2))
+        sizes = {"vocab_size": V, "hidden_size": H}
+        return ModelSpec("Toy4ForCausalLM", V, H, 256, PartSpec("token_embedding", sizes, "wte"), layers,
+                         (PlanEntry(0), PlanEntry(1)), norm.named("ln_f"),
+                         PartSpec("lm_head", dict(sizes, tied_to="wte"), "lm_head"))
+
+    register_norm("centred_norm", CentredNorm)
+    register_block("parallel", ParallelBlock)
+    register_architecture("Toy4ForCausalLM", dict, build)
+    try:
+        raw = {"architectures": ["Toy4ForCausalLM"]}
+        SEED, STD, NSTD = 3, 0.2, 0.1
+        # the plain model, float64, from the plain parts and the weights by name
+        _, spec = resolve(raw)
+        w = {ws.name: random_tensor(ws, SEED, STD, NSTD).double() for ws in Decoder(spec, "float32", "cpu").weight_specs()
+             if ws.alias_of is None}           # (the head is tied to the embedding table)
+        assert sorted(w) == sorted(["wte.weight", "ln_f.gain", "ln_f.bias"] + [
+            f"blocks.{i}.{n}" for i in range(2) for n in ("ln.gain", "ln.bias", "attn.q_proj.weight", "attn.k_proj.weight",
+                                                          "attn.v_proj.weight", "attn.o_proj.weight", "mlp.gate_proj.weight",
+                                                          "mlp.up_proj.weight", "mlp.down_proj.weight")])
+        if dtype == "bfloat16":
+            w = {k: (t.to(torch.bfloat16).double() if t.dim() == 2 else t) for k, t in w.items()}
+        cos, sin = plain.rope_table_fast(256, HD, THETA, position_factor=FACTOR)
+
+        def centred(x, pre):
+            c = x - x.mean(dim=-1, keepdim=True)
+            return c / torch.sqrt((c * c).mean(dim=-1, keepdim=True) + EPS) * w[f"{pre}.gain"] + w[f"{pre}.bias"]
+
+        def reference(tokens):
+            T = len(tokens)
+            x = w["wte.weight"][list(tokens)]
+            for i in range(2):
+                pre = f"blocks.{i}"
+                h = centred(x, f"{pre}.ln")
+                q = plain.linear(h, w[f"{pre}.attn.q_proj.weight"]).reshape(T, NQ, HD)
+                k = plain.linear(h, w[f"{pre}.attn.k_proj.weight"]).reshape(T, NKV, HD)
+                v = plain.linear(h, w[f"{pre}.attn.v_proj.weight"]).reshape(T, NKV, HD)
+                q, k = (plain.apply_rope_interleaved(t, range(T), cos, sin) for t in (q, k))
+                a = plain.attention_fast(q, k, v, range(T)).reshape(T, NQ * HD)
+                x = x + plain.linear(a, w[f"{pre}.attn.o_proj.weight"]) + plain.swiglu(
+                    h, w[f"{pre}.mlp.gate_proj.weight"], w[f"{pre}.mlp.up_proj.weight"], w[f"{pre}.mlp.down_proj.weight"])
+            return plain.linear(centred(x, "ln_f"), w["wte.weight"])
+
+        a, b = random_tokens(70, V, 11), random_tokens(29, V, 12)
+        ref_a, ref_b = reference(a), reference(b)
+        tol = 1e-4 if dtype == "float32" else 3e-2      # bfloat16: the plain model here rounds nothing but the weights
+        engine = EngineConfig(dtype=dtype, kv_block_size=8, max_cache_tokens=256, max_num_seqs=3,
+                              max_num_batched_tokens=80, use_graphs=True)
+        _, dec = random_model(raw, engine, seed=SEED, std=STD, norm_std=NSTD)
+        assert dec.graph_safe
+        runner = build_runner(dec, engine)
+        for g in runner.cache.groups:
+            for t in g.tensors.values():
+                t.fill_(float("nan"))
+        whole = runner.step([StepEntry("a", a, list(range(70)))]).cpu()
+        assert rel_err(whole, ref_a) < tol
+        runner.finish("a")
+        for graphs in (False, True, True, True):
+            got_a, got_b, at_a, at_b = [], [], 0, 0
+            for na, nb in [(7, 2), (2, 0), (19, 11), (1, 1), (40, 14), (1, 1)]:
+                ents = [StepEntry("a", a[at_a:at_a + na], list(range(na)))]
+                if nb:
+                    ents.append(StepEntry("b", b[at_b:at_b + nb], list(range(nb))))
+                out = runner.step(ents, use_graph=graphs).cpu()
+                got_a.append(out[:na])
+                got_b.append(out[na:])
+                at_a, at_b = at_a + na, at_b + nb
+            assert at_a == 70 and at_b == 29
+            assert rel_err(torch.cat(got_a), ref_a) < tol and rel_err(torch.cat(got_b), ref_b) < tol
+            runner.finish("a")
+            runner.finish("b")
+        assert runner.graph_steps >= 8
+        # through the entry point, with runs of chained decode steps: the plain model's greedy tokens
+        eng = Engine(config=raw, dtype=dtype, weights_seed=SEED, init_std=STD, norm_std=NSTD, kv_block_size=8,
+                     max_cache_tokens=256, max_num_seqs=3, max_num_batched_tokens=32, decode_burst=32)
+        out = eng.generate([a[:20], b[:9]], SamplingParams.greedy(40, ignore_eos=True))
+        assert any(g.bursts > 0 for g in eng.runner._graphs.values())
+        for p, o in zip([a[:20], b[:9]], out):
+            ref = reference(p + o)
+            for k, tok in enumerate(o):
+                row = ref[len(p) + k - 1]
+                assert float(row.max() - row[tok]) <= 2 * tol * float(row.abs().max()), k
+    finally:
+        NORMS.unregister("centred_norm")
+        BLOCKS.unregister("parallel")
+        unregister_architecture("Toy4ForCausalLM")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_chained_decode_steps_with_several_cache_groups(dtype):
     """A toy architecture whose three attention layers keep caches of three kinds (every position;
     a window of 20; every position with other kv heads): three cache groups with pools of their own
