@@ -370,7 +370,8 @@ def test_linear_swiglu_epilogue(dtype, M, K, N):
 
 
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 40, 64])
-@pytest.mark.parametrize("K,N", [(64, 250), (2048, 2560), (176, 96), (4096, 64), (5120, 520), (2048, 11264), (300, 4100)])
+@pytest.mark.parametrize("K,N", [(64, 250), (2048, 2560), (176, 96), (4096, 64), (5120, 520), (2048, 11264), (300, 4100),
+                                 (1024, 12300)])
 def test_linear_norm_f32(M, K, N):
     """Float32, few rows: the norm inside the product's kernel against norm, then product, in double;
     with the SiLU-gate epilogue and with a residual; and a row gives the same bits alone and in a batch."""
@@ -403,8 +404,11 @@ def test_linear_norm_f32(M, K, N):
     ops().linear_norm_f32(x[m:m + 1].contiguous(), nw, eps, w, alone)
     assert torch.equal(alone, out[m:m + 1])
     assert not ops().linear_norm_f32_ok(65, N, K, K)
-    # the norm as two kernels (what steps of more rows take): the same BITS, with every epilogue, also
+    # the norm as two kernels (what steps of more rows take, and wide products, where a workgroup of
+    # the plain product owns two or three column tiles): the same BITS, with every epilogue, also
     # when the rows sit among many others (the tiled product) and when they are gathered
+    tiles = -(-N // 16)
+    assert ops().linear_f32_col_tiles(M, N, K) == (min(3, -(-tiles // 256)) if M <= 16 and tiles > 256 else 1)
     hp, inv = ops().norm_prescale_f32(x, nw, eps)
     assert rel(hp, (x * nw).double().cpu()) == 0.0
     two = torch.full((M, N), float("nan"), device=DEV)

@@ -251,7 +251,14 @@ constexpr int FR_WAVES = 8, FR_THREADS = FR_WAVES * TL_WAVE, FR_MAX_MT = 4;
 // are loaded, their squares are added up on the way (per k block and row in a fixed order, the
 // blocks in ascending order, so a row's factor depends on nothing but the row), and the factor is
 // applied to the block sums' total.  That saves the norm's kernel in front of the product.
-template <bool SWIGLU, int COLS, bool NORM = false, bool WIDE = false>
+//
+// CT (one row tile only): a workgroup owns CT column tiles side by side.  The activations of a k block,
+// which weigh as much as one tile's weights, are fetched once for all of them, and a wide product
+// (gate and up, the output head) becomes one or two rounds of workgroups instead of three to eight.
+// The weights come as a chain of pieces, the block's tiles and then the wave's next block, each
+// requested while the piece before it is multiplied.  A tile's block sums are what they are with one
+// tile a workgroup, bit for bit.
+template <bool SWIGLU, int COLS, bool NORM = false, bool WIDE = false, int CT = 1>
 __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* __restrict__ a,
                                                                    const float* __restrict__ w,
                                                                    float* __restrict__ out,
@@ -267,14 +274,16 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
   // this one is multiplied, and the registers that takes are those of the next block's weights, which
   // are requested behind the block's last row tile instead.
   static_assert(!(NORM && WIDE), "the norm rides in the product of one row tile");
-  extern __shared__ float rows_smem[];      // [m tiles][k blocks][16 rows][COLS columns], NORM: + [m tiles][k blocks][16]
+  static_assert(CT >= 1 && CT <= 3 && !(WIDE && CT > 1) && !(NORM && CT > 1), "several column tiles go with one row tile and no norm");
+  extern __shared__ float rows_smem[];      // [m tiles][CT][k blocks][16 rows][COLS columns], NORM: + [m tiles][k blocks][16]
   const int nkb = (K + F_KBLOCK - 1) / F_KBLOCK;
   const int mt0 = WIDE ? blockIdx.y * tiles_wg : 0;                       // first row tile of this workgroup
   const int mts = WIDE ? min(tiles_wg, (M + 15) / 16 - mt0) : (M + 15) / 16;   // and how many it owns
   const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
   const int l16 = lane % 16, kk = lane / 16;
-  const int n0 = blockIdx.x * COLS;
-  const float* wrow = w + (int64_t)min(n0 + l16 % COLS, N - 1) * K;
+  const int n0 = blockIdx.x * COLS * CT;
+  auto wrow_of = [&](int ct) { return w + (int64_t)min(n0 + ct * COLS + l16 % COLS, N - 1) * K; };
+  const float* wrow = wrow_of(0);
   // A k block that lies wholly inside K is loaded without a predicate per load (each would be a
   // branch of its own, and the waits around branches are placed for the worst case); only the last,
   // partial block of an inner size that is no multiple of 256 takes the predicated loads.  The loop
@@ -292,16 +301,33 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
     if (wave * F_KBLOCK + F_KBLOCK <= K) load16(std::true_type{}, wv, wrow, wave * F_KBLOCK);
     else load16(std::false_type{}, wv, wrow, wave * F_KBLOCK);
   }
-  float* ss_smem = rows_smem + mts * nkb * 16 * COLS;
-  // one row tile of one k block: the block sum of 16 rows x COLS columns goes to LDS
-  auto multiply = [&](f32x4 (&av)[16], int mt, int b) {
+  float* ss_smem = rows_smem + mts * CT * nkb * 16 * COLS;
+  // one row tile and column tile of one k block: the block sum of 16 rows x COLS columns goes to LDS
+  auto multiply = [&](f32x4 (&av)[16], int mt, int b, int ct = 0) {
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int g = 0; g < 16; ++g)
 #pragma unroll
       for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wv[g][e], av[g][e], acc, 0, 0, 0);
     // lane (l16, kk): row m = l16, columns 4 kk + r
-    if (kk * 4 < COLS) *(f32x4*)(&rows_smem[((mt * nkb + b) * 16 + l16) * COLS + kk * 4]) = acc;
+    if (kk * 4 < COLS) *(f32x4*)(&rows_smem[(((mt * CT + ct) * nkb + b) * 16 + l16) * COLS + kk * 4]) = acc;
+  };
+  // NORM: the rows times the norm's weights, their squares added up on the way (one row tile of one k block)
+  auto scale_rows = [&](auto whole, f32x4 (&av)[16], int mt, int b) {
+    f32x4 nw[16];
+    load16(whole, nw, norm_w, b * F_KBLOCK);      // 4 * K bytes, from the caches
+    float ss = 0.f;
+#pragma unroll
+    for (int g = 0; g < 16; ++g)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        ss = __builtin_fmaf(av[g][e], av[g][e], ss);
+        av[g][e] *= nw[g][e];
+      }
+    // the four lanes of a row (one per k quarter): every lane gets (s0 + s1) + (s2 + s3)
+    ss += __shfl_xor(ss, 16, TL_WAVE);
+    ss += __shfl_xor(ss, 32, TL_WAVE);
+    if (kk == 0) ss_smem[(mt * nkb + b) * 16 + l16] = ss;
   };
   auto block = [&](auto whole, auto next_whole, int b) {
     const int kb = b * F_KBLOCK;
@@ -325,26 +351,24 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
         }
       }
       if (b + FR_WAVES < nkb) load16(next_whole, wv, wrow, kb + FR_WAVES * F_KBLOCK);
+    } else if constexpr (CT > 1) {
+      // one row tile, no norm
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) {
+        const bool more = ct + 1 < CT || b + FR_WAVES < nkb;
+        if (ct + 1 < CT) load16(whole, wnext, wrow_of(ct + 1), kb);
+        else if (b + FR_WAVES < nkb) load16(next_whole, wnext, wrow, kb + FR_WAVES * F_KBLOCK);
+        multiply(av, 0, b, ct);
+        if (more) {
+#pragma unroll
+          for (int g = 0; g < 16; ++g) wv[g] = wnext[g];
+        }
+      }
     } else {
       if (!NORM && b + FR_WAVES < nkb) load16(next_whole, wnext, wrow, kb + FR_WAVES * F_KBLOCK);
       for (int mt = 0; mt < mts; ++mt) {
         if (mt > 0) load16(whole, av, a_row(mt), kb);
-        if constexpr (NORM) {
-          f32x4 nw[16];
-          load16(whole, nw, norm_w, kb);      // 4 * K bytes, from the caches
-          float ss = 0.f;
-#pragma unroll
-          for (int g = 0; g < 16; ++g)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              ss = __builtin_fmaf(av[g][e], av[g][e], ss);
-              av[g][e] *= nw[g][e];
-            }
-          // the four lanes of a row (one per k quarter): every lane gets (s0 + s1) + (s2 + s3)
-          ss += __shfl_xor(ss, 16, TL_WAVE);
-          ss += __shfl_xor(ss, 32, TL_WAVE);
-          if (kk == 0) ss_smem[(mt * nkb + b) * 16 + l16] = ss;
-        }
+        if constexpr (NORM) scale_rows(whole, av, mt, b);
         multiply(av, mt, b);
       }
       if constexpr (NORM) {
@@ -362,16 +386,16 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
     else block(std::false_type{}, std::false_type{}, b);
   }
   __syncthreads();
-  for (int e = tid; e < mts * 16 * COLS; e += FR_THREADS) {
-    const int mt = e / (16 * COLS), r = (e % (16 * COLS)) / COLS, c = e % COLS;
+  for (int e = tid; e < mts * CT * 16 * COLS; e += FR_THREADS) {
+    const int tile = e / (16 * COLS), mt = tile / CT, ct = tile % CT, r = (e % (16 * COLS)) / COLS, c = e % COLS;
     float t = 0.f;
-    for (int b = 0; b < nkb; ++b) t += rows_smem[((mt * nkb + b) * 16 + r) * COLS + c];
+    for (int b = 0; b < nkb; ++b) t += rows_smem[((tile * nkb + b) * 16 + r) * COLS + c];
     if constexpr (NORM) {
       float q = 0.f;
       for (int b = 0; b < nkb; ++b) q += ss_smem[(mt * nkb + b) * 16 + r];
       t *= f32_norm_factor(q, K, eps);
     }
-    const int m = (mt0 + mt) * 16 + r, n = n0 + c;
+    const int m = (mt0 + mt) * 16 + r, n = n0 + ct * COLS + c;
     if constexpr (!NORM) {
       if (row_scale && m < M) t *= row_scale[m];    // the factor of a norm in front (norm_prescale_f32_kernel)
     }
@@ -1590,6 +1614,19 @@ static int launch_skinny_out(const SkinnyArgs& p, int out_dtype, bool swiglu, hi
   return TL_ERR_ARG;
 }
 
+// Column tiles a workgroup of the float32 few-row kernel owns: one, or, with one row tile and more
+// than 256 column tiles of 16, as many (up to three: four would not leave the registers for a piece of
+// weights ahead) as bring the workgroups down to one to three rounds over the 256 compute units,
+// while the block sums fit into LDS.
+static int f32_rows_col_tiles(int M, int N, int K, int cols) {
+  if (M > 16 || cols != 16) return 1;
+  const int tiles = (N + 15) / 16, nkb = (K + F_KBLOCK - 1) / F_KBLOCK;
+  int ct = tiles > 256 ? (tiles + 255) / 256 : 1;
+  if (ct > 3) ct = 3;
+  while (ct > 1 && (size_t)nkb * 16 * 16 * ct * sizeof(float) > 96 * 1024) --ct;
+  return ct;
+}
+
 }  // namespace
 
 extern "C" {
@@ -1602,6 +1639,14 @@ int tl_linear_norm_f32_ok(int M, int N, int K, int64_t lda) {
   const int cols = (N + 7) / 8 <= 256 ? 8 : 16;
   const size_t smem = (size_t)mts * nkb * 16 * (cols + 1) * sizeof(float);
   return M > 0 && M <= 16 * FR_MAX_MT && K % 4 == 0 && lda % 4 == 0 && smem <= 96 * 1024;
+}
+
+// Column tiles the plain float32 few-row product gives a workgroup at these sizes.  More than one: the
+// product is so wide that a norm in front of it is cheaper as a kernel of its own (tl_norm_prescale_f32)
+// with its factors applied to this product's sums than inside tl_linear_norm_f32, which fetches a
+// workgroup's activation rows once per column tile; the bits are the same either way.
+int tl_linear_f32_col_tiles(int M, int N, int K) {
+  return f32_rows_col_tiles(M, N, K, (N + 7) / 8 <= 256 ? 8 : 16);
 }
 
 int tl_linear_norm_f32(const float* x, const float* norm_w, float eps, const float* w, float* out,
@@ -1691,30 +1736,42 @@ int tl_linear_tile(const void* a, const void* w, void* out, const float* residua
         groups *= 2;
     }
     const int tiles_wg = (mts + groups - 1) / groups;
-    const size_t rows_smem = (size_t)tiles_wg * nkb * 16 * cols * sizeof(float);
+    const int ct = f32_rows_col_tiles(M, N, K, cols);
+    const size_t rows_smem = (size_t)tiles_wg * nkb * 16 * cols * ct * sizeof(float);
     if (M <= 16 * FR_MAX_MT && vec && rows_smem <= 96 * 1024) {
       static bool configured = false;
       if (!configured) {
-        const void* kernels[6] = {(const void*)gemm_f32_rows_kernel<true, 16>, (const void*)gemm_f32_rows_kernel<false, 16>,
-                                  (const void*)gemm_f32_rows_kernel<true, 8>, (const void*)gemm_f32_rows_kernel<false, 8>,
-                                  (const void*)gemm_f32_rows_kernel<true, 16, false, true>,
-                                  (const void*)gemm_f32_rows_kernel<false, 16, false, true>};
+        const void* kernels[10] = {(const void*)gemm_f32_rows_kernel<true, 16>, (const void*)gemm_f32_rows_kernel<false, 16>,
+                                   (const void*)gemm_f32_rows_kernel<true, 8>, (const void*)gemm_f32_rows_kernel<false, 8>,
+                                   (const void*)gemm_f32_rows_kernel<true, 16, false, true>,
+                                   (const void*)gemm_f32_rows_kernel<false, 16, false, true>,
+                                   (const void*)gemm_f32_rows_kernel<true, 16, false, false, 2>,
+                                   (const void*)gemm_f32_rows_kernel<false, 16, false, false, 2>,
+                                   (const void*)gemm_f32_rows_kernel<true, 16, false, false, 3>,
+                                   (const void*)gemm_f32_rows_kernel<false, 16, false, false, 3>};
         for (const void* k : kernels)
           if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024) != hipSuccess)
             return TL_ERR_LAUNCH;
         configured = true;
       }
-      dim3 gr((N + cols - 1) / cols, (mts + tiles_wg - 1) / tiles_wg);
-#define TL_F32_ROWS(SW, CO, WI)                                                                                        \
-  hipLaunchKernelGGL((gemm_f32_rows_kernel<SW, CO, false, WI>), gr, dim3(FR_THREADS), rows_smem, stream, (const float*)a, \
-                     (const float*)w, (float*)out, residual, M, N, K, lda, ldo, (const float*)nullptr, 0.f, row_scale,  \
-                     tiles_wg)
-      if (mts > 1 && swiglu) TL_F32_ROWS(true, 16, true);
-      else if (mts > 1) TL_F32_ROWS(false, 16, true);
-      else if (swiglu && cols == 16) TL_F32_ROWS(true, 16, false);
-      else if (swiglu) TL_F32_ROWS(true, 8, false);
-      else if (cols == 16) TL_F32_ROWS(false, 16, false);
-      else TL_F32_ROWS(false, 8, false);
+      dim3 gr((N + cols * ct - 1) / (cols * ct), (mts + tiles_wg - 1) / tiles_wg);
+#define TL_F32_ROWS(SW, CO, WI, CTI)                                                                                 \
+  hipLaunchKernelGGL((gemm_f32_rows_kernel<SW, CO, false, WI, CTI>), gr, dim3(FR_THREADS), rows_smem, stream,         \
+                     (const float*)a, (const float*)w, (float*)out, residual, M, N, K, lda, ldo, (const float*)nullptr, \
+                     0.f, row_scale, tiles_wg)
+#define TL_F32_ROWS_CT(SW)                                                                                           \
+  do {                                                                                                               \
+    if (ct == 3) TL_F32_ROWS(SW, 16, false, 3);                                                                      \
+    else if (ct == 2) TL_F32_ROWS(SW, 16, false, 2);                                                                 \
+    else TL_F32_ROWS(SW, 16, false, 1);                                                                              \
+  } while (0)
+      if (mts > 1 && swiglu) TL_F32_ROWS(true, 16, true, 1);
+      else if (mts > 1) TL_F32_ROWS(false, 16, true, 1);
+      else if (swiglu && cols == 16) TL_F32_ROWS_CT(true);
+      else if (swiglu) TL_F32_ROWS(true, 8, false, 1);
+      else if (cols == 16) TL_F32_ROWS_CT(false);
+      else TL_F32_ROWS(false, 8, false, 1);
+#undef TL_F32_ROWS_CT
 #undef TL_F32_ROWS
       return tl_launch_status();
     }

@@ -340,6 +340,12 @@ def linear_norm_f32_ok(rows: int, cols: int, inner: int, row_stride: int) -> boo
     return bool(_lib().tl_linear_norm_f32_ok(c_int(rows), c_int(cols), c_int(inner), c_int64(row_stride)))
 
 
+def linear_f32_col_tiles(rows: int, cols: int, inner: int) -> int:
+    """Column tiles a workgroup of the float32 few-row product owns at these sizes (more than one: a
+    wide product, in front of which a norm is cheaper as `norm_prescale_f32` than inside `linear_norm_f32`)."""
+    return int(_lib().tl_linear_f32_col_tiles(c_int(rows), c_int(cols), c_int(inner)))
+
+
 def linear_norm_f32(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: torch.Tensor, out: torch.Tensor,
                     residual: Optional[torch.Tensor] = None, epilogue: Optional[str] = None) -> torch.Tensor:
     """out = rmsnorm(x; norm_weight, eps) @ w.T, then the epilogue of `linear`, all float32 and for few

@@ -33,8 +33,10 @@ class LazyNorm:
             # true float32: the norm inside the few-row product's kernel (measured on whole steps: up
             # to 16 rows it saves time), or as two kernels that give the same bits: norm_weight * x
             # and the rows' factors, then the product with the factor applied to its sums
+            # (a product so wide that a workgroup owns several column tiles takes the two kernels too)
             if (self.rows is None and self.x.shape[0] <= RMSNorm.F32_FUSED_ROWS
-                    and ops.linear_norm_f32_ok(self.x.shape[0], w.shape[0], self.x.shape[1], self.x.stride(0))):
+                    and ops.linear_norm_f32_ok(self.x.shape[0], w.shape[0], self.x.shape[1], self.x.stride(0))
+                    and ops.linear_f32_col_tiles(self.x.shape[0], w.shape[0], self.x.shape[1]) == 1):
                 return ops.linear_norm_f32(self.x, self.weight, self.eps, w, out, epilogue=epilogue)
             h, inv_rms = ops.norm_prescale_f32(self.x, self.weight, self.eps, self.rows)
             return ops.linear(h, w, out, epilogue=epilogue, row_scale=inv_rms)
