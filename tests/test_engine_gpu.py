@@ -673,6 +673,28 @@ def test_command_line_generates_from_prompt_ids(folders):
     assert bad.returncode == 1 and "[Fatal]" in bad.stderr
 
 
+def test_command_line_interactive_loop(folders):
+    """The reference's loop (main.cpp:51-85): lines up to a blank line are one prompt, a blank line
+    alone asks again, the end of the input ends the program with 0.  Without a tokenizer in the folder
+    a prompt is token ids; they may come on several lines."""
+    cfg = CONFIGS["A"][0]
+    w, c = read_weights(folders["A"])
+    p1, p2 = random_tokens(9, cfg["vocab_size"], 41), random_tokens(14, cfg["vocab_size"], 42)
+    text = (" ".join(map(str, p1)) + "\n\n"                                      # one line, then the blank line
+            + "\n"                                                              # an empty prompt
+            + " ".join(map(str, p2[:6])) + "\n" + ",".join(map(str, p2[6:])) + "\n\n")      # two lines
+    for extra in ([], ["--stream"]):
+        proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "tiny_llm"), "--model_path", folders["A"],
+                               "--nodo_sample", "--max_new_tokens=6", "--dtype=float32", "--ignore_eos"] + extra,
+                              input=text, capture_output=True, text=True, timeout=300)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        out = proc.stdout
+        assert out.count("[Input] >") == 4 and out.count("[Output] >") == 2 and "The prompt is empty" in out
+        answers = [blk.strip().splitlines()[0] for blk in out.split("[Output] >")[1:]]
+        assert [[int(t) for t in a.split()] for a in answers] == [plain.greedy_generate(w, c, p1, 6),
+                                                                  plain.greedy_generate(w, c, p2, 6)]
+
+
 def test_tokens_stream_as_they_are_generated(folders):
     """`stream` yields every prompt's tokens in order, each once, with the finish reason at the end;
     together they are what `generate` returns; a bound of one decode step hands over a token at a time."""
