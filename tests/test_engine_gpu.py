@@ -695,6 +695,31 @@ def test_command_line_interactive_loop(folders):
                                                                   plain.greedy_generate(w, c, p2, 6)]
 
 
+def test_command_line_speaks_text_when_the_folder_has_a_tokenizer(folders, tmp_path):
+    """With tokenizer.json in the model folder prompts are text and so is the output
+    (tiny_llm/pipeline/pipeline.cpp:113, 236: encode with special tokens, decode without)."""
+    tokenizers = pytest.importorskip("tokenizers")
+    import shutil
+    cfg = CONFIGS["A"][0]
+    folder = tmp_path / "with_tokenizer"
+    shutil.copytree(folders["A"], folder)
+    vocab = {f"w{i}": i for i in range(cfg["vocab_size"])}
+    tok = tokenizers.Tokenizer(tokenizers.models.WordLevel(vocab, unk_token="w0"))
+    tok.pre_tokenizer = tokenizers.pre_tokenizers.Whitespace()
+    tok.save(str(folder / "tokenizer.json"))
+    w, c = read_weights(str(folder))
+    prompt = random_tokens(10, cfg["vocab_size"], 77)
+    text = " ".join(f"w{t}" for t in prompt) + "\n\n"
+    want = plain.greedy_generate(w, c, prompt, 5)
+    for extra in ([], ["--stream"]):
+        proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "tiny_llm"), "--model_path", str(folder),
+                               "--nodo_sample", "--max_new_tokens=5", "--dtype=float32", "--ignore_eos"] + extra,
+                              input=text, capture_output=True, text=True, timeout=300)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        answer = proc.stdout.split("[Output] >")[1].strip().splitlines()[0]
+        assert answer == " ".join(f"w{t}" for t in want), answer
+
+
 def test_tokens_stream_as_they_are_generated(folders):
     """`stream` yields every prompt's tokens in order, each once, with the finish reason at the end;
     together they are what `generate` returns; a bound of one decode step hands over a token at a time."""
