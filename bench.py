@@ -5,7 +5,8 @@
 A step is one decode step of the whole serving path (scheduler, step function, sampling).  The
 headline is the TinyLlama-1.1B shape in bfloat16 at batch 8 with 512-token prompts.  ONE JSON line is
 printed: decoded tokens per second, the 2,048-token prefill (whole and in portions of 512), the HBM
-roofline of the decode step, decode at batch 1 and 64; the same in true float32; the machine's peaks
+roofline of the decode step, decode at batch 1 and 64, the time of a decode step and of the prefill by
+kernel; the same in true float32; the machine's peaks
 as measured on the spot (a streaming kernel, a loop of matrix instructions); and two soak workloads
 at larger shapes (a mixed batch of 16 requests with prompts cut into portions of 512 at the
 Llama-3-8B shape; 64 requests of 1,024 tokens that nearly fill the cache at the Llama-2-13B shape).
@@ -194,6 +195,41 @@ class Bench:
         eng.scheduler.budget = old
         return min(times[1:])
 
+    def profile_decode(self, batch, prompt_len=PROMPT_LEN, steps=32):
+        """Per-kernel times of a decode step (see kernel_breakdown): `steps` chained steps behind a warm-up."""
+        from tiny_llm_amd import SamplingParams
+        eng = self.engine
+        params = SamplingParams.greedy(3 * steps + 64, ignore_eos=True)
+        ids = [eng.add_request(gen_tokens(prompt_len, self.V, 1000 + i), params) for i in range(batch)]
+        reqs = [eng.requests[i] for i in ids]
+        while any(r.num_computed < prompt_len for r in reqs):
+            eng.step()
+        run0 = eng.steps_run
+        while eng.steps_run - run0 < 2 * steps:             # the shape is captured, its chain of steps too
+            eng.step()
+
+        def run():
+            at = eng.steps_run
+            while eng.steps_run - at < steps:
+                eng.step(max_decode_steps=steps - (eng.steps_run - at))
+        out = kernel_breakdown(run, self.cfg["num_hidden_layers"])
+        for i in ids:
+            eng.abort(i)
+        return out
+
+    def profile_prefill(self, tokens=PREFILL_TOKENS):
+        """Per-kernel times of one whole-prompt prefill step."""
+        from tiny_llm_amd import SamplingParams
+        eng = self.engine
+
+        def once(seed):
+            rid = eng.add_request(gen_tokens(tokens, self.V, seed), SamplingParams.greedy(1, ignore_eos=True))
+            while eng.requests[rid].status != "finished":
+                eng.step()
+        once(91)
+        once(92)
+        return kernel_breakdown(lambda: once(93), self.cfg["num_hidden_layers"])
+
     def soak(self, prompt_lens, new_tokens, budget):
         """All requests at once through the scheduler: prompts in portions under `budget` tokens a
         step beside decoded tokens.  Returns (seconds, steps, preemptions)."""
@@ -212,6 +248,87 @@ class Bench:
         dt = time.perf_counter() - t0
         assert all(len(eng.requests[i].output) == new_tokens for i in ids)
         return dt, steps, sum(eng.requests[i].preemptions for i in ids)
+
+
+def kernel_breakdown(run, layers):
+    """Where a step's time goes, kernel by kernel: `run` executes steps of one kind (decode steps of one
+    batch, or one prefill) under torch's profiler, which also sees the kernels of replayed graphs; what it
+    reports for a kernel reaches from the end of the kernel before it to its own end, so the figures add up
+    to the step.  The kernels of a step are told apart by their order around each layer's attention
+    kernel: before the first one the q/k/v product; between two of them the o product, the gate/up
+    product(s), the down product and the next layer's q/k/v product; behind the last one o, gate/up and
+    down; rotation, the merge of attention's key splits and norms by their names; a product's second
+    kernel (partial sums added up) counts with the product; then the output head, the sampler and, in
+    chained decode steps, the kernel that prepares the next step.  Returns microseconds per step by part,
+    summed over the layers."""
+    import torch
+    from torch.autograd import DeviceType
+    from torch.profiler import ProfilerActivity, profile
+    with profile(activities=[ProfilerActivity.CUDA]) as prof:
+        run()
+        torch.cuda.synchronize()
+    evs = [e for e in prof.events() if e.device_type == DeviceType.CUDA and "emcpy" not in e.name and "emset" not in e.name]
+    evs.sort(key=lambda e: e.time_range.start)
+    starts = [i for i, e in enumerate(evs) if "embedding_kernel" in e.name]
+    is_attention = lambda n: ("attn" in n or "attention" in n or "flash_prefill" in n) and "combine" not in n
+    parts, n_steps = {}, 0
+    for a, z in zip(starts, starts[1:] + [len(evs)]):
+        step = evs[a:z]
+        names = [e.name for e in step]
+        dur = [e.time_range.end - e.time_range.start for e in step]
+        # behind the layers: the head (a product, perhaps with a second kernel), sampler, the next step's metadata
+        tail = len(step)
+        while tail > 0 and ("sample_kernel" in names[tail - 1] or "decode_advance" in names[tail - 1]):
+            tail -= 1
+        head = tail - 1
+        while head > 0 and "splitk_reduce" in names[head]:
+            head -= 1
+        body = list(range(1, head))
+        att = [i for i in body if is_attention(names[i])]
+        if layers <= 0 or len(att) != layers or head <= 0 or "gemm" not in names[head]:
+            continue                                    # not a whole step (the profile began or ended inside one)
+        n_steps += 1
+        add = lambda k, v: parts.__setitem__(k, parts.get(k, 0.0) + v)
+        add("embedding", dur[0])
+        is_product = lambda i: "gemm" in names[i] and "splitk_reduce" not in names[i]
+        last = None
+        for i in body:
+            n = names[i]
+            if "splitk_reduce" in n and last is not None:
+                add(last, dur[i])
+            elif "rope_store" in n:
+                add("rotation", dur[i])
+            elif "combine" in n:
+                add("attention_merge", dur[i])
+            elif is_attention(n):
+                add("attention", dur[i])
+            elif is_product(i):
+                seg = sum(1 for x in att if x < i)                  # attention kernels before this product
+                lo = att[seg - 1] if seg else 0
+                hi = att[seg] if seg < layers else head
+                group = [x for x in body if lo < x < hi and is_product(x)]
+                k = group.index(i)
+                if seg == 0:
+                    last = "qkv"
+                elif seg < layers:
+                    last = "o" if k == 0 else "qkv" if k == len(group) - 1 else "down" if k == len(group) - 2 else "gate_up"
+                else:
+                    last = "o" if k == 0 else "down" if k == len(group) - 1 else "gate_up"
+                add(last, dur[i])
+            elif "norm" in n:
+                add("norm", dur[i])
+            else:
+                add("other", dur[i])
+        for i in range(head, tail):
+            add("lm_head", dur[i])
+        for i in range(tail, len(step)):
+            add("sample" if "sample_kernel" in names[i] else "next_step", dur[i])
+    if not n_steps:
+        return None
+    out = {k: round(v / n_steps, 1) for k, v in parts.items()}
+    out["sum"] = round(sum(parts.values()) / n_steps, 1)
+    out["steps_seen"] = n_steps
+    return out
 
 
 def decode_rooflines(cfg, dtype, batch, seconds, ctx_tokens):
@@ -258,6 +375,9 @@ def tinyllama_figures(args, dtype, peaks):
                            "frac": round(achieved / HBM_GBS, 4)}
         if peaks:
             out["roofline"]["frac_measured"] = round(achieved / peaks["hbm_read_GBs"], 4)
+        if args.only in ("all", "headline", "fp32", "kernels"):
+            out["kernels_us"] = {"decode": b.profile_decode(args.batch, prompt_len=args.prompt_len),
+                                 "prefill": b.profile_prefill()}
         out["points"] = {}
         if args.only in ("all", "headline", "fp32"):
             for n in (1, 64):
@@ -447,6 +567,8 @@ def run(args):
             line[f"roofline_b{n}"] = fig[f"roofline_b{n}"]
     if "prefill_chunked_512" in fig:
         line["prefill_chunked_512"] = fig["prefill_chunked_512"]
+    if "kernels_us" in fig:
+        line["kernels_us"] = fig["kernels_us"]
     if peaks:
         line["measured_peaks"] = peaks
     if args.only == "all":
@@ -454,7 +576,8 @@ def run(args):
         line["fp32"] = {"decode_b8": round(f32["value"], 1), "ms_per_step_b8": round(f32["ms_per_step"], 4),
                         "decode_b1": f32["points"]["decode_b1"], "decode_b64": f32["points"]["decode_b64"],
                         "steps": f32["steps"], "prefill": f32["prefill"], "prefill_chunked_512": f32["prefill_chunked_512"],
-                        "roofline_b8": f32["roofline"], "roofline_b1": f32["roofline_b1"], "roofline_b64": f32["roofline_b64"]}
+                        "roofline_b8": f32["roofline"], "roofline_b1": f32["roofline_b1"], "roofline_b64": f32["roofline_b64"],
+                        "kernels_us": f32.get("kernels_us")}
         line["workloads"] = {"llama3_8b_mixed16": soak_llama3_8b(args), "llama3_8b_prefill": prefill_llama3_8b(args),
                              "llama2_13b_64x1024": soak_llama2_13b(args),
                              "llama3_8b_mixed16_fp32": soak_llama3_8b(args, "fp32"),
@@ -474,9 +597,10 @@ def main():
     ap.add_argument("--soak-layers", type=int, default=0, help="fewer layers for the two larger shapes (0: all)")
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--only", default="all",
-                    choices=["all", "headline", "decode", "prefill", "fp32", "peaks", "llama3_8b", "llama3_8b_prefill", "llama2_13b", "host"],
+                    choices=["all", "headline", "decode", "prefill", "fp32", "kernels", "peaks", "llama3_8b", "llama3_8b_prefill", "llama2_13b", "host"],
                     help="all: everything in one line; headline: the bfloat16 TinyLlama figures only; decode / prefill: "
-                         "one of them (profiling); fp32: the float32 figures as the headline; peaks / llama3_8b / "
+                         "one of them (profiling); fp32: the float32 figures as the headline; kernels: decode with the time of "
+                         "a step by kernel (torch's profiler); peaks / llama3_8b / "
                          "llama2_13b: that part alone; host: a step's wall time against its time on the GPU")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
