@@ -20,6 +20,8 @@ decode-only steps by (requests, bound on the context), other steps by capacities
 no cache slot, padding query tiles hold no token, padding rows of the output are
 dropped.  Eager and captured steps share the layout routine, the model code and
 the sampler; a captured step only has its sizes rounded up and its buffers static.
+A model that holds a part which may not be captured still runs as graphs: one for each
+run of stages that may be, the other stages eagerly between them on the same buffers.
 """
 from __future__ import annotations
 
@@ -57,7 +59,8 @@ class SampleSpec:
 @dataclass
 class StepContext:
     """Who is in the batch and where each token sits; device tensors are int32.
-    In a captured step the sizes are capacities and the host copies are not meaningful."""
+    In a captured step the sizes are capacities, and the host copies are this step's only while a
+    part runs eagerly (a step's first run, or a part that may not be captured)."""
     num_tokens: int
     num_requests: int
     tokens: torch.Tensor            # [T]

@@ -109,9 +109,10 @@ class LayerCache:
 class Part:
     """Base of every part: declares weights, receives them, computes."""
 
-    # True if `forward` only enqueues device work whose shape depends on nothing but the batch
-    # size (no host reads of step data, no host loops over requests): such a part may be
-    # captured in a HIP graph for decode steps.  Parts defined elsewhere default to False.
+    # True if `forward` only enqueues device work whose shape depends on nothing but the step's
+    # capacities (no host reads of step data, no host loops over requests): such a part may be
+    # captured in a HIP graph.  Parts defined elsewhere default to False: their layer then runs
+    # eagerly between the graphs of the layers around it, with the step's host copies in `ctx`.
     graph_safe = False
 
     def __init__(self, prefix: str, dtype: torch.dtype, device: torch.device):
