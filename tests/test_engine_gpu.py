@@ -206,8 +206,8 @@ def test_preemption_recomputes_and_gives_the_same_tokens(folders):
     tight = Engine(folders["A"], dtype="float32", max_num_seqs=4, kv_block_size=16, num_kv_blocks=9)
     out = tight.generate(prompts, sp)            # 3 x 70 tokens need 15 blocks, 9 exist
     assert out == roomy
-    assert sum(r.preemptions for r in tight.requests.values()) >= 1
-    assert all(r.finish_reason == "length" for r in tight.requests.values())
+    assert len(tight.scheduler.finished) == 3 and sum(r.preemptions for r in tight.scheduler.finished) >= 1
+    assert all(r.finish_reason == "length" for r in tight.scheduler.finished)
     tight.runner.cache.audit()
     assert tight.runner.cache.free_blocks() == [9]
 
@@ -435,7 +435,7 @@ def test_a_request_that_cannot_go_on_even_alone_ends_with_capacity(folders):
     eng = Engine(folders["A"], dtype="float32", max_num_seqs=2, kv_block_size=16, num_kv_blocks=3)
     prompt = random_tokens(40, cfg["vocab_size"], 41)
     out = eng.generate([prompt], SamplingParams.greedy(30, ignore_eos=True))[0]
-    req = next(iter(eng.requests.values()))
+    req = eng.scheduler.finished[-1]
     assert req.finish_reason == "capacity" and len(out) == 3 * 16 - 40 + 1      # 48 cached tokens, one more chosen
     assert out == plain.greedy_generate(w, c, prompt, len(out))
     assert eng.runner.cache.free_blocks() == [3]
@@ -457,12 +457,12 @@ def test_preemption_in_bfloat16_with_seeded_sampling(folders):
     poison(tight)
     log = spy_on_steps(tight)
     out = tight.generate(prompts, sps)
-    assert sum(r.preemptions for r in tight.requests.values()) >= 1
+    assert sum(r.preemptions for r in tight.scheduler.finished) >= 1
     assert all(len(o) == 40 for o in out)
     tight.runner.cache.audit()
     assert tight.runner.cache.free_blocks() == [9]
     # a preempted request is recomputed from position 0; what it had generated stays its own
-    worst, n = check_logged_logits(log, {r.req_id: r.tokens for r in tight.requests.values()}, w, c, torch.bfloat16, 2e-2)
+    worst, n = check_logged_logits(log, {r.req_id: r.tokens for r in tight.scheduler.finished}, w, c, torch.bfloat16, 2e-2)
     print(f"preemption in bfloat16: {n} rows , worst rel err {worst:.2e}")
     assert n == 120
     refs = [plain.llama_forward(w, c, p + o, act_dtype=torch.bfloat16) for p, o in zip(prompts, out)]
@@ -718,6 +718,34 @@ def test_command_line_speaks_text_when_the_folder_has_a_tokenizer(folders, tmp_p
         assert proc.returncode == 0, proc.stderr[-2000:]
         answer = proc.stdout.split("[Output] >")[1].strip().splitlines()[0]
         assert answer == " ".join(f"w{t}" for t in want), answer
+
+
+def test_finished_requests_are_let_go(folders):
+    """`generate` forgets its requests when it returns; a request added by hand stays until it is
+    released, and beyond the bound the oldest finished ones go by themselves; the scheduler's record
+    of finished requests is bounded too."""
+    from tiny_llm_amd import Engine, SamplingParams
+    cfg, eng_kw, _ = CONFIGS["A"]
+    eng = Engine(folders["A"], dtype="float32", max_num_seqs=4, **eng_kw)
+    eng.FINISHED_KEPT = 6
+    eng.scheduler.finished = type(eng.scheduler.finished)(maxlen=5)
+    p = random_tokens(7, cfg["vocab_size"], 3)
+    eng.generate([p, p], SamplingParams.greedy(3, ignore_eos=True))
+    assert eng.requests == {}
+    rid = eng.add_request(p, SamplingParams.greedy(2, ignore_eos=True))
+    assert eng.release(rid) is None                   # live: it stays
+    while eng.has_unfinished():
+        eng.step()
+    assert eng.requests[rid].finish_reason == "length"
+    kept = eng.release(rid)
+    assert kept.output and rid not in eng.requests and eng.release(rid) is None
+    ids = []
+    for _ in range(10):
+        ids.append(eng.add_request(p, SamplingParams.greedy(1, ignore_eos=True)))
+        while eng.has_unfinished():
+            eng.step()
+    assert len(eng.requests) <= 7 and ids[-1] in eng.requests and ids[0] not in eng.requests
+    assert len(eng.scheduler.finished) == 5
 
 
 def test_tokens_stream_as_they_are_generated(folders):

@@ -136,7 +136,7 @@ def test_random_schedule(seed):
         w, c = read_weights(folder, round_to=rounded)
         tol = 2 * TOL[dtype]
         for i, (p, o) in enumerate(zip(prompts, out)):
-            assert len(o) == news[i], (i, eng.requests[i].finish_reason)
+            assert len(o) == news[i], i
             ref = plain.llama_forward(w, c, p + o, act_dtype=rounded)
             for k, tok in enumerate(o):
                 row = ref[len(p) + k - 1]
@@ -210,7 +210,7 @@ def test_random_windowed_architecture(seed):
         runner = build_runner(dec, whole)
         tol = 2 * TOL[dtype]
         for i, (p, o) in enumerate(zip(prompts, out)):
-            assert len(o) == news[i], (i, eng.requests[i].finish_reason)
+            assert len(o) == news[i], i
             toks = p + o
             ref = runner.step([StepEntry("w", toks, list(range(len(p) - 1, len(toks) - 1)))]).float().cpu()
             runner.finish("w")

@@ -19,6 +19,11 @@ from .step import SampleSpec, StepEntry
 
 
 class Engine:
+    # Finished requests stay in `requests` (their tokens, their finish reason) until their caller
+    # has had them: `generate` and `stream` let go of theirs at the end, `release` does it for the
+    # caller of `add_request`; beyond this many the oldest finished ones go by themselves.
+    FINISHED_KEPT = 4096
+
     def __init__(self, model_path: Optional[str] = None, *, config: Optional[Mapping] = None,
                  engine_config: Optional[EngineConfig] = None, weights_seed: int = 0,
                  init_std: Optional[float] = None, norm_std: float = 0.0, **engine_kwargs):
@@ -61,7 +66,17 @@ class Engine:
             return req_id
         self.scheduler.add(req)
         self.requests[req_id] = req
+        if len(self.requests) > self.FINISHED_KEPT:
+            for old in [k for k, r in self.requests.items() if r.status == "finished"][:len(self.requests) - self.FINISHED_KEPT]:
+                del self.requests[old]
         return req_id
+
+    def release(self, req_id: Hashable) -> Optional[Request]:
+        """Forgets a finished request (the caller has its tokens) and returns it; a live one stays."""
+        r = self.requests.get(req_id)
+        if r is None or r.status != "finished":
+            return None
+        return self.requests.pop(req_id)
 
     def abort(self, req_id: Hashable) -> None:
         self.scheduler.abort(req_id)
@@ -127,6 +142,8 @@ class Engine:
                     closed[i] = closed[i] or ended
                     yield i, fresh, (r.finish_reason if ended else None)
             if not self.scheduler.has_work():
+                for rid in ids:
+                    self.release(rid)
                 return
             self.step(max_decode_steps)
 

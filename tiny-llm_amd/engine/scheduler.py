@@ -96,6 +96,8 @@ class StepPlan:
 
 
 class Scheduler:
+    FINISHED_KEPT = 4096
+
     def __init__(self, cache: CacheManager, max_num_seqs: int, max_num_batched_tokens: int, max_model_len: int,
                  eos_token_id=None):
         """eos_token_id: one id, several, or None (nothing ends a request but its length)."""
@@ -106,7 +108,8 @@ class Scheduler:
         self.eos_token_id = eos_token_id
         self.waiting: Deque[Request] = deque()
         self.running: List[Request] = []       # in order of admission
-        self.finished: List[Request] = []
+        # the requests that finished last (a bounded record: a serving process finishes without end)
+        self.finished: Deque[Request] = deque(maxlen=self.FINISHED_KEPT)
 
     @property
     def eos_token_id(self):
