@@ -449,11 +449,14 @@ def test_norm_prescale_f32_any_inner_size(K):
     assert torch.equal(alone, out[7:8])
 
 
-@pytest.mark.parametrize("K,N", [(200, 90), (1000, 72), (5632, 130), (256, 8), (258, 34)])
+@pytest.mark.parametrize("K,N", [(200, 90), (1000, 72), (5632, 130), (256, 8), (258, 34), (700, 48), (2308, 24),
+                                 (1536, 2050)])
 def test_linear_row_alone_equals_row_in_batch_fp32(K, N):
     """In float32 a row gives the same bits alone, among a few rows and among many: the tiled kernel
     (more than 16 rows, or an inner size that is no multiple of 4) and the few-row kernel add in one
-    order.  With residual and with the SiLU-gate epilogue too."""
+    order, also where the few-row kernel puts two k blocks into one matrix tile (up to 8 rows and 2,048
+    columns; an odd number of blocks, a last block that is not whole).  With residual and with the
+    SiLU-gate epilogue too."""
     g = torch.Generator().manual_seed(5 + K)
     a = torch.randn(70, K, generator=g).to(DEV)
     w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(DEV)
@@ -469,6 +472,8 @@ def test_linear_row_alone_equals_row_in_batch_fp32(K, N):
         full = run(slice(0, 70))
         assert torch.equal(full[37:38], run(slice(37, 38)))
         assert torch.equal(full[30:43], run(slice(30, 43)))
+        assert torch.equal(full[30:38], run(slice(30, 38)))
+        assert torch.equal(full[11:14], run(slice(11, 14)))
         assert torch.equal(full[3:67], run(slice(3, 67)))
         ref = a.double() @ w.double().T
         if kwargs.get("residual"):

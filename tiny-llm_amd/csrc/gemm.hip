@@ -258,7 +258,15 @@ constexpr int FR_WAVES = 8, FR_THREADS = FR_WAVES * TL_WAVE, FR_MAX_MT = 4;
 // The weights come as a chain of pieces, the block's tiles and then the wave's next block, each
 // requested while the piece before it is multiplied.  A tile's block sums are what they are with one
 // tile a workgroup, bit for bit.
-template <bool SWIGLU, int COLS, bool NORM = false, bool WIDE = false, int CT = 1>
+//
+// PAIR (8 columns, at most 8 rows, no norm): the matrix tile of 16 x 16 then holds two k blocks at
+// once.  Operand rows 0 to 7 are the 8 columns (and the 8 activation rows) at the k of one block, rows
+// 8 to 15 the same columns and rows at the k of the next; the two diagonal 8 x 8 blocks of the result
+// are the two block sums, each accumulated from zero in the order it has everywhere else, and the
+// rest of the tile is dropped.  Without it the second half of the tile repeats the first: every load
+// instruction then fetches half of what it could, and 8 columns are what bounds these products,
+// since a workgroup is as fast as its loads.  A wave takes pairs of blocks instead of blocks.
+template <bool SWIGLU, int COLS, bool NORM = false, bool WIDE = false, int CT = 1, bool PAIR = false>
 __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* __restrict__ a,
                                                                    const float* __restrict__ w,
                                                                    float* __restrict__ out,
@@ -275,12 +283,17 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
   // are requested behind the block's last row tile instead.
   static_assert(!(NORM && WIDE), "the norm rides in the product of one row tile");
   static_assert(CT >= 1 && CT <= 3 && !(WIDE && CT > 1) && !(NORM && CT > 1), "several column tiles go with one row tile and no norm");
+  static_assert(!PAIR || (COLS == 8 && !NORM && !WIDE && CT == 1), "pairs of k blocks: 8 columns, one row tile of at most 8 rows");
   extern __shared__ float rows_smem[];      // [m tiles][CT][k blocks][16 rows][COLS columns], NORM: + [m tiles][k blocks][16]
   const int nkb = (K + F_KBLOCK - 1) / F_KBLOCK;
   const int mt0 = WIDE ? blockIdx.y * tiles_wg : 0;                       // first row tile of this workgroup
   const int mts = WIDE ? min(tiles_wg, (M + 15) / 16 - mt0) : (M + 15) / 16;   // and how many it owns
   const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
   const int l16 = lane % 16, kk = lane / 16;
+  // a wave's unit of work: a k block, or a pair of them, of which this lane feeds the first or the second
+  constexpr int UNIT = PAIR ? 2 : 1;
+  const int second = PAIR ? l16 / 8 : 0;
+  const int units = (nkb + UNIT - 1) / UNIT;
   const int n0 = blockIdx.x * COLS * CT;
   auto wrow_of = [&](int ct) { return w + (int64_t)min(n0 + ct * COLS + l16 % COLS, N - 1) * K; };
   const float* wrow = wrow_of(0);
@@ -295,11 +308,11 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
       else dst[g] = load_k4<true>(row, k0 + g * 16 + kk * 4, K);
     }
   };
-  auto a_row = [&](int mt) { return a + (int64_t)min((mt0 + mt) * 16 + l16, M - 1) * lda; };
+  auto a_row = [&](int mt) { return a + (int64_t)min((mt0 + mt) * 16 + (PAIR ? l16 % 8 : l16), M - 1) * lda; };
   f32x4 wv[16], wnext[WIDE ? 1 : 16];
-  if (wave < nkb) {
-    if (wave * F_KBLOCK + F_KBLOCK <= K) load16(std::true_type{}, wv, wrow, wave * F_KBLOCK);
-    else load16(std::false_type{}, wv, wrow, wave * F_KBLOCK);
+  if (wave < units) {
+    if ((wave + 1) * UNIT * F_KBLOCK <= K) load16(std::true_type{}, wv, wrow, (wave * UNIT + second) * F_KBLOCK);
+    else load16(std::false_type{}, wv, wrow, (wave * UNIT + second) * F_KBLOCK);
   }
   float* ss_smem = rows_smem + mts * CT * nkb * 16 * COLS;
   // one row tile and column tile of one k block: the block sum of 16 rows x COLS columns goes to LDS
@@ -310,7 +323,11 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
 #pragma unroll
       for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(wv[g][e], av[g][e], acc, 0, 0, 0);
     // lane (l16, kk): row m = l16, columns 4 kk + r
-    if (kk * 4 < COLS) *(f32x4*)(&rows_smem[(((mt * CT + ct) * nkb + b) * 16 + l16) * COLS + kk * 4]) = acc;
+    if constexpr (PAIR) {     // rows 0..7 x columns 0..7: this lane's block is the first; 8..15 x 8..15: the second
+      if ((l16 < 8) == (kk < 2) && b < nkb) *(f32x4*)(&rows_smem[(b * 16 + l16 % 8) * COLS + (kk % 2) * 4]) = acc;
+    } else {
+      if (kk * 4 < COLS) *(f32x4*)(&rows_smem[(((mt * CT + ct) * nkb + b) * 16 + l16) * COLS + kk * 4]) = acc;
+    }
   };
   // NORM: the rows times the norm's weights, their squares added up on the way (one row tile of one k block)
   auto scale_rows = [&](auto whole, f32x4 (&av)[16], int mt, int b) {
@@ -329,7 +346,9 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
     ss += __shfl_xor(ss, 32, TL_WAVE);
     if (kk == 0) ss_smem[(mt * nkb + b) * 16 + l16] = ss;
   };
-  auto block = [&](auto whole, auto next_whole, int b) {
+  constexpr int AHEAD = FR_WAVES * UNIT * F_KBLOCK;        // from a wave's unit to its next
+  auto block = [&](auto whole, auto next_whole, int u) {
+    const int b = u * UNIT + second;          // this lane's k block
     const int kb = b * F_KBLOCK;
     // (NORM keeps the norm's weights in registers beside the rows instead of the next block's
     // weights; those are requested once this block is done.  The norm's products have the hidden
@@ -350,14 +369,14 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
           multiply(av2, mt + 1, b);
         }
       }
-      if (b + FR_WAVES < nkb) load16(next_whole, wv, wrow, kb + FR_WAVES * F_KBLOCK);
+      if (u + FR_WAVES < units) load16(next_whole, wv, wrow, kb + AHEAD);
     } else if constexpr (CT > 1) {
       // one row tile, no norm
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct) {
-        const bool more = ct + 1 < CT || b + FR_WAVES < nkb;
+        const bool more = ct + 1 < CT || u + FR_WAVES < units;
         if (ct + 1 < CT) load16(whole, wnext, wrow_of(ct + 1), kb);
-        else if (b + FR_WAVES < nkb) load16(next_whole, wnext, wrow, kb + FR_WAVES * F_KBLOCK);
+        else if (u + FR_WAVES < units) load16(next_whole, wnext, wrow, kb + AHEAD);
         multiply(av, 0, b, ct);
         if (more) {
 #pragma unroll
@@ -365,25 +384,25 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
         }
       }
     } else {
-      if (!NORM && b + FR_WAVES < nkb) load16(next_whole, wnext, wrow, kb + FR_WAVES * F_KBLOCK);
+      if (!NORM && u + FR_WAVES < units) load16(next_whole, wnext, wrow, kb + AHEAD);
       for (int mt = 0; mt < mts; ++mt) {
         if (mt > 0) load16(whole, av, a_row(mt), kb);
         if constexpr (NORM) scale_rows(whole, av, mt, b);
         multiply(av, mt, b);
       }
       if constexpr (NORM) {
-        if (b + FR_WAVES < nkb) load16(next_whole, wv, wrow, kb + FR_WAVES * F_KBLOCK);
+        if (u + FR_WAVES < units) load16(next_whole, wv, wrow, kb + AHEAD);
       } else {
 #pragma unroll
         for (int g = 0; g < 16; ++g) wv[g] = wnext[g];
       }
     }
   };
-  for (int b = wave; b < nkb; b += FR_WAVES) {
-    const bool whole = (b + 1) * F_KBLOCK <= K, next_whole = (b + FR_WAVES + 1) * F_KBLOCK <= K;
-    if (whole && next_whole) block(std::true_type{}, std::true_type{}, b);
-    else if (whole) block(std::true_type{}, std::false_type{}, b);
-    else block(std::false_type{}, std::false_type{}, b);
+  for (int u = wave; u < units; u += FR_WAVES) {
+    const bool whole = (u + 1) * UNIT * F_KBLOCK <= K, next_whole = (u + FR_WAVES + 1) * UNIT * F_KBLOCK <= K;
+    if (whole && next_whole) block(std::true_type{}, std::true_type{}, u);
+    else if (whole) block(std::true_type{}, std::false_type{}, u);
+    else block(std::false_type{}, std::false_type{}, u);
   }
   __syncthreads();
   for (int e = tid; e < mts * CT * 16 * COLS; e += FR_THREADS) {
@@ -1741,7 +1760,9 @@ int tl_linear_tile(const void* a, const void* w, void* out, const float* residua
     if (M <= 16 * FR_MAX_MT && vec && rows_smem <= 96 * 1024) {
       static bool configured = false;
       if (!configured) {
-        const void* kernels[10] = {(const void*)gemm_f32_rows_kernel<true, 16>, (const void*)gemm_f32_rows_kernel<false, 16>,
+        const void* kernels[12] = {(const void*)gemm_f32_rows_kernel<true, 8, false, false, 1, true>,
+                                   (const void*)gemm_f32_rows_kernel<false, 8, false, false, 1, true>,
+                                   (const void*)gemm_f32_rows_kernel<true, 16>, (const void*)gemm_f32_rows_kernel<false, 16>,
                                    (const void*)gemm_f32_rows_kernel<true, 8>, (const void*)gemm_f32_rows_kernel<false, 8>,
                                    (const void*)gemm_f32_rows_kernel<true, 16, false, true>,
                                    (const void*)gemm_f32_rows_kernel<false, 16, false, true>,
@@ -1755,10 +1776,11 @@ int tl_linear_tile(const void* a, const void* w, void* out, const float* residua
         configured = true;
       }
       dim3 gr((N + cols * ct - 1) / (cols * ct), (mts + tiles_wg - 1) / tiles_wg);
-#define TL_F32_ROWS(SW, CO, WI, CTI)                                                                                 \
-  hipLaunchKernelGGL((gemm_f32_rows_kernel<SW, CO, false, WI, CTI>), gr, dim3(FR_THREADS), rows_smem, stream,         \
-                     (const float*)a, (const float*)w, (float*)out, residual, M, N, K, lda, ldo, (const float*)nullptr, \
-                     0.f, row_scale, tiles_wg)
+#define TL_F32_ROWS_K(...)                                                                                          \
+  hipLaunchKernelGGL((gemm_f32_rows_kernel<__VA_ARGS__>), gr, dim3(FR_THREADS), rows_smem, stream, (const float*)a, \
+                     (const float*)w, (float*)out, residual, M, N, K, lda, ldo, (const float*)nullptr, 0.f, row_scale, \
+                     tiles_wg)
+#define TL_F32_ROWS(SW, CO, WI, CTI) TL_F32_ROWS_K(SW, CO, false, WI, CTI)
 #define TL_F32_ROWS_CT(SW)                                                                                           \
   do {                                                                                                               \
     if (ct == 3) TL_F32_ROWS(SW, 16, false, 3);                                                                      \
@@ -1768,11 +1790,14 @@ int tl_linear_tile(const void* a, const void* w, void* out, const float* residua
       if (mts > 1 && swiglu) TL_F32_ROWS(true, 16, true, 1);
       else if (mts > 1) TL_F32_ROWS(false, 16, true, 1);
       else if (swiglu && cols == 16) TL_F32_ROWS_CT(true);
+      else if (swiglu && M <= 8) TL_F32_ROWS_K(true, 8, false, false, 1, true);      // cols == 8: pairs of k blocks
       else if (swiglu) TL_F32_ROWS(true, 8, false, 1);
       else if (cols == 16) TL_F32_ROWS_CT(false);
+      else if (M <= 8) TL_F32_ROWS_K(false, 8, false, false, 1, true);
       else TL_F32_ROWS(false, 8, false, 1);
 #undef TL_F32_ROWS_CT
 #undef TL_F32_ROWS
+#undef TL_F32_ROWS_K
       return tl_launch_status();
     }
     // 128 x 128 tiles, or 64 x 64 where those take fewer rounds of workgroups over the 256 compute
