@@ -531,7 +531,62 @@ def host_time(args):
     return out
 
 
+def attention_sweep():
+    """The decode attention kernel (rotation and cache write inside, merge kernel included) alone, at
+    contexts and batches the model runs do not reach, with the key splits the engine would choose:
+    microseconds a call and the bytes of the keys and values it reads per second."""
+    import torch
+    from tiny_llm_amd.kernels import ops
+    dev, page = "cuda:0", 16
+    rows = []
+    for name, nq, nkv, hd in (("tinyllama", 32, 4, 64), ("llama3_8b", 32, 8, 128), ("llama2_13b", 40, 40, 128)):
+        for batch in (1, 8, 64):
+            for ctx in (2048, 8192, 32768, 131072):
+                pages = -(-ctx // page)
+                nbytes = batch * ctx * nkv * hd * 2 * 2
+                if nbytes > 48e9:
+                    continue
+                kc = torch.randn(batch * pages + 1, nkv, page, hd, device=dev, dtype=torch.bfloat16)
+                vc = torch.randn_like(kc)
+                table = (torch.randperm(batch * pages, device=dev).to(torch.int32) + 1).view(batch, pages).contiguous()
+                pos = torch.full((batch,), ctx - 1, device=dev, dtype=torch.int32)
+                qkv = torch.randn(batch, (nq + 2 * nkv) * hd, device=dev, dtype=torch.bfloat16)
+                out = torch.empty(batch, nq * hd, device=dev, dtype=torch.bfloat16)
+                cos, sin = torch.randn(ctx + 8, hd // 2, device=dev), torch.randn(ctx + 8, hd // 2, device=dev)
+                splits = ops.decode_key_splits(batch, ctx, nkv, hd)
+                scratch = torch.empty(splits * batch * nq * (hd + 2), device=dev) if splits > 1 else None
+
+                def call():
+                    ops.flash_attention(qkv[:, :nq * hd], kc, vc, table, None, pos, out, nq, nkv, hd, hd ** -0.5, 0, splits,
+                                        scratch, fused_rope=(cos, sin))
+                for _ in range(2):
+                    call()
+                torch.cuda.synchronize()
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    for _ in range(8):
+                        call()
+                g.replay()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(3):
+                    g.replay()
+                e1.record()
+                torch.cuda.synchronize()
+                us = e0.elapsed_time(e1) * 1e3 / 24
+                rows.append({"heads": name, "batch": batch, "context": ctx, "splits": splits, "us": round(us, 1),
+                             "GBs": round(nbytes / us / 1e3, 1), "hbm_frac": round(nbytes / us / 1e3 / HBM_GBS, 3)})
+                print(f"# {name:10s} batch {batch:3d} context {ctx:6d}: {splits:2d} splits {us:8.1f} us "
+                      f"{nbytes / us / 1e6:6.2f} TB/s", file=sys.stderr, flush=True)
+                del kc, vc
+    return rows
+
+
 def run(args):
+    if args.only == "attention":
+        print(json.dumps({"decode_attention": attention_sweep()}), flush=True)
+        return
     if args.only == "host":
         print(json.dumps({"host_time": host_time(args)}), flush=True)
         return
@@ -597,11 +652,13 @@ def main():
     ap.add_argument("--soak-layers", type=int, default=0, help="fewer layers for the two larger shapes (0: all)")
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--only", default="all",
-                    choices=["all", "headline", "decode", "prefill", "fp32", "kernels", "peaks", "llama3_8b", "llama3_8b_prefill", "llama2_13b", "host"],
+                    choices=["all", "headline", "decode", "prefill", "fp32", "kernels", "peaks", "llama3_8b", "llama3_8b_prefill", "llama2_13b", "host",
+                             "attention"],
                     help="all: everything in one line; headline: the bfloat16 TinyLlama figures only; decode / prefill: "
                          "one of them (profiling); fp32: the float32 figures as the headline; kernels: decode with the time of "
                          "a step by kernel (torch's profiler); peaks / llama3_8b / "
-                         "llama2_13b: that part alone; host: a step's wall time against its time on the GPU")
+                         "llama2_13b: that part alone; host: a step's wall time against its time on the GPU; attention: the "
+                         "decode attention kernel alone at contexts up to 131,072 tokens")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         if int(os.environ.get("RANK", "0")) == 0:

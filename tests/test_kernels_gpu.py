@@ -671,7 +671,7 @@ def _paged_case(dtype, lens, q_lens, nq, nkv, hd, bs, window=0, seed=0, boost=No
         k = torch.randn(L, nkv, hd, generator=g).to(dtype)
         v = torch.randn(L, nkv, hd, generator=g).to(dtype)
         q = torch.randn(L, nq, hd, generator=g).to(dtype)
-        if boost is not None:               # make one far key stand out for the last query
+        if boost is not None and boost < L:     # make one far key stand out for the last query
             far = boost
             k[far] = 0
             k[far, :, 0] = 6.0
@@ -798,6 +798,19 @@ def test_flash_attention_far_key_among_hundreds(n_splits):
     for far in (0, 15, 16, 63, 64, 255, 256, 511, 699):
         out, ref = _paged_case(torch.bfloat16, lens=[700], q_lens=[1], nq=8, nkv=1, hd=64, bs=16, seed=far,
                                boost=far, impl="flash", n_splits=n_splits)
+        assert rel(out, ref) < 8e-3, far
+
+
+@pytest.mark.parametrize("hd,n_splits", [(64, 32), (64, 64), (128, 33), (128, 64)])
+def test_flash_attention_many_splits_over_a_long_context(hd, n_splits):
+    """Thirty-two to sixty-four workgroups share the keys of one request (what the engine asks for at
+    contexts of tens of thousands of tokens), more than the merge kernel takes in one round trip; one
+    key among 5,000 stands out, near the start, at a split's edge, at the end; a second request is so
+    short that most splits hold none of its keys."""
+    for far in (3, 2047, 2048, 4999):
+        out, ref = _paged_case(torch.bfloat16, lens=[5000, 70], q_lens=[1, 1], nq=8, nkv=2, hd=hd, bs=16, seed=far,
+                               boost=far, impl="flash", n_splits=n_splits)
+        assert not torch.isnan(out).any()
         assert rel(out, ref) < 8e-3, far
 
 

@@ -813,6 +813,40 @@ def flash_waves(head_dim: int, groups: int = 1 << 20) -> int:
 _WAVES: dict = {}
 
 
+def decode_key_splits(num_tokens: int, max_seq_len: int, num_kv_heads: int, head_dim: int) -> int:
+    """Over how many workgroups `flash_attention` shares one query tile's keys out in a decode step of
+    `num_tokens` rows.  The waves of a workgroup take a 64-key tile each per round trip to memory (the
+    next one is on its way while a tile is worked on).  Up to two tiles a wave nothing is split: the
+    partial results of a split are merged by a second kernel, which costs more than a wave's second
+    tile (measured on whole decode steps at contexts of 9 to 16 key tiles: 1.5 % of the step).  Longer
+    contexts are split until a wave has one tile (at 17 to 32 key tiles two tiles a wave with a merge
+    are 3 to 5 % of the step slower than one), as far as that keeps the launch within about 256
+    workgroups (beyond that the splits only queue up) and within the kernel's 64.  One request at
+    131,072 tokens: 36 us with 64 splits, 79 with 16, 1,090 with none (heads of 64, 4 kv heads).
+    A launch of more workgroups than compute units runs in rounds, and a last round that is mostly empty
+    takes as long as a full one (320 workgroups: two rounds for the work of 1.25); where the contexts
+    are long (eight key tiles a wave and more even after it) the keys are split further, 2, 4 or 8 ways,
+    if that fills the rounds better (8 requests x 40 kv heads at 32,768 tokens: 912 us with 4 splits,
+    1,174 with none)."""
+    groups = max(1, num_tokens * num_kv_heads)
+    key_tiles = -(-max_seq_len // 64)
+    room = max(1, 256 // groups)
+    per_wave = -(-key_tiles // flash_waves(head_dim, groups))       # key tiles a wave, unsplit
+    if per_wave <= 2:
+        return 1
+    n_splits = max(1, min(per_wave, room, 64))
+    if groups * n_splits > 256:
+        def rounds_per_split(s):
+            return -(-groups * s // 256) / s
+        best = n_splits
+        for more in (2, 4, 8):
+            s = n_splits * more
+            if s <= 64 and per_wave >= 8 * s and rounds_per_split(s) < 0.95 * rounds_per_split(best):
+                best = s
+        n_splits = best
+    return n_splits
+
+
 PREFILL_TILES = 8     # query tiles (of 16 rows) one workgroup of the prefill attention kernel owns
 
 

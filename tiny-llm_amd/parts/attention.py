@@ -135,18 +135,9 @@ class Attention(Mixer):
         return out if next_norm is None else (out, prepared)
 
     def _splits(self, ctx, T: int, device):
-        """How many workgroups share one query tile's keys.  The waves of a workgroup take a
-        64-key tile each per round trip to memory (the next one is on its way while a tile is
-        worked on).  Up to two tiles a wave nothing is split: the partial results of a split are
-        merged by a second kernel, which costs more than a wave's second tile (measured on whole
-        decode steps at contexts of 9 to 16 key tiles: 1.5 % of the step).  Longer contexts are
-        split until a wave has one tile (at 17 to 32 key tiles two tiles a wave with a merge are
-        3 to 5 % of the step slower than one), as far as that keeps the launch within about 256
-        workgroups (beyond that the splits only queue up)."""
-        key_tiles = -(-ctx.max_seq_len // 64)
-        room = max(1, 256 // max(1, T * self.num_kv_heads))
-        n_splits = -(-key_tiles // ops.flash_waves(self.head_dim, T * self.num_kv_heads))
-        n_splits = 1 if n_splits <= 2 else max(1, min(n_splits, room, 16))
+        """How many workgroups share one query tile's keys (`ops.decode_key_splits`), and the scratch
+        for their partial results."""
+        n_splits = ops.decode_key_splits(T, ctx.max_seq_len, self.num_kv_heads, self.head_dim)
         if n_splits == 1:
             return 1, None
         return n_splits, ops.scratch("attention_partials", (n_splits * T * self.num_heads * (self.head_dim + 2),),
