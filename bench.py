@@ -532,9 +532,10 @@ def host_time(args):
 
 
 def attention_sweep():
-    """The decode attention kernel (rotation and cache write inside, merge kernel included) alone, at
-    contexts and batches the model runs do not reach, with the key splits the engine would choose:
-    microseconds a call and the bytes of the keys and values it reads per second."""
+    """The attention kernels alone at contexts and batches the model runs do not reach, with the key
+    splits the engine would choose.  Decode (rotation and cache write inside, merge kernel included):
+    microseconds a call and the bytes of the keys and values it reads per second.  Prompts, whole and
+    512 tokens at the end of a long context: microseconds and the flops of the two products per second."""
     import torch
     from tiny_llm_amd.kernels import ops
     dev, page = "cuda:0", 16
@@ -580,6 +581,41 @@ def attention_sweep():
                 print(f"# {name:10s} batch {batch:3d} context {ctx:6d}: {splits:2d} splits {us:8.1f} us "
                       f"{nbytes / us / 1e6:6.2f} TB/s", file=sys.stderr, flush=True)
                 del kc, vc
+    # prompt portions: whole prompts, and 512 tokens at the end of a long context
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)
+    for name, nq, nkv, hd in (("tinyllama", 32, 4, 64), ("llama3_8b", 32, 8, 128)):
+        for ctx, new in ((8192, 8192), (32768, 32768), (8192, 512), (32768, 512), (131072, 512)):
+            pages = -(-ctx // page)
+            kc = torch.randn(pages + 1, nkv, page, hd, device=dev, dtype=torch.bfloat16)
+            vc = torch.randn_like(kc)
+            table = (torch.randperm(pages, device=dev).to(torch.int32) + 1).view(1, pages).contiguous()
+            q = torch.randn(new, nq * hd, device=dev, dtype=torch.bfloat16)
+            out = torch.empty_like(q)
+            pos = torch.arange(ctx - new, ctx, device=dev, dtype=torch.int32)
+            waves = ops.prefill_tile_waves(new, nq, nkv)
+            per = (16 // (nq // nkv)) * waves                       # tokens of a query tile group
+            starts = list(range(0, new, per))
+            tiles = (i32([0] * len(starts)), i32(starts), i32([min(per, new - t) for t in starts]))
+            splits = ops.prefill_key_splits(new, ctx, nq, nkv, waves)
+            scratch = torch.empty(max(1, splits * new * nq * (hd + 2)), device=dev)
+
+            def call():
+                ops.flash_prefill(q, kc, vc, table, tiles, pos, out, nq, nkv, hd, hd ** -0.5, 0, waves, splits, scratch)
+            call()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(3):
+                call()
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / 3
+            flops = 4.0 * sum(range(ctx - new + 1, ctx + 1)) * nq * hd      # row p sees p + 1 keys; two products
+            rows.append({"heads": name, "prompt_rows": new, "context": ctx, "splits": splits, "us": round(us, 1),
+                         "TFLOPs": round(flops / us / 1e6, 1), "frac": round(flops / us / 1e6 / PEAK_TFLOPS["bf16"], 3)})
+            print(f"# {name:10s} {new:5d} prompt tokens ending at {ctx:6d}: {splits} splits {us:9.1f} us "
+                  f"{flops / us / 1e6:6.1f} TFLOP/s", file=sys.stderr, flush=True)
+            del kc, vc
     return rows
 
 

@@ -793,6 +793,17 @@ def test_flash_prefill_far_key_among_hundreds():
             assert rel(out, ref) < 8e-3, far
 
 
+@pytest.mark.parametrize("hd", [64, 128])
+def test_flash_prefill_eight_splits_over_a_long_context(hd):
+    """A portion of 40 tokens at the end of 5,000, its keys shared out over eight workgroups (what the
+    engine asks for from 32,768 tokens of context on), beside a portion that is a whole short prompt."""
+    for far in (3, 2047, 2048, 4960, 4999):
+        out, ref = _paged_case(torch.bfloat16, lens=[5000, 90], q_lens=[40, 90], nq=8, nkv=2, hd=hd, bs=16, seed=far,
+                               boost=far, impl="prefill4", n_splits=8)
+        assert not torch.isnan(out).any()
+        assert rel(out, ref) < 8e-3, far
+
+
 @pytest.mark.parametrize("n_splits", [1, 2, 7])
 def test_flash_attention_far_key_among_hundreds(n_splits):
     for far in (0, 15, 16, 63, 64, 255, 256, 511, 699):

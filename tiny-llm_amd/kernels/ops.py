@@ -853,15 +853,17 @@ PREFILL_TILES = 8     # query tiles (of 16 rows) one workgroup of the prefill at
 def prefill_key_splits(num_tokens: int, max_seq_len: int, num_heads: int, num_kv_heads: int, tile_waves: int) -> int:
     """Over how many workgroups `flash_prefill` shares the key tiles of a query tile out: 1 unless the
     step has few query tiles (fewer than two workgroups a compute unit) and contexts of 16 key tiles and
-    more; then one split per 8 key tiles of the longest context, at most 4.  (Chosen by the time of whole
-    steps: timed alone, with keys and values in the caches, fewer and larger workgroups look faster
-    than they are in a model.  A whole prompt of 2,048 tokens has two workgroups a compute unit without
-    any split: 7.4 -> 7.05 ms.)"""
+    more; then one split per 8 key tiles of the longest context, at most 4 (8 from 32,768 tokens of
+    context on: a portion of 512 tokens at 131,072 takes 1.30 ms with 8, 1.42 with 4, 2.29 with none).
+    (Chosen by the time of whole steps: timed alone, with keys and values in the caches, fewer and larger
+    workgroups look faster than they are in a model.  A whole prompt of 2,048 tokens has two workgroups a
+    compute unit without any split: 7.4 -> 7.05 ms.)"""
     tiles = -(-num_tokens // (tile_waves * (16 // (num_heads // num_kv_heads))))
     key_tiles = -(-max_seq_len // 64)
     if tiles * num_kv_heads >= 512 or key_tiles < 16:
         return 1
-    return max(1, min(4, key_tiles // 8, 1024 // max(1, tiles * num_kv_heads)))
+    most, launch = (8, 2048) if key_tiles >= 512 else (4, 1024)      # splits, workgroups of the launch
+    return max(1, min(most, key_tiles // 8, launch // max(1, tiles * num_kv_heads)))
 
 
 def prefill_tile_waves(num_tokens: int, num_heads: int, num_kv_heads: int) -> int:
