@@ -420,6 +420,54 @@ def soak_llama3_8b(args, dtype="bf16"):
             "preemptions": pre, "pass": passes, "first_pass_seconds": round(cold, 3)}
 
 
+def long_context_llama3_8b(args):
+    """The Llama-3-8B shape far beyond its own context: 8 requests of 32,000 tokens and one of 131,000,
+    prompts in portions of 2,048, then decode steps; what a step reads (weights and the live
+    requests' keys and values) over its time."""
+    import torch
+    from tiny_llm_amd import SamplingParams
+    cfg = dict(LLAMA3_8B, max_position_embeddings=140000)
+    layers_full = cfg["num_hidden_layers"]
+    if args.soak_layers:
+        cfg["num_hidden_layers"] = min(layers_full, args.soak_layers)
+    out = {"model": "Llama-3-8B shape", "dtype": "bf16", "layers": cfg["num_hidden_layers"], "layers_full": layers_full,
+           "chunk": 2048}
+    for batch, prompt in ((8, 32000), (1, 131000)):
+        b = Bench(cfg, "bf16", batch, 512, 16, budget=2048, prompt_len=prompt)
+        eng = b.engine
+        params = SamplingParams.greedy(400, ignore_eos=True)            # nobody ends inside the run
+        b.sync()
+        t0 = time.perf_counter()
+        ids = [eng.add_request(gen_tokens(prompt, b.V, 1000 + i), params) for i in range(batch)]
+        reqs = [eng.requests[i] for i in ids]
+        steps = 0
+        while any(r.num_computed < prompt for r in reqs):
+            eng.step()
+            steps += 1
+        b.sync()
+        t1 = time.perf_counter()
+        run0 = eng.steps_run
+        while eng.steps_run - run0 < 8:
+            eng.step(max_decode_steps=8)
+        b.sync()
+        t2, run0 = time.perf_counter(), eng.steps_run
+        while eng.steps_run - run0 < 32:
+            eng.step(max_decode_steps=32 - (eng.steps_run - run0))
+        b.sync()
+        ms = (time.perf_counter() - t2) / 32 * 1e3
+        assert len(eng.scheduler.running) == batch
+        _, weight_bytes, kv_per_token, _ = model_numbers(cfg, ELT["bf16"])
+        nbytes = weight_bytes + sum(r.num_tokens for r in reqs) * kv_per_token
+        out[f"batch{batch}_context{prompt}"] = {
+            "prefill_steps": steps, "prefill_tok_s": round(batch * prompt / (t1 - t0), 1), "decode_ms": round(ms, 3),
+            "decode_tok_s": round(batch / ms * 1e3, 1), "GB_a_step": round(nbytes / 1e9, 1),
+            "GBs": round(nbytes / ms / 1e6, 1), "hbm_frac": round(nbytes / ms / 1e6 / HBM_GBS, 3)}
+        for i in ids:
+            eng.abort(i)
+        b.close()
+    return out
+
+
 def prefill_llama3_8b(args):
     """Whole prompts of 4,096 and 8,192 tokens at the Llama-3-8B shape, one step each."""
     cfg = dict(LLAMA3_8B)
@@ -630,6 +678,9 @@ def run(args):
     if args.only == "peaks":
         print(json.dumps({"measured_peaks": peaks}), flush=True)
         return
+    if args.only == "long_context":
+        print(json.dumps({"llama3_8b_long_context": long_context_llama3_8b(args)}), flush=True)
+        return
     if args.only in ("llama3_8b", "llama2_13b", "llama3_8b_prefill"):
         fn = {"llama3_8b": soak_llama3_8b, "llama2_13b": soak_llama2_13b, "llama3_8b_prefill": prefill_llama3_8b}[args.only]
         res = fn(args) if args.only == "llama3_8b_prefill" else fn(args, args.dtype)
@@ -689,12 +740,13 @@ def main():
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--only", default="all",
                     choices=["all", "headline", "decode", "prefill", "fp32", "kernels", "peaks", "llama3_8b", "llama3_8b_prefill", "llama2_13b", "host",
-                             "attention"],
+                             "attention", "long_context"],
                     help="all: everything in one line; headline: the bfloat16 TinyLlama figures only; decode / prefill: "
                          "one of them (profiling); fp32: the float32 figures as the headline; kernels: decode with the time of "
                          "a step by kernel (torch's profiler); peaks / llama3_8b / "
                          "llama2_13b: that part alone; host: a step's wall time against its time on the GPU; attention: the "
-                         "decode attention kernel alone at contexts up to 131,072 tokens")
+                         "attention kernels alone at contexts up to 131,072 tokens; long_context: the Llama-3-8B shape with "
+                         "8 requests of 32,000 tokens and one of 131,000")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         if int(os.environ.get("RANK", "0")) == 0:
