@@ -44,3 +44,18 @@ def test_more_context_never_means_fewer_splits(waves):
     for rows, kv, hd in ((1, 4, 64), (8, 4, 64), (8, 40, 128), (16, 8, 128), (3, 5, 96)):
         got = [ops.decode_key_splits(rows, ctx, kv, hd) for ctx in (64, 640, 1280, 4224, 8192, 32768, 131072)]
         assert got == sorted(got) and 1 <= got[0] and got[-1] <= 64
+
+
+def test_prompt_portions_split_their_keys_where_it_was_measured_to_pay():
+    heads = dict(num_heads=32, num_kv_heads=8)
+    assert ops.prefill_key_splits(2048, 2048, tile_waves=8, **heads) == 1          # a whole prompt: enough workgroups
+    assert ops.prefill_key_splits(512, 512, tile_waves=4, **heads) == 1            # 8 key tiles: too short
+    assert ops.prefill_key_splits(512, 8192, tile_waves=4, **heads) == 4
+    assert ops.prefill_key_splits(512, 131072, tile_waves=4, **heads) == 8         # from 32,768 tokens of context on
+    assert ops.prefill_key_splits(2048, 32768, tile_waves=8, **heads) == 1
+    assert ops.prefill_key_splits(8192, 131072, tile_waves=8, **heads) == 4        # the same quarter of the keys together
+    assert ops.prefill_key_splits(131072, 131072, tile_waves=8, **heads) == 1      # a whole prompt of that length
+    for rows in (16, 100, 512, 2048, 8192):
+        for ctx in (rows, 4096, 32768, 131072):
+            if ctx >= rows:
+                assert 1 <= ops.prefill_key_splits(rows, ctx, tile_waves=4, **heads) <= 8
