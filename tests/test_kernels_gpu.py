@@ -103,7 +103,8 @@ def test_lm_head_last_rows_reference_vector():
                                    (5, 9000, 72), (8, 64, 4100), (12, 96, 8200), (16, 72, 12300), (7, 64, 8200),
                                    (5, 64, 2500), (16, 96, 3302), (17, 2048, 32000), (40, 64, 16390),
                                    (64, 2048, 32000), (33, 128, 128256), (12, 96, 1500), (16, 2048, 2048),
-                                   (10, 64, 20000), (8, 128, 40004), (4, 2048, 1100), (36, 2048, 2560)])
+                                   (10, 64, 20000), (8, 128, 40004), (4, 2048, 1100), (36, 2048, 2560), (8, 64, 28672),
+                                   (16, 72, 27650)])
 def test_linear_sizes(dtype, M, K, N):
     if dtype == torch.bfloat16 and K % 8:
         K = K + 8 - K % 8
@@ -355,7 +356,8 @@ def test_linear_split_k(M, K, N):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("M,K,N", [(1, 64, 352), (9, 96, 400), (64, 2048, 96), (65, 176, 128), (300, 256, 1030)])
+@pytest.mark.parametrize("M,K,N", [(1, 64, 352), (9, 96, 400), (64, 2048, 96), (65, 176, 128), (300, 256, 1030),
+                                   (8, 64, 28672), (16, 72, 27648), (12, 64, 22010)])
 def test_linear_swiglu_epilogue(dtype, M, K, N):
     g = torch.Generator().manual_seed(M + N)
     a = torch.randn(M, K, generator=g).to(dtype)

@@ -1613,7 +1613,18 @@ static int launch_skinny(const SkinnyArgs& p, hipStream_t stream) {
         if (ct == 3) return launch_skinny_tile<1, 3, TO, PRO, SWIGLU>(q, stream);
         return launch_skinny_tile<1, 4, TO, PRO, SWIGLU>(q, stream);
       }
-      if (ct > 4 && p.M >= 8) return launch_skinny_tile<1, 2, TO, PRO, SWIGLU>(p, stream);
+      if (ct > 4 && p.M >= 8) {
+        // several rounds of two column tiles: as many columns a workgroup (17 to 32, even) as make whole
+        // rounds of 256 workgroups (28,672 columns: 1,024 workgroups of 28 instead of 896 of 32, which
+        // are four rounds as well)
+        SkinnyArgs q = p;
+        const int rounds = (p.N + 256 * 2 * S_COLS - 1) / (256 * 2 * S_COLS);
+        const int cw = (p.N + rounds * 256 - 1) / (rounds * 256);
+        q.cols_wg = cw + (cw & 1);
+        // (a product that prepares a norm keeps whole tiles: its parts are counted per 16 columns)
+        if (q.cols_wg <= S_COLS || q.cols_wg >= 2 * S_COLS || p.emit_operand) q.cols_wg = 0;
+        return launch_skinny_tile<1, 2, TO, PRO, SWIGLU>(q, stream);
+      }
     }
     return launch_skinny_tile<1, 1, TO, PRO, SWIGLU>(p, stream);
   }
