@@ -1358,7 +1358,7 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
     for (int u = 0; u < UN; ++u) {
       // MFMA i of the block covers k = i*32 .. i*32+31, lane group g its 8 k from g*8: one load
       // instruction then reads 64 contiguous bytes of each of the 16 weight rows
-      if (HALF && u > 0 && blk + u * S_WAVES >= nblk) continue;      // the same for the whole wave: no such block
+      if (u > 0 && blk + u * S_WAVES >= nblk) continue;      // the same for the whole wave: no such block
       const int kb = (blk + u * S_WAVES) * KBLK + kh + g * 8;
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct)
@@ -1367,7 +1367,7 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
     }
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
-      if (HALF && u > 0 && blk + u * S_WAVES >= nblk) continue;
+      if (u > 0 && blk + u * S_WAVES >= nblk) continue;
       const int kb = (blk + u * S_WAVES) * KBLK + kh + g * 8;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -1389,7 +1389,7 @@ __global__ __launch_bounds__(S_THREADS) void gemm_skinny_bf16_kernel(const Skinn
   auto multiply = [&](const Stage& st, int blk) {
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
-      if (HALF && u > 0 && blk + u * S_WAVES >= nblk) continue;      // nothing was loaded for it
+      if (u > 0 && blk + u * S_WAVES >= nblk) continue;      // nothing was loaded for it
       const int kb = (blk + u * S_WAVES) * KBLK + kh + g * 8;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -1613,7 +1613,12 @@ static int launch_skinny(const SkinnyArgs& p, hipStream_t stream) {
         if (ct == 3) return launch_skinny_tile<1, 3, TO, PRO, SWIGLU>(q, stream);
         return launch_skinny_tile<1, 4, TO, PRO, SWIGLU>(q, stream);
       }
-      if (ct > 4 && p.M >= 8) {
+      // (below 8 rows too where one tile would leave the last of the kernel's stages, 16 k blocks of 128
+      // over the eight waves, half empty or emptier at a long inner size: inner size 5120 x 27,648
+      // columns at 1 row, 52 us against 61)
+      const int tail_blocks = ((p.K + S_KBLK - 1) / S_KBLK) % (2 * S_WAVES);
+      const bool half_empty_stage = p.K > 4096 && tail_blocks >= 1 && tail_blocks <= S_WAVES;
+      if (ct > 4 && (p.M >= 8 || half_empty_stage)) {
         // several rounds of two column tiles: as many columns a workgroup (17 to 32, even) as make whole
         // rounds of 256 workgroups (28,672 columns: 1,024 workgroups of 28 instead of 896 of 32, which
         // are four rounds as well)
