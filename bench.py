@@ -468,6 +468,27 @@ def long_context_llama3_8b(args):
     return out
 
 
+def decode_larger_shapes(args):
+    """Decode steps at the Llama-3-8B and Llama-2-13B shapes, 512-token prompts, by batch: a step's time
+    against the bytes it has to read."""
+    out = {}
+    for name, shape in (("llama3_8b", LLAMA3_8B), ("llama2_13b", LLAMA2_13B)):
+        cfg = dict(shape)
+        if args.soak_layers:
+            cfg["num_hidden_layers"] = min(cfg["num_hidden_layers"], args.soak_layers)
+        b = Bench(cfg, "bf16", 64, 160, 16, budget=4096)
+        out[name] = {"layers": cfg["num_hidden_layers"], "layers_full": shape["num_hidden_layers"]}
+        for batch in (1, 8, 16, 32, 64):
+            dt, ctx = b.decode(batch, 64, 8)
+            r = decode_rooflines(cfg, "bf16", batch, dt / 64, ctx)
+            out[name][f"batch{batch}"] = {"ms": r["ms"], "tok_s": round(batch * 64 / dt, 1), "GBs": r["GBs"],
+                                         "hbm_frac": r["hbm_frac"]}
+            print(f"# {name} batch {batch:2d}: {dt / 64 * 1e3:7.3f} ms a step, {r['GBs']:7.1f} GB/s ({r['hbm_frac']:.3f} of "
+                  f"{HBM_GBS / 1e3:.0f} TB/s)", file=sys.stderr, flush=True)
+        b.close()
+    return out
+
+
 def prefill_llama3_8b(args):
     """Whole prompts of 4,096 and 8,192 tokens at the Llama-3-8B shape, one step each."""
     cfg = dict(LLAMA3_8B)
@@ -678,6 +699,9 @@ def run(args):
     if args.only == "peaks":
         print(json.dumps({"measured_peaks": peaks}), flush=True)
         return
+    if args.only == "decode_shapes":
+        print(json.dumps({"decode_larger_shapes": decode_larger_shapes(args)}), flush=True)
+        return
     if args.only == "long_context":
         print(json.dumps({"llama3_8b_long_context": long_context_llama3_8b(args)}), flush=True)
         return
@@ -740,13 +764,13 @@ def main():
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--only", default="all",
                     choices=["all", "headline", "decode", "prefill", "fp32", "kernels", "peaks", "llama3_8b", "llama3_8b_prefill", "llama2_13b", "host",
-                             "attention", "long_context"],
+                             "attention", "long_context", "decode_shapes"],
                     help="all: everything in one line; headline: the bfloat16 TinyLlama figures only; decode / prefill: "
                          "one of them (profiling); fp32: the float32 figures as the headline; kernels: decode with the time of "
                          "a step by kernel (torch's profiler); peaks / llama3_8b / "
                          "llama2_13b: that part alone; host: a step's wall time against its time on the GPU; attention: the "
                          "attention kernels alone at contexts up to 131,072 tokens; long_context: the Llama-3-8B shape with "
-                         "8 requests of 32,000 tokens and one of 131,000")
+                         "8 requests of 32,000 tokens and one of 131,000; decode_shapes: decode steps at the two larger shapes by batch")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         if int(os.environ.get("RANK", "0")) == 0:
