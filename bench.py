@@ -152,7 +152,10 @@ class Bench:
         Returns (seconds, cached tokens read per step summed over the batch)."""
         from tiny_llm_amd import SamplingParams
         eng = self.engine
-        params = SamplingParams.greedy(warmup + steps + 64, ignore_eos=True)      # nobody ends inside the run
+        # nobody ends inside the run: requests whose prompt is done decode while the others' prompts are
+        # still computed, a token per step of that phase
+        ahead = -(-batch * prompt_len // eng.scheduler.budget)
+        params = SamplingParams.greedy(warmup + steps + 64 + ahead, ignore_eos=True)
         ids = [eng.add_request(gen_tokens(prompt_len, self.V, 1000 + i), params) for i in range(batch)]
         reqs = [eng.requests[i] for i in ids]
         while any(r.num_computed < prompt_len for r in reqs):
@@ -355,7 +358,8 @@ def tinyllama_figures(args, dtype, peaks):
     steps, warmup = args.steps, args.warmup
     if dtype == "fp32":
         steps, warmup = min(steps, 64), min(warmup, 8)       # the 32-bit path is for checking: a shorter run
-    b = Bench(cfg, dtype, max(args.batch, 64), warmup + steps + 80, args.block_size, prompt_len=args.prompt_len)
+    ahead = -(-max(args.batch, 64) * args.prompt_len // 4096)        # tokens decoded while other prompts are computed
+    b = Bench(cfg, dtype, max(args.batch, 64), warmup + steps + 80 + ahead, args.block_size, prompt_len=args.prompt_len)
     out = {}
     if args.only in ("all", "headline", "fp32", "prefill"):
         pf = b.prefill(3)
