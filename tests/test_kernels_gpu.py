@@ -455,14 +455,14 @@ def test_norm_prescale_f32_any_inner_size(K):
                                  (1536, 2050)])
 def test_linear_row_alone_equals_row_in_batch_fp32(K, N):
     """In float32 a row gives the same bits alone, among a few rows and among many: the tiled kernel
-    (more than 16 rows, or an inner size that is no multiple of 4) and the few-row kernel add in one
+    (more than 256 rows, or an inner size that is no multiple of 4) and the few-row kernel add in one
     order, also where the few-row kernel puts two k blocks into one matrix tile (up to 8 rows and 2,048
     columns; an odd number of blocks, a last block that is not whole).  With residual and with the
     SiLU-gate epilogue too."""
     g = torch.Generator().manual_seed(5 + K)
-    a = torch.randn(70, K, generator=g).to(DEV)
+    a = torch.randn(300, K, generator=g).to(DEV)       # 300 rows: the tiled kernel whatever the other sizes
     w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(DEV)
-    res = torch.randn(70, N, generator=g).to(DEV)
+    res = torch.randn(300, N, generator=g).to(DEV)
     for kwargs in ({}, {"residual": True}, {"epilogue": "swiglu"}):
         width = N // 2 if "epilogue" in kwargs else N
         def run(rows):
@@ -471,7 +471,9 @@ def test_linear_row_alone_equals_row_in_batch_fp32(K, N):
             r = res[rows].contiguous() if kwargs.get("residual") else None
             ops().linear(x, w, out, r, epilogue=kwargs.get("epilogue"))
             return out
-        full = run(slice(0, 70))
+        full = run(slice(0, 300))
+        assert torch.equal(full[100:230], run(slice(100, 230)))      # 65 to 256 rows: either kernel, by estimate
+        assert torch.equal(full[0:256], run(slice(0, 256)))
         assert torch.equal(full[37:38], run(slice(37, 38)))
         assert torch.equal(full[30:43], run(slice(30, 43)))
         assert torch.equal(full[30:38], run(slice(30, 38)))
