@@ -410,7 +410,8 @@ def test_linear_norm_f32(M, K, N):
     # the plain product owns two or three column tiles): the same BITS, with every epilogue, also
     # when the rows sit among many others (the tiled product) and when they are gathered
     tiles = -(-N // 16)
-    assert ops().linear_f32_col_tiles(M, N, K) == (min(3, -(-tiles // 256)) if M <= 16 and tiles > 256 else 1)
+    ct = ops().linear_f32_col_tiles(M, N, K)
+    assert (2 <= ct <= 3) if M <= 16 and tiles > 256 else ct == 1
     hp, inv = ops().norm_prescale_f32(x, nw, eps)
     assert rel(hp, (x * nw).double().cpu()) == 0.0
     two = torch.full((M, N), float("nan"), device=DEV)

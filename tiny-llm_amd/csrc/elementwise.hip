@@ -120,8 +120,12 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const int32_t* __restrict
                                   const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                   const int32_t* __restrict__ slot_mapping, T* __restrict__ k_cache,
                                   T* __restrict__ v_cache, int nq, int nkv, int hd, int rot,
-                                  int block_size, int64_t row_stride, int interleaved) {
+                                  int block_size, int64_t row_stride, int interleaved, int heads_wg) {
+  // blockIdx.y: a run of `heads_wg` of the token's q and k heads (a k head brings its v head along), so
+  // that a step of few tokens still is a launch of many workgroups
   const int t = blockIdx.x;
+  const int head0 = blockIdx.y * heads_wg, head1 = min(nq + nkv, head0 + heads_wg);
+  const int kv0 = max(head0, nq) - nq, kv1 = max(head1, nq) - nq;        // the kv heads among them
   const int pos = positions[t];
   const int half = rot / 2;
   const int slot = slot_mapping ? slot_mapping[t] : -1;
@@ -138,8 +142,8 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const int32_t* __restrict
                            (uintptr_t)sin_t) & 15) == 0;
     if (rot == hd && half % 8 == 0 && row_stride % 8 == 0 && aligned && !interleaved) {
       const int chunks = half / 8;
-      for (int i = threadIdx.x; i < (nq + nkv) * chunks; i += kThreads) {
-        const int head = i / chunks, j = (i - head * chunks) * 8;
+      for (int i = threadIdx.x; i < (head1 - head0) * chunks; i += kThreads) {
+        const int head = head0 + i / chunks, j = (i % chunks) * 8;
         bf16_t* h = (bf16_t*)row + (int64_t)head * hd;
         const bf16x8 a8 = *(const bf16x8*)(h + j), b8 = *(const bf16x8*)(h + j + half);
         const f32x4 c0 = *(const f32x4*)(cs + j), c1 = *(const f32x4*)(cs + j + 4);
@@ -162,8 +166,8 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const int32_t* __restrict
         }
       }
       if (slot < 0) return;
-      for (int i = threadIdx.x; i < nkv * hd / 8; i += kThreads) {
-        const int head = (i * 8) / hd, j = i * 8 - head * hd;
+      for (int i = threadIdx.x; i < (kv1 - kv0) * (hd / 8); i += kThreads) {
+        const int head = kv0 + i / (hd / 8), j = (i % (hd / 8)) * 8;
         *(bf16x8*)((bf16_t*)v_cache + ((blk * nkv + head) * block_size + in_blk) * hd + j) =
             *(const bf16x8*)((const bf16_t*)row + (int64_t)(nq + nkv + head) * hd + j);
       }
@@ -171,9 +175,9 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const int32_t* __restrict
     }
   }
   // rotated pairs of q and k heads
-  const int pairs = (nq + nkv) * half;
+  const int pairs = (head1 - head0) * half;
   for (int i = threadIdx.x; i < pairs; i += kThreads) {
-    const int head = i / half, j = i - head * half;
+    const int head = head0 + i / half, j = i % half;
     const int ia = interleaved ? 2 * j : j, ib = interleaved ? 2 * j + 1 : j + half;
     T* h = row + (int64_t)head * hd;
     const float a = to_f32(h[ia]), b = to_f32(h[ib]);
@@ -192,12 +196,12 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const int32_t* __restrict
   if (slot < 0) return;
   // dims of k beyond the rotated part, and all of v, are copied as they are
   const int tail = hd - rot;
-  for (int i = threadIdx.x; i < nkv * tail; i += kThreads) {
-    const int head = i / tail, j = rot + (i - head * tail);
+  for (int i = threadIdx.x; i < (kv1 - kv0) * tail; i += kThreads) {
+    const int head = kv0 + i / tail, j = rot + i % tail;
     k_cache[((blk * nkv + head) * block_size + in_blk) * hd + j] = row[(int64_t)(nq + head) * hd + j];
   }
-  for (int i = threadIdx.x; i < nkv * hd; i += kThreads) {
-    const int head = i / hd, j = i - head * hd;
+  for (int i = threadIdx.x; i < (kv1 - kv0) * hd; i += kThreads) {
+    const int head = kv0 + i / hd, j = i % hd;
     v_cache[((blk * nkv + head) * block_size + in_blk) * hd + j] = row[(int64_t)(nq + nkv + head) * hd + j];
   }
 }
@@ -343,9 +347,16 @@ int tl_rope_store(void* qkv, const int32_t* positions, const float* cos_t, const
   if (interleaved != 0 && interleaved != 1) return TL_ERR_ARG;
   if (rot > 0 && (!cos_t || !sin_t)) return TL_ERR_ARG;
   if (slot_mapping && (!k_cache || !v_cache)) return TL_ERR_ARG;
-  TL_DISPATCH_T(dtype, hipLaunchKernelGGL(rope_store_kernel<T>, dim3(n_tokens), dim3(kThreads), 0, stream,
+  // about 256 workgroups where the tokens alone are fewer: the heads of a token shared out
+  const int heads = nq + nkv;
+  int groups = n_tokens >= 256 ? 1 : (256 + n_tokens - 1) / n_tokens;
+  if (groups > heads) groups = heads;
+  const int heads_wg = (heads + groups - 1) / groups;
+  groups = (heads + heads_wg - 1) / heads_wg;
+  TL_DISPATCH_T(dtype, hipLaunchKernelGGL(rope_store_kernel<T>, dim3(n_tokens, groups), dim3(kThreads), 0, stream,
                                           (T*)qkv, positions, cos_t, sin_t, slot_mapping, (T*)k_cache,
-                                          (T*)v_cache, nq, nkv, hd, rot, block_size, row_stride, interleaved);)
+                                          (T*)v_cache, nq, nkv, hd, rot, block_size, row_stride, interleaved,
+                                          heads_wg);)
   return tl_launch_status();
 }
 

@@ -275,7 +275,10 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
                                                                    const float* __restrict__ norm_w = nullptr,
                                                                    float eps = 0.f,
                                                                    const float* __restrict__ row_scale = nullptr,
-                                                                   int tiles_wg = FR_MAX_MT) {
+                                                                   int tiles_wg = FR_MAX_MT, int cols_wg = 0) {
+  // cols_wg (even, with CT column tiles of which the last is partly used): the columns a workgroup owns
+  // where whole tiles would not make whole rounds of 256 workgroups; the tile's other columns repeat
+  // the last one and are dropped.
   // WIDE (more than 16 rows): blockIdx.y picks a group of `tiles_wg` row tiles, so that a product with
   // few column tiles still gives every compute unit a workgroup with whole matrix tiles (16 columns)
   // instead of half-used ones (8 columns); the activations of the next row tile are requested before
@@ -294,8 +297,9 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
   constexpr int UNIT = PAIR ? 2 : 1;
   const int second = PAIR ? l16 / 8 : 0;
   const int units = (nkb + UNIT - 1) / UNIT;
-  const int n0 = blockIdx.x * COLS * CT;
-  auto wrow_of = [&](int ct) { return w + (int64_t)min(n0 + ct * COLS + l16 % COLS, N - 1) * K; };
+  const int cw = cols_wg > 0 ? cols_wg : COLS * CT;
+  const int n0 = blockIdx.x * cw;
+  auto wrow_of = [&](int ct) { return w + (int64_t)min(n0 + min(ct * COLS + l16 % COLS, cw - 1), N - 1) * K; };
   const float* wrow = wrow_of(0);
   // A k block that lies wholly inside K is loaded without a predicate per load (each would be a
   // branch of its own, and the waits around branches are placed for the worst case); only the last,
@@ -420,9 +424,9 @@ __global__ __launch_bounds__(FR_THREADS) void gemm_f32_rows_kernel(const float* 
     }
     if constexpr (SWIGLU) {   // columns (2j, 2j+1) = (gate_j, up_j); N and n0 are even
       const float u = __shfl_down(t, 1, TL_WAVE);
-      if (m < M && n < N && (c & 1) == 0) out[(int64_t)m * ldo + n / 2] = swiglu_pair(t, u);
+      if (m < M && n < N && ct * COLS + c < cw && (c & 1) == 0) out[(int64_t)m * ldo + n / 2] = swiglu_pair(t, u);
     } else {
-      if (m < M && n < N) {
+      if (m < M && n < N && ct * COLS + c < cw) {
         const int64_t at = (int64_t)m * ldo + n;
         out[at] = residual ? t + residual[at] : t;
       }
@@ -1650,16 +1654,24 @@ static int launch_skinny_out(const SkinnyArgs& p, int out_dtype, bool swiglu, hi
 }
 
 // Column tiles a workgroup of the float32 few-row kernel owns: one, or, with one row tile and more
-// than 256 column tiles of 16, as many (up to three: four would not leave the registers for a piece of
-// weights ahead) as bring the workgroups down to one to three rounds over the 256 compute units,
-// while the block sums fit into LDS.
-static int f32_rows_col_tiles(int M, int N, int K, int cols) {
+// than 256 column tiles of 16, up to three (four would not leave the registers for a piece of weights
+// ahead) while the block sums fit into LDS, and of them as many columns (*cols_wg, even; 0: all) as make
+// whole rounds of 256 workgroups: 5,120 columns are one round of 20, 15,360 two rounds of 30, 28,672
+// three rounds of 38, where whole tiles would leave the last round a quarter full.
+static int f32_rows_col_tiles(int M, int N, int K, int cols, int* cols_wg = nullptr) {
+  if (cols_wg) *cols_wg = 0;
   if (M > 16 || cols != 16) return 1;
   const int tiles = (N + 15) / 16, nkb = (K + F_KBLOCK - 1) / F_KBLOCK;
-  int ct = tiles > 256 ? (tiles + 255) / 256 : 1;
-  if (ct > 3) ct = 3;
-  while (ct > 1 && (size_t)nkb * 16 * 16 * ct * sizeof(float) > 96 * 1024) --ct;
-  return ct;
+  if (tiles <= 256) return 1;
+  for (int rounds = 1; rounds <= 1024; ++rounds) {
+    int cw = (N + 256 * rounds - 1) / (256 * rounds);
+    cw += cw & 1;
+    const int ct = (cw + 15) / 16;
+    if (ct > 3 || (size_t)nkb * 16 * 16 * ct * sizeof(float) > 96 * 1024) continue;
+    if (cols_wg && cw < 16 * ct && ct > 1) *cols_wg = cw;
+    return ct;
+  }
+  return 1;
 }
 
 }  // namespace
@@ -1771,7 +1783,8 @@ int tl_linear_tile(const void* a, const void* w, void* out, const float* residua
         groups *= 2;
     }
     const int tiles_wg = (mts + groups - 1) / groups;
-    const int ct = f32_rows_col_tiles(M, N, K, cols);
+    int cols_wg = 0;
+    const int ct = f32_rows_col_tiles(M, N, K, cols, &cols_wg);
     const size_t rows_smem = (size_t)tiles_wg * nkb * 16 * cols * ct * sizeof(float);
     // Up to 64 rows the few-row kernel; up to 256 where it is estimated faster than the tiled kernel, whose few
     // tiles each walk the whole inner size (measured at inner size 2048: 87 us a round of up to 352 tiles of
@@ -1803,11 +1816,12 @@ int tl_linear_tile(const void* a, const void* w, void* out, const float* residua
             return TL_ERR_LAUNCH;
         configured = true;
       }
-      dim3 gr((N + cols * ct - 1) / (cols * ct), (mts + tiles_wg - 1) / tiles_wg);
+      const int cw = cols_wg > 0 ? cols_wg : cols * ct;
+      dim3 gr((N + cw - 1) / cw, (mts + tiles_wg - 1) / tiles_wg);
 #define TL_F32_ROWS_K(...)                                                                                          \
   hipLaunchKernelGGL((gemm_f32_rows_kernel<__VA_ARGS__>), gr, dim3(FR_THREADS), rows_smem, stream, (const float*)a, \
                      (const float*)w, (float*)out, residual, M, N, K, lda, ldo, (const float*)nullptr, 0.f, row_scale, \
-                     tiles_wg)
+                     tiles_wg, cols_wg)
 #define TL_F32_ROWS(SW, CO, WI, CTI) TL_F32_ROWS_K(SW, CO, false, WI, CTI)
 #define TL_F32_ROWS_CT(SW)                                                                                           \
   do {                                                                                                               \
