@@ -10,7 +10,10 @@ kernel; the same in true float32; the machine's peaks
 as measured on the spot (a streaming kernel, a loop of matrix instructions); and two soak workloads
 at larger shapes (a mixed batch of 16 requests with prompts cut into portions of 512 at the
 Llama-3-8B shape; 64 requests of 1,024 tokens that nearly fill the cache at the Llama-2-13B shape).
-`--only` picks a part (for profiling).
+`--only` picks a part (for profiling), or one of the measurements that are not part of the line:
+`attention` (the attention kernels alone at contexts up to 131,072 tokens), `long_context` (the Llama-3-8B
+shape with 8 requests of 32,000 tokens and one of 131,000), `decode_shapes` (decode steps at the two larger
+shapes by batch), `host` (a step's wall time against its time on the GPU).
 """
 import argparse
 import json
