@@ -882,6 +882,26 @@ def test_attention_f32_gives_the_same_bits_however_the_work_is_cut():
     assert torch.equal(tail.cpu()[0], base.cpu()[299]) and torch.equal(tail.cpu()[1], base.cpu()[376])
 
 
+@pytest.mark.parametrize("nq,nkv,hd,window", [(8, 4, 64, 0), (4, 4, 32, 0), (16, 2, 128, 0), (8, 4, 48, 300)])
+def test_attention_f32_of_many_query_tiles_has_the_bits_of_few(nq, nkv, hd, window):
+    """A step of a thousand query tiles and more (whole prompts) runs a wave per tile, four neighbouring
+    tiles a workgroup; the same rows as a step of chunks given to workgroups of their own (what decode
+    steps run), and in tiles of one token: the same bits, and the plain result within rounding."""
+    per = 16 // (nq // nkv)
+    lens = [per * (1024 // nkv), 700, 65, 1]        # whole prompts: at least 1,024 tiles x kv heads
+    assert sum(-(-n // per) for n in lens) * nkv >= 1024
+    kw = dict(lens=lens, q_lens=lens, nq=nq, nkv=nkv, hd=hd, bs=16, seed=11, window=window, impl="f32")
+    many, ref = _paged_case(torch.float32, **kw)
+    assert not torch.isnan(many).any()
+    assert rel(many, ref) < 2e-6
+    chunks = -(-max(lens) // 256)
+    few, _ = _paged_case(torch.float32, n_splits=chunks, **kw)
+    assert torch.equal(many.cpu(), few.cpu())
+    if nq == nkv:      # tiles of one token are tiles of one row per head group only where a tile holds 16 tokens
+        single, _ = _paged_case(torch.float32, tile_tokens=3, **kw)
+        assert torch.equal(many.cpu(), single.cpu())
+
+
 def test_flash_attention_decode_batch():
     """Single decoded tokens of many requests of very different lengths, keys split over workgroups."""
     lens = [1, 2, 63, 64, 65, 127, 128, 129, 500, 1000, 17, 256]

@@ -562,6 +562,135 @@ __device__ __forceinline__ float merge_f32_value(float O, float o, float wa, flo
   return __builtin_fmaf(O, wa, ob);
 }
 
+// One tile of 64 keys at kb for the 16 query rows of a wave: (m, l, O) from scratch.  `finite_row`: any
+// HD finite floats (read in place of value rows outside the request's keys); Vl: the wave's own LDS area.
+template <int HDT>
+__device__ __forceinline__ void attention_f32_tile(int kb, const int32_t* __restrict__ bt, int max_blocks, int block_size,
+                                                   int nkv, int kvh, const float* __restrict__ k_cache,
+                                                   const float* __restrict__ v_cache, const float* __restrict__ finite_row,
+                                                   const f32x4 (&qf)[HDT], float c_log2, bool row_valid, int pos, int row_lo,
+                                                   int kv_begin, int kv_end, float* Vl, float& m_t, float& l_t,
+                                                   f32x4 (&o)[HDT]) {
+  constexpr int HD = HDT * 16;
+  const int lane = threadIdx.x % TL_WAVE, l16 = lane % 16, kk = lane / 16;
+  // Everything the tile needs from memory is requested together, in two rounds (page numbers,
+  // then rows): loads are unconditional, with the index clamped into the table; a conditional
+  // load would become a branch, and every branch one more round trip in a row.  A key row
+  // outside the request's keys is read from row 0 of page 0 (its scores are masked below,
+  // whatever they are); a value row outside from the query rows of this tile's first token
+  // (finite numbers: its probabilities are exact zeros, and stale pages may hold NaN, for which
+  // 0 * NaN is NaN).  Nothing is selected into loaded registers, which would make the wave wait
+  // for the rows where the select stands.
+  constexpr int VPRE = (HD < A32_VW ? HD : A32_VW) / 4;
+  const int vkey = kb + lane;
+  const bool v_in_range = vkey >= kv_begin && vkey < kv_end;
+  bool k_in[4];
+  int page_k[4];
+#pragma unroll
+  for (int st = 0; st < 4; ++st) {
+    const int key = kb + st * 16 + l16;
+    k_in[st] = key < kv_end;
+    page_k[st] = bt[min(key / block_size, max_blocks - 1)];
+  }
+  const int page_v = bt[min(vkey / block_size, max_blocks - 1)];
+  auto row_of = [&](int page, int key, bool in) {
+    const int64_t off = (((int64_t)max(page, 0) * nkv + kvh) * block_size + (key - (key / block_size) * block_size)) * HD;
+    return in ? off : (int64_t)0;
+  };
+  const float* vrow = v_in_range ? v_cache + row_of(page_v, vkey, true) : finite_row;
+  f32x4 vpre[VPRE];
+#pragma unroll
+  for (int ch = 0; ch < VPRE; ++ch) vpre[ch] = *(const f32x4*)(vrow + ch * 4);
+  // ---- scores S^T = K Q^T: lane (l16, kk) of subtile st holds keys kb + 16 st + 4 kk + r of row l16
+  f32x4 sc[4];
+  constexpr int STB = HDT <= 4 ? 4 : 2;       // subtiles whose key rows are in registers together
+#pragma unroll
+  for (int s0 = 0; s0 < 4; s0 += STB) {
+    f32x4 kf[STB][HDT];
+#pragma unroll
+    for (int si = 0; si < STB; ++si) {
+      const float* krow = k_cache + row_of(page_k[s0 + si], kb + (s0 + si) * 16 + l16, k_in[s0 + si]);
+#pragma unroll
+      for (int g4 = 0; g4 < HDT; ++g4) kf[si][g4] = *(const f32x4*)(krow + g4 * 16 + kk * 4);
+    }
+#pragma unroll
+    for (int si = 0; si < STB; ++si) {
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int g4 = 0; g4 < HDT; ++g4) {
+        const f32x4 kv = kf[si][g4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(kv[e], qf[g4][e], acc, 0, 0, 0);
+      }
+      sc[s0 + si] = acc;
+    }
+  }
+  // ---- the tile's softmax from scratch
+  m_t = -INFINITY;
+#pragma unroll
+  for (int st = 0; st < 4; ++st)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int key = kb + st * 16 + kk * 4 + r;
+      const bool vis = row_valid && key <= pos && key >= row_lo;
+      sc[st][r] = vis ? sc[st][r] * c_log2 : -INFINITY;
+      m_t = fmaxf(m_t, sc[st][r]);
+    }
+  m_t = fmaxf(max_over_rows(m_t), kNegBig);
+  l_t = 0.f;
+#pragma unroll
+  for (int st = 0; st < 4; ++st)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      sc[st][r] = __builtin_amdgcn_exp2f(sc[st][r] - m_t);
+      l_t += sc[st][r];
+    }
+  l_t = sum_over_rows(l_t);
+  // ---- O^T = V^T P^T, the values staged 64 columns at a time (lane = key row)
+#pragma unroll
+  for (int dt = 0; dt < HDT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  {
+#pragma unroll
+    for (int dh = 0; dh < (HD + A32_VW - 1) / A32_VW; ++dh) {
+      constexpr int full = A32_VW / 4;
+      const int chunks = min(full, (HD - dh * A32_VW) / 4);
+      if (dh > 0) {       // this wave's reads of the columns staged before are done
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      }
+#pragma unroll
+      for (int ch = 0; ch < full; ++ch)
+        if (ch < chunks) {
+          f32x4 v;
+          if (dh == 0) v = vpre[ch < VPRE ? ch : 0];
+          else v = *(const f32x4*)(vrow + dh * A32_VW + ch * 4);
+          *(f32x4*)(&Vl[lane * A32_VS + ch * 4]) = v;
+        }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+      for (int dl = 0; dl < A32_VW / 16; ++dl) {
+        const int dt = dh * (A32_VW / 16) + dl;
+        if (dt < HDT) {
+#pragma unroll
+          for (int st = 0; st < 4; ++st)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const float vf = Vl[(st * 16 + kk * 4 + r) * A32_VS + dl * 16 + l16];
+              o[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf, sc[st][r], o[dt], 0, 0, 0);
+            }
+        }
+      }
+    }
+    // the area is free for the wave's next tile
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
+}
+
 template <int HDT>
 __global__ __launch_bounds__(A32_THREADS) void attention_f32_kernel(
     const float* __restrict__ q, int64_t q_stride, const float* __restrict__ k_cache,
@@ -621,124 +750,11 @@ __global__ __launch_bounds__(A32_THREADS) void attention_f32_kernel(
   for (int c = c_first; c < c_last; ++c) {
     const int t_lo = max(c * A32_CHUNK, first_tile), t_hi = min((c + 1) * A32_CHUNK, last_tile);
     for (int t = t_lo + wave; t < t_hi; t += A32_WAVES) {
-      const int kb = t * FA_KT;
-      // Everything the tile needs from memory is requested together, in two rounds (page numbers,
-      // then rows): loads are unconditional, with the index clamped into the table; a conditional
-      // load would become a branch, and every branch one more round trip in a row.  A key row
-      // outside the request's keys is read from row 0 of page 0 (its scores are masked below,
-      // whatever they are); a value row outside from the query rows of this tile's first token
-      // (finite numbers: its probabilities are exact zeros, and stale pages may hold NaN, for which
-      // 0 * NaN is NaN).  Nothing is selected into loaded registers, which would make the wave wait
-      // for the rows where the select stands.
-      constexpr int VPRE = (HD < A32_VW ? HD : A32_VW) / 4;
-      const int vkey = kb + lane;
-      const bool v_in_range = vkey >= kv_begin && vkey < kv_end;
-      bool k_in[4];
-      int page_k[4];
-#pragma unroll
-      for (int st = 0; st < 4; ++st) {
-        const int key = kb + st * 16 + l16;
-        k_in[st] = key < kv_end;
-        page_k[st] = bt[min(key / block_size, max_blocks - 1)];
-      }
-      const int page_v = bt[min(vkey / block_size, max_blocks - 1)];
-      auto row_of = [&](int page, int key, bool in) {
-        const int64_t off = (((int64_t)max(page, 0) * nkv + kvh) * block_size + (key - (key / block_size) * block_size)) * HD;
-        return in ? off : (int64_t)0;
-      };
-      const float* vrow = v_in_range ? v_cache + row_of(page_v, vkey, true) : q + (int64_t)tok0 * q_stride + (int64_t)kvh * G * HD;
-      f32x4 vpre[VPRE];
-#pragma unroll
-      for (int ch = 0; ch < VPRE; ++ch) vpre[ch] = *(const f32x4*)(vrow + ch * 4);
-      // ---- scores S^T = K Q^T: lane (l16, kk) of subtile st holds keys kb + 16 st + 4 kk + r of row l16
-      f32x4 sc[4];
-      constexpr int STB = HDT <= 4 ? 4 : 2;       // subtiles whose key rows are in registers together
-#pragma unroll
-      for (int s0 = 0; s0 < 4; s0 += STB) {
-        f32x4 kf[STB][HDT];
-#pragma unroll
-        for (int si = 0; si < STB; ++si) {
-          const float* krow = k_cache + row_of(page_k[s0 + si], kb + (s0 + si) * 16 + l16, k_in[s0 + si]);
-#pragma unroll
-          for (int g4 = 0; g4 < HDT; ++g4) kf[si][g4] = *(const f32x4*)(krow + g4 * 16 + kk * 4);
-        }
-#pragma unroll
-        for (int si = 0; si < STB; ++si) {
-          f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-          for (int g4 = 0; g4 < HDT; ++g4) {
-            const f32x4 kv = kf[si][g4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(kv[e], qf[g4][e], acc, 0, 0, 0);
-          }
-          sc[s0 + si] = acc;
-        }
-      }
-      // ---- the tile's softmax from scratch
-      float m_t = -INFINITY;
-#pragma unroll
-      for (int st = 0; st < 4; ++st)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int key = kb + st * 16 + kk * 4 + r;
-          const bool vis = row_valid && key <= pos && key >= row_lo;
-          sc[st][r] = vis ? sc[st][r] * c_log2 : -INFINITY;
-          m_t = fmaxf(m_t, sc[st][r]);
-        }
-      m_t = fmaxf(max_over_rows(m_t), kNegBig);
-      float l_t = 0.f;
-#pragma unroll
-      for (int st = 0; st < 4; ++st)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          sc[st][r] = __builtin_amdgcn_exp2f(sc[st][r] - m_t);
-          l_t += sc[st][r];
-        }
-      l_t = sum_over_rows(l_t);
-      // ---- O^T = V^T P^T, the values staged 64 columns at a time (lane = key row)
+      float m_t, l_t;
       f32x4 o[HDT];
-#pragma unroll
-      for (int dt = 0; dt < HDT; ++dt) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-      {
-#pragma unroll
-        for (int dh = 0; dh < (HD + A32_VW - 1) / A32_VW; ++dh) {
-          constexpr int full = A32_VW / 4;
-          const int chunks = min(full, (HD - dh * A32_VW) / 4);
-          if (dh > 0) {       // this wave's reads of the columns staged before are done
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-          }
-#pragma unroll
-          for (int ch = 0; ch < full; ++ch)
-            if (ch < chunks) {
-              f32x4 v;
-              if (dh == 0) v = vpre[ch < VPRE ? ch : 0];
-              else v = *(const f32x4*)(vrow + dh * A32_VW + ch * 4);
-              *(f32x4*)(&Vl[lane * A32_VS + ch * 4]) = v;
-            }
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-          __builtin_amdgcn_wave_barrier();
-          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-          for (int dl = 0; dl < A32_VW / 16; ++dl) {
-            const int dt = dh * (A32_VW / 16) + dl;
-            if (dt < HDT) {
-#pragma unroll
-              for (int st = 0; st < 4; ++st)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                  const float vf = Vl[(st * 16 + kk * 4 + r) * A32_VS + dl * 16 + l16];
-                  o[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf, sc[st][r], o[dt], 0, 0, 0);
-                }
-            }
-          }
-        }
-        // the area is free for the wave's next tile
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      }
+      attention_f32_tile<HDT>(t * FA_KT, bt, max_blocks, block_size, nkv, kvh, k_cache, v_cache,
+                              q + (int64_t)tok0 * q_stride + (int64_t)kvh * G * HD, qf, c_log2, row_valid, pos, row_lo,
+                              kv_begin, kv_end, Vl, m_t, l_t, o);
       // ---- the tile's (m, l, O) to its slot: lane (l16, kk) holds row l16, dims 16 dt + 4 kk + r
       const int slot = t - c * A32_CHUNK;
 #pragma unroll
@@ -782,6 +798,89 @@ __global__ __launch_bounds__(A32_THREADS) void attention_f32_kernel(
       }
     }
   }
+}
+
+// The same function for steps of many query tiles (prompts): a WAVE owns a query tile of 16 rows and walks
+// all its key tiles alone, merging them in registers in the one order (tiles of a chunk ascending from
+// "nothing", chunks ascending from "nothing"): the very operations attention_f32_kernel applies per
+// element, so the bits are the same.  The four waves of a workgroup own neighbouring query tiles of one kv
+// head, walk nearly the same keys at nearly the same time and find each other's key and value rows in the
+// compute unit's cache; with one tile a workgroup every 16 rows fetched all their keys from the L2, and a
+// whole prompt was bound by that (2,048 tokens, heads of 64: 537 us a layer).
+template <int HDT>
+__global__ __launch_bounds__(A32_THREADS) void attention_f32_rows_kernel(
+    const float* __restrict__ q, int64_t q_stride, const float* __restrict__ k_cache,
+    const float* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int max_blocks,
+    const int32_t* __restrict__ tile_req, const int32_t* __restrict__ tile_tok0,
+    const int32_t* __restrict__ tile_ntok, const int32_t* __restrict__ positions, float* __restrict__ out,
+    int64_t out_stride, int nq, int nkv, int block_size, float scale, int window, int n_tiles) {
+  constexpr int HD = HDT * 16;
+  extern __shared__ __attribute__((aligned(16))) float smem32[];
+  const int tid = threadIdx.x, lane = tid % TL_WAVE, wave = tid / TL_WAVE;
+  const int l16 = lane % 16, kk = lane / 16;
+  const int tile = blockIdx.x * A32_WAVES + wave, kvh = blockIdx.y;
+  if (tile >= n_tiles) return;                     // whole waves; the kernel has no workgroup barrier
+  const int G = nq / nkv, TW = 16 / G;
+  const int req = tile_req ? tile_req[tile] : tile, tok0 = tile_req ? tile_tok0[tile] : tile;
+  const int ntok = tile_req ? tile_ntok[tile] : 1;
+  if (ntok <= 0) return;                           // a padding tile
+  const int32_t* bt = block_tables + (int64_t)req * max_blocks;
+  float* Vl = smem32 + wave * FA_KT * A32_VS;
+
+  const int tok_local = l16 / G, hh = l16 % G;
+  const bool row_valid = tok_local < TW && tok_local < ntok;
+  const int tok = tok0 + (row_valid ? tok_local : 0);
+  const int pos = row_valid ? positions[tok] : -1;
+  const int row_lo = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
+  const int hi = row_max_i32(pos), lo = row_min_i32(row_valid ? row_lo : 0x7fffffff);
+  const int kv_end = hi + 1, kv_begin = lo;
+  const int first_tile = kv_begin / FA_KT, last_tile = (kv_end + FA_KT - 1) / FA_KT;
+  const int c_first = first_tile / A32_CHUNK, c_last = (last_tile + A32_CHUNK - 1) / A32_CHUNK;
+
+  f32x4 qf[HDT];
+  {
+    const float* qrow = q + (int64_t)tok * q_stride + (int64_t)(kvh * G + hh) * HD;
+#pragma unroll
+    for (int g4 = 0; g4 < HDT; ++g4)
+      qf[g4] = row_valid ? *(const f32x4*)(qrow + g4 * 16 + kk * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const float c_log2 = scale * 1.44269504088896341f;
+  const float* finite_row = q + (int64_t)tok0 * q_stride + (int64_t)kvh * G * HD;
+
+  // lane (l16, kk) holds row l16, dims 16 dt + 4 kk + r of the running result
+  float Mrun = kNegBig, Lrun = 0.f;
+  f32x4 Orun[HDT];
+#pragma unroll
+  for (int dt = 0; dt < HDT; ++dt) Orun[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int c = c_first; c < c_last; ++c) {
+    const int t_lo = max(c * A32_CHUNK, first_tile), t_hi = min((c + 1) * A32_CHUNK, last_tile);
+    float Mc = kNegBig, Lc = 0.f, wa, wb;
+    f32x4 Oc[HDT];
+#pragma unroll
+    for (int dt = 0; dt < HDT; ++dt) Oc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int t = t_lo; t < t_hi; ++t) {
+      float m_t, l_t;
+      f32x4 o[HDT];
+      attention_f32_tile<HDT>(t * FA_KT, bt, max_blocks, block_size, nkv, kvh, k_cache, v_cache, finite_row, qf, c_log2,
+                              row_valid, pos, row_lo, kv_begin, kv_end, Vl, m_t, l_t, o);
+      merge_f32(Mc, Lc, m_t, l_t, wa, wb);
+#pragma unroll
+      for (int dt = 0; dt < HDT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) Oc[dt][r] = merge_f32_value(Oc[dt][r], o[dt][r], wa, wb);
+    }
+    merge_f32(Mrun, Lrun, Mc, Lc, wa, wb);
+#pragma unroll
+    for (int dt = 0; dt < HDT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) Orun[dt][r] = merge_f32_value(Orun[dt][r], Oc[dt][r], wa, wb);
+  }
+  if (!row_valid) return;
+  float* orow = out + (int64_t)tok * out_stride + (int64_t)(kvh * G + hh) * HD;
+#pragma unroll
+  for (int dt = 0; dt < HDT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) orow[dt * 16 + kk * 4 + r] = Lrun > 0.f ? Orun[dt][r] / Lrun : 0.f;
 }
 
 // Merges the chunks that attention_f32_kernel left in `part` [chunks][tokens][heads][hd + 2], in
@@ -1317,6 +1416,31 @@ int tl_attention_f32(const float* q, int64_t q_stride, const float* k_cache, con
   if (!tile_req && (tile_tok0 || tile_ntok || n_tiles != n_tokens)) return TL_ERR_ARG;
   if (tile_req && (!tile_tok0 || !tile_ntok)) return TL_ERR_ARG;
   const size_t smem = (size_t)(A32_WAVES * FA_KT * A32_VS + A32_CHUNK * 16 * (hd + 4) + A32_CHUNK * 16 * 2) * sizeof(float);
+  // Many query tiles (prompts): a wave a tile, four neighbouring tiles a workgroup; few (decode steps, small
+  // steps): a workgroup a tile, its waves sharing the key tiles out.  The same bits either way.
+  if (n_chunks == 1 && (int64_t)n_tiles * nkv >= 1024) {
+    const size_t smem_rows = (size_t)A32_WAVES * FA_KT * A32_VS * sizeof(float);
+#define TL_A32_ROWS(HDT)                                                                                          \
+  case HDT: {                                                                                                     \
+    static bool configured = false;                                                                               \
+    if (!configured) {                                                                                            \
+      if (hipFuncSetAttribute((const void*)attention_f32_rows_kernel<HDT>,                                        \
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_rows) != hipSuccess)          \
+        return TL_ERR_LAUNCH;                                                                                     \
+      configured = true;                                                                                          \
+    }                                                                                                             \
+    hipLaunchKernelGGL(attention_f32_rows_kernel<HDT>, dim3((n_tiles + A32_WAVES - 1) / A32_WAVES, nkv),           \
+                       dim3(A32_THREADS), smem_rows, stream, q, q_stride, k_cache, v_cache, block_tables,          \
+                       max_blocks, tile_req, tile_tok0, tile_ntok, positions, out, out_stride, nq, nkv,            \
+                       block_size, scale, window, n_tiles);                                                        \
+  } break;
+    switch (hd / 16) {
+      TL_A32_ROWS(1) TL_A32_ROWS(2) TL_A32_ROWS(3) TL_A32_ROWS(4)
+      TL_A32_ROWS(5) TL_A32_ROWS(6) TL_A32_ROWS(7) TL_A32_ROWS(8)
+    }
+#undef TL_A32_ROWS
+    return tl_launch_status();
+  }
 #define TL_A32_CASE(HDT)                                                                                          \
   case HDT: {                                                                                                     \
     static bool configured = false;                                                                               \
