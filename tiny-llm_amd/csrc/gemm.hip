@@ -1788,7 +1788,7 @@ int tl_linear_tile(const void* a, const void* w, void* out, const float* residua
     const size_t rows_smem = (size_t)tiles_wg * nkb * 16 * cols * ct * sizeof(float);
     // Up to 64 rows the few-row kernel; up to 256 where it is estimated faster than the tiled kernel, whose few
     // tiles each walk the whole inner size (measured at inner size 2048: 87 us a round of up to 352 tiles of
-    // 64 x 64, 204 us a round of 128 x 128; the few-row kernel 0.62 us per row tile and million weights:
+    // 64 x 64, 204 us a round of 128 x 128; the few-row kernel 0.66 us per row tile and million weights:
     // 2048 x 2048 at 128 rows 25 us against 89, 5632 x 2048 at 256 rows 124 against 232).  The bits are the same.
     bool few_rows = M <= 16 * FR_MAX_MT;
     if (!few_rows && M <= 256) {
@@ -1796,7 +1796,10 @@ int tl_linear_tile(const void* a, const void* w, void* out, const float* residua
       const bool small_tiles = (double)ceil_div64(small_t, 256) / (4 * 0.6) < (double)ceil_div64(big_t, 256);
       const double tiled_us = (K / 2048.0) * (small_tiles ? 87.0 * (small_t > 352 ? small_t / 352.0 : 1.0)
                                                           : 204.0 * (double)ceil_div64(big_t, 256));
-      few_rows = 0.62 * mts * ((double)N * K / 1e6) + 8.0 < tiled_us;
+      // (a long inner size leaves LDS for the block sums of one or two row tiles a workgroup only, and the
+      // weights are then fetched once per row tile: 14336 x 4096 at 256 rows 876 us against 657)
+      const double per_tile = tiles_wg >= 4 ? 0.66 : (tiles_wg >= 2 ? 0.8 : 0.98);
+      few_rows = per_tile * mts * ((double)N * K / 1e6) + 8.0 < tiled_us;
     }
     if (few_rows && vec && rows_smem <= 96 * 1024) {
       static bool configured = false;
