@@ -1770,7 +1770,7 @@ int tl_linear_tile(const void* a, const void* w, void* out, const float* residua
     const int mts = (M + 15) / 16;
     // One row tile: 8 columns a workgroup where that still is one round of workgroups over the 256
     // compute units (a workgroup fills a compute unit: more than 256 of them would run in two rounds).
-    // More row tiles (17 to 64 rows): whole matrix tiles of 16 columns, and the row tiles shared out
+    // More row tiles (17 to 64 rows, up to 256 by the estimate below): whole matrix tiles of 16 columns, and the row tiles shared out
     // over as many groups of workgroups (1, 2 or 4) as it takes to give every compute unit a
     // workgroup and to fit the block sums into LDS.
     int cols = (N + 7) / 8 <= 256 ? 8 : 16, groups = 1;
